@@ -1,0 +1,167 @@
+"""Writes tests/golden/*.npz from the reference implementation (CPU, this container only).
+
+Run once as ``python tests/golden/make_golden.py`` with the reference checkout at
+/root/reference.  It covers only what closed forms cannot pin:
+
+  * kfac_*.npz     multi-step KfacGradientMaker runs (orchestration, EMA state, MC sampling
+                   under a fixed seed) on the tiny MLP / CNN of the reference's test/conftest.py
+  * shampoo_*.npz  multi-step ShampooGradientMaker run (in-place ridge accumulation,
+                   power-iteration start vectors under a fixed seed)
+  * power_*.npz    ComputePower outputs for well- and ill-conditioned inputs
+
+The fixtures hold inputs and expected outputs only.
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+sys.path.insert(0, '/root/reference')
+import asdl  # noqa: E402
+from asdl.precondition import PreconditioningConfig, KfacGradientMaker, ShampooGradientMaker  # noqa: E402
+from asdl.precondition.shampoo import ComputePower  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def get_mlp(in_dim=5, hid=4, out=4):
+    return nn.Sequential(nn.Linear(in_dim, hid), nn.ReLU(), nn.Linear(hid, hid), nn.ReLU(), nn.Linear(hid, out))
+
+
+def get_cnn(in_dim=5, hid=4, out=4):
+    return nn.Sequential(nn.Conv2d(in_dim, hid, kernel_size=2), nn.ReLU(), nn.Conv2d(hid, hid, kernel_size=2),
+                         nn.ReLU(), nn.Flatten(), nn.Linear(hid * 2 * 2, out))
+
+
+def get_cnn2(in_dim=3, hid=6, out=5):
+    # padded / strided convolutions with bias, 8x8 inputs
+    return nn.Sequential(nn.Conv2d(in_dim, hid, 3, 1, 1), nn.ReLU(), nn.Conv2d(hid, hid, 3, 2, 1), nn.ReLU(),
+                         nn.Conv2d(hid, 8, 1, 2, 0, bias=False), nn.ReLU(), nn.Flatten(), nn.Linear(8 * 2 * 2, out))
+
+
+def state_arrays(model, prefix):
+    return {f'{prefix}{k}': v.detach().numpy().copy() for k, v in model.state_dict().items()}
+
+
+def run_kfac(tag, model, xs, ts, fisher_type, ema_decay, damping, seed=None, curv_interval=None, prec_interval=1):
+    out = {}
+    out.update(state_arrays(model, 'init/'))
+    config = PreconditioningConfig(data_size=xs[0].shape[0], damping=damping, ema_decay=ema_decay,
+                                   curvature_upd_interval=curv_interval, preconditioner_upd_interval=prec_interval)
+    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    for step, (x, t) in enumerate(zip(xs, ts)):
+        opt.zero_grad(set_to_none=True)
+        dummy_y = gm.setup_model_call(model, x)
+        gm.setup_loss_call(F.cross_entropy, dummy_y, t)
+        y, loss = gm.forward_and_backward()
+        out[f'step{step}/x'] = x.numpy()
+        out[f'step{step}/t'] = t.numpy()
+        out[f'step{step}/loss'] = loss.detach().numpy()
+        out[f'step{step}/y'] = y.detach().numpy()
+        for name, p in model.named_parameters():
+            out[f'step{step}/grad/{name}'] = p.grad.detach().numpy().copy()
+        for name, m in model.named_modules():
+            fisher = getattr(m, 'fisher', None)
+            if fisher is None or fisher.kron is None:
+                continue
+            for key in ['A', 'B', 'A_inv', 'B_inv']:
+                v = getattr(fisher.kron, key)
+                if v is not None:
+                    out[f'step{step}/kron/{name}/{key}'] = v.detach().numpy().copy()
+        opt.step()
+    np.savez_compressed(os.path.join(HERE, f'kfac_{tag}.npz'), **out)
+    print('wrote', tag, len(out))
+
+
+def run_shampoo(tag, model, xs, ts, damping, ema_decay, curv_interval, prec_interval, seed):
+    out = {}
+    out.update(state_arrays(model, 'init/'))
+    config = PreconditioningConfig(damping=damping, ema_decay=ema_decay, curvature_upd_interval=curv_interval,
+                                   preconditioner_upd_interval=prec_interval)
+    gm = ShampooGradientMaker(model, config)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    torch.manual_seed(seed)
+    for step, (x, t) in enumerate(zip(xs, ts)):
+        opt.zero_grad(set_to_none=True)
+        dummy_y = gm.setup_model_call(model, x)
+        gm.setup_loss_call(F.cross_entropy, dummy_y, t)
+        y, loss = gm.forward_and_backward()
+        out[f'step{step}/x'] = x.numpy()
+        out[f'step{step}/t'] = t.numpy()
+        out[f'step{step}/loss'] = loss.detach().numpy()
+        for name, p in model.named_parameters():
+            out[f'step{step}/grad/{name}'] = p.grad.detach().numpy().copy()
+        for i, prec in enumerate(gm.preconditioners):
+            for j, (s, pm) in enumerate(zip(prec.statistics, prec.preconditioners)):
+                out[f'step{step}/stat/{i}/{j}'] = s.numpy().copy()
+                out[f'step{step}/prec/{i}/{j}'] = pm.numpy().copy()
+        opt.step()
+    out['seed'] = np.array(seed)
+    np.savez_compressed(os.path.join(HERE, f'shampoo_{tag}.npz'), **out)
+    print('wrote shampoo', tag, len(out))
+
+
+def run_power():
+    out = {}
+    g = torch.Generator().manual_seed(7)
+    cases = {}
+    X = torch.randn(64, 24, generator=g)
+    cases['wellcond_p4'] = (X.T @ X / 64, 4, 1e-6)
+    X = torch.randn(6, 24, generator=g)
+    cases['rankdef_p4'] = (X.T @ X / 6, 4, 1e-6)
+    cases['rankdef_p4_eps12'] = (X.T @ X / 6, 4, 1e-12)
+    X = torch.randn(40, 16, generator=g)
+    cases['wellcond_p2'] = (X.T @ X, 2, 1e-4)
+    cases['wellcond_p8'] = (X.T @ X, 8, 1e-6)
+    cases['tiny_init'] = (1e-12 * torch.eye(12) + 1e-3 * torch.diag(torch.rand(12, generator=g)), 4, 1e-6)
+    for seed, (name, (mat, p, eps)) in enumerate(cases.items()):
+        torch.manual_seed(100 + seed)
+        v0 = torch.rand(mat.shape[0]) * 2 - 1          # the draw PowerIter makes first
+        torch.manual_seed(100 + seed)
+        m = mat.clone()
+        root = ComputePower(m, p, ridge_epsilon=eps)
+        out[f'{name}/in'] = mat.numpy()
+        out[f'{name}/p'] = np.array(p)
+        out[f'{name}/eps'] = np.array(eps)
+        out[f'{name}/v0'] = v0.numpy()
+        out[f'{name}/root'] = root.numpy()
+        out[f'{name}/mat_after'] = m.numpy()
+    np.savez_compressed(os.path.join(HERE, 'power.npz'), **out)
+    print('wrote power', len(out))
+
+
+def main():
+    torch.manual_seed(0)
+    bs = 8
+    xs = [torch.randn(bs, 5) for _ in range(3)]
+    ts = [torch.randint(4, (bs,)) for _ in range(3)]
+    for fisher_type, seed in [('fisher_emp', None), ('fisher_mc', 1)]:
+        for ema in [-1, 0.3]:
+            torch.manual_seed(11)
+            run_kfac(f'mlp_{fisher_type}_ema{ema}', get_mlp(), xs, ts, fisher_type, ema, 1e-2, seed=seed)
+    xs = [torch.randn(bs, 5, 4, 4) for _ in range(3)]
+    for fisher_type, seed in [('fisher_emp', None), ('fisher_mc', 1)]:
+        torch.manual_seed(12)
+        run_kfac(f'cnn_{fisher_type}_ema-1', get_cnn(), xs, ts, fisher_type, -1, 1e-2, seed=seed)
+    xs = [torch.randn(bs, 3, 8, 8) for _ in range(4)]
+    ts = [torch.randint(5, (bs,)) for _ in range(4)]
+    torch.manual_seed(13)
+    run_kfac('cnn2_fisher_emp_ema0.5_int2', get_cnn2(), xs, ts, 'fisher_emp', 0.5, 1e-3, curv_interval=1, prec_interval=2)
+    torch.manual_seed(14)
+    run_kfac('cnn2_fisher_emp_ema-1_int2', get_cnn2(), xs, ts, 'fisher_emp', -1, 1e-3, prec_interval=2)
+
+    xs = [torch.randn(bs, 5) for _ in range(4)]
+    ts = [torch.randint(4, (bs,)) for _ in range(4)]
+    torch.manual_seed(15)
+    run_shampoo('mlp', get_mlp(), xs, ts, damping=1e-6, ema_decay=-1, curv_interval=1, prec_interval=2, seed=21)
+    torch.manual_seed(16)
+    run_shampoo('mlp_ema', get_mlp(), xs, ts, damping=1e-4, ema_decay=0.1, curv_interval=None, prec_interval=1, seed=22)
+    run_power()
+
+
+if __name__ == '__main__':
+    main()

@@ -1,0 +1,36 @@
+"""Tiny models shared by the oracle tests and the GPU end-to-end tests (the same shapes as
+the fixtures of the reference's test/conftest.py:11-25, plus a padded / strided CNN)."""
+import torch.nn as nn
+
+
+def get_mlp(in_dim=5, hid=4, out=4):
+    return nn.Sequential(nn.Linear(in_dim, hid), nn.ReLU(), nn.Linear(hid, hid), nn.ReLU(), nn.Linear(hid, out))
+
+
+def get_cnn(in_dim=5, hid=4, out=4):
+    return nn.Sequential(nn.Conv2d(in_dim, hid, kernel_size=2), nn.ReLU(), nn.Conv2d(hid, hid, kernel_size=2),
+                         nn.ReLU(), nn.Flatten(), nn.Linear(hid * 2 * 2, out))
+
+
+def get_cnn2(in_dim=3, hid=6, out=5):
+    return nn.Sequential(nn.Conv2d(in_dim, hid, 3, 1, 1), nn.ReLU(), nn.Conv2d(hid, hid, 3, 2, 1), nn.ReLU(),
+                         nn.Conv2d(hid, 8, 1, 2, 0, bias=False), nn.ReLU(), nn.Flatten(), nn.Linear(8 * 2 * 2, out))
+
+
+GOLDEN_KFAC = {
+    # tag: (model factory, fisher_type, ema_decay, damping, seed, curvature interval, preconditioner interval)
+    'mlp_fisher_emp_ema-1': (get_mlp, 'fisher_emp', -1, 1e-2, None, None, 1),
+    'mlp_fisher_emp_ema0.3': (get_mlp, 'fisher_emp', 0.3, 1e-2, None, None, 1),
+    'mlp_fisher_mc_ema-1': (get_mlp, 'fisher_mc', -1, 1e-2, 1, None, 1),
+    'mlp_fisher_mc_ema0.3': (get_mlp, 'fisher_mc', 0.3, 1e-2, 1, None, 1),
+    'cnn_fisher_emp_ema-1': (get_cnn, 'fisher_emp', -1, 1e-2, None, None, 1),
+    'cnn_fisher_mc_ema-1': (get_cnn, 'fisher_mc', -1, 1e-2, 1, None, 1),
+    'cnn2_fisher_emp_ema0.5_int2': (get_cnn2, 'fisher_emp', 0.5, 1e-3, None, 1, 2),
+    'cnn2_fisher_emp_ema-1_int2': (get_cnn2, 'fisher_emp', -1, 1e-3, None, None, 2),
+}
+
+GOLDEN_SHAMPOO = {
+    # tag: (damping, ema_decay, curvature interval, preconditioner interval)
+    'mlp': (1e-6, -1, 1, 2),
+    'mlp_ema': (1e-4, 0.1, None, 1),
+}

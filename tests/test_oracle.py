@@ -1,0 +1,277 @@
+"""Pins the CPU oracle: closed forms, invariants, library routines, brute force, and the golden
+runs written from the reference (tests/golden/make_golden.py)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from conftest import GOLDEN
+from models_small import GOLDEN_KFAC, GOLDEN_SHAMPOO, get_mlp
+from oracle import cpu_ref as R
+
+
+def relerr(a, b):
+    return float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-300))
+
+
+# ----------------------------------------------------------------- factors
+def test_linear_factors_closed_form():
+    torch.manual_seed(0)
+    a = torch.randn(3, 7, 11)
+    g = torch.randn(3, 7, 5)
+    A = R.linear_cov_kron_A(a)
+    B = R.linear_cov_kron_B(g)
+    a2 = a.reshape(-1, 11).double()
+    assert A.shape == (11, 11) and B.shape == (5, 5)
+    assert relerr(A, a2.T @ a2) < 1e-6
+    torch.testing.assert_close(A, A.T)
+    assert abs(float(A.trace()) - float((a ** 2).sum())) < 1e-3
+    assert relerr(B, g.reshape(-1, 5).double().T @ g.reshape(-1, 5).double()) < 1e-6
+
+
+def test_single_datum_kron_is_exact_fisher():
+    # test/grad_maker/test_fisher.py:152-156: for one datum kron(B, A) equals the weight block of
+    # the per-example-gradient outer product and the bias block equals B.
+    torch.manual_seed(1)
+    lin = nn.Linear(5, 4)
+    x = torch.randn(1, 5)
+    y = lin(x)
+    gy = torch.randn(1, 4)
+    gw, gb = torch.autograd.grad(y, [lin.weight, lin.bias], gy)
+    A = R.linear_cov_kron_A(x)
+    B = R.linear_cov_kron_B(gy)
+    torch.testing.assert_close(torch.outer(gw.flatten(), gw.flatten()), torch.kron(B, A))
+    torch.testing.assert_close(torch.outer(gb, gb), B)
+
+
+def _brute_im2col(x, kh, kw, sy, sx, ph, pw):
+    n, c, h, w = x.shape
+    ho = (h + 2 * ph - kh) // sy + 1
+    wo = (w + 2 * pw - kw) // sx + 1
+    out = torch.zeros(n, c * kh * kw, ho * wo, dtype=x.dtype)
+    for b in range(n):
+        for ci in range(c):
+            for ky in range(kh):
+                for kx in range(kw):
+                    for oy in range(ho):
+                        for ox in range(wo):
+                            iy, ix = oy * sy + ky - ph, ox * sx + kx - pw
+                            if 0 <= iy < h and 0 <= ix < w:
+                                out[b, (ci * kh + ky) * kw + kx, oy * wo + ox] = x[b, ci, iy, ix]
+    return out
+
+
+@pytest.mark.parametrize('k,s,p,hw', [((2, 2), (1, 1), (0, 0), (4, 4)), ((3, 3), (1, 1), (1, 1), (6, 5)),
+                                        ((3, 3), (2, 2), (1, 1), (7, 8)), ((1, 1), (2, 2), (0, 0), (6, 6)),
+                                        ((7, 7), (2, 2), (3, 3), (12, 12)), ((3, 2), (2, 1), (0, 1), (9, 6))])
+def test_im2col_vs_unfold_and_brute_force(k, s, p, hw):
+    torch.manual_seed(2)
+    x = torch.randn(2, 3, *hw)
+    col = R.im2col_2d(x, k, s, p)
+    torch.testing.assert_close(col, F.unfold(x, k, padding=p, stride=s))
+    torch.testing.assert_close(col, _brute_im2col(x, *k, *s, *p))
+    A = R.conv_cov_kron_A(x, k, s, p)
+    bf = _brute_im2col(x.double(), *k, *s, *p)
+    ref = sum(bf[i] @ bf[i].T for i in range(2)) / bf.shape[-1]
+    assert relerr(A, ref) < 1e-6
+
+
+def test_conv_B_not_divided_by_out_size():
+    torch.manual_seed(3)
+    g = torch.randn(2, 4, 3, 3)
+    B = R.conv_cov_kron_B(g)
+    ref = torch.zeros(4, 4, dtype=torch.float64)
+    for n in range(2):
+        for y in range(3):
+            for x in range(3):
+                v = g[n, :, y, x].double()
+                ref += torch.outer(v, v)
+    assert relerr(B, ref) < 1e-6
+
+
+def test_single_datum_conv_fisher_bias_block():
+    torch.manual_seed(4)
+    conv = nn.Conv2d(3, 4, 2)
+    x = torch.randn(1, 3, 4, 4)
+    y = conv(x)
+    gy = torch.randn_like(y)
+    gw, gb = torch.autograd.grad(y, [conv.weight, conv.bias], gy)
+    # sum over positions of per-position outer products: dW = sum_pos g_pos x_pos^T
+    col = R.im2col_2d(x, (2, 2), (1, 1), (0, 0))[0]
+    torch.testing.assert_close(gw.view(4, -1), gy.flatten(2)[0] @ col.T)
+    torch.testing.assert_close(gb, gy.sum(dim=(0, 2, 3)))
+
+
+# ----------------------------------------------------------------- damping, inverse, mvp
+def test_kron_damping_formula_and_special_cases():
+    torch.manual_seed(5)
+    X = torch.randn(20, 6)
+    Y = torch.randn(20, 3)
+    A, B = X.T @ X, Y.T @ Y
+    dA, dB = R.kron_damping(A, B, 0.04)
+    pi = ((A.trace() / 6) / (B.trace() / 3)) ** 0.5          # test_fisher.py:267-273
+    assert abs(dA - max(0.2 * float(pi), 1e-7)) < 1e-6 and abs(dB - max(0.2 / float(pi), 1e-7)) < 1e-6
+    assert abs(dA * dB - 0.04) < 1e-6
+    assert R.kron_damping(A, torch.zeros(3, 3), 0.04) == (0.04, 0.04)      # pi = inf
+    assert R.kron_damping(torch.zeros(6, 6), B, 0.04) == (0.04, 0.04)      # pi = 0
+    dA, dB = R.kron_damping(A * 1e-20, B, 1e-12)
+    assert dA == 1e-7                                                      # eps floor
+
+
+def test_cholesky_inv_identity_and_input_unchanged():
+    torch.manual_seed(6)
+    X = torch.randn(10, 30)
+    A = X @ X.T
+    A0 = A.clone()
+    inv = R.cholesky_inv(A, 0.5)
+    torch.testing.assert_close(A, A0)
+    Ad = A + 0.5 * torch.eye(10)
+    torch.testing.assert_close(Ad @ inv, torch.eye(10), atol=1e-4, rtol=0)
+    assert relerr(inv, torch.linalg.inv(Ad.double())) < 1e-5
+    with pytest.raises(torch.linalg.LinAlgError):
+        R.cholesky_inv(-torch.eye(4), 0.1)
+
+
+def test_kron_update_inv_skips_zero_factor():
+    A = torch.eye(3)
+    Ai, Bi = R.kron_update_inv(A, torch.zeros(2, 2), 0.1)
+    assert Bi is None and Ai is not None
+
+
+def test_kron_mvp_is_kronecker_inverse():
+    torch.manual_seed(7)
+    Ai = torch.randn(5, 5)
+    Ai = Ai @ Ai.T
+    Bi = torch.randn(3, 3)
+    Bi = Bi @ Bi.T
+    G = torch.randn(3, 5)
+    b = torch.randn(3)
+    w, bb = R.kron_mvp(Ai, Bi, G, b)
+    torch.testing.assert_close(w.flatten(), torch.kron(Bi, Ai) @ G.flatten(), atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(bb, Bi @ b)
+    conv_g = torch.randn(3, 5, 1, 1)
+    torch.testing.assert_close(R.kron_mvp(Ai, Bi, conv_g).flatten(), w.new_tensor(torch.kron(Bi, Ai) @ conv_g.flatten()),
+                               atol=1e-4, rtol=1e-4)
+
+
+# ----------------------------------------------------------------- Shampoo pieces
+def test_power_iter_converges_to_lambda_max():
+    torch.manual_seed(8)
+    X = torch.randn(50, 12).double()
+    S = X.T @ X
+    lam, iters = R.power_iter(S, torch.rand(12).double() * 2 - 1, error_tolerance=1e-12, num_iters=10000)
+    assert abs(float(lam) - float(torch.linalg.eigvalsh(S)[-1])) / float(lam) < 1e-6
+
+
+@pytest.mark.parametrize('p', [2, 4, 8])
+def test_compute_power_closed_form(p):
+    torch.manual_seed(9)
+    X = torch.randn(60, 10).double()
+    S = X.T @ X / 60
+    S0 = S.clone()
+    root, iters, err = R.compute_power(S, p, torch.rand(10).double() * 2 - 1, ridge_epsilon=1e-6)
+    lam = torch.linalg.eigvalsh(S0)[-1]
+    # ridge stays in the statistic (shampoo.py:498-499)
+    assert relerr(S, S0 + 1e-6 * lam * torch.eye(10).double()) < 1e-6
+    w, V = torch.linalg.eigh(S)
+    ref = V @ torch.diag(w ** (-1.0 / p)) @ V.T
+    assert relerr(root, ref) < 1e-5
+    assert relerr(torch.linalg.matrix_power(root, p) @ S, torch.eye(10).double()) < 1e-5
+    assert 0 < iters < 100
+
+
+def test_mat_power_generic_exponent():
+    torch.manual_seed(10)
+    M = torch.randn(4, 4).double() * 0.5
+    for p in [1, 2, 3, 4, 6, 8]:
+        assert relerr(R.mat_power(M, p), torch.linalg.matrix_power(M, p)) < 1e-12
+
+
+def test_compute_power_matches_reference_golden():
+    z = np.load(os.path.join(GOLDEN, 'power.npz'))
+    names = sorted({k.split('/')[0] for k in z.files})
+    assert len(names) >= 6
+    for name in names:
+        mat = torch.from_numpy(z[f'{name}/in']).clone()
+        root, iters, err = R.compute_power(mat, int(z[f'{name}/p']), torch.from_numpy(z[f'{name}/v0']),
+                                           ridge_epsilon=float(z[f'{name}/eps']))
+        torch.testing.assert_close(root, torch.from_numpy(z[f'{name}/root']), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(mat, torch.from_numpy(z[f'{name}/mat_after']), rtol=1e-6, atol=1e-12)
+
+
+def test_shampoo_statistics_and_precondition_closed_form():
+    torch.manual_seed(11)
+    G = torch.randn(4, 6)
+    stats = [torch.zeros(4, 4), torch.zeros(6, 6)]
+    R.shampoo_statistics(G, stats)
+    torch.testing.assert_close(stats[0], G @ G.T)
+    torch.testing.assert_close(stats[1], G.T @ G)
+    R.shampoo_statistics(G, stats, ema_decay=0.25)
+    torch.testing.assert_close(stats[0], G @ G.T)             # 0.75 S + 0.25 S
+    P0, P1 = torch.randn(4, 4), torch.randn(6, 6)
+    torch.testing.assert_close(R.shampoo_precondition(G, [P0, P1]), P0.T @ G @ P1)
+
+
+# ----------------------------------------------------------------- golden end-to-end runs
+def _load_model(factory, z):
+    model = factory()
+    sd = {k[len('init/'):]: torch.from_numpy(z[k]) for k in z.files if k.startswith('init/')}
+    model.load_state_dict(sd)
+    return model
+
+
+@pytest.mark.parametrize('tag', sorted(GOLDEN_KFAC))
+def test_kfac_oracle_matches_reference_golden(tag):
+    factory, fisher_type, ema, damping, seed, ci, pi = GOLDEN_KFAC[tag]
+    z = np.load(os.path.join(GOLDEN, f'kfac_{tag}.npz'))
+    model = _load_model(factory, z)
+    n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
+    x0 = torch.from_numpy(z['step0/x'])
+    orc = R.KfacOracle(model, data_size=x0.shape[0], damping=damping, ema_decay=ema, fisher_type=fisher_type,
+                       seed=seed, curvature_upd_interval=ci, preconditioner_upd_interval=pi)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    for step in range(n_steps):
+        opt.zero_grad(set_to_none=True)
+        x = torch.from_numpy(z[f'step{step}/x'])
+        t = torch.from_numpy(z[f'step{step}/t'])
+        y, loss = orc.forward_and_backward(x, t)
+        torch.testing.assert_close(loss, torch.from_numpy(z[f'step{step}/loss']), rtol=1e-5, atol=1e-6)
+        for name, p in model.named_parameters():
+            ref = torch.from_numpy(z[f'step{step}/grad/{name}'])
+            assert relerr(p.grad, ref) < 2e-4, (tag, step, name, relerr(p.grad, ref))
+        for key in z.files:
+            if not key.startswith(f'step{step}/kron/'):
+                continue
+            _, _, mname, which = key.split('/')
+            got = getattr(orc, which).get(mname)
+            assert got is not None, key
+            assert relerr(got, torch.from_numpy(z[key])) < 2e-4, (tag, key)
+        opt.step()
+
+
+@pytest.mark.parametrize('tag', sorted(GOLDEN_SHAMPOO))
+def test_shampoo_oracle_matches_reference_golden(tag):
+    damping, ema, ci, pi = GOLDEN_SHAMPOO[tag]
+    z = np.load(os.path.join(GOLDEN, f'shampoo_{tag}.npz'))
+    model = _load_model(get_mlp, z)
+    orc = R.ShampooOracle(model, damping=damping, ema_decay=ema, curvature_upd_interval=ci,
+                          preconditioner_upd_interval=pi)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    torch.manual_seed(int(z['seed']))
+    n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
+    for step in range(n_steps):
+        opt.zero_grad(set_to_none=True)
+        x = torch.from_numpy(z[f'step{step}/x'])
+        t = torch.from_numpy(z[f'step{step}/t'])
+        orc.forward_and_backward(x, t)
+        for i in range(len(orc.params)):
+            for j in range(2):
+                torch.testing.assert_close(orc.stats[i][j], torch.from_numpy(z[f'step{step}/stat/{i}/{j}']),
+                                           rtol=1e-4, atol=1e-12)
+                assert relerr(orc.precs[i][j], torch.from_numpy(z[f'step{step}/prec/{i}/{j}'])) < 1e-4
+        for name, p in model.named_parameters():
+            assert relerr(p.grad, torch.from_numpy(z[f'step{step}/grad/{name}'])) < 1e-4, (tag, step, name)
+        opt.step()
