@@ -1,0 +1,165 @@
+// Shared device helpers for the gfx950 kernels: MFMA fragment types, the layout of a 32x32
+// accumulator tile, LDS transpose reads, and the symmetric epilogue used by both SYRK kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/asdl_amd.h"
+
+namespace ak {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// v_mfma_f32_32x32x16_bf16: lane l feeds A[i = l%32][k = 8*(l/32) + e] and B[k][j = l%32],
+// e = 0..7; accumulator register r of lane l is C[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32].
+__device__ __forceinline__ floatx16 mfma_bf16(bf16x8 a, bf16x8 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+// v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32];
+// same accumulator layout.
+__device__ __forceinline__ floatx16 mfma_f32(float a, float b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane j receives element (j % 4) of the
+// 8 bytes addressed by lanes 4e + j/4, e = 0..3.  With lanes 4e..4e+3 pointing at row k0+e of a
+// [k][i] tile (16 consecutive i), lane j ends up with column i0 + j for k0..k0+3.
+__device__ __forceinline__ short4v lds_read_tr16(const void* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (short4v __attribute__((address_space(3)))*)(p));
+}
+
+__device__ __forceinline__ bf16x8 pack_bf16x8(short4v lo, short4v hi) {
+  short8v v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// Upper-triangular tile enumeration: linear id -> (ti, tj), ti <= tj < T, row-major.
+__device__ __forceinline__ void decode_upper_tile(int id, int T, int& ti, int& tj) {
+  int row = 0, len = T;
+  while (id >= len) { id -= len; ++row; --len; }
+  ti = row;
+  tj = row + id;
+}
+
+// Symmetric epilogue for one wave's accumulators of a BT x BT output tile at (ti, tj), ti <= tj.
+// acc[a][b] is the 32x32 MFMA tile at rows row0 + 32a, cols col0 + 32b of the WG tile.
+// Writes C[i][j] = beta*C[i][j] + alpha*acc and, off the diagonal tile, the mirror C[j][i].
+template <int TI, int TJ>
+__device__ __forceinline__ void syrk_epilogue(floatx16 (&acc)[TI][TJ], float* __restrict__ C, int64_t ldc,
+                                              int64_t d, int64_t gi0, int64_t gj0, bool diag_tile,
+                                              float alpha, float beta, int lane) {
+  const int g = lane >> 5, l32 = lane & 31;
+  const bool vec_mirror = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+#pragma unroll
+  for (int a = 0; a < TI; ++a) {
+#pragma unroll
+    for (int b = 0; b < TJ; ++b) {
+      const int64_t gj = gj0 + 32 * b + l32;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t gi = gi0 + 32 * a + 8 * q + 4 * g;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float x = alpha * acc[a][b][4 * q + e];
+          if (beta != 0.f && gj < d && gi + e < d) x += beta * C[(gi + e) * ldc + gj];
+          v[e] = x;
+        }
+        if (gj < d) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (gi + e < d) C[(gi + e) * ldc + gj] = v[e];
+          if (!diag_tile) {
+            if (vec_mirror && gi + 3 < d) {
+              floatx4 w = {v[0], v[1], v[2], v[3]};
+              *reinterpret_cast<floatx4*>(C + gj * ldc + gi) = w;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (gi + e < d) C[gj * ldc + gi + e] = v[e];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Split-K partial tile store / load in accumulator order: [(a,b,q)][thread] float4, coalesced.
+template <int TI, int TJ>
+__device__ __forceinline__ void store_partial(floatx16 (&acc)[TI][TJ], float* __restrict__ wsTile, int tid) {
+#pragma unroll
+  for (int a = 0; a < TI; ++a)
+#pragma unroll
+    for (int b = 0; b < TJ; ++b)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        floatx4 w = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]};
+        reinterpret_cast<floatx4*>(wsTile)[((a * TJ + b) * 4 + q) * 256 + tid] = w;
+      }
+}
+
+template <int TI, int TJ>
+__device__ __forceinline__ void add_partial(floatx16 (&acc)[TI][TJ], const float* __restrict__ wsTile, int tid) {
+#pragma unroll
+  for (int a = 0; a < TI; ++a)
+#pragma unroll
+    for (int b = 0; b < TJ; ++b)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        floatx4 w = reinterpret_cast<const floatx4*>(wsTile)[((a * TJ + b) * 4 + q) * 256 + tid];
+        acc[a][b][4 * q] += w[0];
+        acc[a][b][4 * q + 1] += w[1];
+        acc[a][b][4 * q + 2] += w[2];
+        acc[a][b][4 * q + 3] += w[3];
+      }
+}
+
+// Sums the split-K partials of every upper tile and applies the symmetric epilogue.
+// grid.x = number of upper tiles, 256 threads.
+template <int TI, int TJ>
+__global__ __launch_bounds__(256) void syrk_finalize_kernel(const float* __restrict__ ws, int nsplit, int T,
+                                                            float* __restrict__ C, int64_t ldc, int64_t d,
+                                                            float alpha, float beta) {
+  constexpr int BT = 64 * TI;
+  static_assert(TI == TJ, "square tiles");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave >> 1, wc = wave & 1;
+  int ti, tj;
+  decode_upper_tile(blockIdx.x, T, ti, tj);
+  const int ntiles = gridDim.x;
+  floatx16 acc[TI][TJ];
+#pragma unroll
+  for (int a = 0; a < TI; ++a)
+#pragma unroll
+    for (int b = 0; b < TJ; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  for (int s = 0; s < nsplit; ++s)
+    add_partial<TI, TJ>(acc, ws + (static_cast<size_t>(s) * ntiles + blockIdx.x) * (BT * BT), tid);
+  syrk_epilogue<TI, TJ>(acc, C, ldc, d, static_cast<int64_t>(ti) * BT + 32 * TI * wr,
+                        static_cast<int64_t>(tj) * BT + 32 * TJ * wc, ti == tj, alpha, beta, lane);
+}
+
+inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_ERR_LAUNCH; }
+
+// Split-K factor shared by the SYRK front ends: enough work groups to fill 256 CUs twice over
+// while every split still runs a useful number of k-steps.
+inline int pick_nsplit(int64_t ntiles, int64_t ksteps) {
+  int64_t want = (640 + ntiles - 1) / ntiles;
+  int64_t cap = ksteps / 8;
+  if (cap < 1) cap = 1;
+  int64_t s = want < cap ? want : cap;
+  if (s > 128) s = 128;
+  if (s < 1) s = 1;
+  return static_cast<int>(s);
+}
+
+}  // namespace ak

@@ -1,0 +1,205 @@
+// fp32 MFMA GEMM tile kernel shared by the dense products (precondition, Newton iteration)
+// and by the blocked Cholesky inverse, which needs triangular-aware contraction ranges.
+//
+// C[M,N] <- alpha * op(A) op(B) + beta * C, row-major, v_mfma_f32_32x32x2_f32 (true fp32 products,
+// fp32 accumulation).  One work group = 4 waves (2x2) = one 128x128 tile, BK = 16.
+// An operand whose contraction index is contiguous in memory is kept in LDS as [row][16 + 4] and
+// read as two ds_read_b128 per lane (8 k values); one whose row/column index is contiguous is kept
+// as [k][128 + 4] and read with conflict-free ds_read_b32.  No transposed copies are made.
+#pragma once
+#include "common.hpp"
+
+namespace ak {
+
+enum KMode {
+  K_FULL = 0,
+  K_LE_J = 1,     // contraction limited to k <= column tile (B^T lower triangular)
+  K_GE_J = 2,     // k >= column tile start (B lower triangular)
+  K_LE_I = 3,     // k <= row tile (A lower triangular)
+  K_GE_MAXIJ = 4  // k >= max(row tile, column tile) start (A^T A with A lower triangular)
+};
+enum TileMode {
+  TILE_ALL = 0,
+  TILE_LOWER = 1,         // only tiles with ti >= tj, only elements with i >= j are written
+  TILE_LOWER_MIRROR = 2   // tiles with ti >= tj, mirrored into the upper triangle
+};
+
+struct GemmParams {
+  const float* A;
+  const float* B;
+  float* C;
+  float* const* C_list;     // optional: per-batch output pointers (overrides C / sC)
+  int64_t lda, ldb, ldc;
+  int64_t sA, sB, sC;       // batch strides in elements
+  int M, N, K;
+  int transA, transB;
+  float alpha, beta;
+  int kmode, tile_mode;
+  const int* active;        // optional per-batch flags: batch z runs only if active[z*active_stride] != 0
+  int active_stride;
+};
+
+constexpr int GBT = 128, GBK = 16;
+constexpr int G_KC_STRIDE = GBK + 4;    // [row][k] layout
+constexpr int G_IC_STRIDE = GBT + 4;    // [k][row] layout
+constexpr int G_PANEL = GBT * G_KC_STRIDE > GBK * G_IC_STRIDE ? GBT * G_KC_STRIDE : GBK * G_IC_STRIDE;
+
+// Loads this thread's two 16-byte chunks of a 128 x 16 operand panel.
+//  kcontig: memory rows are the 128 tile rows, 16 k values contiguous.
+//  else   : memory rows are the 16 k values, 128 tile rows contiguous.
+__device__ __forceinline__ void gemm_fetch(floatx4 (&reg)[2], const float* __restrict__ P, int64_t ld, bool kcontig,
+                                           int r0, int r_end, int k0, int k_end, bool vec_ok, int tid) {
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int c = tid + 256 * u;
+    int outer, inner, o_end, i_end;
+    if (kcontig) { outer = r0 + (c >> 2); inner = k0 + 4 * (c & 3); o_end = r_end; i_end = k_end; }
+    else { outer = k0 + (c >> 5); inner = r0 + 4 * (c & 31); o_end = k_end; i_end = r_end; }
+    floatx4 v = {0.f, 0.f, 0.f, 0.f};
+    if (outer < o_end && inner < i_end) {
+      const float* src = P + static_cast<int64_t>(outer) * ld + inner;
+      if (vec_ok && inner + 4 <= i_end) {
+        v = *reinterpret_cast<const floatx4*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (inner + e < i_end) v[e] = src[e];
+      }
+    }
+    reg[u] = v;
+  }
+}
+
+__device__ __forceinline__ void gemm_stash(const floatx4 (&reg)[2], float* __restrict__ lds, bool kcontig, int tid) {
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int c = tid + 256 * u;
+    const int off = kcontig ? (c >> 2) * G_KC_STRIDE + 4 * (c & 3) : (c >> 5) * G_IC_STRIDE + 4 * (c & 31);
+    *reinterpret_cast<floatx4*>(lds + off) = reg[u];
+  }
+}
+
+// Reads the 8 k values (k = 8g + m) of tile row `row` for this lane.
+__device__ __forceinline__ void gemm_frag(float (&f)[8], const float* __restrict__ lds, bool kcontig, int row, int g) {
+  if (kcontig) {
+    const floatx4* q = reinterpret_cast<const floatx4*>(lds + row * G_KC_STRIDE + 8 * g);
+    const floatx4 lo = q[0], hi = q[1];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+  } else {
+#pragma unroll
+    for (int m = 0; m < 8; ++m) f[m] = lds[(8 * g + m) * G_IC_STRIDE + row];
+  }
+}
+
+static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(16))) float lds[2][2][G_PANEL];
+  const int z = blockIdx.z;
+  if (p.active != nullptr && p.active[static_cast<int64_t>(z) * p.active_stride] == 0) return;
+  const int tj = blockIdx.x, ti = blockIdx.y;
+  if (p.tile_mode != TILE_ALL && ti < tj) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave >> 1, wc = wave & 1, g = lane >> 5, l32 = lane & 31;
+
+  int kbeg = 0, kend = p.K;
+  switch (p.kmode) {
+    case K_LE_J: kend = min(p.K, (tj + 1) * GBT); break;
+    case K_GE_J: kbeg = tj * GBT; break;
+    case K_LE_I: kend = min(p.K, (ti + 1) * GBT); break;
+    case K_GE_MAXIJ: kbeg = max(ti, tj) * GBT; break;
+    default: break;
+  }
+  const float* __restrict__ A = p.A + static_cast<int64_t>(z) * p.sA;
+  const float* __restrict__ B = p.B + static_cast<int64_t>(z) * p.sB;
+  float* __restrict__ C = p.C_list != nullptr ? p.C_list[z] : p.C + static_cast<int64_t>(z) * p.sC;
+  const bool a_kc = (p.transA == 0), b_kc = (p.transB != 0);
+  const bool a_vec = (p.lda % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
+  const bool b_vec = (p.ldb % 4 == 0) && ((reinterpret_cast<uintptr_t>(B) & 15) == 0);
+  const int i0 = ti * GBT, j0 = tj * GBT;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  const int nk = kbeg < kend ? (kend - kbeg + GBK - 1) / GBK : 0;
+  floatx4 ra[2], rb[2];
+  if (nk > 0) {
+    gemm_fetch(ra, A, p.lda, a_kc, i0, p.M, kbeg, kend, a_vec, tid);
+    gemm_fetch(rb, B, p.ldb, b_kc, j0, p.N, kbeg, kend, b_vec, tid);
+    gemm_stash(ra, lds[0][0], a_kc, tid);
+    gemm_stash(rb, lds[0][1], b_kc, tid);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) {
+      const int k0 = kbeg + (kt + 1) * GBK;
+      gemm_fetch(ra, A, p.lda, a_kc, i0, p.M, k0, kend, a_vec, tid);
+      gemm_fetch(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, b_vec, tid);
+    }
+    float fa[2][8], fb[2][8];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) gemm_frag(fa[a], lds[buf][0], a_kc, 64 * wr + 32 * a + l32, g);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) gemm_frag(fb[b], lds[buf][1], b_kc, 64 * wc + 32 * b + l32, g);
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) acc[a][b] = mfma_f32(fa[a][m], fb[b][m], acc[a][b]);
+    if (kt + 1 < nk) {
+      gemm_stash(ra, lds[buf ^ 1][0], a_kc, tid);
+      gemm_stash(rb, lds[buf ^ 1][1], b_kc, tid);
+    }
+    __syncthreads();
+  }
+
+  const bool lower_only = (p.tile_mode == TILE_LOWER);
+  const bool mirror = (p.tile_mode == TILE_LOWER_MIRROR) && (ti != tj);
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int gj = j0 + 64 * wc + 32 * b + l32;
+      if (gj >= p.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gi = i0 + 64 * wr + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (gi >= p.M) continue;
+        if (lower_only && gi < gj) continue;
+        float v = p.alpha * acc[a][b][r];
+        float* dst = C + static_cast<int64_t>(gi) * p.ldc + gj;
+        if (p.beta != 0.f) v += p.beta * *dst;
+        *dst = v;
+        if (mirror) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
+      }
+    }
+}
+
+inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
+  if (p.M <= 0 || p.N <= 0 || batch <= 0) return AK_OK;
+  dim3 grid((p.N + GBT - 1) / GBT, (p.M + GBT - 1) / GBT, batch);
+  hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, p);
+  return check_launch();
+}
+
+inline GemmParams make_gemm(int transA, int transB, int M, int N, int K, float alpha, const float* A, int64_t lda,
+                            const float* B, int64_t ldb, float beta, float* C, int64_t ldc) {
+  GemmParams p;
+  p.A = A; p.B = B; p.C = C; p.C_list = nullptr;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.sA = p.sB = p.sC = 0;
+  p.M = M; p.N = N; p.K = K;
+  p.transA = transA; p.transB = transB;
+  p.alpha = alpha; p.beta = beta;
+  p.kmode = K_FULL; p.tile_mode = TILE_ALL;
+  p.active = nullptr; p.active_stride = 0;
+  return p;
+}
+
+}  // namespace ak

@@ -1,0 +1,241 @@
+"""torch.Tensor front ends of the C ABI (include/asdl_amd.h).
+
+Every function takes tensors that live on a ROCm device, passes raw device pointers and the
+calling thread's current HIP stream to libasdl_amd.so, and returns without synchronising.
+There is no CPU path: a CPU tensor raises.
+"""
+import ctypes
+import threading
+
+import torch
+
+from . import _lib
+
+AK_F32, AK_BF16 = 0, 1
+
+_ws_lock = threading.Lock()
+_workspaces = {}
+_ptr_cache = {}
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError('asdl_amd kernels run on a ROCm device only; got a tensor on '
+                               f'{t.device}. There is no CPU fallback.')
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float32:
+        return AK_F32
+    if t.dtype == torch.bfloat16:
+        return AK_BF16
+    raise TypeError(f'unsupported dtype {t.dtype}: the kernels take float32 or bfloat16 inputs')
+
+
+def workspace(nbytes, device):
+    """A cached scratch buffer per (device, stream); grows geometrically, never shrinks.
+    Kernels on one stream run in order, so consecutive calls may share it."""
+    if nbytes <= 0:
+        return None, 0
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream().cuda_stream)
+    with _ws_lock:
+        buf = _workspaces.get(key)
+        if buf is None or buf.numel() < nbytes:
+            size = max(nbytes, 1 << 20)
+            if buf is not None:
+                size = max(size, int(buf.numel() * 1.5))
+            buf = torch.empty(size, dtype=torch.uint8, device=device)
+            _workspaces[key] = buf
+    return buf, buf.numel()
+
+
+def _ws_args(nbytes, device):
+    buf, size = workspace(nbytes, device)
+    if buf is None:
+        return ctypes.c_void_p(0), 0, None
+    return ctypes.c_void_p(buf.data_ptr()), size, buf
+
+
+def device_ptr_array(tensors):
+    """int64 device tensor holding the data pointers of ``tensors`` (cached by pointer tuple)."""
+    ptrs = tuple(t.data_ptr() for t in tensors)
+    dev = tensors[0].device
+    key = (dev.index, ptrs)
+    arr = _ptr_cache.get(key)
+    if arr is None:
+        if len(_ptr_cache) > 4096:
+            _ptr_cache.clear()
+        arr = torch.tensor(ptrs, dtype=torch.int64).to(dev)
+        _ptr_cache[key] = arr
+    return arr
+
+
+# ------------------------------------------------------------------------------ factors
+def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
+    """out <- beta*out + alpha * x^T x for x = [M, d] (rows may be strided, columns contiguous)."""
+    _require_gpu(x, out)
+    if x.ndim != 2:
+        raise ValueError(f'x.ndim has to be 2. Got {x.ndim}.')
+    if x.stride(1) != 1 and x.shape[1] > 1:
+        x = x.contiguous()
+    M, d = x.shape
+    ldx = x.stride(0) if M > 1 else max(d, x.stride(0))
+    if ldx < d:
+        x = x.contiguous()
+        ldx = d
+    if out is None:
+        out = torch.empty(d, d, dtype=torch.float32, device=x.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
+        raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
+    lib = _lib.load()
+    need = lib.ak_syrk_tn_ws_bytes(M, d)
+    ws, ws_bytes, keep = _ws_args(need, x.device)
+    rc = lib.ak_syrk_tn(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), M, d, ldx, alpha, beta,
+                        ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_syrk_tn')
+    return out
+
+
+def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
+    """out <- beta*out + alpha * sum_{n,pos} patch patch^T for x = [N, C, H, W] (NCHW contiguous),
+    patches ordered (c, ky, kx); no division by the output size (fold it into alpha)."""
+    _require_gpu(x, out)
+    if x.ndim != 4:
+        raise ValueError(f'x.ndim has to be 4. Got {x.ndim}.')
+    x = x.contiguous()
+    N, C, H, W = x.shape
+    kh, kw = kernel_size
+    sh, sw = stride
+    ph, pw = padding
+    d = C * kh * kw
+    if out is None:
+        out = torch.empty(d, d, dtype=torch.float32, device=x.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
+        raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
+    lib = _lib.load()
+    need = lib.ak_conv_syrk_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)
+    ws, ws_bytes, keep = _ws_args(need, x.device)
+    rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw, ph, pw,
+                          alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_conv_syrk')
+    return out
+
+
+def syrk_nt(x, out=None, alpha=1.0, beta=0.0):
+    """out <- beta*out + alpha * sum_n x_n x_n^T for x = [d, K] or [N, d, K] (K contiguous)."""
+    if x.ndim == 2:
+        x = x.unsqueeze(0)
+    if x.ndim != 3:
+        raise ValueError(f'x.ndim has to be 2 or 3. Got {x.ndim}.')
+    return conv_syrk(x.unsqueeze(2), (1, 1), (1, 1), (0, 0), out=out, alpha=alpha, beta=beta)
+
+
+# ------------------------------------------------------------------------------ damping / inverse
+def kron_damping(A_list, B_list, damping, eps=1e-7):
+    """Returns (lam [batch, 2] float32, nonzero [batch, 2] int32), both on the device."""
+    _require_gpu(*A_list, *B_list)
+    dev = A_list[0].device
+    batch = len(A_list)
+    for t in list(A_list) + list(B_list):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.ndim != 2 or t.shape[0] != t.shape[1]:
+            raise ValueError('factors have to be contiguous square float32 matrices')
+    dims = torch.tensor([[a.shape[0], b.shape[0]] for a, b in zip(A_list, B_list)], dtype=torch.int64).to(dev)
+    lam = torch.empty(batch, 2, dtype=torch.float32, device=dev)
+    nonzero = torch.empty(batch, 2, dtype=torch.int32, device=dev)
+    pa, pb = device_ptr_array(A_list), device_ptr_array(B_list)
+    rc = _lib.load().ak_kron_damping(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(pb.data_ptr()),
+                                     ctypes.c_void_p(dims.data_ptr()), batch, damping, eps,
+                                     ctypes.c_void_p(lam.data_ptr()), ctypes.c_void_p(nonzero.data_ptr()), _stream())
+    _lib.check(rc, 'ak_kron_damping')
+    return lam, nonzero
+
+
+def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1, info=None):
+    """outs[b] <- (mats[b] + lam[b*lam_stride] I)^-1 for same-size matrices; returns the device
+    ``info`` tensor (int32 [batch], 0 = ok, k > 0 = leading minor k not positive definite)."""
+    _require_gpu(*mats, *outs, lam, active)
+    d = mats[0].shape[0]
+    batch = len(mats)
+    dev = mats[0].device
+    for t in list(mats) + list(outs):
+        if t.dtype != torch.float32 or t.shape != (d, d) or not t.is_contiguous():
+            raise ValueError('matrices have to be contiguous float32 [d, d] tensors of one size')
+    if info is None:
+        info = torch.empty(batch, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    need = lib.ak_chol_inv_ws_bytes(d, batch)
+    ws, ws_bytes, keep = _ws_args(need, dev)
+    pa, po = device_ptr_array(mats), device_ptr_array(outs)
+    rc = lib.ak_chol_inv_batched(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(po.data_ptr()), d, batch,
+                                 ctypes.c_void_p(lam.data_ptr()), lam_stride,
+                                 ctypes.c_void_p(active.data_ptr()) if active is not None else ctypes.c_void_p(0),
+                                 active_stride, ctypes.c_void_p(info.data_ptr()), ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_chol_inv_batched')
+    return info
+
+
+def cholesky_inv(X, damping=1e-7):
+    """(X + damping I)^-1; raises torch.linalg.LinAlgError when X + damping I is not positive
+    definite (reads the device info word, i.e. synchronises)."""
+    _require_gpu(X)
+    lam = torch.full((1,), float(damping), dtype=torch.float32, device=X.device)
+    out = torch.empty_like(X)
+    info = chol_inv_batched([X.contiguous()], [out], lam)
+    k = int(info.item())
+    if k != 0:
+        raise torch.linalg.LinAlgError(
+            f'cholesky_inv: the leading minor of order {k} is not positive-definite')
+    return out
+
+
+# ------------------------------------------------------------------------------ products
+def gemm(A, B, out=None, transA=False, transB=False, alpha=1.0, beta=0.0):
+    """out <- alpha * op(A) op(B) + beta * out for float32 matrices with contiguous rows."""
+    _require_gpu(A, B, out)
+    for t in (A, B):
+        if t.dtype != torch.float32 or t.ndim != 2 or t.stride(1) != 1:
+            raise ValueError('gemm operands have to be float32 matrices with contiguous rows')
+    M = A.shape[1] if transA else A.shape[0]
+    K = A.shape[0] if transA else A.shape[1]
+    K2 = B.shape[1] if transB else B.shape[0]
+    N = B.shape[0] if transB else B.shape[1]
+    if K != K2:
+        raise ValueError(f'inner dimensions differ: {K} vs {K2}')
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=A.device)
+        beta = 0.0
+    if out.data_ptr() in (A.data_ptr(), B.data_ptr()):
+        raise ValueError('gemm cannot run in place')
+    rc = _lib.load().ak_gemm_f32(int(transA), int(transB), M, N, K, alpha, ctypes.c_void_p(A.data_ptr()),
+                                 max(A.stride(0), A.shape[1]), ctypes.c_void_p(B.data_ptr()),
+                                 max(B.stride(0), B.shape[1]), beta, ctypes.c_void_p(out.data_ptr()),
+                                 max(out.stride(0), N), 1, 0, 0, 0, _stream())
+    _lib.check(rc, 'ak_gemm_f32')
+    return out
+
+
+def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
+    """grad_w <- grad_scale * B_inv @ view(grad_w, [dB, dA]) @ A_inv, grad_b <- grad_scale * B_inv @ grad_b,
+    both in place."""
+    _require_gpu(B_inv, A_inv, grad_w, grad_b)
+    dB, dA = B_inv.shape[0], A_inv.shape[0]
+    if grad_w.numel() != dB * dA or not grad_w.is_contiguous() or grad_w.dtype != torch.float32:
+        raise ValueError('grad_w has to be a contiguous float32 tensor with dB * dA elements')
+    if grad_b is not None and (grad_b.numel() != dB or not grad_b.is_contiguous() or grad_b.dtype != torch.float32):
+        raise ValueError('grad_b has to be a contiguous float32 vector with dB elements')
+    lib = _lib.load()
+    ws, ws_bytes, keep = _ws_args(lib.ak_kron_precond_ws_bytes(dB, dA), grad_w.device)
+    rc = lib.ak_kron_precond(ctypes.c_void_p(B_inv.data_ptr()), ctypes.c_void_p(A_inv.data_ptr()),
+                             ctypes.c_void_p(grad_w.data_ptr()), dB, dA,
+                             ctypes.c_void_p(grad_b.data_ptr()) if grad_b is not None else ctypes.c_void_p(0),
+                             grad_scale, ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_kron_precond')
+    return grad_w, grad_b

@@ -1,0 +1,140 @@
+/*
+ * asdl_amd.h -- C ABI of the MI355X (gfx950) kernels behind the K-FAC / Shampoo
+ * curvature path of kazukiosawa/asdl.
+ *
+ * The reference has no FFI: its hot path is a chain of ATen calls made from Python.
+ * Each entry point below replaces one such chain; the comment above it cites the
+ * reference lines (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - Every pointer except `const char*` results is a DEVICE pointer unless stated.
+ *   - Matrices are row-major with an explicit leading dimension in elements.
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.  All work
+ *     is enqueued on that stream; no entry point synchronises the device.
+ *   - The caller owns every buffer, including workspaces.  Workspace sizes come from
+ *     the matching ak_*_ws_bytes() query.  Nothing here allocates or frees device memory.
+ *   - Return value: 0 ok; <0 bad argument (see ak_error_string).  Numerical failures
+ *     (non positive-definite input) are reported through a device `info` word, like
+ *     LAPACK's info, because they are only known once the stream has run.
+ *   - Thread safety: entry points keep no mutable global state and may be called from
+ *     any host thread (autograd hooks run on the engine's device thread).
+ */
+#ifndef ASDL_AMD_H
+#define ASDL_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AK_F32 0
+#define AK_BF16 1
+
+#define AK_OK 0
+#define AK_ERR_ARG -1        /* null pointer, negative size, unknown dtype */
+#define AK_ERR_WORKSPACE -2  /* workspace missing or too small */
+#define AK_ERR_UNSUPPORTED -3
+#define AK_ERR_LAUNCH -4     /* hipGetLastError() reported a launch failure */
+
+typedef void* ak_stream_t;
+
+int ak_version(void);
+const char* ak_error_string(int code);
+
+/* ---- Kronecker-factor statistics -------------------------------------------------- */
+
+/* C <- beta*C + alpha * X^T X, X = [M, d] row-major (leading dimension ldx), C = [d, d] fp32,
+ * full symmetric on exit (upper triangle computed, mirrored).  beta == 0 never reads C.
+ * Replaces Linear.cov_kron_A / cov_kron_B  (asdl/operations/linear.py:75-77, 87-89), the
+ * `.mul_(cov_scale)` and `results[key] += value` passes (asdl/operations/operation.py:133-137,
+ * 199-201, 264-266) and the EMA pre-scale Kron.mul_ (asdl/symmatrix.py:448-453), and the 2-D
+ * statistic G^T G of Shampoo (asdl/precondition/shampoo.py:331-339). */
+size_t ak_syrk_tn_ws_bytes(int64_t M, int64_t d);
+int ak_syrk_tn(const void* X, int dtype, int64_t M, int64_t d, int64_t ldx,
+               float alpha, float beta, float* C, int64_t ldc,
+               void* ws, size_t ws_bytes, ak_stream_t stream);
+
+/* A <- beta*A + alpha * sum_{n,oy,ox} p p^T with p the (c,ky,kx)-ordered patch of x at output
+ * position (oy,ox): the unfold is fused, the [n, c*kh*kw, h_out*w_out] tensor is never written.
+ * x = [N, C, H, W] contiguous NCHW, zero padding (ph,pw), stride (sh,sw), dilation 1, groups 1.
+ * A = [d, d] fp32 with d = C*kh*kw.  The caller folds 1/out_size into alpha.
+ * Replaces im2col_2d (asdl/utils.py:51-71) + Conv2d.cov_kron_A (asdl/operations/conv.py:80-88).
+ * With kh=kw=1, H=1, W=h_out*w_out it is sum_n G_n G_n^T for out_grads [N, C, hw], i.e.
+ * Conv2d.cov_kron_B (asdl/operations/conv.py:99-103), and with N=1 it is X X^T for a row-major
+ * [d, M] matrix (Shampoo's G G^T, asdl/precondition/shampoo.py:331-339). */
+size_t ak_conv_syrk_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W,
+                             int kh, int kw, int sh, int sw, int ph, int pw);
+int ak_conv_syrk(const void* x, int dtype, int64_t N, int64_t C, int64_t H, int64_t W,
+                 int kh, int kw, int sh, int sw, int ph, int pw,
+                 float alpha, float beta, float* A, int64_t lda,
+                 void* ws, size_t ws_bytes, ak_stream_t stream);
+
+/* ---- damping ---------------------------------------------------------------------- */
+
+/* For each pair b < batch: tr(A_b), tr(B_b), the pi split
+ *   pi = sqrt((trA/dA)/(trB/dB)); lamA = max(sqrt(damping)*pi, eps), lamB = max(sqrt(damping)/pi, eps)
+ *   (lamA = lamB = damping when pi is 0 or inf), and the all-zero test of each factor.
+ * A_list / B_list: device arrays of device pointers (dense, ld = dim).  dims: device int64 [batch,2].
+ * lam_out: device float [batch,2]; nonzero_out: device int [batch,2] (1 when the factor has a
+ * non-zero entry).  One launch, no host synchronisation.
+ * Replaces the head of Kron.update_inv (asdl/symmatrix.py:499-510, 516, 527) and
+ * Operation.cov_kron_damping (asdl/operations/operation.py:457-466). */
+int ak_kron_damping(const float* const* A_list, const float* const* B_list, const int64_t* dims,
+                    int batch, float damping, float eps, float* lam_out, int* nonzero_out,
+                    ak_stream_t stream);
+
+/* ---- damped inverse --------------------------------------------------------------- */
+
+/* out_b <- (A_b + lam_b I)^-1 for b < batch; all matrices d x d fp32 dense (ld = d); A_b is not
+ * modified.  Blocked Cholesky (LDS-resident diagonal blocks, fp32 MFMA panel/trailing updates),
+ * triangular inverse, and L^-T L^-1, all on `stream`.  lam: device float array with element
+ * stride lam_stride.  info: device int [batch]; 0 ok, k > 0 means the leading minor of order k is
+ * not positive definite (LAPACK potrf convention); out_b is then undefined.  If skip_flags is
+ * non-NULL (device int, stride skip_stride) matrices whose flag is 0 are left untouched
+ * (the reference skips all-zero factors).
+ * Replaces cholesky_inv (asdl/utils.py:91-96) as called from asdl/symmatrix.py:518, 529 and
+ * asdl/operations/operation.py:273-275. */
+size_t ak_chol_inv_ws_bytes(int64_t d, int batch);
+int ak_chol_inv_batched(const float* const* A_list, float* const* out_list, int64_t d, int batch,
+                        const float* lam, int lam_stride, const int* skip_flags, int skip_stride,
+                        int* info, void* ws, size_t ws_bytes, ak_stream_t stream);
+
+/* ---- dense fp32 products ---------------------------------------------------------- */
+
+/* C <- alpha * op(A) op(B) + beta * C, fp32 MFMA, row-major; op = identity (0) or transpose (1);
+ * C = [M, N], op(A) = [M, K], op(B) = [K, N].  batch > 1 strides all three by the given element
+ * strides.  Replaces the mm calls of Kron.mvp (asdl/symmatrix.py:536-548), the tensordot chain of
+ * Preconditioner.precondition (asdl/precondition/shampoo.py:351-367) and the matmuls of
+ * ComputePower / MatPower (asdl/precondition/shampoo.py:518-527, 561-586). */
+int ak_gemm_f32(int transA, int transB, int64_t M, int64_t N, int64_t K, float alpha,
+                const float* A, int64_t lda, const float* B, int64_t ldb, float beta,
+                float* C, int64_t ldc, int batch, int64_t strideA, int64_t strideB, int64_t strideC,
+                ak_stream_t stream);
+
+/* G <- grad_scale * Binv G Ainv (G = [dB, dA] in place), bias <- grad_scale * Binv bias when
+ * bias != NULL.  ws holds the [dB, dA] intermediate.  Replaces Kron.mvp(use_inv, inplace)
+ * (asdl/symmatrix.py:536-548) and the grad_scale pre-multiply of
+ * NaturalGradientMaker._precondition_module (asdl/precondition/natural_gradient.py:535-538). */
+size_t ak_kron_precond_ws_bytes(int64_t dB, int64_t dA);
+int ak_kron_precond(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA,
+                    float* bias, float grad_scale, void* ws, size_t ws_bytes, ak_stream_t stream);
+
+/* ---- Shampoo inverse p-th root ---------------------------------------------------- */
+
+/* out <- (S + r I)^(-1/p), r = ridge_eps * lambda_max(S), by power iteration from start vector v0
+ * followed by the coupled Newton iteration; S (n x n fp32 dense) keeps the ridge on exit, as in
+ * the reference.  Convergence tests run on the device: once the error is below tol, or grows by
+ * more than 1.2x (then the previous root is kept), the remaining launches return immediately.
+ * stats: device float [4] = {lambda_max, power iterations, newton iterations, final error}.
+ * Replaces ComputePower / PowerIter / MatPower (asdl/precondition/shampoo.py:465-586). */
+size_t ak_inv_root_ws_bytes(int64_t n);
+int ak_inv_root_newton(float* S, int64_t n, int p, float ridge_eps, const float* v0,
+                       int max_power_iter, float power_tol, int max_iter, float tol,
+                       float* out, float* stats, void* ws, size_t ws_bytes, ak_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

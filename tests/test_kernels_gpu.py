@@ -1,0 +1,263 @@
+"""Parity of every HIP kernel (through the C ABI) with the CPU oracle on identical seeded inputs.
+
+Tolerances (relative Frobenius error): Kronecker factors 1e-5 for fp32 inputs, 5e-3 for bf16 inputs
+(the oracle is fed the same bf16-rounded values upcast to fp32; fp32 accumulation leaves only
+summation-order differences, so the bf16 cases are in fact held to 1e-5 as well); damped inverses
+1e-4 against the fp32 oracle where the matrix is well conditioned, otherwise both are compared with
+an fp64 inverse; preconditioned gradients 1e-3.
+"""
+import pytest
+import torch
+
+from oracle import cpu_ref as R
+
+pytestmark = pytest.mark.gpu
+
+TOL_FACTOR_F32 = 1e-5
+TOL_FACTOR_BF16 = 5e-3
+TOL_INV = 1e-4
+TOL_PRECOND = 1e-3
+
+
+def relerr(a, b):
+    a = a.detach().double().cpu()
+    b = b.detach().double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+
+
+@pytest.fixture(scope='module')
+def K():
+    from asdl_amd import kernels
+    return kernels
+
+
+def _inputs(shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(*shape, generator=g)
+    if dtype == torch.bfloat16:
+        x = x.to(torch.bfloat16)
+    return x
+
+
+# ------------------------------------------------------------------ syrk_tn (Linear A / B, Shampoo G^T G)
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('M,d', [(128, 784), (128, 512), (128, 10), (1, 5), (37, 129), (1000, 300), (4096, 64),
+                                 (70000, 40), (513, 1024)])
+def test_syrk_tn_matches_oracle(K, dtype, M, d):
+    x = _inputs((M, d), dtype, seed=M * 7 + d)
+    ref = R.linear_cov_kron_A(x.float().double())
+    print(f'syrk_tn dtype={dtype} M={M} d={d}', flush=True)
+    out = K.syrk_tn(x.cuda())
+    torch.cuda.synchronize()
+    tol = TOL_FACTOR_F32 if dtype == torch.float32 else TOL_FACTOR_BF16
+    assert relerr(out, ref) < min(tol, 1e-5)
+    assert torch.equal(out, out.T)
+
+
+def test_syrk_tn_alpha_beta_ema_and_strided_rows(K):
+    x = _inputs((300, 200), torch.float32, 3)
+    xs = x[:, :150]                                    # ldx = 200 > d = 150
+    C0 = _inputs((150, 150), torch.float32, 4)
+    C0 = C0 + C0.T
+    ref = 0.7 * C0.double() + 0.3 / 64 * R.linear_cov_kron_A(xs.double())
+    out = C0.cuda().clone()
+    K.syrk_tn(x.cuda()[:, :150], out=out, alpha=0.3 / 64, beta=0.7)
+    assert relerr(out, ref) < TOL_FACTOR_F32
+    # beta == 0 must not read the destination
+    out = torch.full((150, 150), float('nan'), device='cuda')
+    K.syrk_tn(x.cuda()[:, :150], out=out, alpha=1.0, beta=0.0)
+    assert relerr(out, R.linear_cov_kron_A(xs.double())) < TOL_FACTOR_F32
+
+
+def test_syrk_tn_3d_input_rows_flatten(K):
+    x = _inputs((4, 9, 33), torch.bfloat16, 5)
+    ref = R.linear_cov_kron_A(x.float().double())
+    out = K.syrk_tn(x.cuda().flatten(end_dim=1))
+    assert relerr(out, ref) < 1e-5
+
+
+def test_cpu_tensor_is_refused(K):
+    with pytest.raises(RuntimeError):
+        K.syrk_tn(torch.randn(4, 4))
+
+
+# ------------------------------------------------------------------ conv_syrk (fused unfold)
+CONV_CASES = [
+    # N, C, H, W, k, s, p
+    (2, 5, 4, 4, (2, 2), (1, 1), (0, 0)),          # the reference's test CNN
+    (3, 4, 4, 3, (2, 2), (1, 1), (0, 0)),
+    (4, 3, 32, 32, (3, 3), (1, 1), (1, 1)),        # CIFAR stem
+    (2, 16, 16, 16, (3, 3), (2, 2), (1, 1)),
+    (2, 3, 30, 30, (7, 7), (2, 2), (3, 3)),        # ImageNet stem geometry
+    (3, 64, 7, 7, (3, 3), (1, 1), (1, 1)),         # 7x7 maps, ragged rows
+    (2, 32, 14, 14, (1, 1), (1, 1), (0, 0)),       # 1x1 conv: flattened
+    (2, 32, 14, 14, (1, 1), (2, 2), (0, 0)),       # 1x1 stride 2 (downsample)
+    (2, 6, 9, 6, (3, 2), (2, 1), (0, 1)),          # asymmetric everything
+    (1, 150, 8, 8, (3, 3), (1, 1), (1, 1)),        # d = 1350: many tiles
+    (2, 20, 5, 70, (3, 3), (1, 1), (1, 1)),        # W_out > 64: column chunks
+    (2, 4, 10, 10, (3, 3), (3, 3), (0, 0)),        # stride 3: generic gather path
+]
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('case', CONV_CASES, ids=[str(c) for c in CONV_CASES])
+def test_conv_syrk_matches_oracle(K, dtype, case):
+    N, C, H, W, k, s, p = case
+    x = _inputs((N, C, H, W), dtype, seed=N + 10 * C + H)
+    ref = R.conv_cov_kron_A(x.float().double(), k, s, p)
+    out_size = ((H + 2 * p[0] - k[0]) // s[0] + 1) * ((W + 2 * p[1] - k[1]) // s[1] + 1)
+    print(f'conv_syrk dtype={dtype} case={case}', flush=True)
+    out = K.conv_syrk(x.cuda(), k, s, p, alpha=1.0 / out_size)
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5
+    assert torch.equal(out, out.T)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('N,C,hw', [(2, 4, (3, 3)), (8, 64, (7, 7)), (4, 130, (14, 14)), (2, 1000, (1, 1)),
+                                    (3, 17, (28, 28)), (1, 257, (5, 9))])
+def test_conv_B_factor_matches_oracle(K, dtype, N, C, hw):
+    g = _inputs((N, C, *hw), dtype, seed=C)
+    ref = R.conv_cov_kron_B(g.float().double())
+    print(f'conv B dtype={dtype} N={N} C={C} hw={hw}', flush=True)
+    out = K.syrk_nt(g.cuda().flatten(start_dim=2))
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5
+
+
+def test_conv_syrk_ema_accumulate(K):
+    x = _inputs((2, 8, 6, 6), torch.float32, 1)
+    A0 = R.conv_cov_kron_A(x, (3, 3), (1, 1), (1, 1))
+    x2 = _inputs((2, 8, 6, 6), torch.float32, 2)
+    ref = 0.9 * A0.double() + 0.1 * R.conv_cov_kron_A(x2.double(), (3, 3), (1, 1), (1, 1))
+    out = A0.cuda().clone()
+    K.conv_syrk(x2.cuda(), (3, 3), (1, 1), (1, 1), out=out, alpha=0.1 / 36, beta=0.9)
+    assert relerr(out, ref) < TOL_FACTOR_F32
+
+
+# ------------------------------------------------------------------ damping
+def test_kron_damping_matches_oracle(K):
+    torch.manual_seed(0)
+    pairs = []
+    for dA, dB in [(6, 3), (200, 17), (5, 5), (4, 4), (3, 2), (1000, 64)]:
+        X = torch.randn(2 * dA, dA)
+        Y = torch.randn(2 * dB, dB) * 0.1
+        pairs.append((X.T @ X, Y.T @ Y))
+    pairs[2] = (pairs[2][0], torch.zeros(5, 5))                      # pi = inf
+    pairs[3] = (torch.zeros(4, 4), pairs[3][1])                      # pi = 0
+    offdiag = torch.zeros(3, 3)
+    offdiag[0, 2] = offdiag[2, 0] = 1.0                              # zero diagonal, non-zero matrix
+    pairs[4] = (offdiag, pairs[4][1])
+    lam, nz = K.kron_damping([a.cuda() for a, _ in pairs], [b.cuda() for _, b in pairs], 1e-3)
+    lam, nz = lam.cpu(), nz.cpu()
+    for i, (A, B) in enumerate(pairs):
+        ra, rb = R.kron_damping(A, B, 1e-3)
+        assert abs(float(lam[i, 0]) - ra) <= 1e-5 * abs(ra), (i, lam[i], ra)
+        assert abs(float(lam[i, 1]) - rb) <= 1e-5 * abs(rb), (i, lam[i], rb)
+        assert bool(nz[i, 0]) == (not bool(torch.all(A == 0)))
+        assert bool(nz[i, 1]) == (not bool(torch.all(B == 0)))
+
+
+# ------------------------------------------------------------------ damped inverse
+@pytest.mark.parametrize('d', [1, 2, 10, 63, 64, 65, 128, 147, 200, 512, 576, 1000, 1152])
+def test_chol_inv_matches_oracle(K, d):
+    g = torch.Generator().manual_seed(d)
+    X = torch.randn(2 * d + 3, d, generator=g)
+    A = X.T @ X / (2 * d + 3)
+    lam = 0.05
+    ref32 = R.cholesky_inv(A, lam)
+    ref64 = torch.linalg.inv(A.double() + lam * torch.eye(d, dtype=torch.float64))
+    print(f'chol_inv d={d}', flush=True)
+    Ag = A.cuda()
+    out = K.cholesky_inv(Ag, lam)
+    torch.cuda.synchronize()
+    assert torch.equal(Ag.cpu(), A), 'input must be left unchanged'
+    assert relerr(out, ref32) < TOL_INV
+    assert relerr(out, ref64) < TOL_INV
+    resid = (A.double() + lam * torch.eye(d, dtype=torch.float64)) @ out.double().cpu() - torch.eye(d, dtype=torch.float64)
+    assert float(resid.abs().max()) < 1e-4
+    assert torch.equal(out, out.T)
+
+
+def test_chol_inv_rank_deficient_vs_fp64(K):
+    # d > M: conditioning, not the algorithm, limits accuracy; both fp32 results are judged against fp64
+    g = torch.Generator().manual_seed(11)
+    d, M = 384, 96
+    X = torch.randn(M, d, generator=g)
+    A = X.T @ X / M
+    lam = 1e-3
+    ref64 = torch.linalg.inv(A.double() + lam * torch.eye(d, dtype=torch.float64))
+    e_ref = relerr(R.cholesky_inv(A, lam), ref64)
+    e_hip = relerr(K.cholesky_inv(A.cuda(), lam), ref64)
+    print(f'rank deficient: oracle fp32 err {e_ref:.3e}, hip err {e_hip:.3e}', flush=True)
+    # cond(A + lam I) ~ 1e4: eps * cond ~ 1e-3 is the fp32 floor for any algorithm
+    assert e_hip < max(8 * e_ref, 1e-4)
+
+
+def test_chol_inv_batched_skip_and_info(K):
+    g = torch.Generator().manual_seed(5)
+    d = 96
+    mats = []
+    for _ in range(4):
+        X = torch.randn(200, d, generator=g)
+        mats.append((X.T @ X / 200).cuda())
+    mats[2] = -torch.eye(d).cuda()                                   # not positive definite
+    lam = torch.tensor([0.1, 0.2, 0.3, 0.4], device='cuda')
+    active = torch.tensor([1, 0, 1, 1], dtype=torch.int32, device='cuda')
+    outs = [torch.full((d, d), 7.0, device='cuda') for _ in range(4)]
+    info = K.chol_inv_batched(mats, outs, lam, active=active).cpu()
+    assert info[0] == 0 and info[3] == 0
+    assert info[2] == 1                                              # first leading minor fails
+    assert torch.all(outs[1] == 7.0)                                 # skipped: untouched
+    for b in (0, 3):
+        assert relerr(outs[b], R.cholesky_inv(mats[b].cpu(), float(lam[b]))) < TOL_INV
+    with pytest.raises(torch.linalg.LinAlgError):
+        K.cholesky_inv(mats[2], 0.5)
+    # failure in a later block is reported with its global index
+    A = torch.eye(100)
+    A[70, 70] = -5.0
+    info = K.chol_inv_batched([A.cuda()], [torch.empty(100, 100, device='cuda')], torch.zeros(1, device='cuda')).cpu()
+    assert int(info[0]) == 71
+
+
+# ------------------------------------------------------------------ products
+@pytest.mark.parametrize('tA', [False, True])
+@pytest.mark.parametrize('tB', [False, True])
+@pytest.mark.parametrize('M,N,K_', [(5, 7, 3), (130, 257, 65), (512, 384, 1000)])
+def test_gemm_matches_fp64(K, tA, tB, M, N, K_):
+    g = torch.Generator().manual_seed(M + N)
+    A = torch.randn((K_, M) if tA else (M, K_), generator=g)
+    B = torch.randn((N, K_) if tB else (K_, N), generator=g)
+    C0 = torch.randn(M, N, generator=g)
+    ref = 0.5 * (A.double().T if tA else A.double()) @ (B.double().T if tB else B.double()) - 2.0 * C0.double()
+    out = C0.cuda().clone()
+    K.gemm(A.cuda(), B.cuda(), out=out, transA=tA, transB=tB, alpha=0.5, beta=-2.0)
+    assert relerr(out, ref) < 1e-5
+
+
+@pytest.mark.parametrize('dB,dA,bias', [(4, 5, True), (10, 784, True), (512, 512, True), (64, 147, False),
+                                        (300, 1152, False)])
+def test_kron_precond_matches_oracle(K, dB, dA, bias):
+    g = torch.Generator().manual_seed(dB * 3 + dA)
+    Bi = torch.randn(dB, dB, generator=g)
+    Bi = Bi @ Bi.T / dB
+    Ai = torch.randn(dA, dA, generator=g)
+    Ai = Ai @ Ai.T / dA
+    G = torch.randn(dB, dA, generator=g)
+    b = torch.randn(dB, generator=g) if bias else None
+    if bias:
+        rw, rb = R.kron_mvp(Ai.double(), Bi.double(), G.double(), b.double())
+    else:
+        rw, rb = R.kron_mvp(Ai.double(), Bi.double(), G.double()), None
+    Gg = G.cuda()
+    bg = b.cuda() if bias else None
+    K.kron_precond(Bi.cuda(), Ai.cuda(), Gg, bg, grad_scale=1.0)
+    assert relerr(Gg, rw) < TOL_PRECOND
+    assert relerr(Gg, rw) < 1e-5
+    if bias:
+        assert relerr(bg, rb) < 1e-5
+    # conv-shaped gradient and grad_scale
+    if dA % 9 == 0:
+        G4 = G.view(dB, dA // 9, 3, 3).contiguous().cuda()
+        K.kron_precond(Bi.cuda(), Ai.cuda(), G4, None, grad_scale=0.5)
+        assert relerr(G4.view(dB, dA), 0.5 * rw) < 1e-5
