@@ -34,9 +34,9 @@ _SIGNATURES = {
                             c_ptr, c_i64, c_int, c_i64, c_i64, c_i64, c_ptr]),
     'ak_kron_precond_ws_bytes': (c_size, [c_i64, c_i64]),
     'ak_kron_precond': (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr, c_size, c_ptr]),
-    'ak_inv_root_ws_bytes': (c_size, [c_i64]),
-    'ak_inv_root_newton': (c_int, [c_ptr, c_i64, c_int, c_f32, c_ptr, c_int, c_f32, c_int, c_f32, c_ptr, c_ptr,
-                                   c_ptr, c_size, c_ptr]),
+    'ak_inv_root_ws_bytes': (c_size, [c_i64, c_int]),
+    'ak_inv_root_newton': (c_int, [c_ptr, c_i64, c_int, c_i64, c_int, c_f32, c_ptr, c_int, c_f32, c_int, c_f32,
+                                   c_ptr, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
 }
 
 
@@ -60,8 +60,6 @@ def load():
     import torch  # noqa: F401  (makes the process use the HIP runtime PyTorch ships)
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in _SIGNATURES.items():
-        if not hasattr(lib, name) and name.startswith('ak_inv_root'):
-            continue  # TEMP until newton.hip lands
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

@@ -1,0 +1,140 @@
+"""Hook engine: the ``extend`` context attaches one Operation per supported leaf module and calls
+it from a forward hook and from a hook on the gradient of the module's output
+(role of asdl/core.py:20-97, 130-244)."""
+from contextlib import contextmanager, nullcontext
+
+import torch
+import torch.nn as nn
+
+from .matrices import *
+from .operations import *
+from .operations import FWD_OPS, BWD_OPS
+from .utils import record_original_requires_grad
+
+_supported_module_classes = (nn.Linear, nn.Conv2d)
+
+__all__ = ['extend', 'no_centered_cov', 'module_wise_assignments', 'modules_to_assign']
+
+
+@contextmanager
+def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, stream=None) -> OperationContext:
+    handles = []
+    cxt = OperationContext(vectors=vectors)
+    use_stream = torch.cuda.is_available() and stream is not None
+
+    def stream_cxt():
+        return torch.cuda.stream(stream) if use_stream else nullcontext()
+
+    try:
+        for module, names in module_wise_assignments(model, *op_names, ignore_modules=ignore_modules, map_rule=map_rule):
+            if len(names) == 0:
+                continue
+            op_class = get_op_class(module)
+            if op_class is None:
+                continue
+            names = [n for n in names if n in op_class.supported_operations]
+            cxt.register_operation(module, op_class(module, names, model_for_kernel=model))
+            has_fwd = any(n in FWD_OPS for n in names)
+            has_bwd = any(n in BWD_OPS for n in names)
+            if not (has_fwd or has_bwd):
+                continue
+
+            def forward_hook(_module, in_data, out_data, _has_bwd=has_bwd):
+                with stream_cxt():
+                    cxt.call_operations_in_forward(_module, in_data[0].detach(), out_data.detach())
+                if _has_bwd and out_data.requires_grad:
+                    def grad_hook(grad, _m=_module):
+                        if not cxt.is_operation_registered(_m):
+                            return None          # context already closed
+                        with stream_cxt():
+                            cxt.call_operations_in_backward(_m, grad.detach())
+                        return None
+                    handles.append(out_data.register_hook(grad_hook))
+            handles.append(module.register_forward_hook(forward_hook))
+        if not cxt.is_operation_registered(model):
+            cxt.register_operation(model, Operation(model, []))
+        yield cxt
+    finally:
+        for handle in handles:
+            handle.remove()
+        cxt.clear_operations()
+
+
+def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, vectors=None, stream=None,
+                    calc_inv=False) -> OperationContext:
+    """Maps Fisher shapes to operations (asdl/core.py:83-97); only SHAPE_KRON has kernels here."""
+    if cvp:
+        raise NotImplementedError('covariance-vector products are not on this path')
+
+    def map_rule(shape):
+        if shape == SHAPE_KRON:
+            return OP_COV_KRON_INV if calc_inv else OP_COV_KRON
+        raise NotImplementedError(
+            f'Fisher shape "{shape}" has no MI355X kernel in this build; only "{SHAPE_KRON}" is supported. '
+            'Exclude such modules with PreconditioningConfig(ignore_modules=[...]).')
+    return extend(model, *shapes, ignore_modules=ignore_modules, map_rule=map_rule, vectors=vectors, stream=stream)
+
+
+def named_supported_modules(model):
+    for name, module in model.named_modules():
+        if isinstance(module, _supported_module_classes):
+            yield name, module
+
+
+def module_wise_assignments(model, *assign_rules, ignore_modules=None, map_rule=None, named=False):
+    """Yields (name,) module, [values] following the rule priorities of asdl/core.py:130-244:
+    module instance > name substring > module class > the bare string rules."""
+    if any(not isinstance(rule, (str, tuple)) for rule in assign_rules):
+        raise TypeError(f'every assign rule has to be {str} or {tuple}.')
+    ignore_modules = [] if ignore_modules is None else ignore_modules
+    if map_rule is None:
+        def map_rule(x):
+            return x
+
+    common, specified = [], {}
+    for rule in assign_rules:
+        if isinstance(rule, str):
+            common.append(rule)
+            continue
+        if len(rule) < 2:
+            raise ValueError(f'Tuple length has to be >= 2. Given: {rule}.')
+        key, values = rule[0], rule[1:]
+        if any(not isinstance(v, str) for v in values):
+            raise TypeError(f'All values have to be {str}. Given: {values}.')
+        if key in specified:
+            raise ValueError(f'({key}, _) is already assigned.')
+        specified[key] = list(values)
+
+    for name, module in named_supported_modules(model):
+        if any(module is m for m in ignore_modules if isinstance(m, nn.Module)):
+            continue
+        if any(isinstance(module, cls) for cls in ignore_modules if isinstance(cls, type)):
+            continue
+        if any(keyword in name for keyword in ignore_modules if isinstance(keyword, str)):
+            continue
+        requires_grad = False
+        for attr in ['weight', 'bias']:
+            param = getattr(module, attr, None)
+            if param is not None:
+                requires_grad = requires_grad or param.requires_grad
+                record_original_requires_grad(param)
+        if not requires_grad:
+            continue
+        info = (name, module) if named else (module,)
+        if module in specified:
+            values = specified[module]
+        elif any(isinstance(key, str) and key in name for key in specified):
+            values = specified[next(key for key in specified if isinstance(key, str) and key in name)]
+        elif module.__class__ in specified:
+            values = specified[module.__class__]
+        else:
+            if len(common) == 0:
+                continue
+            values = common
+        yield (*info, [map_rule(v) for v in values])
+
+
+def modules_to_assign(model, value, *assign_rules, ignore_modules=None, named=False):
+    for info in module_wise_assignments(model, *assign_rules, ignore_modules=ignore_modules, named=named):
+        if value in info[-1]:
+            yield (info[0], info[1]) if named else info[0]

@@ -1,0 +1,379 @@
+// Shampoo's inverse p-th root of a batch of same-size symmetric PSD statistics:
+//   out <- (S + r I)^(-1/p),  r = ridge_eps * lambda_max(S),
+// power iteration for lambda_max followed by the coupled Newton iteration, with every convergence
+// test evaluated on the device.  The host enqueues the maximum number of iterations; each kernel
+// first reads its matrix's `active` word and returns at once when that matrix has converged (or
+// stopped because its error grew by more than 1.2x, in which case the previous root is kept).
+// All products are fp32 MFMA GEMM tiles (gemm_f32.hpp); reductions are two-stage and deterministic.
+#include "gemm_f32.hpp"
+
+namespace ak {
+
+constexpr int RCHUNKS = 64;   // partial-reduction chunks per matrix
+
+struct RootState {
+  // per matrix, all device memory
+  float* sv;        // current eigenvalue estimate
+  float* nrm2;      // squared norm of the current power-iteration vector
+  float* err;       // current Newton error max|M - I|
+  float* zscale;
+  float* partial;   // [batch, RCHUNKS]
+  int* pi_active;   // power iteration still running
+  int* pi_iters;
+  int* active;      // Newton iteration still running
+  int* commit;      // last Newton step accepted
+  int* count;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+// grid (batch): v <- v0, norm, flags
+static __global__ __launch_bounds__(256) void root_init_kernel(RootState st, const float* __restrict__ v0,
+                                                               float* __restrict__ v, int64_t n) {
+  __shared__ float red[4];
+  const int z = blockIdx.x;
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += 256) {
+    const float x = v0[z * n + i];
+    v[z * n + i] = x;
+    s += x * x;
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    st.nrm2[z] = red[0] + red[1] + red[2] + red[3];
+    st.sv[z] = 0.f;
+    st.pi_active[z] = 1;
+    st.pi_iters[z] = 0;
+    st.active[z] = 0;
+    st.commit[z] = 0;
+    st.count[z] = 0;
+  }
+}
+
+// grid (ceil(n/4), batch): mv[row] = S[row,:] . v / ||v||   (one wave per row)
+static __global__ __launch_bounds__(256) void power_matvec_kernel(RootState st, const float* __restrict__ S,
+                                                                  int64_t strideS, const float* __restrict__ v,
+                                                                  float* __restrict__ mv, int64_t n) {
+  const int z = blockIdx.y;
+  if (st.pi_active[z] == 0) return;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= n) return;
+  const int lane = threadIdx.x & 63;
+  const float* __restrict__ Sr = S + z * strideS + row * n;
+  const float* __restrict__ vz = v + z * n;
+  float s = 0.f;
+  for (int64_t k = lane; k < n; k += 64) s += Sr[k] * vz[k];
+  s = wave_sum(s);
+  if (lane == 0) mv[z * n + row] = s / sqrtf(st.nrm2[z]);
+}
+
+// grid (batch): s_v = (v/||v||) . mv; error = |s_v - sv|; v <- mv
+static __global__ __launch_bounds__(256) void power_update_kernel(RootState st, float* __restrict__ v,
+                                                                  const float* __restrict__ mv, int64_t n, float tol,
+                                                                  int max_iters) {
+  __shared__ float red[8];
+  const int z = blockIdx.x;
+  if (st.pi_active[z] == 0) return;
+  const float inv_norm = 1.f / sqrtf(st.nrm2[z]);
+  float dot = 0.f, nn = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += 256) {
+    const float m = mv[z * n + i];
+    dot += v[z * n + i] * inv_norm * m;
+    nn += m * m;
+    v[z * n + i] = m;
+  }
+  dot = wave_sum(dot);
+  nn = wave_sum(nn);
+  if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = dot; red[4 + (threadIdx.x >> 6)] = nn; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float s_v = red[0] + red[1] + red[2] + red[3];
+    const float error = fabsf(s_v - st.sv[z]);
+    st.sv[z] = s_v;
+    st.nrm2[z] = red[4] + red[5] + red[6] + red[7];
+    const int it = st.pi_iters[z] + 1;
+    st.pi_iters[z] = it;
+    if (!(error > tol && it < max_iters)) st.pi_active[z] = 0;
+  }
+}
+
+// grid (RCHUNKS, batch): S += ridge I (in place), partial sum of squares of the ridged matrix
+static __global__ __launch_bounds__(256) void root_ridge_kernel(RootState st, float* __restrict__ S, int64_t strideS,
+                                                                int64_t n, float ridge_eps) {
+  __shared__ float red[4];
+  const int z = blockIdx.y;
+  float* __restrict__ Sz = S + z * strideS;
+  const float ridge = ridge_eps * st.sv[z];
+  const int64_t total = n * n;
+  float s = 0.f;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
+    float x = Sz[i];
+    if (i % (n + 1) == 0) {
+      x += ridge;
+      Sz[i] = x;
+    }
+    s += x * x;
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) st.partial[z * RCHUNKS + blockIdx.x] = red[0] + red[1] + red[2] + red[3];
+}
+
+// grid (batch)
+static __global__ void root_zscale_kernel(RootState st, int p) {
+  const int z = blockIdx.x;
+  if (threadIdx.x != 0) return;
+  float s = 0.f;
+  for (int c = 0; c < RCHUNKS; ++c) s += st.partial[z * RCHUNKS + c];
+  st.zscale[z] = (1.f + p) / (2.f * sqrtf(s));
+}
+
+// grid (RCHUNKS, batch): M = z S, root = z^(1/p) I, partial max |M - I|
+static __global__ __launch_bounds__(256) void root_start_kernel(RootState st, const float* __restrict__ S,
+                                                                int64_t strideS, float* __restrict__ M,
+                                                                float* __restrict__ root, int64_t strideR, int64_t n,
+                                                                int p) {
+  __shared__ float red[4];
+  const int z = blockIdx.y;
+  const float zs = st.zscale[z];
+  const float r0 = powf(zs, 1.0f / p);
+  const int64_t total = n * n;
+  float e = 0.f;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
+    const bool diag = (i % (n + 1) == 0);
+    const float m = zs * S[z * strideS + i];
+    M[z * total + i] = m;
+    root[z * strideR + i] = diag ? r0 : 0.f;
+    e = fmaxf(e, fabsf(m - (diag ? 1.f : 0.f)));
+  }
+  e = wave_max(e);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = e;
+  __syncthreads();
+  if (threadIdx.x == 0) st.partial[z * RCHUNKS + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// grid (batch)
+static __global__ void root_begin_kernel(RootState st, float tol, int max_iter) {
+  const int z = blockIdx.x;
+  if (threadIdx.x != 0) return;
+  float e = 0.f;
+  for (int c = 0; c < RCHUNKS; ++c) e = fmaxf(e, st.partial[z * RCHUNKS + c]);
+  st.err[z] = e;
+  st.active[z] = (e > tol && max_iter > 0) ? 1 : 0;
+}
+
+// grid (RCHUNKS, batch): T = (1 + 1/p) I - M / p
+static __global__ __launch_bounds__(256) void newton_tmp_kernel(RootState st, const float* __restrict__ M,
+                                                                float* __restrict__ T, int64_t n, int p) {
+  const int z = blockIdx.y;
+  if (st.active[z] == 0) return;
+  const int64_t total = n * n;
+  const float alpha = -1.0f / p;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
+    const bool diag = (i % (n + 1) == 0);
+    T[z * total + i] = (diag ? (1.f - alpha) : 0.f) + alpha * M[z * total + i];
+  }
+}
+
+// grid (RCHUNKS, batch): partial max |Mnew - I|
+static __global__ __launch_bounds__(256) void newton_err_kernel(RootState st, const float* __restrict__ Mnew, int64_t n) {
+  __shared__ float red[4];
+  const int z = blockIdx.y;
+  if (st.active[z] == 0) return;
+  const int64_t total = n * n;
+  float e = 0.f;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
+    const float m = Mnew[z * total + i];
+    const float d = fabsf(m - ((i % (n + 1) == 0) ? 1.f : 0.f));
+    e = (d > e || d != d) ? d : e;        // NaN propagates, as torch.max does
+  }
+  float o;
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) { o = __shfl_xor(e, s); e = (o > e || o != o) ? o : e; }
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = e;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float r = red[0];
+    for (int w = 1; w < 4; ++w) r = (red[w] > r || red[w] != red[w]) ? red[w] : r;
+    st.partial[z * RCHUNKS + blockIdx.x] = r;
+  }
+}
+
+// grid (batch): accept / reject the step and decide whether to go on
+static __global__ void newton_decide_kernel(RootState st, float tol, int max_iter) {
+  const int z = blockIdx.x;
+  if (threadIdx.x != 0) return;
+  st.commit[z] = 0;
+  if (st.active[z] == 0) return;
+  float e = st.partial[z * RCHUNKS];
+  for (int c = 1; c < RCHUNKS; ++c) {
+    const float x = st.partial[z * RCHUNKS + c];
+    e = (x > e || x != x) ? x : e;
+  }
+  const float err = st.err[z];
+  if (e > err * 1.2f) {          // diverging: keep the previous root (NaN compares false, like the reference)
+    st.active[z] = 0;
+    return;
+  }
+  st.commit[z] = 1;
+  st.err[z] = e;
+  const int c = st.count[z] + 1;
+  st.count[z] = c;
+  if (!(e > tol && c < max_iter)) st.active[z] = 0;
+}
+
+// grid (RCHUNKS, batch): root <- newroot, M <- Mnew where the step was accepted
+static __global__ __launch_bounds__(256) void newton_commit_kernel(RootState st, float* __restrict__ root,
+                                                                   int64_t strideR, const float* __restrict__ newroot,
+                                                                   float* __restrict__ M, const float* __restrict__ Mnew,
+                                                                   int64_t n) {
+  const int z = blockIdx.y;
+  if (st.commit[z] == 0) return;
+  const int64_t total = n * n;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
+    root[z * strideR + i] = newroot[z * total + i];
+    M[z * total + i] = Mnew[z * total + i];
+  }
+}
+
+// grid (batch)
+static __global__ void root_stats_kernel(RootState st, float* __restrict__ stats) {
+  const int z = blockIdx.x;
+  if (threadIdx.x != 0) return;
+  stats[4 * z] = st.sv[z];
+  stats[4 * z + 1] = static_cast<float>(st.pi_iters[z]);
+  stats[4 * z + 2] = static_cast<float>(st.count[z]);
+  stats[4 * z + 3] = st.err[z];
+}
+
+static size_t root_state_floats(int batch) { return static_cast<size_t>(batch) * (4 + RCHUNKS + 5) + 16; }
+
+}  // namespace ak
+
+extern "C" size_t ak_inv_root_ws_bytes(int64_t n, int batch) {
+  if (n <= 0 || batch <= 0) return 0;
+  // M, Mnew, newroot, four product buffers, two vectors, state
+  return (static_cast<size_t>(batch) * (7 * n * n + 2 * n) + ak::root_state_floats(batch)) * sizeof(float);
+}
+
+extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
+                                  const float* v0, int max_power_iter, float power_tol, int max_iter, float tol,
+                                  float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
+                                  ak_stream_t stream) {
+  using namespace ak;
+  if (S == nullptr || v0 == nullptr || out == nullptr || stats == nullptr || n < 2 || batch <= 0 || p < 1 ||
+      n > (1 << 20) || strideS < n * n || strideOut < n * n)
+    return AK_ERR_ARG;
+  if (ws == nullptr || ws_bytes < ak_inv_root_ws_bytes(n, batch)) return AK_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t nn = n * n;
+  float* w = static_cast<float*>(ws);
+  float* M = w;        w += batch * nn;
+  float* Mnew = w;     w += batch * nn;
+  float* newroot = w;  w += batch * nn;
+  float* buf[4];
+  for (int i = 0; i < 4; ++i) { buf[i] = w; w += batch * nn; }
+  float* v = w;        w += batch * n;
+  float* mv = w;       w += batch * n;
+  RootState st;
+  st.sv = w; w += batch;
+  st.nrm2 = w; w += batch;
+  st.err = w; w += batch;
+  st.zscale = w; w += batch;
+  st.partial = w; w += static_cast<size_t>(batch) * RCHUNKS;
+  st.pi_active = reinterpret_cast<int*>(w); w += batch;
+  st.pi_iters = reinterpret_cast<int*>(w); w += batch;
+  st.active = reinterpret_cast<int*>(w); w += batch;
+  st.commit = reinterpret_cast<int*>(w); w += batch;
+  st.count = reinterpret_cast<int*>(w); w += batch;
+
+  const dim3 gb(batch), gc(RCHUNKS, batch), b256(256);
+  hipLaunchKernelGGL(root_init_kernel, gb, b256, 0, s, st, v0, v, n);
+  const dim3 gmv(static_cast<unsigned>((n + 3) / 4), batch);
+  for (int it = 0; it < max_power_iter; ++it) {
+    hipLaunchKernelGGL(power_matvec_kernel, gmv, b256, 0, s, st, S, strideS, v, mv, n);
+    hipLaunchKernelGGL(power_update_kernel, gb, b256, 0, s, st, v, mv, n, power_tol, max_power_iter);
+  }
+  hipLaunchKernelGGL(root_ridge_kernel, gc, b256, 0, s, st, S, strideS, n, ridge_eps);
+  hipLaunchKernelGGL(root_zscale_kernel, gb, dim3(64), 0, s, st, p);
+  hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, M, out, strideOut, n, p);
+  hipLaunchKernelGGL(root_begin_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
+
+  const int N = static_cast<int>(n);
+  auto mm = [&](const float* A, int64_t sA, const float* B, int64_t sB, float* C, int64_t sC) {
+    GemmParams g = make_gemm(0, 0, N, N, N, 1.f, A, n, B, n, 0.f, C, n);
+    g.sA = sA; g.sB = sB; g.sC = sC;
+    g.active = st.active; g.active_stride = 1;
+    return launch_gemm(g, batch, s);
+  };
+  for (int it = 0; it < max_iter; ++it) {
+    float* T = buf[0];
+    hipLaunchKernelGGL(newton_tmp_kernel, gc, b256, 0, s, st, M, T, n, p);
+    int rc = mm(out, strideOut, T, nn, newroot, nn);            // new_root = root T
+    if (rc != AK_OK) return rc;
+    // T^p with the multiplication order of MatPower
+    const float* tp = nullptr;
+    if ((p & (p - 1)) == 0) {
+      const float* cur = T;
+      int which = 1;
+      for (int done = 1; done < p; done *= 2) {
+        float* dst = buf[which];
+        rc = mm(cur, nn, cur, nn, dst, nn);
+        if (rc != AK_OK) return rc;
+        cur = dst;
+        which = (which == 1) ? 2 : 1;
+      }
+      tp = cur;
+    } else {
+      const float* base = T;        // squares ping-pong in buf[0]/buf[1], the running power in buf[2]/buf[3]
+      const float* power = nullptr;
+      int sq = 1, pw = 2;
+      for (int q = p; q > 0; q /= 2) {
+        if (q & 1) {
+          if (power == nullptr) {
+            power = base;
+          } else {
+            float* dst = buf[pw];
+            rc = mm(base, nn, power, nn, dst, nn);
+            if (rc != AK_OK) return rc;
+            power = dst;
+            pw = (pw == 2) ? 3 : 2;
+          }
+        }
+        if (q / 2 > 0) {
+          float* dst = buf[sq];
+          if (power == base) {      // keep the value `power` points at alive
+            float* keep = buf[pw];
+            hipMemcpyAsync(keep, base, sizeof(float) * batch * nn, hipMemcpyDeviceToDevice, s);
+            power = keep;
+            pw = (pw == 2) ? 3 : 2;
+          }
+          rc = mm(base, nn, base, nn, dst, nn);
+          if (rc != AK_OK) return rc;
+          base = dst;
+          sq = (sq == 1) ? 0 : 1;
+        }
+      }
+      tp = power;
+    }
+    rc = mm(tp, nn, M, nn, Mnew, nn);                           // M' = T^p M
+    if (rc != AK_OK) return rc;
+    hipLaunchKernelGGL(newton_err_kernel, gc, b256, 0, s, st, Mnew, n);
+    hipLaunchKernelGGL(newton_decide_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
+    hipLaunchKernelGGL(newton_commit_kernel, gc, b256, 0, s, st, out, strideOut, newroot, M, Mnew, n);
+  }
+  hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
+  return check_launch();
+}

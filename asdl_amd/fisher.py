@@ -1,0 +1,280 @@
+"""FisherMaker: forward, (sampled / exact / empirical) backward under the hooks, and extraction of
+``module.fisher`` (behaviour of asdl/fisher.py:29-205, 419-521 for the Kronecker-factored shape)."""
+from dataclasses import dataclass
+from typing import Any, List, Tuple, Union
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+from .core import no_centered_cov
+from .grad_maker import GradientMaker, LOSS_CROSS_ENTROPY, LOSS_MSE
+from .matrices import *
+from .operations import OperationContext
+from .symmatrix import SymMatrix, batched_update_inv
+from .utils import skip_param_grad
+
+__all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
+
+_supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
+_invalid_data_size = -1
+
+
+@dataclass
+class FisherConfig:
+    fisher_type: str
+    fisher_shapes: List[Any]
+    loss_type: str = None
+    n_mc_samples: int = 1
+    var: float = 1.
+    seed: int = None
+    fisher_attr: str = 'fisher'
+    fvp_attr: str = 'fvp'
+    ignore_modules: List[Any] = None
+    data_size: int = _invalid_data_size
+    scale: float = 1.
+    is_distributed: bool = False
+    all_reduce: bool = False
+    is_master: bool = True
+    ignore_index: int = -1
+
+
+class FisherMaker(GradientMaker):
+    _loss_reduction = 'sum'
+
+    def __init__(self, model, config):
+        super().__init__(model)
+        self.config: FisherConfig = config
+
+    def zero_fisher(self, fvp=False):
+        attr = self.config.fvp_attr if fvp else self.config.fisher_attr
+        for module in self.model.modules():
+            if hasattr(module, attr):
+                delattr(module, attr)
+
+    @property
+    def is_fisher_emp(self):
+        return False
+
+    @property
+    def do_local_accumulate(self) -> bool:
+        raise NotImplementedError
+
+    def forward_and_backward(self, data_size=_invalid_data_size, scale=None, accumulate=False, calc_loss_grad=False,
+                             calc_inv=False, fvp=False, damping=None, vec=None,
+                             accumulate_prescale=1.0) -> Union[Tuple[Any, Tensor], Any]:
+        """Same arguments as asdl/fisher.py:69-77 plus ``accumulate_prescale``: with accumulate=True
+        the existing factors are multiplied by it inside the kernel that adds the new statistic
+        (the EMA decay), instead of in a separate pass beforehand."""
+        if accumulate and calc_inv:
+            raise ValueError('accumulate and calc_inv cannot be True at the same time.')
+        if fvp:
+            raise NotImplementedError('Fisher-vector products are not on this path')
+        model = self.model
+        config = self.config
+        fisher_shapes = config.fisher_shapes
+        if isinstance(fisher_shapes, str):
+            fisher_shapes = [fisher_shapes]
+        if data_size == _invalid_data_size:
+            data_size = config.data_size
+        if data_size == _invalid_data_size:
+            raise ValueError('data_size is not specified.')
+        if scale is None:
+            scale = config.scale
+        scale /= data_size
+
+        if not accumulate:
+            self.zero_fisher()
+        if config.seed is not None:
+            torch.random.manual_seed(config.seed)
+
+        loss_grad_with_fisher = calc_loss_grad and self.is_fisher_emp
+        loss_grad_after_fisher = calc_loss_grad and not self.is_fisher_emp
+        inv_with_fisher = calc_inv and not self.do_local_accumulate
+        inv_after_fisher = calc_inv and self.do_local_accumulate
+
+        with no_centered_cov(model, fisher_shapes, ignore_modules=config.ignore_modules,
+                             calc_inv=inv_with_fisher) as cxt:
+            if accumulate:
+                self._register_fisher(cxt, accumulate_prescale)
+            if damping is not None:
+                cxt.set_damping(damping)
+            cxt.set_cov_scale(scale)
+
+            self.call_model()
+            loss = None
+            if self.is_fisher_emp or calc_loss_grad:
+                self.call_loss()
+                loss = self._loss
+
+            def closure(nll_expr, retain_graph=False):
+                with skip_param_grad(model, disable=loss_grad_with_fisher):
+                    nll_expr().backward(retain_graph=retain_graph or loss_grad_after_fisher)
+
+            if self.is_fisher_emp:
+                closure(lambda: loss)
+            else:
+                self._fisher_loop(closure)
+            cxt.finish_registered()
+            self._extract_fisher(cxt)
+
+        if inv_after_fisher:
+            self.replace_fisher_with_inv(damping)
+        if loss_grad_after_fisher:
+            loss.backward()
+        if calc_loss_grad:
+            # the loss was summed over the batch: divide gradients and loss by the data size
+            for p in model.parameters():
+                if p.grad is not None:
+                    p.grad.div_(data_size)
+            loss.div_(data_size)
+        return self._model_output, loss
+
+    def _register_fisher(self, cxt: OperationContext, prescale=1.0):
+        attr = self.config.fisher_attr
+        for module in self.model.modules():
+            fisher = getattr(module, attr, None)
+            if fisher is not None and cxt.is_operation_registered(module):
+                cxt.register_symmatrix(module, fisher, first_beta=prescale)
+
+    def _extract_fisher(self, cxt: OperationContext):
+        attr = self.config.fisher_attr
+        for module in self.model.modules():
+            if getattr(module, attr, None) is None and cxt.is_operation_registered(module):
+                fisher = cxt.cov_symmatrix(module, pop=True)
+                if fisher is not None:
+                    setattr(module, attr, fisher)
+
+    def replace_fisher_with_inv(self, damping):
+        attr = self.config.fisher_attr
+        krons = []
+        for module in self.model.modules():
+            fisher: SymMatrix = getattr(module, attr, None)
+            if fisher is not None and fisher.has_kron:
+                krons.append(fisher.kron)
+        batched_update_inv(krons, damping=damping, replace=True)
+
+    def _fisher_loop(self, closure):
+        raise NotImplementedError
+
+    def get_fisher_tensor(self, module: nn.Module, *keys) -> Union[torch.Tensor, None]:
+        data = getattr(module, self.config.fisher_attr, None)
+        if data is None:
+            return None
+        for key in keys:
+            data = getattr(data, key, None)
+        if data is not None and not isinstance(data, torch.Tensor):
+            raise TypeError(f'data have to be {torch.Tensor}, got {type(data)}.')
+        return data
+
+
+class FisherExactCrossEntropy(FisherMaker):
+    """asdl/fisher.py:419-440."""
+
+    @property
+    def do_local_accumulate(self) -> bool:
+        if self._logits is not None:
+            return self._logits.shape[-1] > 1
+        return True
+
+    def _fisher_loop(self, closure):
+        logits = self._logits
+        log_probs = F.log_softmax(logits, dim=-1)
+        log_probs = log_probs.view(-1, log_probs.size(-1))
+        n, n_classes = log_probs.shape
+        with torch.no_grad():
+            sqrt_probs = torch.sqrt(F.softmax(logits, dim=-1)).view(n, n_classes)
+        for i in range(n_classes):
+            targets = torch.full((n,), i, device=logits.device, dtype=torch.long)
+
+            def nll_expr():
+                nll = F.nll_loss(log_probs, targets, reduction='none', ignore_index=self.config.ignore_index)
+                return nll.mul(sqrt_probs[:, i]).sum()
+            closure(nll_expr, retain_graph=i < n_classes - 1)
+
+
+class FisherMCCrossEntropy(FisherMaker):
+    """asdl/fisher.py:443-459."""
+
+    @property
+    def do_local_accumulate(self) -> bool:
+        return self.config.n_mc_samples > 1
+
+    def _fisher_loop(self, closure):
+        logits = self._logits
+        n_mc_samples = self.config.n_mc_samples
+        probs = F.softmax(logits, dim=-1)
+        log_probs = F.log_softmax(logits, dim=-1)
+        dist = torch.distributions.Categorical(probs)
+        for i in range(n_mc_samples):
+            with torch.no_grad():
+                targets = self.sample_targets(dist, i)
+            closure(lambda: F.nll_loss(log_probs.view(-1, log_probs.size(-1)), targets.view(-1), reduction='sum',
+                                       ignore_index=self.config.ignore_index) / n_mc_samples,
+                    retain_graph=i < n_mc_samples - 1)
+
+    def sample_targets(self, dist, i):
+        """One draw of the model's predictive distribution; override to replay fixed targets."""
+        return dist.sample()
+
+
+class FisherExactMSE(FisherMaker):
+    """asdl/fisher.py:462-473."""
+
+    @property
+    def do_local_accumulate(self) -> bool:
+        if self._logits is not None:
+            return self._logits.shape[-1] > 1
+        return True
+
+    def _fisher_loop(self, closure):
+        logits = self._logits
+        n_dims = logits.size(-1)
+        for i in range(n_dims):
+            closure(lambda: logits[:, i].sum(), retain_graph=i < n_dims - 1)
+
+
+class FisherMCMSE(FisherMaker):
+    """asdl/fisher.py:476-490."""
+
+    @property
+    def do_local_accumulate(self) -> bool:
+        return self.config.n_mc_samples > 1
+
+    def _fisher_loop(self, closure):
+        logits = self._logits
+        n_mc_samples = self.config.n_mc_samples
+        dist = torch.distributions.normal.Normal(logits, scale=np.sqrt(self.config.var))
+        for i in range(n_mc_samples):
+            with torch.no_grad():
+                targets = dist.sample()
+            closure(lambda: 0.5 * F.mse_loss(logits, targets, reduction='sum') / n_mc_samples,
+                    retain_graph=i < n_mc_samples - 1)
+
+
+class FisherEmp(FisherMaker):
+    """asdl/fisher.py:493-500."""
+
+    @property
+    def do_local_accumulate(self) -> bool:
+        return False
+
+    @property
+    def is_fisher_emp(self):
+        return True
+
+
+def get_fisher_maker(model: nn.Module, config: FisherConfig):
+    fisher_type = config.fisher_type
+    loss_type = config.loss_type
+    if fisher_type not in _supported_types:
+        raise ValueError(f'Invalid fisher_type: {fisher_type}. {_supported_types} are supported.')
+    if fisher_type == FISHER_EMP:
+        return FisherEmp(model, config)
+    if loss_type not in [LOSS_CROSS_ENTROPY, LOSS_MSE]:
+        raise ValueError(f'Invalid loss_type: {loss_type}. {[LOSS_CROSS_ENTROPY, LOSS_MSE]} are supported.')
+    if fisher_type == FISHER_EXACT:
+        return FisherExactCrossEntropy(model, config) if loss_type == LOSS_CROSS_ENTROPY else FisherExactMSE(model, config)
+    return FisherMCCrossEntropy(model, config) if loss_type == LOSS_CROSS_ENTROPY else FisherMCMSE(model, config)

@@ -16,6 +16,32 @@ AK_F32, AK_BF16 = 0, 1
 _ws_lock = threading.Lock()
 _workspaces = {}
 _ptr_cache = {}
+_timing_sink = None      # when set to a list, factor launches append (name, flops, start event, end event)
+
+
+def set_timing_sink(sink):
+    """Benchmark instrumentation: with a list as sink every factor-statistics launch is bracketed by
+    two events on the launching stream and recorded with its algorithmic FLOP count M*d*(d+1)."""
+    global _timing_sink
+    _timing_sink = sink
+
+
+class _Timed:
+    def __init__(self, name, flops):
+        self.name, self.flops = name, flops
+
+    def __enter__(self):
+        if _timing_sink is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _timing_sink is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            _timing_sink.append((self.name, self.flops, self.start, end))
+        return False
 
 
 def _require_gpu(*tensors):
@@ -97,8 +123,9 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     lib = _lib.load()
     need = lib.ak_syrk_tn_ws_bytes(M, d)
     ws, ws_bytes, keep = _ws_args(need, x.device)
-    rc = lib.ak_syrk_tn(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), M, d, ldx, alpha, beta,
-                        ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
+    with _Timed('syrk_tn', M * d * (d + 1)):
+        rc = lib.ak_syrk_tn(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), M, d, ldx, alpha, beta,
+                            ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
     _lib.check(rc, 'ak_syrk_tn')
     return out
 
@@ -123,8 +150,10 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     lib = _lib.load()
     need = lib.ak_conv_syrk_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)
     ws, ws_bytes, keep = _ws_args(need, x.device)
-    rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw, ph, pw,
-                          alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
+    h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
+        rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw, ph, pw,
+                              alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
     _lib.check(rc, 'ak_conv_syrk')
     return out
 
@@ -239,3 +268,35 @@ def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
                              grad_scale, ws, ws_bytes, _stream())
     _lib.check(rc, 'ak_kron_precond')
     return grad_w, grad_b
+
+
+# ------------------------------------------------------------------------------ Shampoo inverse root
+def inv_root_newton(S, p, ridge_eps, v0, out=None, max_power_iter=100, power_tol=1e-6, max_iter=100, tol=1e-6):
+    """out[b] <- (S[b] + ridge_eps * lambda_max I)^(-1/p) for S = [batch, n, n] (or [n, n]); S keeps the
+    ridge.  v0 = [batch, n] start vectors of the power iteration.  Returns (out, stats) with
+    stats = [batch, 4] = (lambda_max, power iterations, newton iterations, final error) on the device."""
+    _require_gpu(S, v0, out)
+    single = S.ndim == 2
+    S3 = S.unsqueeze(0) if single else S
+    batch, n = S3.shape[0], S3.shape[1]
+    if S3.dtype != torch.float32 or S3.shape[2] != n or S3.stride(2) != 1 or S3.stride(1) != n:
+        raise ValueError('S has to be float32 [batch, n, n] with dense matrices')
+    if n < 2:
+        raise ValueError('n has to be >= 2 (the inverse root of a 1 x 1 statistic is defined as the identity)')
+    v0 = v0.reshape(batch, n).to(torch.float32).contiguous()
+    if out is None:
+        out = torch.empty(batch, n, n, dtype=torch.float32, device=S.device)
+    out3 = out.unsqueeze(0) if out.ndim == 2 else out
+    if out3.dtype != torch.float32 or out3.shape != (batch, n, n) or out3.stride(2) != 1 or out3.stride(1) != n:
+        raise ValueError('out has to be float32 [batch, n, n] with dense matrices')
+    stats = torch.empty(batch, 4, dtype=torch.float32, device=S.device)
+    lib = _lib.load()
+    ws, ws_bytes, keep = _ws_args(lib.ak_inv_root_ws_bytes(n, batch), S.device)
+    strideS = S3.stride(0) if batch > 1 else n * n
+    strideO = out3.stride(0) if batch > 1 else n * n
+    rc = lib.ak_inv_root_newton(ctypes.c_void_p(S3.data_ptr()), n, batch, strideS, int(p), float(ridge_eps),
+                                ctypes.c_void_p(v0.data_ptr()), int(max_power_iter), float(power_tol), int(max_iter),
+                                float(tol), ctypes.c_void_p(out3.data_ptr()), strideO,
+                                ctypes.c_void_p(stats.data_ptr()), ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_inv_root_newton')
+    return (out3[0] if single and out.ndim == 3 else out), stats

@@ -1,0 +1,208 @@
+"""K-FAC gradient maker on one GPU (behaviour of asdl/precondition/natural_gradient.py:28-128,
+323-543, 859-900 for the Kronecker-factored shape).
+
+Host-side differences from the reference, all result-preserving:
+* the EMA pre-scale ``curv *= (1 - ema_decay)`` is folded into the factor kernels,
+* inverses of all layers are taken in one batched pass with one host synchronisation,
+* layer ownership across ranks (the reference's partitions) does not exist: one process, one GPU.
+"""
+from typing import Any, List, Union
+
+import torch
+import torch.distributed as dist
+from torch import nn
+
+from .core import module_wise_assignments, modules_to_assign
+from .fisher import FisherConfig, get_fisher_maker
+from .grad_maker import LOSS_CROSS_ENTROPY
+from .matrices import *
+from .prec_grad_maker import PreconditionedGradientMaker, PreconditioningConfig
+from .symmatrix import SymMatrix, batched_update_inv
+
+_invalid_ema_decay = -1
+_module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KFE, SHAPE_UNIT_WISE, SHAPE_DIAG]
+_kernel_shapes = [SHAPE_KRON]
+
+__all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
+
+
+def _bias_requires_grad(module):
+    return hasattr(module, 'bias') and module.bias is not None and module.bias.requires_grad
+
+
+class NaturalGradientMaker(PreconditionedGradientMaker):
+    _supported_classes = (nn.Linear, nn.Conv2d, nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm, nn.Embedding)
+
+    def __init__(self, model, config: PreconditioningConfig, fisher_type: str = FISHER_MC,
+                 fisher_shape: Union[str, List[Any]] = SHAPE_KRON, loss_type: str = LOSS_CROSS_ENTROPY,
+                 scale: float = 1, grad_scale: float = 1, n_mc_samples: int = 1, var: float = 1., seed: int = None):
+        from torch.nn.parallel import DistributedDataParallel as DDP
+        if isinstance(model, DDP):
+            raise TypeError(f'{DDP} is not supported.')
+        if dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1:
+            raise NotImplementedError('this build runs on one GPU: layer-partitioned preconditioning across ranks '
+                                      'is not implemented')
+        super().__init__(model, config)
+        if isinstance(fisher_shape, str):
+            fisher_shape = [fisher_shape]
+        if not self.do_accumulate and config.curvature_upd_ratio is not None:
+            raise ValueError('curvature_upd_ratio cannot be specified when no curvature accumulation is performed.')
+
+        unsupported = [m for m in self.module_dict.values() if not isinstance(m, (nn.Linear, nn.Conv2d))]
+        if unsupported:
+            kinds = sorted({type(m).__name__ for m in unsupported})
+            raise NotImplementedError(
+                f'{kinds} modules would get a unit-wise / diagonal Fisher in the reference; this build has kernels '
+                f'for the Kronecker-factored shape of Linear and Conv2d only. Pass '
+                f'PreconditioningConfig(ignore_modules=[...]) to leave them un-preconditioned.')
+
+        self.named_modules_for_curvature = []
+        self.modules_for_curvature = []
+        self.shape_for = {}
+        for name, module, shapes in module_wise_assignments(self.module_dict, *fisher_shape, named=True):
+            if len(shapes) != 1:
+                raise ValueError(f'Each module has to be assigned one Fisher shape. '
+                                 f'{name} is assigned {len(shapes)} shapes.')
+            if shapes[0] not in _kernel_shapes:
+                raise NotImplementedError(f'Fisher shape "{shapes[0]}" (module {name}) is not on this path.')
+            self.modules_for_curvature.append(module)
+            self.named_modules_for_curvature.append((name, module))
+            self.shape_for[module] = shapes[0]
+            self.shape_for[name] = shapes[0]
+        self._named_modules_for = {}
+
+        fisher_config = FisherConfig(fisher_type=fisher_type, fisher_shapes=fisher_shape, loss_type=loss_type,
+                                     n_mc_samples=n_mc_samples, ignore_modules=config.ignore_modules, var=var,
+                                     seed=seed)
+        self.fisher_maker = get_fisher_maker(model, fisher_config)
+        self.fisher_type = fisher_type
+        self.fisher_shape = fisher_shape
+        self.scale = scale
+        self.grad_scale = grad_scale
+        self.world_rank = 0
+        self.world_size = 1
+
+    def do_forward_and_backward(self, step=None):
+        return not self.do_update_curvature(step)
+
+    def named_modules_for(self, shape):
+        if shape not in self._named_modules_for:
+            self._named_modules_for[shape] = list(modules_to_assign(self.model, shape, *self.fisher_shape,
+                                                                    ignore_modules=self.config.ignore_modules,
+                                                                    named=True))
+        return self._named_modules_for[shape]
+
+    def modules_for(self, shape):
+        return [m for _, m in self.named_modules_for(shape)]
+
+    @property
+    def _fisher_attr(self):
+        return self.fisher_maker.config.fisher_attr
+
+    def _get_module_fisher(self, module):
+        return getattr(module, self._fisher_attr, None)
+
+    def _get_module_symmatrix(self, module, shape):
+        fisher = self._get_module_fisher(module)
+        if fisher is None:
+            return None
+        if shape in [SHAPE_KRON, SHAPE_SWIFT_KRON]:
+            return fisher.kron
+        raise ValueError(f'Invalid shape: {shape}.')
+
+    @property
+    def do_accumulate(self):
+        return self.config.ema_decay != _invalid_ema_decay
+
+    def update_curvature(self):
+        config = self.config
+        scale = self.scale
+        prescale = 1.0
+        ema_decay = config.ema_decay
+        if ema_decay != _invalid_ema_decay:
+            scale *= ema_decay
+            prescale = 1 - ema_decay          # applied to the old factors inside the factor kernels
+        self.delegate_forward_and_backward(self.fisher_maker, data_size=config.data_size, scale=scale,
+                                           accumulate=self.do_accumulate, calc_loss_grad=True,
+                                           calc_inv=not self.do_accumulate, damping=config.damping,
+                                           accumulate_prescale=prescale)
+
+    def update_preconditioner(self, damping=None, module_name=None, kron=None, zero_curvature=False):
+        if not self.do_accumulate:
+            return
+        if kron is None:
+            kron = ['A', 'B']
+        if damping is None:
+            damping = self.config.damping
+        matrices = []
+        for shape in _kernel_shapes:
+            for name, module in self.named_modules_for(shape):
+                if module_name is not None and name != module_name:
+                    continue
+                if module not in self.modules_for_curvature:
+                    continue
+                matrix = self._get_module_symmatrix(module, shape)
+                if matrix is not None:
+                    matrices.append(matrix)
+        batched_update_inv(matrices, damping, calc_A_inv='A' in kron, calc_B_inv='B' in kron)
+        if zero_curvature:
+            with torch.no_grad():
+                for matrix in matrices:
+                    if 'A' in kron:
+                        matrix.A.mul_(0)
+                    if 'B' in kron:
+                        matrix.B.mul_(0)
+
+    def precondition(self, vectors=None, grad_scale=None, use_inv=True):
+        if vectors is not None:
+            raise NotImplementedError('precondition(vectors=...) is not on this path')
+        if grad_scale is None:
+            grad_scale = self.grad_scale
+        for shape in _kernel_shapes:
+            for module in self.modules_for(shape):
+                if module not in self.modules_for_curvature:
+                    continue
+                self._precondition_module(module, shape, grad_scale=grad_scale, use_inv=use_inv)
+
+    def _precondition_module(self, module, shape=None, vectors=None, vec_weight=None, vec_bias=None,
+                             grad_scale=None, use_inv=True):
+        if grad_scale is None:
+            grad_scale = self.grad_scale
+        if shape is None:
+            shape = self.shape_for.get(module)
+        if shape is None:
+            raise ValueError(f'No shape is assigned to module: {module}.')
+        matrix = self._get_module_symmatrix(module, shape)
+        if matrix is None:
+            raise ValueError(f'Matrix of shape {shape} for module {module} has not been calculated.')
+        if vec_weight is None and module.weight.requires_grad:
+            vec_weight = module.weight.grad
+        if vec_weight is None:
+            raise ValueError(f'weight gradient for module {module} has not been calculated.')
+        if _bias_requires_grad(module):
+            if vec_bias is None:
+                vec_bias = module.bias.grad
+            if vec_bias is None:
+                raise ValueError(f'bias gradient for module {module} has not been calculated.')
+        if grad_scale != 1:
+            vec_weight.data.mul_(grad_scale)
+            if vec_bias is not None:
+                vec_bias.data.mul_(grad_scale)
+        if not use_inv or matrix.has_inv:
+            matrix.mvp(vec_weight=vec_weight, vec_bias=vec_bias, use_inv=use_inv, inplace=True)
+
+
+class KfacGradientMaker(NaturalGradientMaker):
+    """K-FAC (https://arxiv.org/abs/1503.05671) behind the GradientMaker interface; same constructor
+    arguments as asdl/precondition/natural_gradient.py:883-900.
+
+    BatchNorm / LayerNorm modules (unit-wise Fisher in the reference) and ``swift=True`` have no
+    kernels in this build: exclude such modules through ``config.ignore_modules``."""
+
+    def __init__(self, model, config: PreconditioningConfig, fisher_type: str = FISHER_MC,
+                 loss_type: str = LOSS_CROSS_ENTROPY, scale: float = 1, grad_scale: float = 1, n_mc_samples: int = 1,
+                 var: float = 1., seed: int = None, swift=False):
+        if swift:
+            raise NotImplementedError('swift=True (SKFAC) is not on this path')
+        super().__init__(model, config, fisher_type=fisher_type, fisher_shape=[SHAPE_KRON], loss_type=loss_type,
+                         scale=scale, grad_scale=grad_scale, n_mc_samples=n_mc_samples, var=var, seed=seed)

@@ -1,0 +1,354 @@
+"""Per-layer operations of the K-FAC path and the context that stores their results.
+
+Mirrors the operator seam of the reference (asdl/operations/operation.py:87-548 for Operation,
+:551-964 for OperationContext, asdl/operations/linear.py and conv.py for the layer classes) for the
+two operations on this path, OP_COV_KRON and OP_COV_KRON_INV.  Differences that come from running
+on the GPU kernels:
+
+* cov_kron_A / cov_kron_B take optional ``out``, ``alpha``, ``beta`` and compute
+  ``out <- beta*out + alpha*factor`` in one launch, so the reference's separate
+  ``.mul_(cov_scale)``, ``results[key] += value`` and EMA pre-scale passes disappear.
+* Conv2d.preprocess_in_data returns a lazy UnfoldedInput; the unfold happens inside the kernel.
+* With OP_COV_KRON_INV the inverses are not taken inside the backward hook: the context queues the
+  (A, B) pairs and inverts them all in one batched pass (OperationContext.flush_inverses).
+"""
+import warnings
+from typing import Dict
+
+import torch
+import torch.nn as nn
+
+from . import kernels
+from .symmatrix import Kron, SymMatrix, batched_update_inv
+from .utils import UnfoldedInput, im2col_2d
+
+OP_COV_KRON = 'cov_kron'
+OP_COV_KRON_INV = 'cov_kron_inv'
+OP_SAVE_INPUTS = 'save_inputs'
+OP_SAVE_OUTPUTS = 'save_outputs'
+OP_SAVE_OUTGRADS = 'save_outgrads'
+
+ALL_OPS = [OP_COV_KRON, OP_COV_KRON_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS]
+FWD_OPS = [OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_COV_KRON, OP_COV_KRON_INV]
+BWD_OPS = [OP_SAVE_OUTGRADS, OP_COV_KRON, OP_COV_KRON_INV]
+
+__all__ = ['Operation', 'Linear', 'Conv2d', 'OperationContext', 'get_op_class', 'ALL_OPS', 'FWD_OPS', 'BWD_OPS',
+           'OP_COV_KRON', 'OP_COV_KRON_INV', 'OP_SAVE_INPUTS', 'OP_SAVE_OUTPUTS', 'OP_SAVE_OUTGRADS']
+
+_FACTOR_CACHE_ATTR = '_asdl_amd_factor_cache'
+
+
+class Operation:
+    supported_operations = set(ALL_OPS)
+
+    def __init__(self, module, op_names, model_for_kernel=None):
+        if hasattr(module, 'weight'):
+            requires_grad = module.weight.requires_grad
+            if hasattr(module, 'bias') and module.bias is not None:
+                requires_grad = requires_grad or module.bias.requires_grad
+            if not requires_grad:
+                raise ValueError(f'One of weight or bias has to require grad (module: {module}).')
+        self._module = module
+        if isinstance(op_names, str):
+            op_names = [op_names]
+        if not isinstance(op_names, list):
+            raise TypeError(f'op_names has to be a list. Got {type(op_names)}.')
+        op_names = set(op_names)
+        for name in op_names:
+            if name not in ALL_OPS:
+                raise ValueError(f'Invalid operation name: {name}. {ALL_OPS} are supported.')
+        self._op_names = op_names
+        self._op_results = {}
+        self._damping = 1.e-7
+        self._cov_scale = 1.
+        self._first_beta = {}       # 'A' / 'B' -> factor applied to a registered matrix at its first update
+        self._touched = set()
+        self._context = None
+
+    # ---- result store (asdl/operations/operation.py:118-160)
+    def accumulate_result(self, value, *keys, extend=False):
+        results = self._op_results
+        for key in keys[:-1]:
+            if results.get(key, None) is None:
+                results[key] = {}
+            results = results[key]
+        key = keys[-1]
+        if results.get(key, None) is None:
+            results[key] = value
+        elif extend:
+            results[key].extend(value)
+        else:
+            results[key] += value
+
+    def get_result(self, *keys, pop=False, default=None):
+        results = self._op_results
+        for key in keys[:-1]:
+            try:
+                results = results[key]
+            except KeyError:
+                return None
+        key = keys[-1]
+        if pop:
+            return results.pop(key, default)
+        return results.get(key, default)
+
+    def clear_results(self):
+        self._op_results = {}
+
+    def set_damping(self, value):
+        self._damping = value
+
+    def set_cov_scale(self, value):
+        self._cov_scale = value
+
+    # ---- fused accumulate into the stored factor
+    def _update_factor(self, key, compute):
+        """compute(out, alpha, beta) writes ``beta*out + alpha*factor`` (allocating when out is None)."""
+        existing = self.get_result(OP_COV_KRON, key)
+        if existing is None:
+            self.accumulate_result(compute(None, self._cov_scale, 0.0), OP_COV_KRON, key)
+        else:
+            beta = self._first_beta.pop(key, 1.0)
+            compute(existing, self._cov_scale, beta)
+        self._touched.add(key)
+
+    def _scratch_factor(self, key, dim, device):
+        """Reusable buffer for a factor that only lives until it has been inverted."""
+        cache = getattr(self._module, _FACTOR_CACHE_ATTR, None)
+        if cache is None:
+            cache = {}
+            setattr(self._module, _FACTOR_CACHE_ATTR, cache)
+        buf = cache.get(key)
+        if buf is None or buf.shape[0] != dim or buf.device != device:
+            buf = torch.empty(dim, dim, dtype=torch.float32, device=device)
+            cache[key] = buf
+        return buf
+
+    def forward_post_process(self, in_data: torch.Tensor, out_data: torch.Tensor):
+        module = self._module
+        op_names = self._op_names
+        if OP_SAVE_INPUTS in op_names:
+            self.accumulate_result([in_data], OP_SAVE_INPUTS, extend=True)
+        if OP_SAVE_OUTPUTS in op_names:
+            self.accumulate_result([out_data], OP_SAVE_OUTPUTS, extend=True)
+        if OP_COV_KRON in op_names:
+            data = self.preprocess_in_data(module, in_data, out_data)
+            self._update_factor('A', lambda out, alpha, beta: self.cov_kron_A(module, data, out=out, alpha=alpha, beta=beta))
+        elif OP_COV_KRON_INV in op_names:
+            data = self.preprocess_in_data(module, in_data, out_data)
+            dim = data.shape[1]
+            first = '_A_tmp' not in self._op_results
+            buf = self._scratch_factor('A', dim, in_data.device)
+            self.cov_kron_A(module, data, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
+            self._op_results['_A_tmp'] = buf
+
+    def backward_pre_process(self, out_grads, vector: torch.Tensor = None):
+        module = self._module
+        op_names = self._op_names
+        if not any(name in BWD_OPS for name in op_names):
+            return
+        grads = self.preprocess_out_grads(module, out_grads)
+        if OP_SAVE_OUTGRADS in op_names:
+            self.accumulate_result([grads], OP_SAVE_OUTGRADS, extend=True)
+        if OP_COV_KRON in op_names:
+            self._update_factor('B', lambda out, alpha, beta: self.cov_kron_B(module, grads, out=out, alpha=alpha, beta=beta))
+        elif OP_COV_KRON_INV in op_names:
+            first = '_B_tmp' not in self._op_results
+            buf = self._scratch_factor('B', grads.shape[1], grads.device)
+            self.cov_kron_B(module, grads, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
+            self._op_results['_B_tmp'] = buf
+            if self._context is not None:
+                self._context.queue_inverse(self)
+
+    def finish_registered(self):
+        """Applies the pending pre-scale to registered factors that no hook touched."""
+        kron = self._op_results.get(OP_COV_KRON)
+        for key, beta in list(self._first_beta.items()):
+            if kron is not None and kron.get(key) is not None and beta != 1.0:
+                kron[key].mul_(beta)
+        self._first_beta = {}
+
+    @staticmethod
+    def preprocess_in_data(module, in_data, out_data):
+        return in_data
+
+    @staticmethod
+    def preprocess_out_grads(module, out_grads):
+        return out_grads
+
+    @staticmethod
+    def cov_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
+        raise NotImplementedError
+
+    @staticmethod
+    def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        raise NotImplementedError
+
+
+class Linear(Operation):
+    """module.weight: f_out x f_in; in_data: n x f_in; out_grads: n x f_out
+    (asdl/operations/linear.py:9-42, 75-89)."""
+
+    @staticmethod
+    def preprocess_in_data(module, in_data, out_data):
+        if in_data.ndim > 2:
+            in_data = in_data.flatten(end_dim=in_data.ndim - 2)
+        return in_data
+
+    @staticmethod
+    def preprocess_out_grads(module, out_grads):
+        if out_grads.ndim > 2:
+            out_grads = out_grads.flatten(end_dim=out_grads.ndim - 2)
+        return out_grads
+
+    @staticmethod
+    def cov_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
+        return kernels.syrk_tn(in_data, out=out, alpha=alpha, beta=beta)      # f_in x f_in
+
+    @staticmethod
+    def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        return kernels.syrk_tn(out_grads, out=out, alpha=alpha, beta=beta)    # f_out x f_out
+
+
+class Conv2d(Operation):
+    """module.weight: c_out x c_in x k_h x k_w; in_data: lazy n x (c_in k_h k_w) x out_size;
+    out_grads: n x c_out x out_size (asdl/operations/conv.py:9-42, 80-103)."""
+
+    @staticmethod
+    def preprocess_in_data(module, in_data, out_data):
+        if isinstance(in_data, UnfoldedInput):
+            return in_data
+        if getattr(module, 'groups', 1) != 1:
+            raise NotImplementedError('grouped convolutions are not supported by the K-FAC factors')
+        return im2col_2d(in_data, module)
+
+    @staticmethod
+    def preprocess_out_grads(module, out_grads):
+        return out_grads.flatten(start_dim=2)
+
+    @staticmethod
+    def cov_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
+        if not isinstance(in_data, UnfoldedInput):
+            # already materialised [n, d, out_size] patches
+            return kernels.syrk_nt(in_data, out=out, alpha=alpha / in_data.shape[-1], beta=beta)
+        return kernels.conv_syrk(in_data.x, in_data.kernel_size, in_data.stride, in_data.padding, out=out,
+                                 alpha=alpha / in_data.out_size, beta=beta)
+
+    @staticmethod
+    def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        return kernels.syrk_nt(out_grads, out=out, alpha=alpha, beta=beta)    # c_out x c_out
+
+
+def get_op_class(module):
+    """asdl/operations/__init__.py:60-79, restricted to the layer types on this path."""
+    if isinstance(module, nn.Linear):
+        return Linear
+    elif isinstance(module, nn.Conv2d):
+        return Conv2d
+    warnings.warn(f'Failed to lookup operations for Module {module}.')
+    return None
+
+
+class OperationContext:
+    def __init__(self, vectors=None):
+        self._operations: Dict[nn.Module, Operation] = {}
+        self._vectors = vectors
+        self._pending_inverse = []
+
+    def is_operation_registered(self, module):
+        return module in self._operations
+
+    def register_operation(self, module, operation):
+        operation._context = self
+        self._operations[module] = operation
+
+    def get_operation(self, module) -> Operation:
+        try:
+            return self._operations[module]
+        except KeyError:
+            raise KeyError(f'No operation is registered to {module}.')
+
+    def clear_operations(self):
+        self._operations.clear()
+        self._pending_inverse = []
+
+    def call_operations_in_forward(self, module, in_data, out_data):
+        self.get_operation(module).forward_post_process(in_data, out_data)
+
+    def call_operations_in_backward(self, module, out_grads):
+        self.get_operation(module).backward_pre_process(out_grads, None)
+
+    def get_result(self, module, *keys, pop=False, default=None):
+        try:
+            return self.get_operation(module).get_result(*keys, pop=pop, default=default)
+        except KeyError:
+            return default
+
+    def set_damping(self, value):
+        for operation in self._operations.values():
+            operation.set_damping(value)
+
+    def set_cov_scale(self, value):
+        for operation in self._operations.values():
+            operation.set_cov_scale(value)
+
+    def clear_batch_grads(self):
+        pass
+
+    def calc_full_cov(self, model, scale=1., calc_inv=False, damping=1e-7):
+        pass  # only needed for the full (non layer-wise) shape
+
+    # ---- deferred, batched inverses
+    def queue_inverse(self, operation):
+        if operation not in self._pending_inverse:
+            self._pending_inverse.append(operation)
+
+    def flush_inverses(self):
+        ops = self._pending_inverse
+        self._pending_inverse = []
+        if not ops:
+            return
+        krons = []
+        for op in ops:
+            A = op._op_results.pop('_A_tmp', None)
+            B = op._op_results.pop('_B_tmp', None)
+            if A is None or B is None:
+                raise RuntimeError('cov_kron_inv: the forward and backward hooks did not both run')
+            prev = op._op_results.get(OP_COV_KRON) or {}
+            krons.append(Kron(A, B, prev.get('A_inv'), prev.get('B_inv')))
+        # every operation in one context shares the damping value
+        batched_update_inv(krons, damping=ops[0]._damping, replace=False)
+        for op, kron in zip(ops, krons):
+            store = op._op_results.setdefault(OP_COV_KRON, {})
+            if kron.A_inv is not None:
+                store['A_inv'] = kron.A_inv
+            if kron.B_inv is not None:
+                store['B_inv'] = kron.B_inv
+
+    # ---- symmatrix exchange (asdl/operations/operation.py:815-876)
+    def cov_symmatrix(self, module, pop=False):
+        self.flush_inverses()
+        cov_kron = self.get_result(module, OP_COV_KRON, pop=pop)
+        if cov_kron is None:
+            return None
+        kwargs = dict(kron_A=cov_kron.pop('A', None), kron_B=cov_kron.pop('B', None),
+                      kron_A_inv=cov_kron.pop('A_inv', None), kron_B_inv=cov_kron.pop('B_inv', None))
+        if all(v is None for v in kwargs.values()):
+            return None
+        return SymMatrix(**kwargs)
+
+    def register_symmatrix(self, module, matrix: SymMatrix, first_beta=1.0):
+        """Places the module's existing factors in the result store so that the hooks accumulate
+        into them in place; ``first_beta`` is the factor they are scaled by at their first update."""
+        operation = self.get_operation(module)
+        if matrix.has_kron:
+            if matrix.kron.has_A:
+                operation.accumulate_result(matrix.kron.A, OP_COV_KRON, 'A')
+                operation._first_beta['A'] = first_beta
+            if matrix.kron.has_B:
+                operation.accumulate_result(matrix.kron.B, OP_COV_KRON, 'B')
+                operation._first_beta['B'] = first_beta
+
+    def finish_registered(self):
+        for operation in self._operations.values():
+            operation.finish_registered()

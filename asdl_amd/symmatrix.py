@@ -1,0 +1,260 @@
+"""Containers of the curvature matrices on the K-FAC path: SymMatrix and its Kronecker part.
+
+Same attributes and call signatures as asdl/symmatrix.py (SymMatrix :94-358, Kron :361-548);
+the arithmetic runs in the HIP kernels.  Only the Kronecker-factored shape is on this path:
+full / layer-wise / KFE / unit-wise / diagonal containers are accepted as opaque attributes but
+have no kernels here.
+"""
+from collections import defaultdict
+
+import torch
+from torch import Tensor
+
+from . import kernels
+
+__all__ = ['SymMatrix', 'Kron', 'batched_update_inv']
+
+_default_damping = 1e-5
+
+
+def _is_all_none(xs):
+    return all(x is None for x in xs)
+
+
+def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_inv=True, eps=1e-7, replace=False):
+    """Kron.update_inv for many Kron objects at once (asdl/symmatrix.py:499-534 per object).
+
+    One damping launch for all pairs, one batched Cholesky inverse per distinct matrix size, and
+    a single device-to-host read at the end for the zero / not-positive-definite flags (the
+    reference synchronises three to five times per layer)."""
+    krons = [k for k in krons if k is not None]
+    if not krons:
+        return
+    for k in krons:
+        if not k.has_data:
+            raise ValueError('data do not exist.')
+        if calc_A_inv and not k.has_A:
+            raise ValueError('A does not exist.')
+        if calc_B_inv and not k.has_B:
+            raise ValueError('B does not exist.')
+        for m in (k.A, k.B):
+            if m is not None and (m.ndim != 2 or m.shape[0] != m.shape[1]):
+                raise NotImplementedError('non-square (swift) Kronecker factors are not on this path')
+    dev = (krons[0].A if krons[0].has_A else krons[0].B).device
+    A_list = [k.A if k.has_A else k.B for k in krons]
+    B_list = [k.B if k.has_B else k.A for k in krons]
+    A_list = [a if a.is_contiguous() else a.contiguous() for a in A_list]
+    B_list = [b if b.is_contiguous() else b.contiguous() for b in B_list]
+    lam, nonzero = kernels.kron_damping(A_list, B_list, float(damping), float(eps))
+    single = [i for i, k in enumerate(krons) if not (k.has_A and k.has_B)]
+    if single:
+        lam[torch.tensor(single, device=dev)] = float(damping)      # no pi split without both factors
+    lam_flat, nz_flat = lam.view(-1), nonzero.view(-1)
+
+    groups = defaultdict(list)   # d -> [(flat index, matrix, kron, 'A'|'B')]
+    for i, k in enumerate(krons):
+        if calc_A_inv:
+            groups[A_list[i].shape[0]].append((2 * i, A_list[i], k, 'A'))
+        if calc_B_inv:
+            groups[B_list[i].shape[0]].append((2 * i + 1, B_list[i], k, 'B'))
+    infos, records = [], []
+    for d in sorted(groups, reverse=True):
+        entries = groups[d]
+        idx = torch.tensor([e[0] for e in entries], device=dev)
+        outs = []
+        for _, mat, k, which in entries:
+            old = getattr(k, which + '_inv')
+            reuse = old is not None and old.shape == mat.shape and old.is_contiguous() and old.dtype == mat.dtype
+            outs.append(old if reuse else torch.empty_like(mat))
+        info = kernels.chol_inv_batched([e[1] for e in entries], outs, lam_flat[idx], 1,
+                                        active=nz_flat[idx].contiguous(), active_stride=1)
+        infos.append(info)
+        records.extend((e[0], e[2], e[3], out) for e, out in zip(entries, outs))
+    host = torch.cat(infos + [nz_flat]).cpu().tolist()        # the one synchronisation
+    info_host, nz_host = host[:len(records)], host[len(records):]
+    for (flat, k, which, out), inf in zip(records, info_host):
+        if not nz_host[flat]:
+            continue                                            # all-zero factor: inverse skipped
+        if inf != 0:
+            raise torch.linalg.LinAlgError(
+                f'cholesky_inv: the leading minor of order {inf} of kron.{which} + damping is not positive-definite')
+        setattr(k, which + '_inv', out)
+        if replace:
+            setattr(k, which, None)
+
+
+class Kron:
+    def __init__(self, A, B, A_inv=None, B_inv=None):
+        self.A: Tensor = A
+        self.B: Tensor = B
+        self.A_inv: Tensor = A_inv
+        self.B_inv: Tensor = B_inv
+        self._A_dim = self._B_dim = None
+
+    def __add__(self, other):
+        if not other.has_data:
+            return self
+        A = (self.A.add(other.A) if self.has_A else other.A) if other.has_A else self.A
+        B = (self.B.add(other.B) if self.has_B else other.B) if other.has_B else self.B
+        return Kron(A, B)
+
+    def __iadd__(self, other):
+        if not other.has_data:
+            return self
+        if other.has_A:
+            if self.has_A:
+                self.A.add_(other.A)
+            else:
+                self.A = other.A
+        if other.has_B:
+            if self.has_B:
+                self.B.add_(other.B)
+            else:
+                self.B = other.B
+        return self
+
+    @property
+    def data(self):
+        return [self.A, self.B]
+
+    @property
+    def has_data(self):
+        return self.has_A or self.has_B
+
+    @property
+    def has_A(self):
+        return self.A is not None
+
+    @property
+    def has_B(self):
+        return self.B is not None
+
+    @property
+    def has_inv(self):
+        return self.A_inv is not None and self.B_inv is not None
+
+    @property
+    def A_dim(self):
+        if self._A_dim is None:
+            if self.A is not None:
+                self._A_dim = self.A.shape[-1]
+            elif self.A_inv is not None:
+                self._A_dim = self.A_inv.shape[-1]
+            else:
+                raise ValueError('A nor A_inv has not been set.')
+        return self._A_dim
+
+    @property
+    def B_dim(self):
+        if self._B_dim is None:
+            if self.B is not None:
+                self._B_dim = self.B.shape[-1]
+            elif self.B_inv is not None:
+                self._B_dim = self.B_inv.shape[-1]
+            else:
+                raise ValueError('B nor B_inv has not been set.')
+        return self._B_dim
+
+    def mul_(self, value):
+        if self.has_A:
+            self.A.mul_(value)
+        if self.has_B:
+            self.B.mul_(value)
+        return self
+
+    def trace(self):
+        return torch.diag(self.A).sum().item() * torch.diag(self.B).sum().item()
+
+    def update_inv(self, damping=_default_damping, calc_A_inv=True, calc_B_inv=True, eps=1e-7, replace=False):
+        batched_update_inv([self], damping, calc_A_inv, calc_B_inv, eps, replace)
+
+    def mvp(self, vec_weight, vec_bias=None, use_inv=False, inplace=False):
+        """B G A (or B^-1 G A^-1) on a weight gradient viewed as [B_dim, -1], and B b on the bias
+        (asdl/symmatrix.py:536-548)."""
+        mat_A = self.A_inv if use_inv else self.A
+        mat_B = self.B_inv if use_inv else self.B
+        direct = inplace and vec_weight.is_contiguous() and vec_weight.dtype == torch.float32
+        w = vec_weight if direct else vec_weight.detach().to(torch.float32).contiguous().clone()
+        b = None
+        if vec_bias is not None:
+            direct_b = inplace and vec_bias.is_contiguous() and vec_bias.dtype == torch.float32
+            b = vec_bias if direct_b else vec_bias.detach().to(torch.float32).contiguous().clone()
+        kernels.kron_precond(mat_B, mat_A, w.data, b.data if b is not None else None, 1.0)
+        if inplace and w is not vec_weight:
+            vec_weight.copy_(w)
+        if vec_bias is not None:
+            if inplace and b is not vec_bias:
+                vec_bias.copy_(b)
+            return w, b
+        return w
+
+
+class SymMatrix:
+    def __init__(self, data=None, inv=None, kron=None, kfe=None, diag=None, unit=None,
+                 kron_A=None, kron_B=None, kron_A_inv=None, kron_B_inv=None):
+        self.data: Tensor = data
+        self.inv: Tensor = inv
+        if not _is_all_none([kron_A, kron_B, kron_A_inv, kron_B_inv]):
+            self.kron = Kron(kron_A, kron_B, kron_A_inv, kron_B_inv)
+        else:
+            self.kron: Kron = kron
+        self.kfe = kfe
+        self.diag = diag
+        self.unit = unit
+
+    def __repr__(self):
+        parts = []
+        if self.has_kron:
+            for key in ('A', 'B', 'A_inv', 'B_inv'):
+                v = getattr(self.kron, key)
+                if v is not None:
+                    parts.append(f'kron.{key} {tuple(v.shape)}')
+        return 'SymMatrix(' + ', '.join(parts) + ')'
+
+    @property
+    def has_data(self):
+        return self.data is not None
+
+    @property
+    def has_kron(self):
+        return self.kron is not None
+
+    @property
+    def has_kfe(self):
+        return self.kfe is not None
+
+    @property
+    def has_diag(self):
+        return self.diag is not None
+
+    @property
+    def has_unit(self):
+        return self.unit is not None
+
+    def _only_kron(self, what):
+        if self.has_data or self.has_kfe or self.has_diag or self.has_unit:
+            raise NotImplementedError(f'{what}: only the Kronecker-factored shape is on this path')
+
+    def __iadd__(self, other):
+        self._only_kron('__iadd__')
+        if other.kron is not None:
+            if self.kron is not None:
+                self.kron += other.kron
+            else:
+                self.kron = other.kron
+        return self
+
+    def mul_(self, value):
+        self._only_kron('mul_')
+        if self.has_kron:
+            self.kron.mul_(value)
+        return self
+
+    def update_inv(self, damping=_default_damping, replace=False):
+        self._only_kron('update_inv')
+        if self.has_kron:
+            self.kron.update_inv(damping, replace=replace)
+
+    def mvp(self, vectors=None, vec_weight=None, vec_bias=None, use_inv=False, inplace=False):
+        raise NotImplementedError('SymMatrix.mvp with a full / layer-wise matrix is not on this path; '
+                                  'use SymMatrix.kron.mvp')

@@ -1,0 +1,169 @@
+"""Headline benchmark: full K-FAC steps per second on ResNet-50, batch 64, one MI355X.
+
+A step = optimizer.zero_grad(); setup_model_call; setup_loss_call; KfacGradientMaker
+.forward_and_backward() (forward, Monte-Carlo Fisher backward with the factor kernels in its hooks,
+pi-damped inverses of all 54 layers, loss backward, preconditioning of every gradient);
+optimizer.step().  bf16 autocast forward/backward, fp32 factors and inverses, factors refreshed every
+step, BatchNorm excluded (Conv2d + Linear only).  Inputs are synthetic N(0,1) images resident in HBM.
+
+Prints ONE JSON line; see --help for the knobs.  The `roofline` object is for the dominant kernel
+family (the factor-statistics SYRK kernels): algorithmic FLOP M*d*(d+1) per launch summed over the
+108 launches of a step, divided by their summed durations measured with events on the launching
+stream inside the timed steps.  `cpu_baseline` times the CPU oracle's K-FAC step (same formulas in
+PyTorch CPU ops) on the host cores of the same box.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+BF16_MFMA_PEAK_TFLOPS = 2500.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--batch', type=int, default=64)
+    ap.add_argument('--fisher', default='fisher_mc', choices=['fisher_mc', 'fisher_emp'])
+    ap.add_argument('--damping', type=float, default=1e-3)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--cpu-batch', type=int, default=16,
+                    help='batch of the CPU baseline sample (its time is scaled to the full batch)')
+    ap.add_argument('--no-factor-timing', action='store_true')
+    return ap.parse_args()
+
+
+def cpu_baseline(args):
+    """One K-FAC step of the CPU oracle on a bounded sample; returns the cpu_baseline object."""
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import bench_models
+    from oracle import cpu_ref
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    model = bench_models.resnet50()
+    bs = args.cpu_batch
+    x = torch.randn(bs, 3, 224, 224)
+    t = torch.randint(0, 1000, (bs,))
+
+    def fwd(inp):
+        with torch.autocast('cpu', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    class Wrapped:
+        def __call__(self, inp):
+            return fwd(inp)
+
+        def parameters(self):
+            return model.parameters()
+
+    orc = cpu_ref.KfacOracle(model, data_size=bs, damping=args.damping, fisher_type=args.fisher,
+                             factor_dtype=torch.float32)
+    orc.model = Wrapped()
+    t0 = time.time()
+    orc.forward_and_backward(x, t)
+    dt = time.time() - t0
+    # forward/backward and factor statistics scale with the batch, inverses and preconditioning do not;
+    # scaling the whole sample linearly therefore over-estimates the CPU time per full step only slightly
+    # less than proportionally -- reported as measured on the sample, and scaled, both.
+    scaled = dt * args.batch / bs
+    return {'value': 1.0 / scaled, 'unit': 'steps/s', 'cores': cores, 'kind': 'port',
+            'sample': f'one K-FAC step of the CPU oracle on ResNet-50 at batch {bs} took {dt:.1f} s; '
+                      f'value = 1 / (that time x {args.batch}/{bs})'}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f'bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}).',
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import bench_models
+    from asdl_amd import PreconditioningConfig, KfacGradientMaker, kernels
+
+    if not torch.cuda.is_available():
+        print('bench.py needs a ROCm GPU.', file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device('cuda:0')
+    torch.manual_seed(0)
+    model = bench_models.resnet50().to(dev)
+    bs = args.batch
+    x = torch.randn(bs, 3, 224, 224).to(dev)
+    t = torch.randint(0, 1000, (bs,)).to(dev)
+    config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=[nn.BatchNorm2d])
+    gm = KfacGradientMaker(model, config, fisher_type=args.fisher)
+    opt = torch.optim.SGD(model.parameters(), lr=1e-4)
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        dummy_y = gm.setup_model_call(fwd, x)
+        gm.setup_loss_call(F.cross_entropy, dummy_y, t)
+        gm.forward_and_backward()
+        opt.step()
+
+    for _ in range(args.warmup):
+        step()
+    sink = None if args.no_factor_timing else []
+    kernels.set_timing_sink(sink)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernels.set_timing_sink(None)
+
+    ms_per_step = elapsed / args.steps * 1e3
+    out = {
+        'metric': 'K-FAC steps/s ResNet-50 bs64',
+        'value': args.steps / elapsed,
+        'unit': 'steps/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': ms_per_step,
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'bf16',
+        'data': 'synthetic',
+        'config': {'workload': f'K-FAC step (factors + pi-damped Cholesky inverses + precondition every step, '
+                               f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
+                               f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
+                               f'BatchNorm ignored',
+                   'batch': bs},
+    }
+    if sink:
+        flops = sum(s[1] for s in sink)
+        secs = sum(s[2].elapsed_time(s[3]) for s in sink) * 1e-3
+        achieved = flops / secs / 1e12
+        out['roofline'] = {'bound': 'mfma', 'achieved': achieved, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
+                           'frac': achieved / BF16_MFMA_PEAK_TFLOPS, 'traffic': None,
+                           'kernel': 'factor statistics (conv_syrk_kernel / syrk_tn_kernel), SYRK FLOP M*d*(d+1)',
+                           'launches_per_step': len(sink) // args.steps,
+                           'factor_ms_per_step': secs / args.steps * 1e3,
+                           'gemm_equiv_tflops': 2 * achieved}
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline(args)
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

@@ -123,16 +123,19 @@ int ak_kron_precond(const float* Binv, const float* Ainv, float* G, int64_t dB, 
 
 /* ---- Shampoo inverse p-th root ---------------------------------------------------- */
 
-/* out <- (S + r I)^(-1/p), r = ridge_eps * lambda_max(S), by power iteration from start vector v0
- * followed by the coupled Newton iteration; S (n x n fp32 dense) keeps the ridge on exit, as in
- * the reference.  Convergence tests run on the device: once the error is below tol, or grows by
- * more than 1.2x (then the previous root is kept), the remaining launches return immediately.
- * stats: device float [4] = {lambda_max, power iterations, newton iterations, final error}.
+/* out_b <- (S_b + r_b I)^(-1/p), r_b = ridge_eps * lambda_max(S_b), for a batch of n x n fp32 statistics
+ * (S_b = S + b*strideS, out_b = out + b*strideOut, dense rows): power iteration from the start vectors
+ * v0 [batch, n] (the reference draws them from U(-1, 1)), then the coupled Newton iteration.  S_b keeps
+ * the ridge on exit, as in the reference.  Convergence tests run on the device: once a matrix's error is
+ * below tol, or grows by more than 1.2x (then its previous root is kept), the remaining launches return
+ * immediately for it.  stats: device float [batch, 4] = {lambda_max, power iterations, newton iterations,
+ * final error}.  n >= 2 (the reference returns the identity for n == 1 without any arithmetic).
  * Replaces ComputePower / PowerIter / MatPower (asdl/precondition/shampoo.py:465-586). */
-size_t ak_inv_root_ws_bytes(int64_t n);
-int ak_inv_root_newton(float* S, int64_t n, int p, float ridge_eps, const float* v0,
-                       int max_power_iter, float power_tol, int max_iter, float tol,
-                       float* out, float* stats, void* ws, size_t ws_bytes, ak_stream_t stream);
+size_t ak_inv_root_ws_bytes(int64_t n, int batch);
+int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
+                       const float* v0, int max_power_iter, float power_tol, int max_iter, float tol,
+                       float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
+                       ak_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,86 @@
+"""Test-only stand-ins for asdl_amd.kernels built on the CPU oracle, so that the host logic
+(hooks, schedules, result store, batching) can be exercised without a GPU.  Installed with
+pytest's monkeypatch; the product never imports this file."""
+import torch
+
+from oracle import cpu_ref as R
+
+
+def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
+    val = alpha * R.linear_cov_kron_A(x.float())
+    if out is None:
+        return val
+    out.copy_(val if beta == 0 else beta * out + val)
+    return out
+
+
+def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
+    col = R.im2col_2d(x.float(), kernel_size, stride, padding)
+    m = col.transpose(0, 1).flatten(start_dim=1)
+    val = alpha * (m @ m.T)
+    if out is None:
+        return val
+    out.copy_(val if beta == 0 else beta * out + val)
+    return out
+
+
+def syrk_nt(x, out=None, alpha=1.0, beta=0.0):
+    if x.ndim == 2:
+        x = x.unsqueeze(0)
+    m = x.float().transpose(0, 1).flatten(start_dim=1)
+    val = alpha * (m @ m.T)
+    if out is None:
+        return val
+    out.copy_(val if beta == 0 else beta * out + val)
+    return out
+
+
+def kron_damping(A_list, B_list, damping, eps=1e-7):
+    lam = torch.empty(len(A_list), 2)
+    nz = torch.empty(len(A_list), 2, dtype=torch.int32)
+    for i, (A, B) in enumerate(zip(A_list, B_list)):
+        lam[i, 0], lam[i, 1] = R.kron_damping(A, B, damping, eps)
+        nz[i, 0] = int(not bool(torch.all(A == 0)))
+        nz[i, 1] = int(not bool(torch.all(B == 0)))
+    return lam, nz
+
+
+def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1, info=None):
+    info = torch.zeros(len(mats), dtype=torch.int32)
+    for b, (m, o) in enumerate(zip(mats, outs)):
+        if active is not None and int(active[b * active_stride]) == 0:
+            continue
+        try:
+            o.copy_(R.cholesky_inv(m, float(lam[b * lam_stride])))
+        except torch.linalg.LinAlgError:
+            info[b] = 1
+    return info
+
+
+def cholesky_inv(X, damping=1e-7):
+    return R.cholesky_inv(X, damping)
+
+
+def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
+    if grad_b is not None:
+        w, b = R.kron_mvp(A_inv, B_inv, grad_w, grad_b)
+        grad_b.copy_(grad_scale * b)
+    else:
+        w = R.kron_mvp(A_inv, B_inv, grad_w)
+    grad_w.copy_(grad_scale * w)
+    return grad_w, grad_b
+
+
+def gemm(A, B, out=None, transA=False, transB=False, alpha=1.0, beta=0.0):
+    val = alpha * ((A.T if transA else A) @ (B.T if transB else B))
+    if out is None:
+        return val
+    out.copy_(val if beta == 0 else beta * out + val)
+    return out
+
+
+def install(monkeypatch):
+    from asdl_amd import kernels
+    for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'cholesky_inv',
+                 'kron_precond', 'gemm']:
+        monkeypatch.setattr(kernels, name, globals()[name])

@@ -1,0 +1,251 @@
+"""Host logic on the CPU: the GradientMaker API, schedules, the hook engine and the K-FAC
+orchestration, with the kernel entry points replaced by oracle-backed stand-ins
+(tests/cpu_backend.py).  Also checks that the C-ABI library loads and exports every declared symbol
+and that the product refuses CPU tensors."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import asdl_amd
+from asdl_amd import (PreconditioningConfig, KfacGradientMaker, GradientMaker, FisherConfig, get_fisher_maker,
+                      get_update_schedule, SHAPE_KRON, FISHER_EMP, FISHER_MC, FISHER_EXACT, LOSS_CROSS_ENTROPY, LOSS_MSE)
+from conftest import GOLDEN
+from models_small import GOLDEN_KFAC, get_mlp, get_cnn
+import cpu_backend
+
+
+def relerr(a, b):
+    return float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-300))
+
+
+# ------------------------------------------------------------------ library / boundary
+def test_library_loads_and_exports_every_declared_symbol():
+    from asdl_amd import _lib
+    lib = _lib.load()
+    declared = _lib.declared_symbols()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), f'{name} is declared in include/asdl_amd.h but not exported'
+        assert name in _lib._SIGNATURES, f'{name} has no ctypes signature'
+    assert lib.ak_version() >= 100
+    assert b'workspace' in lib.ak_error_string(-2)
+
+
+def test_product_refuses_cpu_tensors():
+    from asdl_amd import kernels
+    with pytest.raises(RuntimeError, match='ROCm device'):
+        kernels.syrk_tn(torch.randn(4, 4))
+    with pytest.raises(RuntimeError, match='ROCm device'):
+        kernels.conv_syrk(torch.randn(1, 2, 4, 4), (3, 3), (1, 1), (1, 1))
+    with pytest.raises(RuntimeError, match='ROCm device'):
+        asdl_amd.cholesky_inv(torch.eye(3), 0.1)
+    model = get_mlp()
+    gm = KfacGradientMaker(model, PreconditioningConfig(data_size=2, damping=1e-2), fisher_type=FISHER_EMP)
+    x, t = torch.randn(2, 5), torch.randint(4, (2,))
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+    with pytest.raises(RuntimeError, match='ROCm device'):
+        gm.forward_and_backward()
+
+
+# ------------------------------------------------------------------ GradientMaker API (test/grad_maker/test_grad_maker.py)
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.model = get_mlp()
+
+    def forward(self, inputs, targets=None, flip=False):
+        logits = self.model(inputs)
+        if targets is not None:
+            loss = F.cross_entropy(logits, targets)
+            return (loss, logits) if flip else (logits, loss)
+        return logits
+
+
+def _vanilla(model, x, t):
+    model.zero_grad(set_to_none=True)
+    loss = F.cross_entropy(model(x), t)
+    loss.backward()
+    return loss, [p.grad.clone() for p in model.parameters()]
+
+
+def test_grad_maker_matches_vanilla_autograd_for_every_calling_style():
+    torch.manual_seed(0)
+    model = _Net()
+    x, t = torch.randn(4, 5), torch.randint(4, (4,))
+    ref_loss, ref_grads = _vanilla(model, x, t)
+    gm = GradientMaker(model)
+
+    def check(loss):
+        torch.testing.assert_close(loss, ref_loss)
+        for p, g in zip(model.parameters(), ref_grads):
+            torch.testing.assert_close(p.grad, g)
+
+    model.zero_grad(set_to_none=True)
+    dummy_y = gm.setup_model_call(model, x)
+    gm.setup_loss_call(F.cross_entropy, dummy_y, t)
+    y, loss = gm.forward_and_backward()
+    check(loss)
+    torch.testing.assert_close(y, model(x))
+
+    for flip, idx in [(False, 1), (True, 0)]:
+        model.zero_grad(set_to_none=True)
+        dummy_y = gm.setup_model_call(model, x, targets=t, flip=flip)
+        gm._loss_fn = None
+        gm.setup_loss_repr(dummy_y[idx])
+        y, loss = gm.forward_and_backward()
+        check(loss)
+
+    with pytest.raises(TypeError):
+        gm.setup_loss_repr('not a dummy')
+    with pytest.raises(ValueError):
+        GradientMaker(model).forward_and_backward()
+
+
+def test_dummy_object_replays_attribute_item_and_call():
+    lin = nn.Linear(5, 3)
+    assert asdl_amd.DummyObject().weight[0].numel().eval(lin) == 5
+    d = asdl_amd.DummyObject()
+    assert d['a'][1].eval({'a': [1, 2]}) == 2
+
+
+# ------------------------------------------------------------------ schedules
+def test_update_schedule_and_intervals():
+    s = get_update_schedule(10, update_ratio=0.5)
+    assert len(s) == 10 and sum(s) == 5 and s[0]
+    s = get_update_schedule(10, update_ratio=0.5, warmup_ratio=0.2)
+    assert s[:2] == [True, True] and sum(s) == 5
+    assert get_update_schedule(4, 1.0) == [True] * 4
+    assert get_update_schedule(6, 0.5, interval_type='step') == [True] * 3 + [False] * 3
+    with pytest.raises(ValueError):
+        get_update_schedule(0)
+    with pytest.raises(ValueError):
+        get_update_schedule(10, 1.5)
+    gm = KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1, preconditioner_upd_interval=3,
+                                                            curvature_upd_interval=2, ema_decay=0.1))
+    assert [gm.do_update_preconditioner(s) for s in range(6)] == [True, False, False, True, False, False]
+    assert [gm.do_update_curvature(s) for s in range(4)] == [True, False, True, False]
+    assert gm.state_dict() == {'step': 0}
+    gm.load_state_dict({'step': 5})
+    assert gm.state['step'] == 5
+    gm2 = KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1, num_total_steps=4,
+                                                             preconditioner_upd_ratio=0.5))
+    with pytest.warns(UserWarning):
+        assert gm2.do_update_preconditioner(10) is False
+
+
+def test_config_defaults_match_reference():
+    c = PreconditioningConfig()
+    assert (c.num_total_steps, c.preconditioner_upd_interval, c.preconditioner_warmup_steps) == (None, 1, 0)
+    assert (c.curvature_upd_interval, c.curvature_upd_ratio, c.data_size, c.damping, c.ema_decay) == (None, None, -1, 1e-7, -1)
+    assert c.ignore_modules is None and c.preconditioner_interval_type == 'constant'
+
+
+def test_constructor_errors():
+    from torch.nn.parallel import DistributedDataParallel
+    model = nn.Sequential(nn.Linear(3, 3), nn.BatchNorm1d(3))
+    with pytest.raises(NotImplementedError, match='ignore_modules'):
+        KfacGradientMaker(model, PreconditioningConfig(data_size=1))
+    KfacGradientMaker(model, PreconditioningConfig(data_size=1, ignore_modules=[nn.BatchNorm1d]))
+    with pytest.raises(ValueError):
+        KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1, curvature_upd_ratio=0.5, num_total_steps=10))
+    gm = KfacGradientMaker(get_mlp(), PreconditioningConfig())
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(gm.model, torch.randn(2, 5)), torch.zeros(2, dtype=torch.long))
+    with pytest.raises(ValueError, match='data_size'):
+        gm.forward_and_backward()
+
+
+# ------------------------------------------------------------------ K-FAC orchestration vs the reference's golden runs
+@pytest.mark.parametrize('tag', sorted(GOLDEN_KFAC))
+def test_kfac_host_logic_matches_reference_golden(tag, monkeypatch):
+    cpu_backend.install(monkeypatch)
+    factory, fisher_type, ema, damping, seed, ci, pi = GOLDEN_KFAC[tag]
+    z = np.load(os.path.join(GOLDEN, f'kfac_{tag}.npz'))
+    model = factory()
+    model.load_state_dict({k[len('init/'):]: torch.from_numpy(z[k]) for k in z.files if k.startswith('init/')})
+    bs = z['step0/x'].shape[0]
+    config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema, curvature_upd_interval=ci,
+                                   preconditioner_upd_interval=pi)
+    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
+    for step in range(n_steps):
+        opt.zero_grad(set_to_none=True)
+        x, t = torch.from_numpy(z[f'step{step}/x']), torch.from_numpy(z[f'step{step}/t'])
+        dummy_y = gm.setup_model_call(model, x)
+        gm.setup_loss_call(F.cross_entropy, dummy_y, t)
+        y, loss = gm.forward_and_backward()
+        torch.testing.assert_close(loss, torch.from_numpy(z[f'step{step}/loss']), rtol=1e-5, atol=1e-6)
+        for name, p in model.named_parameters():
+            assert relerr(p.grad, torch.from_numpy(z[f'step{step}/grad/{name}'])) < 2e-4, (tag, step, name)
+        for key in z.files:
+            if key.startswith(f'step{step}/kron/'):
+                _, _, mname, which = key.split('/')
+                got = getattr(model.get_submodule(mname).fisher.kron, which)
+                assert got is not None, key
+                assert relerr(got, torch.from_numpy(z[key])) < 2e-4, key
+        for name, m in model.named_modules():
+            if isinstance(m, (nn.Linear, nn.Conv2d)) and ema == -1:
+                assert m.fisher.kron.A is None and m.fisher.kron.B is None    # only inverses are kept
+        opt.step()
+    assert gm.state_dict() == {'step': n_steps}
+
+
+# ------------------------------------------------------------------ FisherMaker invariants (test/grad_maker/test_fisher.py)
+@pytest.mark.parametrize('network', ['mlp', 'cnn'])
+@pytest.mark.parametrize('fisher_type', [FISHER_EMP, FISHER_MC, FISHER_EXACT])
+@pytest.mark.parametrize('loss_type', [LOSS_CROSS_ENTROPY, LOSS_MSE])
+def test_fisher_maker_invariants(network, fisher_type, loss_type, monkeypatch):
+    cpu_backend.install(monkeypatch)
+    torch.manual_seed(0)
+    model = get_mlp() if network == 'mlp' else get_cnn()
+    bs = 4
+    x = torch.randn(bs, 5) if network == 'mlp' else torch.randn(bs, 5, 4, 4)
+    t = torch.randint(4, (bs,)) if loss_type == LOSS_CROSS_ENTROPY else torch.randn(bs, 4)
+    loss_fn = F.cross_entropy if loss_type == LOSS_CROSS_ENTROPY else F.mse_loss
+    fm = get_fisher_maker(model, FisherConfig(fisher_type=fisher_type, fisher_shapes=[SHAPE_KRON], data_size=1,
+                                              loss_type=loss_type, seed=1))
+    fm.setup_loss_call(loss_fn, fm.setup_model_call(model, x), t)
+    mods = [m for m in model.modules() if isinstance(m, (nn.Linear, nn.Conv2d))]
+
+    def snap():
+        return [(m.fisher.kron.A.clone(), m.fisher.kron.B.clone()) for m in mods]
+
+    fm.forward_and_backward()
+    first = snap()
+    for m, (A, B) in zip(mods, first):
+        in_dim = m.in_features if isinstance(m, nn.Linear) else m.in_channels * 4
+        out_dim = m.out_features if isinstance(m, nn.Linear) else m.out_channels
+        assert A.shape == (in_dim, in_dim) and B.shape == (out_dim, out_dim)
+        torch.testing.assert_close(A, A.T)
+        torch.testing.assert_close(B, B.T)
+    for k in [2, 3]:                                     # test_accumulate
+        fm.forward_and_backward(accumulate=True)
+        for (A, B), (A1, B1) in zip(snap(), first):
+            torch.testing.assert_close(A, A1 * k)
+            torch.testing.assert_close(B, B1 * k)
+    fm.forward_and_backward(scale=0.1)                   # test_scale
+    for (A, B), (A1, B1) in zip(snap(), first):
+        torch.testing.assert_close(A, A1 * 0.1)
+    fm.forward_and_backward(data_size=32)                # test_data_size
+    for (A, B), (A1, B1) in zip(snap(), first):
+        torch.testing.assert_close(B, B1 / 32)
+    damping = 1.0                                        # test_inv
+    fm.forward_and_backward(calc_inv=True, damping=damping)
+    for m, (A, B) in zip(mods, first):
+        kron = m.fisher.kron
+        assert kron.A is None and kron.B is None and kron.A_inv is not None and kron.B_inv is not None
+        pi = torch.sqrt((A.trace() / A.shape[0]) / (B.trace() / B.shape[0]))
+        dA, dB = max(damping ** 0.5 * pi, 1e-7), max(damping ** 0.5 / pi, 1e-7)
+        torch.testing.assert_close(torch.eye(A.shape[0]), (A + dA * torch.eye(A.shape[0])) @ kron.A_inv)
+        torch.testing.assert_close(torch.eye(B.shape[0]), (B + dB * torch.eye(B.shape[0])) @ kron.B_inv)
+    N, damping = 10, 10.0                                # test_inv_data_size
+    fm.forward_and_backward(calc_inv=True, damping=damping * N * N)
+    inv1 = [(m.fisher.kron.A_inv.clone(), m.fisher.kron.B_inv.clone()) for m in mods]
+    fm.forward_and_backward(data_size=N, calc_inv=True, damping=damping)
+    for m, (Ai, Bi) in zip(mods, inv1):
+        torch.testing.assert_close(m.fisher.kron.A_inv, Ai * N)
+        torch.testing.assert_close(m.fisher.kron.B_inv, Bi * N)

@@ -1,0 +1,236 @@
+"""End-to-end K-FAC parity on the GPU: KfacGradientMaker (HIP kernels) against the reference's
+golden runs and against the CPU oracle on identical seeded inputs.
+
+Tolerances: inverses 1e-4, preconditioned gradients 1e-3 (relative Frobenius norm); looser only
+where the test says why.
+"""
+import copy
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from asdl_amd import PreconditioningConfig, KfacGradientMaker, FISHER_EMP, FISHER_MC
+from conftest import GOLDEN
+from models_small import GOLDEN_KFAC
+from oracle import cpu_ref as R
+import bench_models
+
+pytestmark = pytest.mark.gpu
+TOL_INV, TOL_GRAD = 1e-4, 1e-3
+
+
+def relerr(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+
+
+@pytest.mark.parametrize('tag', sorted(GOLDEN_KFAC))
+def test_kfac_gpu_matches_reference_golden(tag):
+    factory, fisher_type, ema, damping, seed, ci, pi = GOLDEN_KFAC[tag]
+    z = np.load(os.path.join(GOLDEN, f'kfac_{tag}.npz'))
+    sd = {k[len('init/'):]: torch.from_numpy(z[k]) for k in z.files if k.startswith('init/')}
+    model = factory()
+    model.load_state_dict(sd)
+    bs = z['step0/x'].shape[0]
+    replay = None
+    if fisher_type == FISHER_MC:
+        # the sampled targets depend on the CPU RNG stream: draw them with the oracle and replay them
+        cpu_model = copy.deepcopy(model)
+        orc = R.KfacOracle(cpu_model, data_size=bs, damping=damping, ema_decay=ema, fisher_type=fisher_type, seed=seed,
+                           curvature_upd_interval=ci, preconditioner_upd_interval=pi)
+        cpu_opt = torch.optim.SGD(cpu_model.parameters(), lr=0.05)
+        replay = []
+    model = model.cuda()
+    config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema, curvature_upd_interval=ci,
+                                   preconditioner_upd_interval=pi)
+    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
+    for step in range(n_steps):
+        x, t = torch.from_numpy(z[f'step{step}/x']), torch.from_numpy(z[f'step{step}/t'])
+        if replay is not None:
+            cpu_opt.zero_grad(set_to_none=True)
+            orc.forward_and_backward(x, t)
+            cpu_opt.step()
+            targets = orc.last_mc_targets.cuda()
+            gm.fisher_maker.sample_targets = lambda dist, i, _t=targets: _t
+        opt.zero_grad(set_to_none=True)
+        dummy_y = gm.setup_model_call(model, x.cuda())
+        gm.setup_loss_call(F.cross_entropy, dummy_y, t.cuda())
+        print(f'golden {tag} step {step}', flush=True)
+        y, loss = gm.forward_and_backward()
+        torch.testing.assert_close(loss.cpu(), torch.from_numpy(z[f'step{step}/loss']), rtol=1e-4, atol=1e-5)
+        for key in z.files:
+            if key.startswith(f'step{step}/kron/'):
+                _, _, mname, which = key.split('/')
+                got = getattr(model.get_submodule(mname).fisher.kron, which)
+                assert got is not None, key
+                assert relerr(got, torch.from_numpy(z[key])) < 5e-4, (key, relerr(got, torch.from_numpy(z[key])))
+        for name, p in model.named_parameters():
+            assert relerr(p.grad, torch.from_numpy(z[f'step{step}/grad/{name}'])) < TOL_GRAD, (tag, step, name)
+        opt.step()
+
+
+def _run_pair(model_cpu, x, t, damping, ema=-1, steps=1, autocast=False, fisher_type=FISHER_EMP, tol_grad=TOL_GRAD,
+              tol_inv=TOL_INV, check_inv=True):
+    """Runs the product on the GPU and the oracle on the CPU on identical inputs; returns max errors."""
+    bs = x.shape[0]
+    model_gpu = copy.deepcopy(model_cpu).cuda()
+    ignore = [nn.BatchNorm2d, nn.BatchNorm1d, nn.LayerNorm]
+    config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema, ignore_modules=ignore)
+    gm = KfacGradientMaker(model_gpu, config, fisher_type=fisher_type)
+    orc = R.KfacOracle(model_cpu, data_size=bs, damping=damping, ema_decay=ema, fisher_type=fisher_type,
+                       factor_dtype=torch.float32)
+    worst_g = worst_i = 0.0
+    for step in range(steps):
+        model_cpu.zero_grad(set_to_none=True)
+        model_gpu.zero_grad(set_to_none=True)
+        if autocast:
+            def fwd_cpu(inp):
+                with torch.autocast('cpu', dtype=torch.bfloat16):
+                    return model_cpu(inp).float()
+
+            def fwd_gpu(inp):
+                with torch.autocast('cuda', dtype=torch.bfloat16):
+                    return model_gpu(inp).float()
+        else:
+            fwd_cpu, fwd_gpu = model_cpu, model_gpu
+        y_ref, loss_ref = _oracle_step(orc, fwd_cpu, x, t)
+        dummy_y = gm.setup_model_call(fwd_gpu, x.cuda())
+        gm.setup_loss_call(F.cross_entropy, dummy_y, t.cuda())
+        y, loss = gm.forward_and_backward()
+        assert abs(float(loss) - float(loss_ref)) < 1e-3 * max(1.0, abs(float(loss_ref)))
+        for (name, m_cpu), (_, m_gpu) in zip(model_cpu.named_modules(), model_gpu.named_modules()):
+            if not isinstance(m_cpu, (nn.Linear, nn.Conv2d)):
+                continue
+            if check_inv:
+                for which, store in (('A_inv', orc.A_inv), ('B_inv', orc.B_inv)):
+                    e = relerr(getattr(m_gpu.fisher.kron, which), store[name])
+                    worst_i = max(worst_i, e)
+                    assert e < tol_inv, (name, which, e)
+            for pn, p_cpu in m_cpu.named_parameters(recurse=False):
+                e = relerr(getattr(m_gpu, pn).grad, p_cpu.grad)
+                worst_g = max(worst_g, e)
+                assert e < tol_grad, (name, pn, e)
+    return worst_g, worst_i
+
+
+class _CallableModel:
+    """Lets KfacOracle call an autocast wrapper while still iterating the module's parameters."""
+
+    def __init__(self, module, fn):
+        self._module, self._fn = module, fn
+
+    def __call__(self, x):
+        return self._fn(x)
+
+    def parameters(self):
+        return self._module.parameters()
+
+
+def _oracle_step(orc, fwd, x, t):
+    module = orc.model
+    orc.model = _CallableModel(module, fwd)
+    try:
+        return orc.forward_and_backward(x, t)
+    finally:
+        orc.model = module
+
+
+def test_config1_mlp_784_512_512_10_batch128():
+    torch.manual_seed(0)
+    model = bench_models.mlp()
+    x, t = torch.randn(128, 784), torch.randint(0, 10, (128,))
+    g, i = _run_pair(model, x, t, damping=0.01)
+    print(f'C1 MLP: worst grad err {g:.2e}, worst inverse err {i:.2e}', flush=True)
+
+
+def test_config1_mlp_ema_three_steps():
+    torch.manual_seed(1)
+    model = bench_models.mlp()
+    x, t = torch.randn(128, 784), torch.randint(0, 10, (128,))
+    _run_pair(model, x, t, damping=0.01, ema=0.05, steps=3)
+
+
+def test_resnet18_cifar_fp32_small_batch():
+    # config 3 geometry (3x3 convs up to d = 4608, stride-2 and 1x1 shortcuts) at batch 8.
+    # layer4 factors are rank deficient (M = 8*16 < d = 4608): the inverse is compared at 1e-3 because
+    # cond(A + lam I) ~ 1e3..1e4 amplifies fp32 rounding in any algorithm.
+    torch.manual_seed(2)
+    model = bench_models.resnet18_cifar()
+    x, t = torch.randn(8, 3, 32, 32), torch.randint(0, 10, (8,))
+    g, i = _run_pair(model, x, t, damping=1e-3, tol_inv=2e-3, tol_grad=5e-3)
+    print(f'ResNet-18: worst grad err {g:.2e}, worst inverse err {i:.2e}', flush=True)
+
+
+def test_small_cnn_bf16_autocast():
+    # bf16 forward/backward through autocast, fp32 factors accumulated from the bf16 activations.  CPU and GPU
+    # bf16 convolutions round differently, so the oracle is fed the very activations / output gradients the GPU
+    # run produced (captured with extra hooks) and the GPU's raw gradients: same inputs, same formulas.
+    torch.manual_seed(3)
+    model = nn.Sequential(nn.Conv2d(3, 16, 3, 1, 1), nn.ReLU(), nn.Conv2d(16, 32, 3, 2, 1), nn.ReLU(),
+                          nn.Conv2d(32, 32, 1), nn.ReLU(), nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
+    bs, damping = 16, 1e-2
+    x, t = torch.randn(bs, 3, 16, 16).cuda(), torch.randint(0, 10, (bs,)).cuda()
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    layers = [(n, m) for n, m in model.named_modules() if isinstance(m, (nn.Linear, nn.Conv2d))]
+    ins, gouts, handles = {}, {}, []
+    for name, m in layers:
+        def fhook(mod, inp, out, name=name):
+            ins[name] = inp[0].detach()
+            out.register_hook(lambda g, name=name: gouts.__setitem__(name, g.detach()))
+        handles.append(m.register_forward_hook(fhook))
+    # raw (mean-reduced) gradients and captured tensors from a plain step
+    model.zero_grad(set_to_none=True)
+    F.cross_entropy(fwd(x), t).backward()
+    raw = {n: p.grad.detach().clone() for n, p in model.named_parameters()}
+    saw_bf16 = any(v.dtype == torch.bfloat16 for v in ins.values())
+    for h in handles:
+        h.remove()
+    assert saw_bf16, 'autocast should hand bf16 activations to the hooks'
+
+    gm = KfacGradientMaker(model, PreconditioningConfig(data_size=bs, damping=damping), fisher_type=FISHER_EMP)
+    model.zero_grad(set_to_none=True)
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
+    gm.forward_and_backward()
+    for name, m in layers:
+        a = ins[name].float().cpu()
+        g = gouts[name].float().cpu() * bs            # hooks saw the mean-reduced loss; K-FAC uses the summed one
+        if isinstance(m, nn.Conv2d):
+            A = R.conv_cov_kron_A(a, m.kernel_size, m.stride, m.padding) / bs
+            B = R.conv_cov_kron_B(g) / bs
+        else:
+            A, B = R.linear_cov_kron_A(a) / bs, R.linear_cov_kron_B(g) / bs
+        A_inv, B_inv = R.kron_update_inv(A, B, damping)
+        assert relerr(m.fisher.kron.A_inv, A_inv) < TOL_INV, (name, relerr(m.fisher.kron.A_inv, A_inv))
+        assert relerr(m.fisher.kron.B_inv, B_inv) < 5e-3, (name, relerr(m.fisher.kron.B_inv, B_inv))
+        w, b = R.kron_mvp(A_inv, B_inv, raw[name + '.weight'].cpu(), raw[name + '.bias'].cpu())
+        assert relerr(m.weight.grad, w) < 1e-2, (name, relerr(m.weight.grad, w))
+        assert relerr(m.bias.grad, b) < 1e-2
+
+
+def test_fisher_attributes_and_steps_without_curvature_update():
+    torch.manual_seed(4)
+    model = bench_models.mlp(20, 16, 5).cuda()
+    config = PreconditioningConfig(data_size=8, damping=1e-2, preconditioner_upd_interval=2)
+    gm = KfacGradientMaker(model, config, fisher_type=FISHER_EMP)
+    x, t = torch.randn(8, 20).cuda(), torch.randint(0, 5, (8,)).cuda()
+    invs = []
+    for step in range(3):
+        model.zero_grad(set_to_none=True)
+        gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+        y, loss = gm.forward_and_backward()
+        kron = model[0].fisher.kron
+        assert kron.A is None and kron.B is None and kron.has_inv
+        assert kron.A_inv.shape == (20, 20) and kron.B_inv.shape == (16, 16) and kron.A_inv.is_cuda
+        invs.append(kron.A_inv.clone())
+    assert torch.equal(invs[0], invs[1])            # step 1 reuses the stale inverse
+    assert gm.state_dict() == {'step': 3}
