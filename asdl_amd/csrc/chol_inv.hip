@@ -1,7 +1,7 @@
 // out <- (A + lam I)^-1 for a batch of same-size symmetric positive definite fp32 matrices.
 //
 // Recursive blocked Cholesky that carries the triangular inverse along:
-//   F(lo, hi): n <= 64  -> one wave factors the block in registers and inverts the factor.
+//   F(lo, hi): n <= 128 -> one work group factors the block in LDS and inverts the factor.
 //              otherwise, with [lo,mid) / [mid,hi) and M11 = L11^-1 already in place,
 //                T1  = A21 M11^T            (= L21; the triangular solve is a product)
 //                A22 -= T1 T1^T             (lower triangle only)
@@ -17,7 +17,7 @@
 
 namespace ak {
 
-constexpr int LEAF = 64;
+constexpr int LEAF = 128;
 
 struct BatchPtrs {
   const float* const* A_list;
@@ -52,59 +52,159 @@ __device__ __forceinline__ float lane_bcast(float v, int src_lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
 }
 
-// One wave per matrix: Cholesky of the n x n (n <= 64) diagonal block at `lo`, then its triangular
-// inverse, both in registers.  Lane i owns row i of the block.  On exit the block holds
-// L^-1 in its lower triangle and zeros above the diagonal.
-static __global__ __launch_bounds__(64) void chol_leaf_kernel(float* __restrict__ W, int64_t strideW, int64_t d, int lo,
-                                                              int n, int* __restrict__ info, const int* active,
-                                                              int active_stride) {
-  const int z = blockIdx.x;
-  if (active != nullptr && active[static_cast<int64_t>(z) * active_stride] == 0) return;
-  const int lane = threadIdx.x;
-  float* __restrict__ blk = W + z * strideW + static_cast<int64_t>(lo) * d + lo;
-  float a[LEAF];
-#pragma unroll
-  for (int j = 0; j < LEAF; ++j) {
-    float v = (j == lane) ? 1.f : 0.f;           // identity padding beyond n
-    if (lane < n && j <= lane) v = blk[static_cast<int64_t>(lane) * d + j];
-    a[j] = v;
-  }
+constexpr int PB = 16;              // panel width inside a leaf
+constexpr int LLD = LEAF + 1;       // LDS leading dimension (bank-conflict free columns)
+constexpr int LEAF_THREADS = 1024;
+constexpr int LEAF_BLOCKS = LEAF / PB;
+constexpr size_t LEAF_LDS_BYTES = (2 * LEAF * LLD + LEAF_BLOCKS * PB * (PB + 1) + 8) * sizeof(float);
+
+// Cholesky factor and its inverse of a PB x PB block held one row per lane (lanes >= PB carry an identity
+// row).  On exit a[] is row `lane` of L and m[] is column `lane` of L^-1.  Returns 0 or the 1-based index of
+// the first non-positive pivot.
+__device__ __forceinline__ int small_chol_inv(float (&a)[PB], float (&m)[PB], int lane) {
   int bad = 0;
-  float inv_diag[LEAF];
+  float inv_diag[PB];
 #pragma unroll
-  for (int k = 0; k < LEAF; ++k) {
+  for (int k = 0; k < PB; ++k) {
     float akk = lane_bcast(a[k], k);
-    if (!(akk > 0.f)) {                           // also catches NaN
+    if (!(akk > 0.f)) {             // also catches NaN
       if (bad == 0) bad = k + 1;
       akk = 1.f;
     }
-    const float lkk = sqrtf(akk);
-    const float inv = 1.0f / lkk;
+    float inv = __builtin_amdgcn_rsqf(akk);                 // hardware rsqrt, then one Newton step:
+    inv = inv * (1.5f - 0.5f * akk * inv * inv);             // keeps the serial pivot chain short
+    const float lkk = akk * inv;
     inv_diag[k] = inv;
     a[k] = (lane > k) ? a[k] * inv : ((lane == k) ? lkk : a[k]);
 #pragma unroll
-    for (int j = k + 1; j < LEAF; ++j) {
+    for (int j = k + 1; j < PB; ++j) {
       const float ljk = lane_bcast(a[k], j);
       a[j] = (lane >= j) ? a[j] - a[k] * ljk : a[j];
     }
   }
-  if (bad != 0 && bad <= n && lane == 0 && info[z] == 0) info[z] = lo + bad;
-  // column `lane` of M = L^-1 by forward substitution down the rows
-  float m[LEAF];
 #pragma unroll
-  for (int i = 0; i < LEAF; ++i) {
+  for (int i = 0; i < PB; ++i) {   // column `lane` of L^-1 by forward substitution down the rows
     float s = (lane == i) ? 1.f : 0.f;
 #pragma unroll
-    for (int k = 0; k < i; ++k) {
-      const float lik = lane_bcast(a[k], i);
-      s -= lik * m[k];
-    }
+    for (int k = 0; k < i; ++k) s -= lane_bcast(a[k], i) * m[k];
     m[i] = (lane <= i) ? s * inv_diag[i] : 0.f;
   }
-  if (lane < n) {
+  return bad;
+}
+
+// One work group (16 waves) per matrix: blocked Cholesky of the n x n (n <= LEAF) diagonal block at `lo`,
+// resident in LDS.  Per 16-column panel: the 16 x 16 diagonal block is factored and inverted in registers
+// by one wave; the panel below it (a product with that small inverse) and the trailing update are LDS
+// products spread over all threads.  Then the blocked triangular inverse, one block diagonal at a time.
+// On exit the block holds L^-1 in its lower triangle and zeros above the diagonal.
+static __global__ __launch_bounds__(LEAF_THREADS) void chol_leaf_kernel(float* __restrict__ W, int64_t strideW,
+                                                                        int64_t d, int lo, int n,
+                                                                        int* __restrict__ info, const int* active,
+                                                                        int active_stride) {
+  extern __shared__ __attribute__((aligned(16))) float leaf_smem[];
+  float (*A)[LLD] = reinterpret_cast<float (*)[LLD]>(leaf_smem);
+  float (*Mi)[LLD] = reinterpret_cast<float (*)[LLD]>(leaf_smem + LEAF * LLD);
+  float (*Sc)[PB][PB + 1] = reinterpret_cast<float (*)[PB][PB + 1]>(leaf_smem + 2 * LEAF * LLD);
+  int* s_bad = reinterpret_cast<int*>(leaf_smem + 2 * LEAF * LLD + LEAF_BLOCKS * PB * (PB + 1));
+  const int z = blockIdx.x;
+  if (active != nullptr && active[static_cast<int64_t>(z) * active_stride] == 0) return;
+  const int tid = threadIdx.x;
+  const int np = (n + PB - 1) / PB;        // panels
+  const int npad = np * PB;
+  float* __restrict__ blk = W + z * strideW + static_cast<int64_t>(lo) * d + lo;
+  for (int i = tid >> 7; i < npad; i += LEAF_THREADS / 128) {
+    const int j = tid & 127;
+    if (j < npad) {
+      float v = (i == j) ? 1.f : 0.f;              // identity padding beyond n
+      if (i < n && j < n) v = (j <= i) ? blk[static_cast<int64_t>(i) * d + j] : 0.f;
+      A[i][j] = v;
+      Mi[i][j] = 0.f;
+    }
+  }
+  if (tid == 0) *s_bad = 0;
+  __syncthreads();
+
+#pragma unroll 1
+  for (int pb = 0; pb < np; ++pb) {
+    const int c0 = PB * pb;
+    if (tid < 64) {
+      const int lane = tid;
+      float a[PB], m[PB];
 #pragma unroll
-    for (int i = 0; i < LEAF; ++i)
-      if (i < n) blk[static_cast<int64_t>(i) * d + lane] = m[i];
+      for (int j = 0; j < PB; ++j) a[j] = (lane < PB && j <= lane) ? A[c0 + lane][c0 + j] : ((j == lane) ? 1.f : 0.f);
+      const int bad = small_chol_inv(a, m, lane);
+      if (lane < PB) {
+#pragma unroll
+        for (int j = 0; j < PB; ++j) {
+          if (j <= lane) A[c0 + lane][c0 + j] = a[j];
+          Sc[0][j][lane] = m[j];
+          Mi[c0 + j][c0 + lane] = m[j];
+        }
+      }
+      if (lane == 0 && bad != 0 && *s_bad == 0) *s_bad = c0 + bad;
+    }
+    __syncthreads();
+    const int r0 = c0 + PB;
+    const int nrows = npad - r0;
+    if (nrows > 0) {
+      float res[2] = {0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {               // panel below: A_below * Wd^T  (Wd = Sc[0])
+        const int i = r0 + (tid >> 4) + 64 * t, j = tid & 15;
+        if (i < npad) {
+          float acc = 0.f;
+#pragma unroll
+          for (int k = 0; k < PB; ++k) acc += A[i][c0 + k] * Sc[0][j][k];
+          res[t] = acc;
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int i = r0 + (tid >> 4) + 64 * t;
+        if (i < npad) A[i][c0 + (tid & 15)] = res[t];
+      }
+      __syncthreads();
+      const int j = r0 + (tid & 127);
+      for (int i = r0 + (tid >> 7); i < npad; i += LEAF_THREADS / 128) {   // trailing update, lower triangle
+        if (j <= i) {
+          float acc = 0.f;
+#pragma unroll
+          for (int k = 0; k < PB; ++k) acc += A[i][c0 + k] * A[j][c0 + k];
+          A[i][j] -= acc;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  if (tid == 0 && *s_bad != 0 && *s_bad <= n && info[z] == 0) info[z] = lo + *s_bad;
+
+  // blocked triangular inverse: block (bi, bj), bi > bj, is -W_ii * sum_{bj <= kb < bi} L_{bi,kb} M_{kb,bj};
+  // all blocks of one block diagonal are independent.
+#pragma unroll 1
+  for (int dist = 1; dist < np; ++dist) {
+    const int nb = np - dist;
+    for (int e = tid; e < nb * PB * PB; e += LEAF_THREADS) {
+      const int bj = e >> 8, ty = (e >> 4) & 15, tx = e & 15, bi = bj + dist;
+      float acc = 0.f;
+      for (int kb = bj; kb < bi; ++kb)
+#pragma unroll
+        for (int k = 0; k < PB; ++k) acc += A[PB * bi + ty][PB * kb + k] * Mi[PB * kb + k][PB * bj + tx];
+      Sc[bj][ty][tx] = acc;
+    }
+    __syncthreads();
+    for (int e = tid; e < nb * PB * PB; e += LEAF_THREADS) {
+      const int bj = e >> 8, ty = (e >> 4) & 15, tx = e & 15, bi = bj + dist;
+      float r = 0.f;
+#pragma unroll
+      for (int k = 0; k < PB; ++k) r += Mi[PB * bi + ty][PB * bi + k] * Sc[bj][k][tx];
+      Mi[PB * bi + ty][PB * bj + tx] = -r;
+    }
+    __syncthreads();
+  }
+  for (int i = tid >> 7; i < n; i += LEAF_THREADS / 128) {
+    const int j = tid & 127;
+    if (j < n) blk[static_cast<int64_t>(i) * d + j] = (j <= i) ? Mi[i][j] : 0.f;
   }
 }
 
@@ -131,8 +231,8 @@ static void run_gemm(CholCtx& c, GemmParams p) {
 static void factor_range(CholCtx& c, int lo, int hi, int64_t t1_off) {
   const int n = hi - lo;
   if (n <= LEAF) {
-    hipLaunchKernelGGL(chol_leaf_kernel, dim3(c.batch), dim3(64), 0, c.stream, c.W, c.strideW, c.d, lo, n, c.info,
-                       c.active, c.active_stride);
+    hipLaunchKernelGGL(chol_leaf_kernel, dim3(c.batch), dim3(LEAF_THREADS), LEAF_LDS_BYTES, c.stream, c.W, c.strideW,
+                       c.d, lo, n, c.info, c.active, c.active_stride);
     return;
   }
   const int nb = (n + LEAF - 1) / LEAF;
@@ -207,6 +307,13 @@ extern "C" int ak_chol_inv_batched(const float* const* A_list, float* const* out
   c.active = skip_flags; c.active_stride = skip_stride;
   c.stream = static_cast<hipStream_t>(stream);
   c.rc = AK_OK;
+  static bool leaf_attr_set = false;     // idempotent; a benign race sets it twice at worst
+  if (!leaf_attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(chol_leaf_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(LEAF_LDS_BYTES)) != hipSuccess)
+      return AK_ERR_LAUNCH;
+    leaf_attr_set = true;
+  }
   BatchPtrs bp{A_list, skip_flags, skip_stride};
   dim3 grid(static_cast<unsigned>((d + 15) / 16), static_cast<unsigned>((d + 63) / 64), batch);
   hipLaunchKernelGGL(chol_copy_in_kernel, grid, dim3(256), 0, c.stream, bp, c.W, c.strideW, d, lam, lam_stride, info);

@@ -122,8 +122,9 @@ __device__ __forceinline__ void add_partial(floatx16 (&acc)[TI][TJ], const float
       }
 }
 
-// Sums the split-K partials of every upper tile and applies the symmetric epilogue.
-// grid.x = number of upper tiles, 256 threads.
+// Sums the split-K partials and applies the symmetric epilogue.  grid (upper tiles, TI*TJ*4): each work
+// group owns one float4 slot (a, b, q) of every thread's accumulators, so a tile is reduced by 4*TI*TJ work
+// groups in parallel; the sum over splits runs in a fixed order (deterministic).
 template <int TI, int TJ>
 __global__ __launch_bounds__(256) void syrk_finalize_kernel(const float* __restrict__ ws, int nsplit, int T,
                                                             float* __restrict__ C, int64_t ldc, int64_t d,
@@ -131,21 +132,38 @@ __global__ __launch_bounds__(256) void syrk_finalize_kernel(const float* __restr
   constexpr int BT = 64 * TI;
   static_assert(TI == TJ, "square tiles");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wr = wave >> 1, wc = wave & 1;
+  const int wr = wave >> 1, wc = wave & 1, g = lane >> 5, l32 = lane & 31;
   int ti, tj;
   decode_upper_tile(blockIdx.x, T, ti, tj);
   const int ntiles = gridDim.x;
-  floatx16 acc[TI][TJ];
+  const int slot = blockIdx.y;                 // (a * TJ + b) * 4 + q
+  const int q = slot & 3, b = (slot >> 2) % TJ, a = (slot >> 2) / TJ;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  const floatx4* src = reinterpret_cast<const floatx4*>(ws) + (static_cast<size_t>(blockIdx.x) * (BT * BT / 4)) +
+                       slot * 256 + tid;
+  const size_t split_stride = static_cast<size_t>(ntiles) * (BT * BT / 4);
+  for (int s = 0; s < nsplit; ++s) {
+    const floatx4 w = src[s * split_stride];
+    acc[0] += w[0]; acc[1] += w[1]; acc[2] += w[2]; acc[3] += w[3];
+  }
+  const int64_t gj = static_cast<int64_t>(tj) * BT + 32 * TJ * wc + 32 * b + l32;
+  const int64_t gi = static_cast<int64_t>(ti) * BT + 32 * TI * wr + 32 * a + 8 * q + 4 * g;
+  if (gj >= d) return;
+  float v[4];
 #pragma unroll
-  for (int a = 0; a < TI; ++a)
+  for (int e = 0; e < 4; ++e) {
+    float x = alpha * acc[e];
+    if (beta != 0.f && gi + e < d) x += beta * C[(gi + e) * ldc + gj];
+    v[e] = x;
+  }
 #pragma unroll
-    for (int b = 0; b < TJ; ++b)
+  for (int e = 0; e < 4; ++e)
+    if (gi + e < d) C[(gi + e) * ldc + gj] = v[e];
+  if (ti != tj) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  for (int s = 0; s < nsplit; ++s)
-    add_partial<TI, TJ>(acc, ws + (static_cast<size_t>(s) * ntiles + blockIdx.x) * (BT * BT), tid);
-  syrk_epilogue<TI, TJ>(acc, C, ldc, d, static_cast<int64_t>(ti) * BT + 32 * TI * wr,
-                        static_cast<int64_t>(tj) * BT + 32 * TJ * wc, ti == tj, alpha, beta, lane);
+    for (int e = 0; e < 4; ++e)
+      if (gi + e < d) C[gj * ldc + gi + e] = v[e];
+  }
 }
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_ERR_LAUNCH; }
@@ -153,11 +171,11 @@ inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_
 // Split-K factor shared by the SYRK front ends: enough work groups to fill 256 CUs twice over
 // while every split still runs a useful number of k-steps.
 inline int pick_nsplit(int64_t ntiles, int64_t ksteps) {
-  int64_t want = (640 + ntiles - 1) / ntiles;
+  int64_t want = (512 + ntiles - 1) / ntiles;
   int64_t cap = ksteps / 8;
   if (cap < 1) cap = 1;
   int64_t s = want < cap ? want : cap;
-  if (s > 128) s = 128;
+  if (s > 256) s = 256;
   if (s < 1) s = 1;
   return static_cast<int>(s);
 }

@@ -38,6 +38,7 @@ struct ConvSyrkParams {
   int RB, CB;    // row blocks per image, column chunks per row
   int64_t total_stages, stages_per_split;
   uint32_t mU, mKK, mKw, mRI, mKwRI, mCPR, mCB, mRBCB;   // magic multipliers for division
+  int RP, dcl, dkx, dr;   // LDS rows staged per pass of the work group, and that step decomposed as (channel, kx, row)
 };
 
 __host__ __device__ inline uint32_t make_magic(uint32_t d) { return static_cast<uint32_t>((0x100000000ull + d - 1) / d); }
@@ -53,31 +54,39 @@ template <typename T> struct Elem;
 template <> struct Elem<uint16_t> { static constexpr int E = 8; typedef uint4_a2 vec_u; };
 template <> struct Elem<float> { static constexpr int E = 4; typedef uint4_a4 vec_u; };
 
-// Fills one panel's planes for the stage (n, oy0, ox0).
+// Fills one panel's planes for the stage (n, oy0, ox0).  Thread t owns 16-byte chunk t % CPR of LDS rows
+// t / CPR, t / CPR + RP, ...; the row index is decoded to (channel, kx, input row) once and then advanced
+// with carries, so the loop body has no divisions.
 template <typename T>
 __device__ __forceinline__ void stage_panel(T* __restrict__ plane, const ConvSyrkParams& p, const T* __restrict__ x,
                                             int64_t n, int c_lo, int nc, int oy0, int ox0, int R_eff, int W_eff,
                                             int tid) {
   constexpr int E = Elem<T>::E;
   const int CPR = p.WC / E;
-  const int RI_eff = (R_eff - 1) * p.sh + p.kh;
+  const int row0 = static_cast<int>(fastdiv(tid, p.mCPR, CPR));
+  if (row0 >= p.RP) return;
+  const int m = tid - row0 * CPR;
   const int kwRI = p.kw * p.RI;
-  const int total = nc * kwRI * CPR;
-  for (int G = tid; G < total; G += 256) {
-    const uint32_t rs = fastdiv(G, p.mCPR, CPR);
-    const int m = G - rs * CPR;
-    const uint32_t cl = fastdiv(rs, p.mKwRI, kwRI);
-    const uint32_t t2 = rs - cl * kwRI;
-    const uint32_t kx = fastdiv(t2, p.mRI, p.RI);
-    const int r = t2 - kx * p.RI;
-    const int c = c_lo + cl;
-    const int iy = oy0 * p.sh - p.ph + r;
-    const int q0 = m * E;
-    const int x0 = (ox0 + q0) * p.sw + static_cast<int>(kx) - p.pw;
+  const int total_rows = nc * kwRI;
+  int cl = static_cast<int>(fastdiv(row0, p.mKwRI, kwRI));
+  const int t2 = row0 - cl * kwRI;
+  int kx = static_cast<int>(fastdiv(t2, p.mRI, p.RI));
+  int r = t2 - kx * p.RI;
+  const int RI_eff = (R_eff - 1) * p.sh + p.kh;
+  const int q0 = m * E;
+  const int xq = (ox0 + q0) * p.sw - p.pw;
+  const int iy0 = oy0 * p.sh - p.ph;
+  const bool q_in = q0 < W_eff, q_full = q0 + E <= W_eff;
+  const T* __restrict__ img = x + n * p.C * p.H * p.W;
+  T* __restrict__ dst = plane + row0 * p.RS + q0;
+  const int dst_step = p.RP * p.RS;
+  for (int rs = row0; rs < total_rows; rs += p.RP, dst += dst_step) {
+    const int iy = iy0 + r;
+    const int x0 = xq + kx;
     uint4 v = {0u, 0u, 0u, 0u};
-    if (r < RI_eff && c < p.C && iy >= 0 && iy < p.H && q0 < W_eff) {
-      const T* src = x + ((n * p.C + c) * p.H + iy) * p.W;
-      const bool inner = (q0 + E <= W_eff) && (x0 >= 0);
+    if (q_in && r < RI_eff && iy >= 0 && iy < p.H) {
+      const T* src = img + (static_cast<int64_t>(c_lo + cl) * p.H + iy) * p.W;
+      const bool inner = q_full && (x0 >= 0);
       if (p.sw == 1 && inner && x0 + E <= p.W) {
         v = *reinterpret_cast<const typename Elem<T>::vec_u*>(src + x0);
       } else if (p.sw == 2 && inner && x0 + 2 * E <= p.W) {
@@ -101,7 +110,10 @@ __device__ __forceinline__ void stage_panel(T* __restrict__ plane, const ConvSyr
         v = *reinterpret_cast<uint4*>(tmp);
       }
     }
-    *reinterpret_cast<uint4*>(plane + rs * p.RS + q0) = v;
+    *reinterpret_cast<uint4*>(dst) = v;
+    r += p.dr; kx += p.dkx; cl += p.dcl;
+    if (r >= p.RI) { r -= p.RI; kx += 1; }
+    if (kx >= p.kw) { kx -= p.kw; cl += 1; }
   }
 }
 
@@ -231,18 +243,24 @@ __global__ __launch_bounds__(256) void conv_syrk_kernel(ConvSyrkParams p) {
 // Host-side geometry shared by the launch and the workspace query.
 struct ConvPlan {
   ConvSyrkParams p;
+  int BT;
   size_t lds_bytes;
   int64_t ntiles;
   size_t ws_need;
 };
 
+static int tile_rows_for(int64_t d) { return d <= 64 ? 64 : 128; }
+
 static bool make_plan(ConvPlan& plan, int esize, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh,
                       int sw, int ph, int pw) {
-  constexpr int BT = 128;
   ConvSyrkParams& p = plan.p;
+  const int BT = tile_rows_for(C * kh * kw);
+  plan.BT = BT;
+  bool flat = false;
   if (kh == 1 && kw == 1 && ph == 0 && pw == 0 && sh == 1 && sw == 1) {  // positions are contiguous: flatten
     W = H * W;
     H = 1;
+    flat = true;
   }
   const int64_t Ho = (H + 2 * ph - kh) / sh + 1, Wo = (W + 2 * pw - kw) / sw + 1;
   if (Ho <= 0 || Wo <= 0) return false;
@@ -251,7 +269,7 @@ static bool make_plan(ConvPlan& plan, int esize, int64_t N, int64_t C, int64_t H
   p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
   p.KK = kh * kw;
   p.d = C * p.KK;
-  const int wc_max = 64;
+  const int wc_max = (flat && esize == 2) ? 128 : 64;
   int WC = static_cast<int>(((Wo + 7) / 8) * 8);
   if (WC > wc_max) WC = wc_max;
   p.WC = WC;
@@ -262,12 +280,16 @@ static bool make_plan(ConvPlan& plan, int esize, int64_t N, int64_t C, int64_t H
   int ncmax = (BT - 1 + p.KK - 1) / p.KK + 1;
   if (ncmax > C) ncmax = static_cast<int>(C);
   p.NCmax = ncmax;
-  const size_t budget = 64 * 1024 - 64;
+  const size_t budget = 80 * 1024 - 64;     // two work groups per CU
   int R = 1;
-  for (int cand = 1; cand <= Ho && cand * WC <= 512; ++cand) {
+  for (int cand = 1; cand <= Ho && cand * WC <= 1024; ++cand) {
     const int RI = (cand - 1) * sh + kh;
     const size_t bytes = 2ull * ncmax * kw * RI * p.RS * esize;
     if (bytes <= budget) R = cand; else break;
+  }
+  {  // equal-sized row blocks: no short last block
+    const int64_t nrb = (Ho + R - 1) / R;
+    R = static_cast<int>((Ho + nrb - 1) / nrb);
   }
   p.R = R;
   p.RI = (R - 1) * sh + kh;
@@ -278,6 +300,7 @@ static bool make_plan(ConvPlan& plan, int esize, int64_t N, int64_t C, int64_t H
   p.CB = static_cast<int>((Wo + WC - 1) / WC);
   p.total_stages = N * p.RB * p.CB;
   if (p.total_stages >= (1ll << 31) || p.d >= (1ll << 24)) return false;
+  if (p.total_stages * p.RB * p.CB >= (1ll << 32)) return false;   // exactness of the magic division
   const int64_t Tn = (p.d + BT - 1) / BT;
   p.T = static_cast<int>(Tn);
   plan.ntiles = Tn * (Tn + 1) / 2;
@@ -292,15 +315,22 @@ static bool make_plan(ConvPlan& plan, int esize, int64_t N, int64_t C, int64_t H
   p.nsplit = nsplit;
   plan.ws_need = nsplit > 1 ? static_cast<size_t>(nsplit) * plan.ntiles * BT * BT * sizeof(float) : 0;
   const int CPR = WC / (16 / esize);
+  p.RP = 256 / CPR;
+  {
+    const int kwRI = kw * p.RI;
+    p.dcl = p.RP / kwRI;
+    const int rem = p.RP - p.dcl * kwRI;
+    p.dkx = rem / p.RI;
+    p.dr = rem - p.dkx * p.RI;
+  }
   p.mU = make_magic(p.U); p.mKK = make_magic(p.KK); p.mKw = make_magic(kw); p.mRI = make_magic(p.RI);
   p.mKwRI = make_magic(kw * p.RI); p.mCPR = make_magic(CPR); p.mCB = make_magic(p.CB);
   p.mRBCB = make_magic(p.RB * p.CB);
   return true;
 }
 
-template <typename T>
-static int launch_conv_syrk(ConvPlan& plan, hipStream_t stream) {
-  constexpr int TI = 2;
+template <typename T, int TI>
+static int launch_conv_syrk_t(ConvPlan& plan, hipStream_t stream) {
   auto kern = conv_syrk_kernel<T, TI>;
   if (plan.lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -310,10 +340,15 @@ static int launch_conv_syrk(ConvPlan& plan, hipStream_t stream) {
   dim3 grid(static_cast<unsigned>(plan.ntiles), static_cast<unsigned>(plan.p.nsplit));
   hipLaunchKernelGGL(kern, grid, dim3(256), plan.lds_bytes, stream, plan.p);
   if (plan.p.nsplit > 1)
-    hipLaunchKernelGGL((syrk_finalize_kernel<TI, TI>), dim3(static_cast<unsigned>(plan.ntiles)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((syrk_finalize_kernel<TI, TI>), dim3(static_cast<unsigned>(plan.ntiles), 4 * TI * TI), dim3(256), 0, stream,
                        static_cast<const float*>(plan.p.ws), plan.p.nsplit, plan.p.T, plan.p.A, plan.p.lda, plan.p.d,
                        plan.p.alpha, plan.p.beta);
   return check_launch();
+}
+
+template <typename T>
+static int launch_conv_syrk(ConvPlan& plan, hipStream_t stream) {
+  return plan.BT == 64 ? launch_conv_syrk_t<T, 1>(plan, stream) : launch_conv_syrk_t<T, 2>(plan, stream);
 }
 
 }  // namespace ak

@@ -39,22 +39,27 @@ struct GemmParams {
   int active_stride;
 };
 
-constexpr int GBT = 128, GBK = 16;
+constexpr int GBT = 128, GBK = 16;     // GBT: granularity of the triangular contraction ranges (both tile sizes)
 constexpr int G_KC_STRIDE = GBK + 4;    // [row][k] layout
-constexpr int G_IC_STRIDE = GBT + 4;    // [k][row] layout
-constexpr int G_PANEL = GBT * G_KC_STRIDE > GBK * G_IC_STRIDE ? GBT * G_KC_STRIDE : GBK * G_IC_STRIDE;
+template <int BT> struct GemmTile {
+  static constexpr int IC_STRIDE = BT + 4;    // [k][row] layout
+  static constexpr int PANEL = BT * G_KC_STRIDE > GBK * IC_STRIDE ? BT * G_KC_STRIDE : GBK * IC_STRIDE;
+  static constexpr int CHUNKS = BT * GBK / 4 / 256;   // 16-byte chunks per thread per panel
+};
 
 // Loads this thread's two 16-byte chunks of a 128 x 16 operand panel.
 //  kcontig: memory rows are the 128 tile rows, 16 k values contiguous.
 //  else   : memory rows are the 16 k values, 128 tile rows contiguous.
-__device__ __forceinline__ void gemm_fetch(floatx4 (&reg)[2], const float* __restrict__ P, int64_t ld, bool kcontig,
-                                           int r0, int r_end, int k0, int k_end, bool vec_ok, int tid) {
+template <int BT>
+__device__ __forceinline__ void gemm_fetch(floatx4 (&reg)[GemmTile<BT>::CHUNKS], const float* __restrict__ P, int64_t ld,
+                                           bool kcontig, int r0, int r_end, int k0, int k_end, bool vec_ok, int tid) {
+  constexpr int RC = BT / 4;      // chunks per k-row in the [k][row] layout
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
+  for (int u = 0; u < GemmTile<BT>::CHUNKS; ++u) {
     const int c = tid + 256 * u;
     int outer, inner, o_end, i_end;
     if (kcontig) { outer = r0 + (c >> 2); inner = k0 + 4 * (c & 3); o_end = r_end; i_end = k_end; }
-    else { outer = k0 + (c >> 5); inner = r0 + 4 * (c & 31); o_end = k_end; i_end = r_end; }
+    else { outer = k0 + c / RC; inner = r0 + 4 * (c % RC); o_end = k_end; i_end = r_end; }
     floatx4 v = {0.f, 0.f, 0.f, 0.f};
     if (outer < o_end && inner < i_end) {
       const float* src = P + static_cast<int64_t>(outer) * ld + inner;
@@ -70,16 +75,20 @@ __device__ __forceinline__ void gemm_fetch(floatx4 (&reg)[2], const float* __res
   }
 }
 
-__device__ __forceinline__ void gemm_stash(const floatx4 (&reg)[2], float* __restrict__ lds, bool kcontig, int tid) {
+template <int BT>
+__device__ __forceinline__ void gemm_stash(const floatx4 (&reg)[GemmTile<BT>::CHUNKS], float* __restrict__ lds,
+                                           bool kcontig, int tid) {
+  constexpr int RC = BT / 4;
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
+  for (int u = 0; u < GemmTile<BT>::CHUNKS; ++u) {
     const int c = tid + 256 * u;
-    const int off = kcontig ? (c >> 2) * G_KC_STRIDE + 4 * (c & 3) : (c >> 5) * G_IC_STRIDE + 4 * (c & 31);
+    const int off = kcontig ? (c >> 2) * G_KC_STRIDE + 4 * (c & 3) : (c / RC) * GemmTile<BT>::IC_STRIDE + 4 * (c % RC);
     *reinterpret_cast<floatx4*>(lds + off) = reg[u];
   }
 }
 
 // Reads the 8 k values (k = 8g + m) of tile row `row` for this lane.
+template <int BT>
 __device__ __forceinline__ void gemm_frag(float (&f)[8], const float* __restrict__ lds, bool kcontig, int row, int g) {
   if (kcontig) {
     const floatx4* q = reinterpret_cast<const floatx4*>(lds + row * G_KC_STRIDE + 8 * g);
@@ -88,12 +97,14 @@ __device__ __forceinline__ void gemm_frag(float (&f)[8], const float* __restrict
     for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
   } else {
 #pragma unroll
-    for (int m = 0; m < 8; ++m) f[m] = lds[(8 * g + m) * G_IC_STRIDE + row];
+    for (int m = 0; m < 8; ++m) f[m] = lds[(8 * g + m) * GemmTile<BT>::IC_STRIDE + row];
   }
 }
 
+template <int TI>
 static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(16))) float lds[2][2][G_PANEL];
+  constexpr int BT = 64 * TI;
+  __shared__ __attribute__((aligned(16))) float lds[2][2][GemmTile<BT>::PANEL];
   const int z = blockIdx.z;
   if (p.active != nullptr && p.active[static_cast<int64_t>(z) * p.active_stride] == 0) return;
   const int tj = blockIdx.x, ti = blockIdx.y;
@@ -102,11 +113,11 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
   const int wr = wave >> 1, wc = wave & 1, g = lane >> 5, l32 = lane & 31;
 
   int kbeg = 0, kend = p.K;
-  switch (p.kmode) {
-    case K_LE_J: kend = min(p.K, (tj + 1) * GBT); break;
-    case K_GE_J: kbeg = tj * GBT; break;
-    case K_LE_I: kend = min(p.K, (ti + 1) * GBT); break;
-    case K_GE_MAXIJ: kbeg = max(ti, tj) * GBT; break;
+  switch (p.kmode) {     // ranges rounded outwards to multiples of GBK; the operands are zero outside their triangle
+    case K_LE_J: kend = min(p.K, (tj + 1) * BT); break;
+    case K_GE_J: kbeg = tj * BT; break;
+    case K_LE_I: kend = min(p.K, (ti + 1) * BT); break;
+    case K_GE_MAXIJ: kbeg = max(ti, tj) * BT; break;
     default: break;
   }
   const float* __restrict__ A = p.A + static_cast<int64_t>(z) * p.sA;
@@ -115,46 +126,46 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
   const bool a_kc = (p.transA == 0), b_kc = (p.transB != 0);
   const bool a_vec = (p.lda % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
   const bool b_vec = (p.ldb % 4 == 0) && ((reinterpret_cast<uintptr_t>(B) & 15) == 0);
-  const int i0 = ti * GBT, j0 = tj * GBT;
+  const int i0 = ti * BT, j0 = tj * BT;
 
-  floatx16 acc[2][2];
+  floatx16 acc[TI][TI];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < TI; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < TI; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   const int nk = kbeg < kend ? (kend - kbeg + GBK - 1) / GBK : 0;
-  floatx4 ra[2], rb[2];
+  floatx4 ra[GemmTile<BT>::CHUNKS], rb[GemmTile<BT>::CHUNKS];
   if (nk > 0) {
-    gemm_fetch(ra, A, p.lda, a_kc, i0, p.M, kbeg, kend, a_vec, tid);
-    gemm_fetch(rb, B, p.ldb, b_kc, j0, p.N, kbeg, kend, b_vec, tid);
-    gemm_stash(ra, lds[0][0], a_kc, tid);
-    gemm_stash(rb, lds[0][1], b_kc, tid);
+    gemm_fetch<BT>(ra, A, p.lda, a_kc, i0, p.M, kbeg, kend, a_vec, tid);
+    gemm_fetch<BT>(rb, B, p.ldb, b_kc, j0, p.N, kbeg, kend, b_vec, tid);
+    gemm_stash<BT>(ra, lds[0][0], a_kc, tid);
+    gemm_stash<BT>(rb, lds[0][1], b_kc, tid);
   }
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) {
       const int k0 = kbeg + (kt + 1) * GBK;
-      gemm_fetch(ra, A, p.lda, a_kc, i0, p.M, k0, kend, a_vec, tid);
-      gemm_fetch(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, b_vec, tid);
+      gemm_fetch<BT>(ra, A, p.lda, a_kc, i0, p.M, k0, kend, a_vec, tid);
+      gemm_fetch<BT>(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, b_vec, tid);
     }
-    float fa[2][8], fb[2][8];
+    float fa[TI][8], fb[TI][8];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) gemm_frag(fa[a], lds[buf][0], a_kc, 64 * wr + 32 * a + l32, g);
+    for (int a = 0; a < TI; ++a) gemm_frag<BT>(fa[a], lds[buf][0], a_kc, 32 * TI * wr + 32 * a + l32, g);
 #pragma unroll
-    for (int b = 0; b < 2; ++b) gemm_frag(fb[b], lds[buf][1], b_kc, 64 * wc + 32 * b + l32, g);
+    for (int b = 0; b < TI; ++b) gemm_frag<BT>(fb[b], lds[buf][1], b_kc, 32 * TI * wc + 32 * b + l32, g);
 #pragma unroll
     for (int m = 0; m < 8; ++m)
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < TI; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) acc[a][b] = mfma_f32(fa[a][m], fb[b][m], acc[a][b]);
+        for (int b = 0; b < TI; ++b) acc[a][b] = mfma_f32(fa[a][m], fb[b][m], acc[a][b]);
     if (kt + 1 < nk) {
-      gemm_stash(ra, lds[buf ^ 1][0], a_kc, tid);
-      gemm_stash(rb, lds[buf ^ 1][1], b_kc, tid);
+      gemm_stash<BT>(ra, lds[buf ^ 1][0], a_kc, tid);
+      gemm_stash<BT>(rb, lds[buf ^ 1][1], b_kc, tid);
     }
     __syncthreads();
   }
@@ -162,14 +173,14 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
   const bool lower_only = (p.tile_mode == TILE_LOWER);
   const bool mirror = (p.tile_mode == TILE_LOWER_MIRROR) && (ti != tj);
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < TI; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const int gj = j0 + 64 * wc + 32 * b + l32;
+    for (int b = 0; b < TI; ++b) {
+      const int gj = j0 + 32 * TI * wc + 32 * b + l32;
       if (gj >= p.N) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int gi = i0 + 64 * wr + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3);
+        const int gi = i0 + 32 * TI * wr + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3);
         if (gi >= p.M) continue;
         if (lower_only && gi < gj) continue;
         float v = p.alpha * acc[a][b][r];
@@ -183,8 +194,16 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
 
 inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return AK_OK;
-  dim3 grid((p.N + GBT - 1) / GBT, (p.M + GBT - 1) / GBT, batch);
-  hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, p);
+  // 128 x 128 tiles when they alone fill the 256 CUs twice over, else 64 x 64 tiles (four times the work groups)
+  const int64_t tiles128 = static_cast<int64_t>((p.N + 127) / 128) * ((p.M + 127) / 128) * batch;
+  const bool lower = p.tile_mode != TILE_ALL;
+  if ((lower ? tiles128 / 2 : tiles128) >= 512) {
+    dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
+    hipLaunchKernelGGL(gemm_f32_kernel<2>, grid, dim3(256), 0, stream, p);
+  } else {
+    dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
+    hipLaunchKernelGGL(gemm_f32_kernel<1>, grid, dim3(256), 0, stream, p);
+  }
   return check_launch();
 }
 

@@ -181,7 +181,7 @@ static int launch_syrk_tn(const void* X, int64_t M, int64_t d, int64_t ldx, floa
   dim3 grid(static_cast<unsigned>(ntiles), static_cast<unsigned>(nsplit));
   hipLaunchKernelGGL((syrk_tn_kernel<T, TI>), grid, dim3(256), 0, stream, p);
   if (nsplit > 1)
-    hipLaunchKernelGGL((syrk_finalize_kernel<TI, TI>), dim3(static_cast<unsigned>(ntiles)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((syrk_finalize_kernel<TI, TI>), dim3(static_cast<unsigned>(ntiles), 4 * TI * TI), dim3(256), 0, stream,
                        static_cast<const float*>(ws), nsplit, static_cast<int>(Tn), C, ldc, d, alpha, beta);
   return check_launch();
 }

@@ -17,6 +17,17 @@ __all__ = ['SymMatrix', 'Kron', 'batched_update_inv']
 _default_damping = 1e-5
 
 
+_side_stream_cache = {}
+
+
+def _side_streams(device, n):
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    pool = _side_stream_cache.setdefault(key, [])
+    while len(pool) < n:
+        pool.append(torch.cuda.Stream(device=device))
+    return pool[:n]
+
+
 def _is_all_none(xs):
     return all(x is None for x in xs)
 
@@ -41,6 +52,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             if m is not None and (m.ndim != 2 or m.shape[0] != m.shape[1]):
                 raise NotImplementedError('non-square (swift) Kronecker factors are not on this path')
     dev = (krons[0].A if krons[0].has_A else krons[0].B).device
+    mats_on_gpu = dev.type == 'cuda'
     A_list = [k.A if k.has_A else k.B for k in krons]
     B_list = [k.B if k.has_B else k.A for k in krons]
     A_list = [a if a.is_contiguous() else a.contiguous() for a in A_list]
@@ -57,8 +69,11 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             groups[A_list[i].shape[0]].append((2 * i, A_list[i], k, 'A'))
         if calc_B_inv:
             groups[B_list[i].shape[0]].append((2 * i + 1, B_list[i], k, 'B'))
-    infos, records = [], []
-    for d in sorted(groups, reverse=True):
+    # Each size group is an independent chain of small launches: spread the groups over a few side streams
+    # (default priority) so that their launch latencies overlap; everything joins the caller's stream again.
+    order = sorted(groups, key=lambda d: d ** 3 * len(groups[d]), reverse=True)
+    prepared = []
+    for d in order:
         entries = groups[d]
         idx = torch.tensor([e[0] for e in entries], device=dev)
         outs = []
@@ -66,10 +81,30 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             old = getattr(k, which + '_inv')
             reuse = old is not None and old.shape == mat.shape and old.is_contiguous() and old.dtype == mat.dtype
             outs.append(old if reuse else torch.empty_like(mat))
-        info = kernels.chol_inv_batched([e[1] for e in entries], outs, lam_flat[idx], 1,
-                                        active=nz_flat[idx].contiguous(), active_stride=1)
+        info = torch.empty(len(entries), dtype=torch.int32, device=dev)
+        prepared.append((entries, outs, lam_flat[idx], nz_flat[idx].contiguous(), info))
+    infos, records = [], []
+    use_streams = mats_on_gpu and len(prepared) > 1
+    if use_streams:
+        main = torch.cuda.current_stream()
+        side = _side_streams(dev, min(4, len(prepared)))
+        start = torch.cuda.Event()
+        start.record(main)
+    for gi, (entries, outs, lam_g, act_g, info) in enumerate(prepared):
+        if use_streams:
+            st = side[gi % len(side)]
+            st.wait_event(start)
+            with torch.cuda.stream(st):
+                kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
+        else:
+            kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
         infos.append(info)
         records.extend((e[0], e[2], e[3], out) for e, out in zip(entries, outs))
+    if use_streams:
+        for st in side:
+            done = torch.cuda.Event()
+            done.record(st)
+            main.wait_event(done)
     host = torch.cat(infos + [nz_flat]).cpu().tolist()        # the one synchronisation
     info_host, nz_host = host[:len(records)], host[len(records):]
     for (flat, k, which, out), inf in zip(records, info_host):

@@ -46,7 +46,9 @@ def kron_damping(A_list, B_list, damping, eps=1e-7):
 
 
 def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1, info=None):
-    info = torch.zeros(len(mats), dtype=torch.int32)
+    if info is None:
+        info = torch.empty(len(mats), dtype=torch.int32)
+    info.zero_()
     for b, (m, o) in enumerate(zip(mats, outs)):
         if active is not None and int(active[b * active_stride]) == 0:
             continue
