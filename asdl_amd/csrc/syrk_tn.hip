@@ -47,14 +47,16 @@ __device__ __forceinline__ uint4 load_chunk(const T* __restrict__ X, int64_t row
 }
 
 template <typename T, int TI>
-__global__ __launch_bounds__(256) void syrk_tn_kernel(SyrkTnParams p) {
+__global__ __launch_bounds__(256, 2) void syrk_tn_kernel(SyrkTnParams p) {
   constexpr int BT = 64 * TI;
   constexpr int BK = TnCfg<T>::BK, PAD = TnCfg<T>::PAD, E = TnCfg<T>::E;
   constexpr int LDSS = BT + PAD;                 // elements per k-row in LDS
   constexpr int CPR = BT / E;                    // 16-byte chunks per k-row
   constexpr int CHUNKS = BK * CPR / 256;         // chunks per thread per panel
+  constexpr int PANEL = BK * LDSS;               // elements per panel buffer
   static_assert(BK * CPR % 256 == 0, "panel must split evenly");
-  __shared__ __attribute__((aligned(16))) T lds[2][2][BK * LDSS];
+  extern __shared__ __attribute__((aligned(16))) unsigned char tn_smem[];
+  T* lds = reinterpret_cast<T*>(tn_smem);        // [buffer][panel][BK * LDSS]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave >> 1, wc = wave & 1;
@@ -69,6 +71,8 @@ __global__ __launch_bounds__(256) void syrk_tn_kernel(SyrkTnParams p) {
 
   const T* __restrict__ X = static_cast<const T*>(p.X);
   const bool vec_ok = (p.ldx % E == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  // whole panels inside the matrix and aligned: plain vector loads, no per-chunk tests
+  const bool fast = vec_ok && (j0 + BT <= p.d);   // j0 >= i0, so this covers the I panel too
 
   floatx16 acc[TI][TI];
 #pragma unroll
@@ -81,21 +85,33 @@ __global__ __launch_bounds__(256) void syrk_tn_kernel(SyrkTnParams p) {
   uint4 regI[CHUNKS], regJ[CHUNKS];
   auto fetch = [&](int kt) {
     const int64_t kb = k_begin + static_cast<int64_t>(kt) * BK;
+    if (fast && kb + BK <= k_end) {
 #pragma unroll
-    for (int u = 0; u < CHUNKS; ++u) {
-      const int c = tid + 256 * u;
-      const int row = c / CPR, cc = c % CPR;
-      regI[u] = load_chunk<T>(X, kb + row, i0 + cc * E, k_end, p.d, p.ldx, vec_ok);
-      if (!diag) regJ[u] = load_chunk<T>(X, kb + row, j0 + cc * E, k_end, p.d, p.ldx, vec_ok);
+      for (int u = 0; u < CHUNKS; ++u) {
+        const int c = tid + 256 * u;
+        const T* src = X + (kb + c / CPR) * p.ldx + (c % CPR) * E;
+        regI[u] = *reinterpret_cast<const uint4*>(src + i0);
+        if (!diag) regJ[u] = *reinterpret_cast<const uint4*>(src + j0);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < CHUNKS; ++u) {
+        const int c = tid + 256 * u;
+        const int row = c / CPR, cc = c % CPR;
+        regI[u] = load_chunk<T>(X, kb + row, i0 + cc * E, k_end, p.d, p.ldx, vec_ok);
+        if (!diag) regJ[u] = load_chunk<T>(X, kb + row, j0 + cc * E, k_end, p.d, p.ldx, vec_ok);
+      }
     }
   };
   auto stash = [&](int buf) {
+    T* pI = lds + (2 * buf) * PANEL;
+    T* pJ = pI + PANEL;
 #pragma unroll
     for (int u = 0; u < CHUNKS; ++u) {
       const int c = tid + 256 * u;
       const int row = c / CPR, cc = c % CPR;
-      *reinterpret_cast<uint4*>(&lds[buf][0][row * LDSS + cc * E]) = regI[u];
-      if (!diag) *reinterpret_cast<uint4*>(&lds[buf][1][row * LDSS + cc * E]) = regJ[u];
+      *reinterpret_cast<uint4*>(&pI[row * LDSS + cc * E]) = regI[u];
+      if (!diag) *reinterpret_cast<uint4*>(&pJ[row * LDSS + cc * E]) = regJ[u];
     }
   };
 
@@ -109,28 +125,40 @@ __global__ __launch_bounds__(256) void syrk_tn_kernel(SyrkTnParams p) {
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) fetch(kt + 1);
-    const T* pI = lds[buf][0];
-    const T* pJ = diag ? lds[buf][0] : lds[buf][1];
+    const T* pI = lds + (2 * buf) * PANEL;
+    const T* pJ = diag ? pI : pI + PANEL;
     if constexpr (sizeof(T) == 2) {
       const int half = (lane >> 4) & 1, j16 = lane & 15;
       const int frag_off = (8 * g + (j16 >> 2)) * LDSS + 16 * half + 4 * (j16 & 3);
-#pragma unroll
-      for (int kk = 0; kk < BK; kk += 16) {
-        bf16x8 fa[TI], fb[TI];
+      const T* qI = pI + frag_off + 32 * TI * wr;
+      const T* qJ = pJ + frag_off + 32 * TI * wc;
+      auto read = [&](bf16x8 (&fa)[TI], bf16x8 (&fb)[TI], int kk) {
 #pragma unroll
         for (int a = 0; a < TI; ++a) {
-          const T* q = pI + kk * LDSS + frag_off + 32 * TI * wr + 32 * a;
+          const T* q = qI + kk * LDSS + 32 * a;
           fa[a] = pack_bf16x8(lds_read_tr16(q), lds_read_tr16(q + 4 * LDSS));
         }
 #pragma unroll
         for (int b = 0; b < TI; ++b) {
-          const T* q = pJ + kk * LDSS + frag_off + 32 * TI * wc + 32 * b;
+          const T* q = qJ + kk * LDSS + 32 * b;
           fb[b] = pack_bf16x8(lds_read_tr16(q), lds_read_tr16(q + 4 * LDSS));
         }
+      };
+      auto mma = [&](const bf16x8 (&fa)[TI], const bf16x8 (&fb)[TI]) {
 #pragma unroll
         for (int a = 0; a < TI; ++a)
 #pragma unroll
           for (int b = 0; b < TI; ++b) acc[a][b] = mfma_bf16(fa[a], fb[b], acc[a][b]);
+      };
+      // ping-pong fragment registers: the reads of one k-step fly during the MFMAs of the previous one
+      bf16x8 fa0[TI], fb0[TI], fa1[TI], fb1[TI];
+      read(fa0, fb0, 0);
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 32) {
+        read(fa1, fb1, kk + 16);
+        mma(fa0, fb0);
+        if (kk + 32 < BK) read(fa0, fb0, kk + 32);
+        mma(fa1, fb1);
       }
     } else {
 #pragma unroll
@@ -179,7 +207,18 @@ static int launch_syrk_tn(const void* X, int64_t M, int64_t d, int64_t ldx, floa
   p.ws = static_cast<float*>(ws); p.T = static_cast<int>(Tn); p.nsplit = nsplit;
   p.rows_per_split = steps_per_split * BK;
   dim3 grid(static_cast<unsigned>(ntiles), static_cast<unsigned>(nsplit));
-  hipLaunchKernelGGL((syrk_tn_kernel<T, TI>), grid, dim3(256), 0, stream, p);
+  constexpr size_t lds_bytes = 4ull * BK * (BT + TnCfg<T>::PAD) * sizeof(T);
+  auto kern = syrk_tn_kernel<T, TI>;
+  if (lds_bytes > 64 * 1024) {
+    static bool attr_set = false;     // idempotent; a benign race sets it twice at worst
+    if (!attr_set) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds_bytes)) != hipSuccess)
+        return AK_ERR_LAUNCH;
+      attr_set = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, stream, p);
   if (nsplit > 1)
     hipLaunchKernelGGL((syrk_finalize_kernel<TI, TI>), dim3(static_cast<unsigned>(ntiles), 4 * TI * TI), dim3(256), 0, stream,
                        static_cast<const float*>(ws), nsplit, static_cast<int>(Tn), C, ldc, d, alpha, beta);

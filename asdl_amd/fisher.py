@@ -118,12 +118,17 @@ class FisherMaker(GradientMaker):
             else:
                 self._fisher_loop(closure)
             cxt.finish_registered()
+            # The inverses only need the factors: enqueue them now (side streams) and, when a loss backward
+            # pass follows, let that pass run on the main stream meanwhile; the flags are read afterwards.
+            deferred = cxt.flush_inverses(defer=loss_grad_after_fisher)
             self._extract_fisher(cxt)
 
         if inv_after_fisher:
             self.replace_fisher_with_inv(damping)
         if loss_grad_after_fisher:
             loss.backward()
+        if deferred is not None:
+            deferred.finish(config.fisher_attr)
         if calc_loss_grad:
             # the loss was summed over the batch: divide gradients and loss by the data size
             for p in model.parameters():

@@ -239,6 +239,26 @@ class Conv2d(Operation):
         return kernels.syrk_nt(out_grads, out=out, alpha=alpha, beta=beta)    # c_out x c_out
 
 
+class DeferredInverses:
+    """Inverses enqueued by OperationContext.flush_inverses(defer=True).  finish(attr) waits for them,
+    raises torch.linalg.LinAlgError for a factor that is not positive definite, and removes from
+    ``module.<attr>.kron`` the inverse of any all-zero factor (which the reference never computes)."""
+
+    def __init__(self, pending, targets):
+        self._pending, self._targets = pending, targets
+
+    def finish(self, attr):
+        self._pending.finish()
+        for module, kron in self._targets:
+            fisher = getattr(module, attr, None)
+            if fisher is None or not fisher.has_kron:
+                continue
+            if kron.A_inv is None:
+                fisher.kron.A_inv = None
+            if kron.B_inv is None:
+                fisher.kron.B_inv = None
+
+
 def get_op_class(module):
     """asdl/operations/__init__.py:60-79, restricted to the layer types on this path."""
     if isinstance(module, nn.Linear):
@@ -303,11 +323,14 @@ class OperationContext:
         if operation not in self._pending_inverse:
             self._pending_inverse.append(operation)
 
-    def flush_inverses(self):
+    def flush_inverses(self, defer=False):
+        """Inverts every queued (A, B) pair in one batched pass.  With ``defer=True`` the launches are only
+        enqueued: the result store receives the output tensors right away and the returned object's
+        finish() must be called before they are used (it reads the zero / not-positive-definite flags)."""
         ops = self._pending_inverse
         self._pending_inverse = []
         if not ops:
-            return
+            return None
         krons = []
         for op in ops:
             A = op._op_results.pop('_A_tmp', None)
@@ -317,17 +340,26 @@ class OperationContext:
             prev = op._op_results.get(OP_COV_KRON) or {}
             krons.append(Kron(A, B, prev.get('A_inv'), prev.get('B_inv')))
         # every operation in one context shares the damping value
-        batched_update_inv(krons, damping=ops[0]._damping, replace=False)
+        pending = batched_update_inv(krons, damping=ops[0]._damping, replace=False, defer=True)
+        if not defer:
+            pending.finish()
+            for op, kron in zip(ops, krons):
+                store = op._op_results.setdefault(OP_COV_KRON, {})
+                if kron.A_inv is not None:
+                    store['A_inv'] = kron.A_inv
+                if kron.B_inv is not None:
+                    store['B_inv'] = kron.B_inv
+            return None
+        outs = {(id(k), which): out for _, k, which, out in pending._records}
         for op, kron in zip(ops, krons):
             store = op._op_results.setdefault(OP_COV_KRON, {})
-            if kron.A_inv is not None:
-                store['A_inv'] = kron.A_inv
-            if kron.B_inv is not None:
-                store['B_inv'] = kron.B_inv
+            store['A_inv'] = outs[(id(kron), 'A')]
+            store['B_inv'] = outs[(id(kron), 'B')]
+        return DeferredInverses(pending, [(op._module, kron) for op, kron in zip(ops, krons)])
 
     # ---- symmatrix exchange (asdl/operations/operation.py:815-876)
     def cov_symmatrix(self, module, pop=False):
-        self.flush_inverses()
+        self.flush_inverses()       # no-op when the caller has already flushed (possibly deferred)
         cov_kron = self.get_result(module, OP_COV_KRON, pop=pop)
         if cov_kron is None:
             return None

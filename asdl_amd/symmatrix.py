@@ -12,7 +12,7 @@ from torch import Tensor
 
 from . import kernels
 
-__all__ = ['SymMatrix', 'Kron', 'batched_update_inv']
+__all__ = ['SymMatrix', 'Kron', 'batched_update_inv', 'PendingInverses']
 
 _default_damping = 1e-5
 
@@ -32,15 +32,52 @@ def _is_all_none(xs):
     return all(x is None for x in xs)
 
 
-def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_inv=True, eps=1e-7, replace=False):
+class PendingInverses:
+    """Inverses that have been enqueued (on side streams) but whose flags have not been read yet.
+    finish() joins the streams into the current one, reads all flags with one device-to-host copy,
+    raises for a matrix that is not positive definite and stores the inverses on the Kron objects."""
+
+    def __init__(self, records, infos, nz_flat, events, replace, keep_alive=None):
+        self._records, self._infos, self._nz_flat = records, infos, nz_flat
+        self._keep_alive = keep_alive      # tensors the side-stream kernels still read
+        self._events, self._replace = events, replace
+        self._done = False
+
+    def finish(self):
+        if self._done:
+            return
+        self._done = True
+        main = torch.cuda.current_stream() if self._events else None
+        for ev in self._events:
+            main.wait_event(ev)
+        host = torch.cat(self._infos + [self._nz_flat]).cpu().tolist()        # the one synchronisation
+        n = len(self._records)
+        info_host, nz_host = host[:n], host[n:]
+        self._keep_alive = None
+        for (flat, k, which, out), inf in zip(self._records, info_host):
+            if not nz_host[flat]:
+                continue                                            # all-zero factor: inverse skipped
+            if inf != 0:
+                raise torch.linalg.LinAlgError(
+                    f'cholesky_inv: the leading minor of order {inf} of kron.{which} + damping is not '
+                    f'positive-definite')
+            setattr(k, which + '_inv', out)
+            if self._replace:
+                setattr(k, which, None)
+
+
+def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_inv=True, eps=1e-7, replace=False,
+                       defer=False):
     """Kron.update_inv for many Kron objects at once (asdl/symmatrix.py:499-534 per object).
 
     One damping launch for all pairs, one batched Cholesky inverse per distinct matrix size, and
     a single device-to-host read at the end for the zero / not-positive-definite flags (the
-    reference synchronises three to five times per layer)."""
+    reference synchronises three to five times per layer).  With ``defer=True`` the launches are
+    enqueued and a PendingInverses is returned: the caller may enqueue unrelated work (the loss
+    backward pass) before calling its finish()."""
     krons = [k for k in krons if k is not None]
     if not krons:
-        return
+        return None
     for k in krons:
         if not k.has_data:
             raise ValueError('data do not exist.')
@@ -83,8 +120,8 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             outs.append(old if reuse else torch.empty_like(mat))
         info = torch.empty(len(entries), dtype=torch.int32, device=dev)
         prepared.append((entries, outs, lam_flat[idx], nz_flat[idx].contiguous(), info))
-    infos, records = [], []
-    use_streams = mats_on_gpu and len(prepared) > 1
+    infos, records, events = [], [], []
+    use_streams = mats_on_gpu and (len(prepared) > 1 or defer)
     if use_streams:
         main = torch.cuda.current_stream()
         side = _side_streams(dev, min(4, len(prepared)))
@@ -104,18 +141,12 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         for st in side:
             done = torch.cuda.Event()
             done.record(st)
-            main.wait_event(done)
-    host = torch.cat(infos + [nz_flat]).cpu().tolist()        # the one synchronisation
-    info_host, nz_host = host[:len(records)], host[len(records):]
-    for (flat, k, which, out), inf in zip(records, info_host):
-        if not nz_host[flat]:
-            continue                                            # all-zero factor: inverse skipped
-        if inf != 0:
-            raise torch.linalg.LinAlgError(
-                f'cholesky_inv: the leading minor of order {inf} of kron.{which} + damping is not positive-definite')
-        setattr(k, which + '_inv', out)
-        if replace:
-            setattr(k, which, None)
+            events.append(done)
+    pending = PendingInverses(records, infos, nz_flat, events, replace, keep_alive=(prepared, lam, nonzero, A_list, B_list))
+    if defer:
+        return pending
+    pending.finish()
+    return None
 
 
 class Kron:
