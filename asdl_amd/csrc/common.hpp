@@ -166,6 +166,20 @@ __global__ __launch_bounds__(256) void syrk_finalize_kernel(const float* __restr
   }
 }
 
+// Division by a run-time constant: q = umulhi(x, ceil(2^32 / d)), exact while x * d < 2^32.
+__host__ __device__ inline uint32_t make_magic(uint32_t d) { return static_cast<uint32_t>((0x100000000ull + d - 1) / d); }
+__device__ __forceinline__ uint32_t fastdiv(uint32_t x, uint32_t magic, uint32_t d) {
+  return d == 1 ? x : __umulhi(x, magic);
+}
+
+// bf16 X^T X with direct global -> LDS panel loads (syrk_dtl.hip).  *_ok tells whether the operand meets its
+// alignment and range requirements; the launcher may still answer AK_ERR_UNSUPPORTED / AK_ERR_WORKSPACE, on
+// which callers take the register-staged kernel.
+bool syrk_dtl_plain_ok(const void* X, int64_t M, int64_t d, int64_t ldx);
+size_t syrk_dtl_plain_ws_bytes(int64_t M, int64_t d, int64_t ldx);
+int syrk_dtl_plain(const void* X, int64_t M, int64_t d, int64_t ldx, float alpha, float beta, float* C, int64_t ldc,
+                   void* ws, size_t ws_bytes, hipStream_t stream);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_ERR_LAUNCH; }
 
 // Split-K factor shared by the SYRK front ends: enough work groups to fill 256 CUs twice over

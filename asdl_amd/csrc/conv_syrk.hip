@@ -51,11 +51,6 @@ struct ConvSyrkParams {
   int RP, dcl, dkx, dr;   // LDS rows staged per pass of the work group, and that step decomposed as (channel, kx, row)
 };
 
-__host__ __device__ inline uint32_t make_magic(uint32_t d) { return static_cast<uint32_t>((0x100000000ull + d - 1) / d); }
-// exact for x * d < 2^32
-__device__ __forceinline__ uint32_t fastdiv(uint32_t x, uint32_t magic, uint32_t d) {
-  return d == 1 ? x : __umulhi(x, magic);
-}
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 __attribute__((aligned(2))) uint4_a2;

@@ -1,0 +1,577 @@
+// bf16 rank-k update C <- beta*C + alpha * U^T U whose panels travel global memory -> LDS without
+// passing through registers (buffer_load_dwordx4 ... lds), for two kinds of U:
+//   plain : U = X, a row-major [M, d] matrix (the contraction index is the strided one);
+//   gather: U = the unfolded input of a convolution, never materialised.  x is [N, H, W, C] (channels
+//           last); row (n,oy,ox) of U holds, for every tap (ky,kx), the C channels of input pixel
+//           (oy*sh - ph + ky, ox*sw - pw + kx), zeros outside the image.  The kernel works in the
+//           column order (c/G, ky, kx, c%G) for a group size G (a multiple of 8 dividing C): 8 consecutive
+//           columns are 16 contiguous bytes of x.  The epilogue applies the permutation to the (c,ky,kx)
+//           order of the dense factor, which stays inside blocks of G*kh*kw columns.  G = C makes the
+//           gathered rows longest (best for the loads), G = 8 keeps a tile's writes within a few cache
+//           lines (best for large factors, whose epilogue would otherwise scatter 4-byte writes).
+//
+// One work group owns one BT x BT tile of the upper triangle and, with split-K, a slice of the M rows.
+// A k-tile is 32 rows.  Per k-tile and panel the LDS holds BT/32 column blocks, each [32 rows][32 cols]
+// bf16 with 64-byte rows: one wave-wide 16-byte load fills 16 rows of a block (lane l -> row l/4,
+// 16-byte chunk l%4), so every lane keeps the same row for all its loads of a k-tile and the 64 bytes per
+// row stay contiguous in global memory.  ds_read_b64_tr_b16 then finds, for the 32 lanes it serves per
+// pass, 4 rows x 64 bytes = 256 consecutive bytes: no bank conflicts and no padding.
+// The loads run STAGES-1 k-tiles ahead of the MFMAs; completion is tracked with s_waitcnt vmcnt, the
+// hand-over between waves with one barrier per k-tile.  Rows and columns outside the matrix (or taps
+// outside the image) are given a byte offset beyond the buffer range, for which the hardware returns
+// zeros, so the main loop has no masks and no branches.
+#include <cmath>
+#include <type_traits>
+#include "common.hpp"
+
+namespace ak {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#define AK_LDS __attribute__((address_space(3)))
+
+constexpr int kDtlBK = 32;              // rows per k-tile
+constexpr int kDtlStages = 4;          // >= 3: the loads run two k-tiles ahead of the one being read
+constexpr uint32_t kDtlRange = 0xFFFFFF00u;   // num_records of the descriptor; larger offsets read as zero
+constexpr uint32_t kDtlOob = 0xFFFFFFFFu;
+
+struct DtlParams {
+  const void* X;
+  float* C;
+  float* ws;
+  int64_t M, d, ldc, rows_per_split;
+  uint32_t row_bytes;      // plain: bytes between rows of X
+  int T, nsplit;
+  float alpha, beta;
+  // gather geometry
+  int Cin, H, W, kw, KK, sh, sw, ph, pw, Ho, Wo;
+  int G;                          // channels per column group
+  uint32_t mWo, mHo, mKw, mBlk, mG;   // magic multipliers: Wo, Ho, kw, G*KK, G
+};
+
+// 16 bytes per lane, global -> LDS at m0 + 16*lane.  The compiler does not see the LDS write: callers
+// order it against LDS reads with s_waitcnt vmcnt + a barrier.
+__device__ __forceinline__ void load_to_lds(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  // gfx9 encoding: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14; expcnt/lgkmcnt left at "no wait"
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
+// Working column v = blk*(G*KK) + tap*G + cg stands for channel c = G*blk + cg and tap (ky,kx).
+__device__ __forceinline__ void decode_column(uint32_t v, const DtlParams& p, uint32_t& c, uint32_t& tap) {
+  const uint32_t blk = fastdiv(v, p.mBlk, p.G * p.KK);
+  const uint32_t rem = v - blk * p.G * p.KK;
+  tap = fastdiv(rem, p.mG, p.G);
+  c = blk * p.G + rem - tap * p.G;
+}
+
+template <bool GATHER>
+__device__ __forceinline__ int64_t out_index(int64_t v, const DtlParams& p) {
+  if constexpr (!GATHER) return v;
+  uint32_t c, tap;
+  decode_column(static_cast<uint32_t>(v), p, c, tap);
+  return static_cast<int64_t>(c * p.KK + tap);
+}
+
+// Writes one wave's accumulators: C[oi][oj] = beta*C + alpha*acc and the mirror off the diagonal tile.
+template <int FR, int FC, bool GATHER>
+__device__ __forceinline__ void dtl_epilogue(floatx16 (&acc)[FR][FC], const DtlParams& p, int64_t gi0, int64_t gj0,
+                                             bool diag_tile, int lane) {
+  if constexpr (!GATHER) {
+    syrk_epilogue<FR, FC>(acc, p.C, p.ldc, p.d, gi0, gj0, diag_tile, p.alpha, p.beta, lane);
+  } else {
+    const int g = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int b = 0; b < FC; ++b) {
+      const int64_t gj = gj0 + 32 * b + l32;
+      if (gj >= p.d) continue;
+      const int64_t oj = out_index<true>(gj, p);
+#pragma unroll
+      for (int a = 0; a < FR; ++a) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t gi = gi0 + 32 * a + 8 * q + 4 * g;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (gi + e >= p.d) continue;
+            const int64_t oi = out_index<true>(gi + e, p);
+            float v = p.alpha * acc[a][b][4 * q + e];
+            float* dst = p.C + oi * p.ldc + oj;
+            if (p.beta != 0.f) v += p.beta * *dst;
+            *dst = v;
+            if (!diag_tile) p.C[oj * p.ldc + oi] = v;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int WR, int WC, int FR, int FC, bool GATHER>
+struct DtlCfg {
+  static constexpr int NW = WR * WC;
+  static constexpr int BT = 32 * FR * WR;
+  static constexpr int NCB = BT / 32;                         // column blocks per panel
+  static constexpr int BLOCK_BYTES = kDtlBK * 64;             // one column block of one k-tile
+  static constexpr int PANEL_BYTES = NCB * BLOCK_BYTES;
+  static constexpr int STAGE_BYTES = 2 * PANEL_BYTES;
+  static constexpr int LDS_BYTES = kDtlStages * STAGE_BYTES;
+  static constexpr int IPW = NCB * (kDtlBK / 16) / NW;        // wave-wide loads per wave, panel and k-tile
+  static_assert(32 * FC * WC == BT, "square work-group tile");
+  static_assert(NCB * (kDtlBK / 16) % NW == 0 && IPW >= 1, "loads must split evenly over the waves");
+};
+
+template <int WR, int WC, int FR, int FC, bool GATHER>
+__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
+  using Cfg = DtlCfg<WR, WC, FR, FC, GATHER>;
+  constexpr int NW = Cfg::NW, BT = Cfg::BT, NCB = Cfg::NCB, IPW = Cfg::IPW, BK = kDtlBK, S = kDtlStages;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char dtl_smem[];
+  AK_LDS unsigned char* lds = (AK_LDS unsigned char*)dtl_smem;
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = wave / WC, wc = wave % WC;
+  int ti, tj;
+  decode_upper_tile(blockIdx.x, p.T, ti, tj);
+  const bool diag = (ti == tj);
+  const int64_t i0 = static_cast<int64_t>(ti) * BT, j0 = static_cast<int64_t>(tj) * BT;
+  const int64_t k_begin = static_cast<int64_t>(blockIdx.y) * p.rows_per_split;
+  int64_t k_end = k_begin + p.rows_per_split;
+  if (k_end > p.M) k_end = p.M;
+  const int rows = k_begin < k_end ? static_cast<int>(k_end - k_begin) : 0;
+  const int nk = (rows + BK - 1) / BK;
+
+  // buffer descriptor: plain mode is based at this split's first row, gather mode at the tensor
+  const unsigned char* base = static_cast<const unsigned char*>(p.X);
+  if constexpr (!GATHER) base += k_begin * static_cast<int64_t>(p.row_bytes);
+  const uint64_t ba = reinterpret_cast<uint64_t>(base);
+  u32x4 rsrc;
+  rsrc[0] = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ba));
+  rsrc[1] = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ba >> 32) & 0xffffu);
+  rsrc[2] = kDtlRange;
+  rsrc[3] = 0x00020000u;
+
+  // this lane's part in the panel loads: one row of the k-tile, IPW 16-byte chunks per panel
+  const int half = wave & 1;                       // rows 16*half .. 16*half+15 of the k-tile
+  const int row_in_tile = 16 * half + (lane >> 2);
+  const int cb0 = (wave >> 1) * IPW;               // first column block this wave loads
+  uint32_t coloff[2][IPW];                         // byte offset of the chunk inside a row (kDtlOob: no such column)
+  int tapy[2][IPW], tapx[2][IPW];
+#pragma unroll
+  for (int P = 0; P < 2; ++P) {
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) {
+      const int64_t v = (P == 0 ? i0 : j0) + 32 * (cb0 + i) + 8 * (lane & 3);
+      tapy[P][i] = tapx[P][i] = 0;
+      if (v >= p.d) {
+        coloff[P][i] = kDtlOob;
+      } else if constexpr (!GATHER) {
+        coloff[P][i] = static_cast<uint32_t>(v) * 2u;
+      } else {
+        uint32_t c, tap;
+        decode_column(static_cast<uint32_t>(v), p, c, tap);
+        const uint32_t ky = fastdiv(tap, p.mKw, p.kw), kx = tap - ky * p.kw;
+        tapy[P][i] = ky;
+        tapx[P][i] = kx;
+        coloff[P][i] = ((ky * p.W + kx) * p.Cin + c) * 2u;
+      }
+    }
+  }
+  const uint32_t lds_lane_blk = lds0 + cb0 * Cfg::BLOCK_BYTES + half * 1024;   // + stage + panel + i*BLOCK_BYTES
+
+  // Row part of the addresses of one k-tile (shared by all loads of the lane), then one load per call.
+  struct RowState { uint32_t rowoff; int iy0, ix0; bool ok; uint32_t sbase; };
+  auto prepare = [&](int kt, int stage) {
+    RowState st;
+    const int r = kt * BK + row_in_tile;           // row of this split
+    st.ok = r < rows;
+    st.iy0 = st.ix0 = 0;
+    if constexpr (!GATHER) {
+      st.rowoff = static_cast<uint32_t>(r) * p.row_bytes;
+    } else {
+      const uint32_t pos = static_cast<uint32_t>(k_begin) + r;
+      const uint32_t q1 = fastdiv(pos, p.mWo, p.Wo);
+      const uint32_t ox = pos - q1 * p.Wo;
+      const uint32_t n = fastdiv(q1, p.mHo, p.Ho);
+      const uint32_t oy = q1 - n * p.Ho;
+      st.iy0 = static_cast<int>(oy) * p.sh - p.ph;
+      st.ix0 = static_cast<int>(ox) * p.sw - p.pw;
+      st.rowoff = static_cast<uint32_t>((static_cast<int>(n * p.H) + st.iy0) * p.W + st.ix0) *
+                  static_cast<uint32_t>(p.Cin * 2);
+    }
+    st.sbase = lds_lane_blk + stage * Cfg::STAGE_BYTES;
+    return st;
+  };
+  auto load_one = [&](const RowState& st, int P, int i) {
+    bool ok = st.ok && coloff[P][i] != kDtlOob;
+    if constexpr (GATHER)
+      ok = ok && static_cast<unsigned>(st.iy0 + tapy[P][i]) < static_cast<unsigned>(p.H) &&
+           static_cast<unsigned>(st.ix0 + tapx[P][i]) < static_cast<unsigned>(p.W);
+    const uint32_t voff = ok ? st.rowoff + coloff[P][i] : kDtlOob;
+    load_to_lds(rsrc, st.sbase + P * Cfg::PANEL_BYTES + i * Cfg::BLOCK_BYTES, voff);
+  };
+
+  floatx16 acc[FR][FC];
+#pragma unroll
+  for (int a = 0; a < FR; ++a)
+#pragma unroll
+    for (int b = 0; b < FC; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  // fragment addressing: lane (g, hl, j) reads row 8g + j/4 (+4 for the second half of the fragment),
+  // bytes 32*hl + 8*(j%4) of its 64-byte row
+  const int g = lane >> 5, hl = (lane >> 4) & 1, j16 = lane & 15;
+  const int frag_lane = (8 * g + (j16 >> 2)) * 64 + hl * 32 + (j16 & 3) * 8;
+  AK_LDS const unsigned char* fragI = lds + frag_lane + wr * FR * Cfg::BLOCK_BYTES;
+  AK_LDS const unsigned char* fragJ = lds + frag_lane + wc * FC * Cfg::BLOCK_BYTES + (diag ? 0 : Cfg::PANEL_BYTES);
+
+  auto tr = [](AK_LDS const unsigned char* q) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((AK_LDS short4v*)(q));
+  };
+  // fragment u of a half k-tile in the order the MFMAs want them: a0, b0 .. b(FC-1), a1 .. a(FR-1)
+  auto read_unit = [&](bf16x8 (&fa)[FR], bf16x8 (&fb)[FC], int soff, int kk, int u) {
+    if (u == 0 || u > FC) {
+      const int a = u == 0 ? 0 : u - FC;
+      AK_LDS const unsigned char* q = fragI + soff + a * Cfg::BLOCK_BYTES + kk * 64;
+      fa[a] = pack_bf16x8(tr(q), tr(q + 256));
+    } else {
+      const int b = u - 1;
+      AK_LDS const unsigned char* q = fragJ + soff + b * Cfg::BLOCK_BYTES + kk * 64;
+      fb[b] = pack_bf16x8(tr(q), tr(q + 256));
+    }
+  };
+
+  // One half k-tile (16 rows): FR*FC MFMAs on the fragments (ca, cb), with the LDS reads of the next half's
+  // fragments (na, nb) and, if NLOAD > 0, the panel loads of a k-tile further ahead spread between them so
+  // that the matrix pipe never waits for their issue.
+  auto half_step = [&](auto nload_tag, const bf16x8 (&ca)[FR], const bf16x8 (&cb)[FC], bf16x8 (&na)[FR],
+                       bf16x8 (&nb)[FC], int soff_next, int kk_next, const RowState& st) {
+    constexpr int NLOAD = decltype(nload_tag)::value;
+    constexpr int NM = FR * FC, NS = NLOAD + FR + FC;
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      const int a = m / FC, b = m % FC;
+      acc[a][b] = mfma_bf16(ca[a], cb[b], acc[a][b]);
+#pragma unroll
+      for (int sidx = (m * NS) / NM; sidx < ((m + 1) * NS) / NM; ++sidx) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (sidx < NLOAD) load_one(st, sidx / IPW, sidx % IPW);
+        else read_unit(na, nb, soff_next, kk_next, sidx - NLOAD);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  auto mainloop = [&](auto diag_tag) {
+    constexpr bool DIAG = decltype(diag_tag)::value;
+    constexpr int LPT = IPW * (DIAG ? 1 : 2);      // loads per wave and k-tile
+#pragma unroll
+    for (int t = 0; t < S - 1; ++t) {              // tiles beyond nk load zeros: the counts stay uniform
+      const RowState st = prepare(t, t);
+#pragma unroll
+      for (int l = 0; l < LPT; ++l) load_one(st, l / IPW, l % IPW);
+    }
+    wait_vmcnt<(S - 2) * LPT>();                   // this wave's loads of k-tile 0 have landed
+    __syncthreads();                               // ... and everybody's
+    bf16x8 fa0[FR], fb0[FC], fa1[FR], fb1[FC];
+#pragma unroll
+    for (int u = 0; u < FR + FC; ++u) read_unit(fa0, fb0, 0, 0, u);
+    int rd = 0, wrs = S - 1;
+    const RowState none{};
+    for (int kt = 0; kt < nk; ++kt) {
+      // first half: MFMAs on rows 0..15 of k-tile kt while rows 16..31 come out of the LDS
+      half_step(std::integral_constant<int, 0>{}, fa0, fb0, fa1, fb1, rd * Cfg::STAGE_BYTES, 16, none);
+      wait_vmcnt<(S - 3) * LPT>();                 // own loads of k-tile kt+1 have landed
+      __syncthreads();                             // everybody's have; nobody reads k-tile kt-1 any more
+      // second half: MFMAs on rows 16..31 while k-tile kt+S-1 is requested into the stage k-tile kt-1
+      // occupied and rows 0..15 of k-tile kt+1 come out of the LDS
+      const RowState st = prepare(kt + S - 1, wrs);
+      rd = (rd + 1 == S) ? 0 : rd + 1;
+      wrs = (wrs + 1 == S) ? 0 : wrs + 1;
+      half_step(std::integral_constant<int, LPT>{}, fa1, fb1, fa0, fb0, rd * Cfg::STAGE_BYTES, 0, st);
+    }
+    wait_vmcnt<0>();                               // drain the zero-fill loads before the LDS is released
+  };
+  if (diag) mainloop(std::true_type{});
+  else mainloop(std::false_type{});
+
+  const int64_t gi0 = i0 + 32 * FR * wr, gj0 = j0 + 32 * FC * wc;
+  if (p.nsplit == 1) {
+    dtl_epilogue<FR, FC, GATHER>(acc, p, gi0, gj0, diag, lane);
+  } else {
+    // partial tile in accumulator order: [(a,b,q)][thread] float4
+    floatx4* dst = reinterpret_cast<floatx4*>(p.ws) +
+                   (static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * (BT * BT / 4);
+#pragma unroll
+    for (int a = 0; a < FR; ++a)
+#pragma unroll
+      for (int b = 0; b < FC; ++b)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          floatx4 w = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]};
+          dst[((a * FC + b) * 4 + q) * (NW * 64) + tid] = w;
+        }
+  }
+}
+
+// Split-K reduction, first stage (only for many splits): work group (tile, slot, g) sums partials
+// [g*group, min((g+1)*group, n)) of its float4 slot and writes the sum as partial g of a second buffer with
+// the same layout.  Fixed summation order.
+template <int NT>
+__global__ __launch_bounds__(NT) void syrk_dtl_reduce_kernel(const floatx4* __restrict__ src, floatx4* __restrict__ dst,
+                                                             int n, int group, size_t tile_f4) {
+  const size_t split_stride = static_cast<size_t>(gridDim.x) * tile_f4;
+  const size_t off = blockIdx.x * tile_f4 + static_cast<size_t>(blockIdx.y) * NT + threadIdx.x;
+  const int s0 = blockIdx.z * group;
+  const int s1 = s0 + group < n ? s0 + group : n;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  int s = s0;
+  for (; s + 4 <= s1; s += 4) {
+    const floatx4 w0 = src[off + (s + 0) * split_stride], w1 = src[off + (s + 1) * split_stride];
+    const floatx4 w2 = src[off + (s + 2) * split_stride], w3 = src[off + (s + 3) * split_stride];
+    acc += w0; acc += w1; acc += w2; acc += w3;
+  }
+  for (; s < s1; ++s) acc += src[off + s * split_stride];
+  dst[off + blockIdx.z * split_stride] = acc;
+}
+
+// Sums the (remaining) partials in a fixed order and applies the epilogue.  grid (tiles, 4*FR*FC): each work
+// group owns one float4 slot (a, b, q) of every thread's accumulators.
+template <int WR, int WC, int FR, int FC, bool GATHER>
+__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_kernel(DtlParams p, const floatx4* __restrict__ part,
+                                                                         int n) {
+  constexpr int NW = WR * WC, BT = 32 * FR * WR;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave / WC, wc = wave % WC, g = lane >> 5, l32 = lane & 31;
+  int ti, tj;
+  decode_upper_tile(blockIdx.x, p.T, ti, tj);
+  const int slot = blockIdx.y;                     // (a * FC + b) * 4 + q
+  const int q = slot & 3, b = (slot >> 2) % FC, a = (slot >> 2) / FC;
+  const size_t tile_f4 = BT * BT / 4;
+  const floatx4* src = part + blockIdx.x * tile_f4 + slot * (NW * 64) + tid;
+  const size_t split_stride = static_cast<size_t>(gridDim.x) * tile_f4;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  int s = 0;
+  for (; s + 4 <= n; s += 4) {
+    const floatx4 w0 = src[(s + 0) * split_stride], w1 = src[(s + 1) * split_stride];
+    const floatx4 w2 = src[(s + 2) * split_stride], w3 = src[(s + 3) * split_stride];
+    acc += w0; acc += w1; acc += w2; acc += w3;
+  }
+  for (; s < n; ++s) acc += src[s * split_stride];
+  const int64_t gj = static_cast<int64_t>(tj) * BT + 32 * FC * wc + 32 * b + l32;
+  const int64_t gi = static_cast<int64_t>(ti) * BT + 32 * FR * wr + 32 * a + 8 * q + 4 * g;
+  if (gj >= p.d) return;
+  const int64_t oj = out_index<GATHER>(gj, p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (gi + e >= p.d) continue;
+    const int64_t oi = out_index<GATHER>(gi + e, p);
+    float v = p.alpha * acc[e];
+    float* dst = p.C + oi * p.ldc + oj;
+    if (p.beta != 0.f) v += p.beta * *dst;
+    *dst = v;
+    if (ti != tj) p.C[oj * p.ldc + oi] = v;
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------
+
+constexpr int kDtlDirectSplits = 24;   // up to this many partials the epilogue pass sums them itself
+
+struct DtlPlan {
+  int bt;          // work-group tile: 64, 128 or 256
+  int T, nsplit;
+  int group, ngroups;   // two-stage reduction: partials per first-stage sum, number of sums (0: single stage)
+  int64_t ntiles, rows_per_split;
+  size_t ws_bytes;
+};
+
+static int g_force_bt = 0, g_force_ns = 0;   // tuning hook (ak_debug_force_syrk_plan); 0: use the model
+
+// Tile size and split-K factor from a small cost model (microseconds, constants measured on MI355X): the
+// k-tiles of one split times the k-tile time of the most loaded CU, a fixed charge per work group, the
+// partial-tile traffic and the reduction passes.
+static DtlPlan dtl_plan(int64_t M, int64_t d, int64_t max_rows_per_split, bool gather) {
+  struct Cand { int bt; int occ; double t_alone, t_shared, t_fix; };
+  // t_alone: k-tile time of a work group that has its CU to itself, t_shared: with `occ` of them on the CU
+  const Cand cands[3] = {{64, 4, 0.20, 0.20, 3.0},
+                         {128, 2, gather ? 0.40 : 0.25, 0.59, 4.0},
+                         {256, 1, gather ? 0.95 : 0.70, gather ? 0.95 : 0.70, 8.0}};
+  const int64_t ktiles = (M + kDtlBK - 1) / kDtlBK;
+  DtlPlan best{};
+  double best_cost = 1e300;
+  for (const Cand& c : cands) {
+    if (g_force_bt != 0 && c.bt != g_force_bt) continue;
+    if (g_force_bt == 0 && c.bt == 64 && d > 192) continue;
+    if (g_force_bt == 0 && c.bt == 256 && d < 1024) continue;
+    const int64_t T = (d + c.bt - 1) / c.bt, ntiles = T * (T + 1) / 2;
+    const int64_t slots = 256 * c.occ;
+    const int64_t ns_cap = ktiles / 4 < 1 ? 1 : (ktiles / 4 > 1024 ? 1024 : ktiles / 4);
+    for (int64_t ns = 1; ns <= ns_cap; ++ns) {
+      if (g_force_ns != 0 && ns != (g_force_ns < ns_cap ? g_force_ns : ns_cap)) continue;
+      const int64_t kt_split = (ktiles + ns - 1) / ns;
+      if (kt_split * kDtlBK > max_rows_per_split) continue;
+      const int64_t ns_eff = (ktiles + kt_split - 1) / kt_split;
+      const int64_t wgs = ntiles * ns_eff, rounds = (wgs + slots - 1) / slots;
+      int64_t per_cu = (wgs + 255) / 256;
+      if (per_cu > c.occ) per_cu = c.occ;
+      const double t_kt = c.occ > 1 ? c.t_alone + (c.t_shared - c.t_alone) * (per_cu - 1) / (c.occ - 1) : c.t_alone;
+      double cost = static_cast<double>(rounds) * (static_cast<double>(kt_split) * t_kt + c.t_fix);
+      if (ns_eff > 1) {
+        const double part_mb = static_cast<double>(wgs) * c.bt * c.bt * 4.0 * 1e-6;
+        cost += 2.0 * part_mb / 5.0;                                // written once, read once, ~5 TB/s out of L2/MALL
+        cost += ns_eff <= kDtlDirectSplits ? 3.0 + 0.08 * ns_eff : 7.0 + 0.3 * std::sqrt(static_cast<double>(ns_eff));
+      }
+      if (cost < best_cost) {
+        best_cost = cost;
+        best.bt = c.bt;
+        best.T = static_cast<int>(T);
+        best.ntiles = ntiles;
+        best.rows_per_split = kt_split * kDtlBK;
+      }
+    }
+  }
+  if (best.bt == 0) {                                               // nothing fits the offset range
+    best.bt = 128;
+    best.T = static_cast<int>((d + 127) / 128);
+    best.ntiles = static_cast<int64_t>(best.T) * (best.T + 1) / 2;
+    best.rows_per_split = ((M + kDtlBK - 1) / kDtlBK) * kDtlBK;
+  }
+  best.nsplit = static_cast<int>((M + best.rows_per_split - 1) / best.rows_per_split);
+  if (best.nsplit < 1) best.nsplit = 1;
+  best.group = best.ngroups = 0;
+  size_t parts = best.nsplit > 1 ? best.nsplit : 0;
+  if (best.nsplit > kDtlDirectSplits) {
+    best.group = static_cast<int>(std::ceil(std::sqrt(static_cast<double>(best.nsplit))));
+    best.ngroups = (best.nsplit + best.group - 1) / best.group;
+    parts += best.ngroups;
+  }
+  best.ws_bytes = parts * best.ntiles * best.bt * best.bt * sizeof(float);
+  return best;
+}
+
+template <int WR, int WC, int FR, int FC, bool GATHER>
+static int dtl_launch_cfg(const DtlParams& p, const DtlPlan& pl, hipStream_t stream) {
+  using Cfg = DtlCfg<WR, WC, FR, FC, GATHER>;
+  auto kern = syrk_dtl_kernel<WR, WC, FR, FC, GATHER>;
+  if (Cfg::LDS_BYTES > 64 * 1024) {
+    static bool attr_set = false;     // idempotent; a race sets it twice at worst
+    if (!attr_set) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              Cfg::LDS_BYTES) != hipSuccess)
+        return AK_ERR_LAUNCH;
+      attr_set = true;
+    }
+  }
+  const unsigned ntiles = static_cast<unsigned>(pl.ntiles);
+  hipLaunchKernelGGL(kern, dim3(ntiles, static_cast<unsigned>(p.nsplit)), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, stream, p);
+  if (p.nsplit > 1) {
+    const size_t tile_f4 = static_cast<size_t>(Cfg::BT) * Cfg::BT / 4;
+    const floatx4* part = reinterpret_cast<const floatx4*>(p.ws);
+    int n = p.nsplit;
+    if (pl.ngroups > 0) {
+      floatx4* sums = reinterpret_cast<floatx4*>(p.ws) + static_cast<size_t>(p.nsplit) * pl.ntiles * tile_f4;
+      hipLaunchKernelGGL((syrk_dtl_reduce_kernel<Cfg::NW * 64>), dim3(ntiles, 4 * FR * FC, pl.ngroups),
+                         dim3(Cfg::NW * 64), 0, stream, part, sums, p.nsplit, pl.group, tile_f4);
+      part = sums;
+      n = pl.ngroups;
+    }
+    hipLaunchKernelGGL((syrk_dtl_finalize_kernel<WR, WC, FR, FC, GATHER>), dim3(ntiles, 4 * FR * FC),
+                       dim3(Cfg::NW * 64), 0, stream, p, part, n);
+  }
+  return check_launch();
+}
+
+template <bool GATHER>
+static int dtl_launch(DtlParams& p, const DtlPlan& pl, void* ws, size_t ws_bytes, hipStream_t stream) {
+  if (pl.ws_bytes > 0 && (ws == nullptr || ws_bytes < pl.ws_bytes)) return AK_ERR_WORKSPACE;
+  p.T = pl.T;
+  p.nsplit = pl.nsplit;
+  p.rows_per_split = pl.rows_per_split;
+  p.ws = static_cast<float*>(ws);
+  if (pl.bt == 64) return dtl_launch_cfg<2, 2, 1, 1, GATHER>(p, pl, stream);
+  if (pl.bt == 256) return dtl_launch_cfg<2, 2, 4, 4, GATHER>(p, pl, stream);
+  return dtl_launch_cfg<2, 2, 2, 2, GATHER>(p, pl, stream);
+}
+
+bool syrk_dtl_plain_ok(const void* X, int64_t M, int64_t d, int64_t ldx) {
+  return M > 0 && d % 8 == 0 && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0 &&
+         ldx * 2 * static_cast<int64_t>(kDtlBK) <= static_cast<int64_t>(kDtlRange);
+}
+
+static int64_t plain_max_rows(int64_t ldx) { return static_cast<int64_t>(kDtlRange) / (ldx * 2); }
+
+size_t syrk_dtl_plain_ws_bytes(int64_t M, int64_t d, int64_t ldx) {
+  return dtl_plan(M, d, plain_max_rows(ldx), false).ws_bytes;
+}
+
+int syrk_dtl_plain(const void* X, int64_t M, int64_t d, int64_t ldx, float alpha, float beta, float* C,
+                   int64_t ldc, void* ws, size_t ws_bytes, hipStream_t stream) {
+  DtlParams p{};
+  p.X = X; p.C = C; p.M = M; p.d = d; p.ldc = ldc;
+  p.row_bytes = static_cast<uint32_t>(ldx * 2);
+  p.alpha = alpha; p.beta = beta;
+  p.Cin = 1; p.KK = 1;
+  const DtlPlan pl = dtl_plan(M, d, plain_max_rows(ldx), false);
+  if (pl.rows_per_split > plain_max_rows(ldx)) return AK_ERR_UNSUPPORTED;
+  return dtl_launch<false>(p, pl, ws, ws_bytes, stream);
+}
+
+static bool nhwc_ok(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw,
+                    int ph, int pw, int64_t& Ho, int64_t& Wo) {
+  if (x == nullptr || N <= 0 || C <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 || ph < 0 ||
+      pw < 0)
+    return false;
+  Ho = (H + 2 * ph - kh) / sh + 1;
+  Wo = (W + 2 * pw - kw) / sw + 1;
+  if (Ho <= 0 || Wo <= 0) return false;
+  return true;
+}
+
+}  // namespace ak
+
+// Not part of the public interface: pins the tile size (64/128/256) and split-K factor of the direct-to-LDS
+// SYRK for tuning runs; (0, 0) restores the cost model.
+extern "C" void ak_debug_force_syrk_plan(int bt, int nsplit) {
+  ak::g_force_bt = bt;
+  ak::g_force_ns = nsplit;
+}
+
+extern "C" size_t ak_conv_syrk_nhwc_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh,
+                                             int sw, int ph, int pw) {
+  int64_t Ho, Wo;
+  if (!ak::nhwc_ok(reinterpret_cast<const void*>(16), N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return 0;
+  return ak::dtl_plan(N * Ho * Wo, C * kh * kw, INT64_MAX, true).ws_bytes;
+}
+
+extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw,
+                                 int sh, int sw, int ph, int pw, float alpha, float beta, float* A, int64_t lda,
+                                 void* ws, size_t ws_bytes, ak_stream_t stream) {
+  int64_t Ho, Wo;
+  if (A == nullptr || !ak::nhwc_ok(x, N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return AK_ERR_ARG;
+  const int64_t d = C * kh * kw, M = N * Ho * Wo;
+  if (lda < d) return AK_ERR_ARG;
+  if (dtype != AK_BF16) return AK_ERR_UNSUPPORTED;
+  // 16-byte chunks must not straddle taps, offsets must fit the 32-bit buffer range, and the magic
+  // divisions by Wo, Ho, C and kw must be exact over their operand ranges
+  if (C % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return AK_ERR_UNSUPPORTED;
+  if (N * H * W * C * 2 > static_cast<int64_t>(ak::kDtlRange)) return AK_ERR_UNSUPPORTED;
+  if (M * (Wo > Ho ? Wo : Ho) >= (1ll << 32) || (d + 256) * d >= (1ll << 32)) return AK_ERR_UNSUPPORTED;
+  ak::DtlParams p{};
+  p.X = x; p.C = A; p.M = M; p.d = d; p.ldc = lda;
+  p.alpha = alpha; p.beta = beta;
+  p.Cin = static_cast<int>(C); p.H = static_cast<int>(H); p.W = static_cast<int>(W);
+  p.kw = kw; p.KK = kh * kw; p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw;
+  p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
+  p.mWo = ak::make_magic(p.Wo); p.mHo = ak::make_magic(p.Ho); p.mKw = ak::make_magic(kw);
+  p.G = d >= 3456 ? 8 : p.Cin;
+  p.mBlk = ak::make_magic(p.G * p.KK); p.mG = ak::make_magic(p.G);
+  const ak::DtlPlan pl = ak::dtl_plan(M, d, INT64_MAX, true);
+  return ak::dtl_launch<true>(p, pl, ws, ws_bytes, static_cast<hipStream_t>(stream));
+}

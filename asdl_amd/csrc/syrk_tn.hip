@@ -233,13 +233,19 @@ extern "C" size_t ak_syrk_tn_ws_bytes(int64_t M, int64_t d) {
   const int64_t ntiles = Tn * (Tn + 1) / 2;
   // upper bound over both dtypes (bf16 has the fewer k-steps, fp32 the more)
   const int ns = ak::pick_nsplit(ntiles, (M + 15) / 16);
-  return ns > 1 ? static_cast<size_t>(ns) * ntiles * 128 * 128 * sizeof(float) : 0;
+  const size_t staged = ns > 1 ? static_cast<size_t>(ns) * ntiles * 128 * 128 * sizeof(float) : 0;
+  const size_t direct = d % 8 == 0 ? ak::syrk_dtl_plain_ws_bytes(M, d, d) : 0;
+  return staged > direct ? staged : direct;
 }
 
 extern "C" int ak_syrk_tn(const void* X, int dtype, int64_t M, int64_t d, int64_t ldx, float alpha, float beta,
                           float* C, int64_t ldc, void* ws, size_t ws_bytes, ak_stream_t stream) {
   if (X == nullptr || C == nullptr || M < 0 || d <= 0 || ldx < d || ldc < d) return AK_ERR_ARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == AK_BF16 && ak::syrk_dtl_plain_ok(X, M, d, ldx)) {
+    const int rc = ak::syrk_dtl_plain(X, M, d, ldx, alpha, beta, C, ldc, ws, ws_bytes, s);
+    if (rc != AK_ERR_UNSUPPORTED && rc != AK_ERR_WORKSPACE) return rc;
+  }
   if (dtype == AK_BF16) return ak::launch_syrk_tn<uint16_t>(X, M, d, ldx, alpha, beta, C, ldc, ws, ws_bytes, s);
   if (dtype == AK_F32) return ak::launch_syrk_tn<float>(X, M, d, ldx, alpha, beta, C, ldc, ws, ws_bytes, s);
   return AK_ERR_ARG;

@@ -130,13 +130,21 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     return out
 
 
+AK_ERR_UNSUPPORTED = -3
+
+
+def _is_channels_last(x):
+    return (x.ndim == 4 and x.shape[1] > 1 and x.is_contiguous(memory_format=torch.channels_last)
+            and not x.is_contiguous())
+
+
 def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
-    """out <- beta*out + alpha * sum_{n,pos} patch patch^T for x = [N, C, H, W] (NCHW contiguous),
-    patches ordered (c, ky, kx); no division by the output size (fold it into alpha)."""
+    """out <- beta*out + alpha * sum_{n,pos} patch patch^T for x = [N, C, H, W], patches ordered (c, ky, kx);
+    no division by the output size (fold it into alpha).  A channels-last bf16 x is read in place
+    (rows gathered from the NHWC memory); anything else goes through the NCHW kernel."""
     _require_gpu(x, out)
     if x.ndim != 4:
         raise ValueError(f'x.ndim has to be 4. Got {x.ndim}.')
-    x = x.contiguous()
     N, C, H, W = x.shape
     kh, kw = kernel_size
     sh, sw = stride
@@ -148,9 +156,22 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
         raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
     lib = _lib.load()
+    h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    if x.dtype == torch.bfloat16 and C % 8 == 0 and _is_channels_last(x):
+        if (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0):
+            return syrk_tn(x.permute(0, 2, 3, 1).reshape(N * H * W, C), out=out, alpha=alpha, beta=beta)
+        need = lib.ak_conv_syrk_nhwc_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)
+        ws, ws_bytes, keep = _ws_args(need, x.device)
+        with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
+            rc = lib.ak_conv_syrk_nhwc(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw,
+                                       ph, pw, alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0),
+                                       ws, ws_bytes, _stream())
+        if rc != AK_ERR_UNSUPPORTED:
+            _lib.check(rc, 'ak_conv_syrk_nhwc')
+            return out
+    x = x.contiguous()
     need = lib.ak_conv_syrk_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)
     ws, ws_bytes, keep = _ws_args(need, x.device)
-    h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
     with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
         rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw, ph, pw,
                               alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())

@@ -224,6 +224,9 @@ class Conv2d(Operation):
 
     @staticmethod
     def preprocess_out_grads(module, out_grads):
+        if kernels._is_channels_last(out_grads):
+            # [n, h, w, c_out] in memory: keep it, the rows of B's statistic are the pixels
+            return out_grads
         return out_grads.flatten(start_dim=2)
 
     @staticmethod
@@ -236,6 +239,10 @@ class Conv2d(Operation):
 
     @staticmethod
     def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        if out_grads.ndim == 4:                                               # channels last
+            n, c, h, w = out_grads.shape
+            rows = out_grads.permute(0, 2, 3, 1).reshape(n * h * w, c)        # a view
+            return kernels.syrk_tn(rows, out=out, alpha=alpha, beta=beta)
         return kernels.syrk_nt(out_grads, out=out, alpha=alpha, beta=beta)    # c_out x c_out
 
 

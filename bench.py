@@ -33,6 +33,8 @@ def parse():
     ap.add_argument('--batch', type=int, default=64)
     ap.add_argument('--fisher', default='fisher_mc', choices=['fisher_mc', 'fisher_emp'])
     ap.add_argument('--damping', type=float, default=1e-3)
+    ap.add_argument('--memory-format', default='channels_last', choices=['channels_last', 'contiguous'],
+                    help='layout of activations and conv weights; the K-FAC step is the same either way')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-batch', type=int, default=16,
                     help='batch of the CPU baseline sample (its time is scaled to the full batch)')
@@ -102,6 +104,9 @@ def main():
     model = bench_models.resnet50().to(dev)
     bs = args.batch
     x = torch.randn(bs, 3, 224, 224).to(dev)
+    if args.memory_format == 'channels_last':
+        model = model.to(memory_format=torch.channels_last)
+        x = x.contiguous(memory_format=torch.channels_last)
     t = torch.randint(0, 1000, (bs,)).to(dev)
     config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=[nn.BatchNorm2d])
     gm = KfacGradientMaker(model, config, fisher_type=args.fisher)
@@ -147,7 +152,7 @@ def main():
         'config': {'workload': f'K-FAC step (factors + pi-damped Cholesky inverses + precondition every step, '
                                f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
-                               f'BatchNorm ignored',
+                               f'BatchNorm ignored, {args.memory_format} activations and weights',
                    'batch': bs},
     }
     if sink:
@@ -156,7 +161,8 @@ def main():
         achieved = flops / secs / 1e12
         out['roofline'] = {'bound': 'mfma', 'achieved': achieved, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
                            'frac': achieved / BF16_MFMA_PEAK_TFLOPS, 'traffic': None,
-                           'kernel': 'factor statistics (conv_syrk_kernel / syrk_tn_kernel), SYRK FLOP M*d*(d+1)',
+                           'kernel': 'factor statistics (syrk_dtl_kernel; conv_syrk_kernel for the 3-channel stem), '
+                                     'SYRK FLOP M*d*(d+1)',
                            'launches_per_step': len(sink) // args.steps,
                            'factor_ms_per_step': secs / args.steps * 1e3,
                            'gemm_equiv_tflops': 2 * achieved}

@@ -71,6 +71,19 @@ int ak_conv_syrk(const void* x, int dtype, int64_t N, int64_t C, int64_t H, int6
                  float alpha, float beta, float* A, int64_t lda,
                  void* ws, size_t ws_bytes, ak_stream_t stream);
 
+/* Same statistic as ak_conv_syrk for a channels-last input: x = [N, H, W, C] contiguous (the memory of a
+ * torch.channels_last NCHW tensor), bf16, C a multiple of 8.  Rows of the unfolded input are gathered
+ * straight from x; A is written in the same (c,ky,kx) order as ak_conv_syrk, so both entry points
+ * are interchangeable replacements of im2col_2d (asdl/utils.py:51-71) + Conv2d.cov_kron_A
+ * (asdl/operations/conv.py:80-88).  AK_ERR_UNSUPPORTED for other dtypes, channel counts or tensors
+ * of 4 GiB and more: callers then use ak_conv_syrk on an NCHW copy. */
+size_t ak_conv_syrk_nhwc_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W,
+                                  int kh, int kw, int sh, int sw, int ph, int pw);
+int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C, int64_t H, int64_t W,
+                      int kh, int kw, int sh, int sw, int ph, int pw,
+                      float alpha, float beta, float* A, int64_t lda,
+                      void* ws, size_t ws_bytes, ak_stream_t stream);
+
 /* ---- damping ---------------------------------------------------------------------- */
 
 /* For each pair b < batch: tr(A_b), tr(B_b), the pi split

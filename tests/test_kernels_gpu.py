@@ -113,6 +113,64 @@ def test_conv_syrk_matches_oracle(K, dtype, case):
     assert torch.equal(out, out.T)
 
 
+NHWC_CASES = [
+    # N, C, H, W, kernel, stride, padding
+    (2, 8, 6, 6, (3, 3), (1, 1), (1, 1)),          # smallest channel count the gather path takes
+    (2, 64, 12, 12, (3, 3), (1, 1), (1, 1)),       # d = 576
+    (3, 64, 7, 7, (3, 3), (1, 1), (1, 1)),         # 7x7 maps: k-tiles straddle rows and images
+    (2, 128, 14, 14, (3, 3), (2, 2), (1, 1)),      # stride 2
+    (2, 32, 14, 14, (1, 1), (1, 1), (0, 0)),       # 1x1 conv: plain rows
+    (2, 32, 14, 14, (1, 1), (2, 2), (0, 0)),       # 1x1 stride 2 (downsample)
+    (2, 16, 9, 6, (3, 2), (2, 1), (0, 1)),         # asymmetric everything
+    (1, 152, 8, 8, (3, 3), (1, 1), (1, 1)),        # d = 1368: edge tiles, C not a power of two
+    (2, 24, 5, 70, (5, 5), (1, 1), (2, 2)),        # 25 taps
+    (5, 40, 33, 35, (3, 3), (1, 1), (1, 1)),       # M = 5775: split-K with a ragged last split
+    (2, 176, 12, 12, (3, 3), (1, 1), (1, 1)),      # d = 1584: 256-wide tiles with an edge tile
+    (2, 12, 6, 6, (3, 3), (1, 1), (1, 1)),         # C % 8 != 0: falls back to the NCHW kernel
+]
+
+
+@pytest.mark.parametrize('case', NHWC_CASES, ids=[str(c) for c in NHWC_CASES])
+def test_conv_syrk_channels_last_matches_oracle(K, case):
+    N, C, H, W, k, s, p = case
+    x = _inputs((N, C, H, W), torch.bfloat16, seed=N + 10 * C + H)
+    ref = R.conv_cov_kron_A(x.float().double(), k, s, p)
+    out_size = ((H + 2 * p[0] - k[0]) // s[0] + 1) * ((W + 2 * p[1] - k[1]) // s[1] + 1)
+    print(f'conv_syrk channels_last case={case}', flush=True)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last)
+    out = K.conv_syrk(xg, k, s, p, alpha=1.0 / out_size)
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5
+    assert torch.equal(out, out.T)
+    # same bits as the NCHW kernel is not required, same statistic is
+    out2 = K.conv_syrk(x.cuda(), k, s, p, alpha=1.0 / out_size)
+    assert relerr(out, out2.double()) < 1e-5
+
+
+def test_conv_syrk_channels_last_ema_accumulate(K):
+    x = _inputs((4, 16, 10, 10), torch.bfloat16, 1)
+    x2 = _inputs((4, 16, 10, 10), torch.bfloat16, 2)
+    A0 = R.conv_cov_kron_A(x.float(), (3, 3), (1, 1), (1, 1))
+    ref = 0.9 * A0.double() + 0.1 * R.conv_cov_kron_A(x2.float().double(), (3, 3), (1, 1), (1, 1))
+    out = A0.cuda().clone()
+    K.conv_syrk(x2.cuda().contiguous(memory_format=torch.channels_last), (3, 3), (1, 1), (1, 1), out=out,
+                alpha=0.1 / 100, beta=0.9)
+    assert relerr(out, ref) < TOL_FACTOR_F32
+
+
+@pytest.mark.parametrize('M,d,ld', [(4096, 64, 64), (20000, 64, 64), (3000, 1000, 1000), (777, 256, 320),
+                                    (100000, 128, 128), (33, 2048, 2048), (3000, 1600, 1600), (1500, 2560, 2568)])
+def test_syrk_tn_bf16_split_k_and_strided(K, M, d, ld):
+    """Shapes that exercise split-K, ragged last splits, edge tiles and a row stride larger than d."""
+    x = _inputs((M, ld), torch.bfloat16, seed=M % 97)
+    ref = x[:, :d].float().double().T @ x[:, :d].float().double()
+    print(f'syrk_tn bf16 M={M} d={d} ld={ld}', flush=True)
+    out = K.syrk_tn(x.cuda()[:, :d])
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5
+    assert torch.equal(out, out.T)
+
+
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('N,C,hw', [(2, 4, (3, 3)), (8, 64, (7, 7)), (4, 130, (14, 14)), (2, 1000, (1, 1)),
                                     (3, 17, (28, 28)), (1, 257, (5, 9))])
