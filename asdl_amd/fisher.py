@@ -20,6 +20,7 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
+EAGER_INVERSE_CHUNK = 10     # (A, B) pairs per batched inverse started during the backward pass
 
 
 @dataclass
@@ -53,6 +54,11 @@ class FisherMaker(GradientMaker):
         for module in self.model.modules():
             if hasattr(module, attr):
                 delattr(module, attr)
+
+    @property
+    def single_backward_pass(self):
+        """True when _fisher_loop (or the empirical-Fisher backward) runs exactly one backward pass."""
+        return self.is_fisher_emp or (self.config.fisher_type == FISHER_MC and self.config.n_mc_samples == 1)
 
     @property
     def is_fisher_emp(self):
@@ -102,6 +108,10 @@ class FisherMaker(GradientMaker):
             if damping is not None:
                 cxt.set_damping(damping)
             cxt.set_cov_scale(scale)
+            if inv_with_fisher and self.single_backward_pass:
+                # every B factor is final when its hook has run: start inverting in chunks, behind the
+                # backward pass that is still producing the others
+                cxt.set_eager_inverse(EAGER_INVERSE_CHUNK)
 
             self.call_model()
             loss = None

@@ -102,6 +102,24 @@ def device_ptr_array(tensors):
     return arr
 
 
+_int_cache = {}
+
+
+def device_ints(values, device, dtype=torch.int64):
+    """Device tensor holding a small tuple of Python ints (nested tuples give a 2-D tensor).  Cached: the
+    same index sets recur every step, and building them anew costs a synchronous host-to-device copy that
+    stalls the host behind everything already enqueued."""
+    dev = torch.device(device)
+    key = (dev.index, dtype, values)
+    t = _int_cache.get(key)
+    if t is None:
+        if len(_int_cache) > 8192:
+            _int_cache.clear()
+        t = torch.tensor(values, dtype=dtype).to(dev)
+        _int_cache[key] = t
+    return t
+
+
 # ------------------------------------------------------------------------------ factors
 def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     """out <- beta*out + alpha * x^T x for x = [M, d] (rows may be strided, columns contiguous)."""
@@ -197,7 +215,7 @@ def kron_damping(A_list, B_list, damping, eps=1e-7):
     for t in list(A_list) + list(B_list):
         if t.dtype != torch.float32 or not t.is_contiguous() or t.ndim != 2 or t.shape[0] != t.shape[1]:
             raise ValueError('factors have to be contiguous square float32 matrices')
-    dims = torch.tensor([[a.shape[0], b.shape[0]] for a, b in zip(A_list, B_list)], dtype=torch.int64).to(dev)
+    dims = device_ints(tuple((a.shape[0], b.shape[0]) for a, b in zip(A_list, B_list)), dev)
     lam = torch.empty(batch, 2, dtype=torch.float32, device=dev)
     nonzero = torch.empty(batch, 2, dtype=torch.int32, device=dev)
     pa, pb = device_ptr_array(A_list), device_ptr_array(B_list)

@@ -62,6 +62,7 @@ class Operation:
         self._damping = 1.e-7
         self._cov_scale = 1.
         self._first_beta = {}       # 'A' / 'B' -> factor applied to a registered matrix at its first update
+        self._n_forward = self._n_backward = 0    # hook calls that contributed to the scratch factors
         self._touched = set()
         self._context = None
 
@@ -141,6 +142,7 @@ class Operation:
             buf = self._scratch_factor('A', dim, in_data.device)
             self.cov_kron_A(module, data, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
             self._op_results['_A_tmp'] = buf
+            self._n_forward += 1
 
     def backward_pre_process(self, out_grads, vector: torch.Tensor = None):
         module = self._module
@@ -157,7 +159,9 @@ class Operation:
             buf = self._scratch_factor('B', grads.shape[1], grads.device)
             self.cov_kron_B(module, grads, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
             self._op_results['_B_tmp'] = buf
-            if self._context is not None:
+            self._n_backward += 1
+            # a module called several times in the forward pass is complete after as many backward hooks
+            if self._context is not None and self._n_backward % max(self._n_forward, 1) == 0:
                 self._context.queue_inverse(self)
 
     def finish_registered(self):
@@ -247,23 +251,27 @@ class Conv2d(Operation):
 
 
 class DeferredInverses:
-    """Inverses enqueued by OperationContext.flush_inverses(defer=True).  finish(attr) waits for them,
-    raises torch.linalg.LinAlgError for a factor that is not positive definite, and removes from
-    ``module.<attr>.kron`` the inverse of any all-zero factor (which the reference never computes)."""
+    """Inverses enqueued by OperationContext.flush_inverses(defer=True), possibly in several chunks.
+    finish(attr) waits for them, raises torch.linalg.LinAlgError for a factor that is not positive definite,
+    and removes from ``module.<attr>.kron`` the inverse of any all-zero factor (which the reference never
+    computes)."""
 
-    def __init__(self, pending, targets):
-        self._pending, self._targets = pending, targets
+    def __init__(self, chunks):
+        self._chunks = chunks            # [(PendingInverses, [(module, kron), ...]), ...]
 
     def finish(self, attr):
-        self._pending.finish()
-        for module, kron in self._targets:
-            fisher = getattr(module, attr, None)
-            if fisher is None or not fisher.has_kron:
-                continue
-            if kron.A_inv is None:
-                fisher.kron.A_inv = None
-            if kron.B_inv is None:
-                fisher.kron.B_inv = None
+        for pending, _ in self._chunks:
+            pending.join()               # all waits first, then the flag reads
+        for pending, targets in self._chunks:
+            pending.finish()
+            for module, kron in targets:
+                fisher = getattr(module, attr, None)
+                if fisher is None or not fisher.has_kron:
+                    continue
+                if kron.A_inv is None:
+                    fisher.kron.A_inv = None
+                if kron.B_inv is None:
+                    fisher.kron.B_inv = None
 
 
 def get_op_class(module):
@@ -281,6 +289,8 @@ class OperationContext:
         self._operations: Dict[nn.Module, Operation] = {}
         self._vectors = vectors
         self._pending_inverse = []
+        self._inverse_chunks = []
+        self._eager_chunk = 0
 
     def is_operation_registered(self, module):
         return module in self._operations
@@ -298,6 +308,7 @@ class OperationContext:
     def clear_operations(self):
         self._operations.clear()
         self._pending_inverse = []
+        self._inverse_chunks = []
 
     def call_operations_in_forward(self, module, in_data, out_data):
         self.get_operation(module).forward_post_process(in_data, out_data)
@@ -326,18 +337,25 @@ class OperationContext:
         pass  # only needed for the full (non layer-wise) shape
 
     # ---- deferred, batched inverses
+    def set_eager_inverse(self, chunk):
+        """With ``chunk`` > 0 a batched inverse is enqueued as soon as that many (A, B) pairs are complete,
+        i.e. while the backward pass that produces the remaining B factors is still running.  Only valid when
+        every factor receives a single contribution (one backward pass); None or 0 waits for flush_inverses."""
+        self._eager_chunk = chunk or 0
+
     def queue_inverse(self, operation):
         if operation not in self._pending_inverse:
             self._pending_inverse.append(operation)
+        if self._eager_chunk and len(self._pending_inverse) >= self._eager_chunk:
+            self._enqueue_pending()
 
-    def flush_inverses(self, defer=False):
-        """Inverts every queued (A, B) pair in one batched pass.  With ``defer=True`` the launches are only
-        enqueued: the result store receives the output tensors right away and the returned object's
-        finish() must be called before they are used (it reads the zero / not-positive-definite flags)."""
+    def _enqueue_pending(self):
+        """Starts the batched inverse of every queued pair (side streams, worker threads) and places the
+        output tensors in the result store; their flags are read by DeferredInverses.finish()."""
         ops = self._pending_inverse
         self._pending_inverse = []
         if not ops:
-            return None
+            return
         krons = []
         for op in ops:
             A = op._op_results.pop('_A_tmp', None)
@@ -348,21 +366,35 @@ class OperationContext:
             krons.append(Kron(A, B, prev.get('A_inv'), prev.get('B_inv')))
         # every operation in one context shares the damping value
         pending = batched_update_inv(krons, damping=ops[0]._damping, replace=False, defer=True)
-        if not defer:
-            pending.finish()
-            for op, kron in zip(ops, krons):
-                store = op._op_results.setdefault(OP_COV_KRON, {})
-                if kron.A_inv is not None:
-                    store['A_inv'] = kron.A_inv
-                if kron.B_inv is not None:
-                    store['B_inv'] = kron.B_inv
-            return None
         outs = {(id(k), which): out for _, k, which, out in pending._records}
         for op, kron in zip(ops, krons):
             store = op._op_results.setdefault(OP_COV_KRON, {})
             store['A_inv'] = outs[(id(kron), 'A')]
             store['B_inv'] = outs[(id(kron), 'B')]
-        return DeferredInverses(pending, [(op._module, kron) for op, kron in zip(ops, krons)])
+        self._inverse_chunks.append((pending, [(op._module, kron) for op, kron in zip(ops, krons)]))
+
+    def flush_inverses(self, defer=False):
+        """Inverts every queued (A, B) pair in batched passes.  With ``defer=True`` the launches are only
+        enqueued: the result store receives the output tensors right away and the returned object's
+        finish() must be called before they are used (it reads the zero / not-positive-definite flags)."""
+        self._enqueue_pending()
+        chunks = self._inverse_chunks
+        self._inverse_chunks = []
+        if not chunks:
+            return None
+        deferred = DeferredInverses(chunks)
+        if defer:
+            return deferred
+        for pending, _ in chunks:
+            pending.join()
+        for pending, targets in chunks:
+            pending.finish()
+            for module, kron in targets:
+                store = self.get_operation(module)._op_results.setdefault(OP_COV_KRON, {})
+                for which in ('A_inv', 'B_inv'):
+                    if getattr(kron, which) is None:
+                        store.pop(which, None)       # all-zero factor: the reference computes no inverse
+        return None
 
     # ---- symmatrix exchange (asdl/operations/operation.py:815-876)
     def cov_symmatrix(self, module, pop=False):

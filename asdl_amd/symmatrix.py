@@ -28,6 +28,22 @@ def _side_streams(device, n):
     return pool[:n]
 
 
+_enqueue_workers = {}
+
+
+def _worker(stream_index):
+    """One enqueue thread per side stream.  The launches of a batched inverse are a few dozen small kernels
+    issued from C without the interpreter lock, so the caller can go on (with the backward pass) while they are
+    being issued; a single thread per stream keeps the jobs of that stream, which share its workspace, in
+    order."""
+    w = _enqueue_workers.get(stream_index)
+    if w is None:
+        from concurrent.futures import ThreadPoolExecutor
+        w = ThreadPoolExecutor(max_workers=1, thread_name_prefix=f'asdl_amd_inv{stream_index}')
+        _enqueue_workers[stream_index] = w
+    return w
+
+
 def _is_all_none(xs):
     return all(x is None for x in xs)
 
@@ -37,19 +53,28 @@ class PendingInverses:
     finish() joins the streams into the current one, reads all flags with one device-to-host copy,
     raises for a matrix that is not positive definite and stores the inverses on the Kron objects."""
 
-    def __init__(self, records, infos, nz_flat, events, replace, keep_alive=None):
+    def __init__(self, records, infos, nz_flat, events, replace, keep_alive=None, futures=()):
         self._records, self._infos, self._nz_flat = records, infos, nz_flat
         self._keep_alive = keep_alive      # tensors the side-stream kernels still read
         self._events, self._replace = events, replace
+        self._futures = list(futures)      # enqueue jobs running on worker threads; each returns an event
         self._done = False
+
+    def join(self):
+        """Makes the current stream wait for the inverses (no host synchronisation beyond the enqueue
+        jobs themselves)."""
+        events = list(self._events) + [f.result() for f in self._futures]
+        self._events, self._futures = [], []
+        if events:
+            main = torch.cuda.current_stream()
+            for ev in events:
+                main.wait_event(ev)
 
     def finish(self):
         if self._done:
             return
         self._done = True
-        main = torch.cuda.current_stream() if self._events else None
-        for ev in self._events:
-            main.wait_event(ev)
+        self.join()
         host = torch.cat(self._infos + [self._nz_flat]).cpu().tolist()        # the one synchronisation
         n = len(self._records)
         info_host, nz_host = host[:n], host[n:]
@@ -97,7 +122,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
     lam, nonzero = kernels.kron_damping(A_list, B_list, float(damping), float(eps))
     single = [i for i, k in enumerate(krons) if not (k.has_A and k.has_B)]
     if single:
-        lam[torch.tensor(single, device=dev)] = float(damping)      # no pi split without both factors
+        lam[kernels.device_ints(tuple(single), dev)] = float(damping)      # no pi split without both factors
     lam_flat, nz_flat = lam.view(-1), nonzero.view(-1)
 
     groups = defaultdict(list)   # d -> [(flat index, matrix, kron, 'A'|'B')]
@@ -112,7 +137,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
     prepared = []
     for d in order:
         entries = groups[d]
-        idx = torch.tensor([e[0] for e in entries], device=dev)
+        idx = kernels.device_ints(tuple(e[0] for e in entries), dev)
         outs = []
         for _, mat, k, which in entries:
             old = getattr(k, which + '_inv')
@@ -120,29 +145,42 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             outs.append(old if reuse else torch.empty_like(mat))
         info = torch.empty(len(entries), dtype=torch.int32, device=dev)
         prepared.append((entries, outs, lam_flat[idx], nz_flat[idx].contiguous(), info))
-    infos, records, events = [], [], []
+    infos, records, events, futures = [], [], [], []
     use_streams = mats_on_gpu and (len(prepared) > 1 or defer)
+
+    def run_group(group):
+        entries, outs, lam_g, act_g, info = group
+        kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
+
     if use_streams:
         main = torch.cuda.current_stream()
         side = _side_streams(dev, min(4, len(prepared)))
         start = torch.cuda.Event()
         start.record(main)
-    for gi, (entries, outs, lam_g, act_g, info) in enumerate(prepared):
-        if use_streams:
-            st = side[gi % len(side)]
-            st.wait_event(start)
-            with torch.cuda.stream(st):
-                kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
-        else:
-            kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
+        per_stream = [prepared[i::len(side)] for i in range(len(side))]
+
+        def run_stream(st, groups_of_stream):
+            with torch.cuda.device(dev), torch.cuda.stream(st):
+                st.wait_event(start)
+                for group in groups_of_stream:
+                    run_group(group)
+                done = torch.cuda.Event()
+                done.record(st)
+            return done
+
+        for si, (st, groups_of_stream) in enumerate(zip(side, per_stream)):
+            if defer:
+                futures.append(_worker(si).submit(run_stream, st, groups_of_stream))
+            else:
+                events.append(run_stream(st, groups_of_stream))
+    else:
+        for group in prepared:
+            run_group(group)
+    for entries, outs, lam_g, act_g, info in prepared:
         infos.append(info)
         records.extend((e[0], e[2], e[3], out) for e, out in zip(entries, outs))
-    if use_streams:
-        for st in side:
-            done = torch.cuda.Event()
-            done.record(st)
-            events.append(done)
-    pending = PendingInverses(records, infos, nz_flat, events, replace, keep_alive=(prepared, lam, nonzero, A_list, B_list))
+    pending = PendingInverses(records, infos, nz_flat, events, replace,
+                              keep_alive=(prepared, lam, nonzero, A_list, B_list), futures=futures)
     if defer:
         return pending
     pending.finish()
