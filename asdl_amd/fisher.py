@@ -20,7 +20,7 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
-EAGER_INVERSE_CHUNK = 10     # (A, B) pairs per batched inverse started during the backward pass
+EAGER_INVERSE_CHUNK = 0      # (A, B) pairs per batched inverse started during the backward pass; 0: one pass after it
 
 
 @dataclass

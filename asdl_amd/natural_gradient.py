@@ -158,11 +158,31 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             raise NotImplementedError('precondition(vectors=...) is not on this path')
         if grad_scale is None:
             grad_scale = self.grad_scale
-        for shape in _kernel_shapes:
-            for module in self.modules_for(shape):
-                if module not in self.modules_for_curvature:
-                    continue
+        work = [(module, shape) for shape in _kernel_shapes for module in self.modules_for(shape)
+                if module in self.modules_for_curvature]
+        grads = [m.weight.grad for m, _ in work if getattr(m, 'weight', None) is not None and m.weight.grad is not None]
+        if len(work) < 4 or not grads or not grads[0].is_cuda:
+            for module, shape in work:
                 self._precondition_module(module, shape, grad_scale=grad_scale, use_inv=use_inv)
+            return
+        # The layers are independent and most of their GEMMs are too small to fill the device: spread them
+        # over the side streams (largest first) and join.  Everything they touch is waited for before returning.
+        from .symmatrix import _side_streams
+        dev = grads[0].device
+        main = torch.cuda.current_stream(dev)
+        side = _side_streams(dev, 4)
+        start = torch.cuda.Event()
+        start.record(main)
+        work.sort(key=lambda mw: -(mw[0].weight.numel() * (mw[0].weight.shape[0] + mw[0].weight[0].numel())))
+        for st in side:
+            st.wait_event(start)
+        for i, (module, shape) in enumerate(work):
+            with torch.cuda.stream(side[i % len(side)]):
+                self._precondition_module(module, shape, grad_scale=grad_scale, use_inv=use_inv)
+        for st in side:
+            done = torch.cuda.Event()
+            done.record(st)
+            main.wait_event(done)
 
     def _precondition_module(self, module, shape=None, vectors=None, vec_weight=None, vec_bias=None,
                              grad_scale=None, use_inv=True):
