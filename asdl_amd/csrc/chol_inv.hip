@@ -52,11 +52,16 @@ __device__ __forceinline__ float lane_bcast(float v, int src_lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
 }
 
-constexpr int PB = 16;              // panel width inside a leaf
-constexpr int LLD = LEAF + 1;       // LDS leading dimension (bank-conflict free columns)
+constexpr int PB = 16;              // base block handled in registers by one wave
+constexpr int LLD = LEAF + 4;       // LDS leading dimension: rows 4 banks apart, so the [row][k] operand reads of the
+                                    // 16x16x4 MFMA (16 rows x 4 k per instruction) touch 64 different banks
 constexpr int LEAF_THREADS = 1024;
-constexpr int LEAF_BLOCKS = LEAF / PB;
-constexpr size_t LEAF_LDS_BYTES = (2 * LEAF * LLD + LEAF_BLOCKS * PB * (PB + 1) + 8) * sizeof(float);
+constexpr int LEAF_WAVES = LEAF_THREADS / 64;
+constexpr int T1_LD = 68;
+// work block, T1 pool (64x64 + 32x32 + 16x16 panels of nested levels) and T2, plus the bad-pivot word
+constexpr int LEAF_T1_FLOATS = 64 * T1_LD + 32 * T1_LD + 16 * T1_LD;
+constexpr int LEAF_T2_FLOATS = 64 * T1_LD;
+constexpr size_t LEAF_LDS_BYTES = (LEAF * LLD + LEAF_T1_FLOATS + LEAF_T2_FLOATS + 8) * sizeof(float);
 
 // Cholesky factor and its inverse of a PB x PB block held one row per lane (lanes >= PB carry an identity
 // row).  On exit a[] is row `lane` of L and m[] is column `lane` of L^-1.  Returns 0 or the 1-based index of
@@ -92,119 +97,122 @@ __device__ __forceinline__ int small_chol_inv(float (&a)[PB], float (&m)[PB], in
   return bad;
 }
 
-// One work group (16 waves) per matrix: blocked Cholesky of the n x n (n <= LEAF) diagonal block at `lo`,
-// resident in LDS.  Per 16-column panel: the 16 x 16 diagonal block is factored and inverted in registers
-// by one wave; the panel below it (a product with that small inverse) and the trailing update are LDS
-// products spread over all threads.  Then the blocked triangular inverse, one block diagonal at a time.
-// On exit the block holds L^-1 in its lower triangle and zeros above the diagonal.
+// v_mfma_f32_16x16x4_f32: lane l feeds A[i = l%16][k = l/16] and B[k = l/16][j = l%16]; accumulator register r of
+// lane l is C[i = 4*(l/16) + r][j = l%16].
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+// Which part of the contraction range a 16x16 output tile (ib, jb) needs when one operand is triangular.
+enum LeafK { LK_FULL, LK_LE_J, LK_GE_J, LK_LE_I };
+
+// C[M x N] (=, -=) alpha * A[M x K] * op(B) for small matrices in LDS, all sizes multiples of 16, one 16x16 output
+// tile per wave and turn.  TB: op(B)[k][j] = B[j][k].  LOWER: only tiles on or below the diagonal (M == N).
+// ACC: C -= product, else C = alpha * product.  The caller synchronises before and after.
+template <int M, int N, int K, bool TB, bool LOWER, bool ACC, LeafK KM>
+__device__ __forceinline__ void leaf_gemm(float* __restrict__ C, int ldc, const float* __restrict__ A, int lda,
+                                          const float* __restrict__ B, int ldb, float alpha, int wave, int lane) {
+  constexpr int TM = M / 16, TN = N / 16;
+  const int li = lane & 15, lk = lane >> 4;
+#pragma unroll 1
+  for (int t = wave; t < TM * TN; t += LEAF_WAVES) {
+    const int ib = t / TN, jb = t % TN;
+    if (LOWER && jb > ib) continue;
+    int k0 = 0, k1 = K;
+    if (KM == LK_LE_J) k1 = 16 * (jb + 1);
+    if (KM == LK_GE_J) k0 = 16 * jb;
+    if (KM == LK_LE_I) k1 = 16 * (ib + 1);
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    const float* pa = A + (16 * ib + li) * lda + lk;
+    const float* pb = TB ? B + (16 * jb + li) * ldb + lk : B + lk * ldb + 16 * jb + li;
+    for (int k = k0; k < k1; k += 4) {
+      const float a = pa[k];
+      const float b = TB ? pb[k] : pb[k * ldb];
+      acc = mfma16(a, b, acc);
+    }
+    float* pc = C + (16 * ib + 4 * lk) * ldc + 16 * jb + li;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (ACC) pc[r * ldc] -= acc[r];
+      else pc[r * ldc] = alpha * acc[r];
+    }
+  }
+}
+
+// Factors the N x N block of Wm at (lo, lo) and leaves the inverse of its Cholesky factor in the lower triangle;
+// same recursion as the global one, on LDS operands.  t1: this level's slice of the T1 pool.
+template <int N>
+__device__ __forceinline__ void leaf_factor(float* __restrict__ Wm, int lo, float* __restrict__ t1,
+                                            float* __restrict__ t2, int* __restrict__ s_bad, int tid) {
+  const int wave = tid >> 6, lane = tid & 63;
+  if constexpr (N == PB) {
+    if (wave == 0) {
+      float a[PB], m[PB];
+#pragma unroll
+      for (int j = 0; j < PB; ++j)
+        a[j] = (lane < PB && j <= lane) ? Wm[(lo + lane) * LLD + lo + j] : ((j == lane) ? 1.f : 0.f);
+      const int bad = small_chol_inv(a, m, lane);
+      if (lane < PB) {
+#pragma unroll
+        for (int j = 0; j < PB; ++j) Wm[(lo + j) * LLD + lo + lane] = m[j];     // m[j] = 0 above the diagonal
+      }
+      if (lane == 0 && bad != 0 && *s_bad == 0) *s_bad = lo + bad;
+    }
+    __syncthreads();
+  } else {
+    constexpr int H = N / 2;
+    leaf_factor<H>(Wm, lo, t1, t2, s_bad, tid);
+    float* W11 = Wm + lo * LLD + lo;
+    float* W21 = Wm + (lo + H) * LLD + lo;
+    float* W22 = Wm + (lo + H) * LLD + lo + H;
+    leaf_gemm<H, H, H, true, false, false, LK_LE_J>(t1, T1_LD, W21, LLD, W11, LLD, 1.f, wave, lane);   // T1 = A21 M11^T
+    __syncthreads();
+    leaf_gemm<H, H, H, true, true, true, LK_FULL>(W22, LLD, t1, T1_LD, t1, T1_LD, 1.f, wave, lane);    // A22 -= T1 T1^T
+    __syncthreads();
+    leaf_factor<H>(Wm, lo + H, t1 + H * T1_LD, t2, s_bad, tid);
+    leaf_gemm<H, H, H, false, false, false, LK_GE_J>(t2, T1_LD, t1, T1_LD, W11, LLD, 1.f, wave, lane); // T2 = T1 M11
+    __syncthreads();
+    leaf_gemm<H, H, H, false, false, false, LK_LE_I>(W21, LLD, W22, LLD, t2, T1_LD, -1.f, wave, lane); // M21 = -M22 T2
+    __syncthreads();
+  }
+}
+
+// One work group (16 waves) per matrix: the n x n (n <= LEAF) diagonal block at `lo`, padded with an identity to
+// a power-of-two multiple of 16, is factored in LDS by the recursion above: 16 x 16 blocks in the registers of one
+// wave, everything else as 16x16x4 fp32 MFMA products over all waves.  On exit the block holds L^-1 in its lower
+// triangle and zeros above the diagonal.
 static __global__ __launch_bounds__(LEAF_THREADS) void chol_leaf_kernel(float* __restrict__ W, int64_t strideW,
                                                                         int64_t d, int lo, int n,
                                                                         int* __restrict__ info, const int* active,
                                                                         int active_stride) {
   extern __shared__ __attribute__((aligned(16))) float leaf_smem[];
-  float (*A)[LLD] = reinterpret_cast<float (*)[LLD]>(leaf_smem);
-  float (*Mi)[LLD] = reinterpret_cast<float (*)[LLD]>(leaf_smem + LEAF * LLD);
-  float (*Sc)[PB][PB + 1] = reinterpret_cast<float (*)[PB][PB + 1]>(leaf_smem + 2 * LEAF * LLD);
-  int* s_bad = reinterpret_cast<int*>(leaf_smem + 2 * LEAF * LLD + LEAF_BLOCKS * PB * (PB + 1));
+  float* Wm = leaf_smem;
+  float* t1 = leaf_smem + LEAF * LLD;
+  float* t2 = t1 + LEAF_T1_FLOATS;
+  int* s_bad = reinterpret_cast<int*>(t2 + LEAF_T2_FLOATS);
   const int z = blockIdx.x;
   if (active != nullptr && active[static_cast<int64_t>(z) * active_stride] == 0) return;
   const int tid = threadIdx.x;
-  const int np = (n + PB - 1) / PB;        // panels
-  const int npad = np * PB;
+  const int npad = n <= 16 ? 16 : (n <= 32 ? 32 : (n <= 64 ? 64 : 128));
   float* __restrict__ blk = W + z * strideW + static_cast<int64_t>(lo) * d + lo;
   for (int i = tid >> 7; i < npad; i += LEAF_THREADS / 128) {
     const int j = tid & 127;
     if (j < npad) {
       float v = (i == j) ? 1.f : 0.f;              // identity padding beyond n
       if (i < n && j < n) v = (j <= i) ? blk[static_cast<int64_t>(i) * d + j] : 0.f;
-      A[i][j] = v;
-      Mi[i][j] = 0.f;
+      Wm[i * LLD + j] = v;
     }
   }
   if (tid == 0) *s_bad = 0;
   __syncthreads();
-
-#pragma unroll 1
-  for (int pb = 0; pb < np; ++pb) {
-    const int c0 = PB * pb;
-    if (tid < 64) {
-      const int lane = tid;
-      float a[PB], m[PB];
-#pragma unroll
-      for (int j = 0; j < PB; ++j) a[j] = (lane < PB && j <= lane) ? A[c0 + lane][c0 + j] : ((j == lane) ? 1.f : 0.f);
-      const int bad = small_chol_inv(a, m, lane);
-      if (lane < PB) {
-#pragma unroll
-        for (int j = 0; j < PB; ++j) {
-          if (j <= lane) A[c0 + lane][c0 + j] = a[j];
-          Sc[0][j][lane] = m[j];
-          Mi[c0 + j][c0 + lane] = m[j];
-        }
-      }
-      if (lane == 0 && bad != 0 && *s_bad == 0) *s_bad = c0 + bad;
-    }
-    __syncthreads();
-    const int r0 = c0 + PB;
-    const int nrows = npad - r0;
-    if (nrows > 0) {
-      float res[2] = {0.f, 0.f};
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {               // panel below: A_below * Wd^T  (Wd = Sc[0])
-        const int i = r0 + (tid >> 4) + 64 * t, j = tid & 15;
-        if (i < npad) {
-          float acc = 0.f;
-#pragma unroll
-          for (int k = 0; k < PB; ++k) acc += A[i][c0 + k] * Sc[0][j][k];
-          res[t] = acc;
-        }
-      }
-      __syncthreads();
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int i = r0 + (tid >> 4) + 64 * t;
-        if (i < npad) A[i][c0 + (tid & 15)] = res[t];
-      }
-      __syncthreads();
-      const int j = r0 + (tid & 127);
-      for (int i = r0 + (tid >> 7); i < npad; i += LEAF_THREADS / 128) {   // trailing update, lower triangle
-        if (j <= i) {
-          float acc = 0.f;
-#pragma unroll
-          for (int k = 0; k < PB; ++k) acc += A[i][c0 + k] * A[j][c0 + k];
-          A[i][j] -= acc;
-        }
-      }
-      __syncthreads();
-    }
-  }
+  if (npad == 16) leaf_factor<16>(Wm, 0, t1, t2, s_bad, tid);
+  else if (npad == 32) leaf_factor<32>(Wm, 0, t1, t2, s_bad, tid);
+  else if (npad == 64) leaf_factor<64>(Wm, 0, t1, t2, s_bad, tid);
+  else leaf_factor<128>(Wm, 0, t1, t2, s_bad, tid);
   if (tid == 0 && *s_bad != 0 && *s_bad <= n && info[z] == 0) info[z] = lo + *s_bad;
-
-  // blocked triangular inverse: block (bi, bj), bi > bj, is -W_ii * sum_{bj <= kb < bi} L_{bi,kb} M_{kb,bj};
-  // all blocks of one block diagonal are independent.
-#pragma unroll 1
-  for (int dist = 1; dist < np; ++dist) {
-    const int nb = np - dist;
-    for (int e = tid; e < nb * PB * PB; e += LEAF_THREADS) {
-      const int bj = e >> 8, ty = (e >> 4) & 15, tx = e & 15, bi = bj + dist;
-      float acc = 0.f;
-      for (int kb = bj; kb < bi; ++kb)
-#pragma unroll
-        for (int k = 0; k < PB; ++k) acc += A[PB * bi + ty][PB * kb + k] * Mi[PB * kb + k][PB * bj + tx];
-      Sc[bj][ty][tx] = acc;
-    }
-    __syncthreads();
-    for (int e = tid; e < nb * PB * PB; e += LEAF_THREADS) {
-      const int bj = e >> 8, ty = (e >> 4) & 15, tx = e & 15, bi = bj + dist;
-      float r = 0.f;
-#pragma unroll
-      for (int k = 0; k < PB; ++k) r += Mi[PB * bi + ty][PB * bi + k] * Sc[bj][k][tx];
-      Mi[PB * bi + ty][PB * bj + tx] = -r;
-    }
-    __syncthreads();
-  }
   for (int i = tid >> 7; i < n; i += LEAF_THREADS / 128) {
     const int j = tid & 127;
-    if (j < n) blk[static_cast<int64_t>(i) * d + j] = (j <= i) ? Mi[i][j] : 0.f;
+    if (j < n) blk[static_cast<int64_t>(i) * d + j] = (j <= i) ? Wm[i * LLD + j] : 0.f;
   }
 }
 

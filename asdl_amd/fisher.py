@@ -20,7 +20,7 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
-EAGER_INVERSE_CHUNK = 0      # (A, B) pairs per batched inverse started during the backward pass; 0: one pass after it
+EAGER_INVERSE = False       # start the bulk of the inverses during a single sampled / empirical backward pass (no gain while the GPU is throughput-bound)
 
 
 @dataclass
@@ -108,10 +108,10 @@ class FisherMaker(GradientMaker):
             if damping is not None:
                 cxt.set_damping(damping)
             cxt.set_cov_scale(scale)
-            if inv_with_fisher and self.single_backward_pass:
-                # every B factor is final when its hook has run: start inverting in chunks, behind the
-                # backward pass that is still producing the others
-                cxt.set_eager_inverse(EAGER_INVERSE_CHUNK)
+            if inv_with_fisher and self.single_backward_pass and EAGER_INVERSE:
+                # every B factor is final when its hook has run: the bulk of the inverses may start behind
+                # the backward pass that is still producing the others
+                cxt.set_eager_inverse(getattr(self, '_inverse_cost_prev', 0))
 
             self.call_model()
             loss = None
@@ -131,6 +131,7 @@ class FisherMaker(GradientMaker):
             # The inverses only need the factors: enqueue them now (side streams) and, when a loss backward
             # pass follows, let that pass run on the main stream meanwhile; the flags are read afterwards.
             deferred = cxt.flush_inverses(defer=loss_grad_after_fisher)
+            self._inverse_cost_prev = cxt.inverse_cost
             self._extract_fisher(cxt)
 
         if inv_after_fisher:

@@ -250,6 +250,9 @@ class Conv2d(Operation):
         return kernels.syrk_nt(out_grads, out=out, alpha=alpha, beta=beta)    # c_out x c_out
 
 
+EAGER_COST_FRACTION = 0.6
+
+
 class DeferredInverses:
     """Inverses enqueued by OperationContext.flush_inverses(defer=True), possibly in several chunks.
     finish(attr) waits for them, raises torch.linalg.LinAlgError for a factor that is not positive definite,
@@ -290,7 +293,9 @@ class OperationContext:
         self._vectors = vectors
         self._pending_inverse = []
         self._inverse_chunks = []
-        self._eager_chunk = 0
+        self._eager_total = 0.0
+        self._eager_done = False
+        self._inverse_cost = 0.0
 
     def is_operation_registered(self, module):
         return module in self._operations
@@ -337,16 +342,31 @@ class OperationContext:
         pass  # only needed for the full (non layer-wise) shape
 
     # ---- deferred, batched inverses
-    def set_eager_inverse(self, chunk):
-        """With ``chunk`` > 0 a batched inverse is enqueued as soon as that many (A, B) pairs are complete,
-        i.e. while the backward pass that produces the remaining B factors is still running.  Only valid when
-        every factor receives a single contribution (one backward pass); None or 0 waits for flush_inverses."""
-        self._eager_chunk = chunk or 0
+    def set_eager_inverse(self, total_cost):
+        """``total_cost``: sum of d^3 over all factors inverted in the previous step (0 or None: unknown).
+        When known, the pairs queued so far are inverted as soon as they hold EAGER_COST_FRACTION of it,
+        i.e. while the backward pass that produces the remaining B factors is still running: in a network
+        whose widest layers come last, the longest chains of the batched inverse start early and only the
+        cheap remainder is left for after the pass.  One early batch only, so that same-size factors still
+        share launches.  Only valid when every factor receives a single contribution (one backward pass)."""
+        self._eager_total = float(total_cost or 0)
+        self._eager_done = False
+
+    @property
+    def inverse_cost(self):
+        """Sum of d^3 over the factors queued for inversion since the context was created."""
+        return self._inverse_cost
 
     def queue_inverse(self, operation):
         if operation not in self._pending_inverse:
             self._pending_inverse.append(operation)
-        if self._eager_chunk and len(self._pending_inverse) >= self._eager_chunk:
+            for key in ('_A_tmp', '_B_tmp'):
+                buf = operation._op_results.get(key)
+                if buf is not None:
+                    self._inverse_cost += float(buf.shape[0]) ** 3
+        if self._eager_total > 0 and not self._eager_done and \
+                self._inverse_cost >= EAGER_COST_FRACTION * self._eager_total:
+            self._eager_done = True
             self._enqueue_pending()
 
     def _enqueue_pending(self):

@@ -18,6 +18,7 @@ _default_damping = 1e-5
 
 
 _side_stream_cache = {}
+N_SIDE_STREAMS = 8     # size groups of a batched inverse that may run side by side
 
 
 def _side_streams(device, n):
@@ -154,7 +155,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
 
     if use_streams:
         main = torch.cuda.current_stream()
-        side = _side_streams(dev, min(4, len(prepared)))
+        side = _side_streams(dev, min(N_SIDE_STREAMS, len(prepared)))
         start = torch.cuda.Event()
         start.record(main)
         per_stream = [prepared[i::len(side)] for i in range(len(side))]
