@@ -232,6 +232,7 @@ struct CholCtx {
 static void run_gemm(CholCtx& c, GemmParams p) {
   p.active = c.active;
   p.active_stride = c.active_stride;
+  p.split = 3;          // large products run on the bf16 matrix cores with fp32-grade accuracy
   const int rc = launch_gemm(p, c.batch, c.stream);
   if (rc != AK_OK) c.rc = rc;
 }

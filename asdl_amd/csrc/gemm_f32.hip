@@ -37,6 +37,22 @@ extern "C" int ak_gemm_f32(int transA, int transB, int64_t M, int64_t N, int64_t
   return ak::launch_gemm(p, batch, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, int64_t K, float alpha,
+                                 const float* A, int64_t lda, const float* B, int64_t ldb, float beta, float* C,
+                                 int64_t ldc, int batch, int64_t strideA, int64_t strideB, int64_t strideC,
+                                 ak_stream_t stream) {
+  if (A == nullptr || B == nullptr || C == nullptr || M < 0 || N < 0 || K < 0 || batch <= 0) return AK_ERR_ARG;
+  if (pieces != 0 && pieces != 2 && pieces != 3) return AK_ERR_ARG;
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return AK_ERR_ARG;
+  const int64_t a_cols = transA ? M : K, b_cols = transB ? K : N;
+  if (lda < a_cols || ldb < b_cols || ldc < N) return AK_ERR_ARG;
+  ak::GemmParams p = ak::make_gemm(transA != 0, transB != 0, static_cast<int>(M), static_cast<int>(N),
+                                   static_cast<int>(K), alpha, A, lda, B, ldb, beta, C, ldc);
+  p.sA = strideA; p.sB = strideB; p.sC = strideC;
+  p.split = pieces;
+  return ak::launch_gemm(p, batch, static_cast<hipStream_t>(stream));
+}
+
 extern "C" size_t ak_kron_precond_ws_bytes(int64_t dB, int64_t dA) {
   if (dB <= 0 || dA <= 0) return 0;
   return static_cast<size_t>(dB * dA + dB) * sizeof(float);
@@ -50,9 +66,14 @@ extern "C" int ak_kron_precond(const float* Binv, const float* Ainv, float* G, i
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* T = static_cast<float*>(ws);
   const int b = static_cast<int>(dB), a = static_cast<int>(dA);
-  int rc = ak::launch_gemm(ak::make_gemm(0, 0, b, a, b, 1.f, Binv, dB, G, dA, 0.f, T, dA), 1, s);
+  // the inverses are symmetric: reading A^-1 as its transpose makes both operands of the second product
+  // contiguous along the contraction index
+  ak::GemmParams g1 = ak::make_gemm(0, 0, b, a, b, 1.f, Binv, dB, G, dA, 0.f, T, dA);
+  ak::GemmParams g2 = ak::make_gemm(0, 1, b, a, a, grad_scale, T, dA, Ainv, dA, 0.f, G, dA);
+  g1.split = g2.split = 3;
+  int rc = ak::launch_gemm(g1, 1, s);
   if (rc != AK_OK) return rc;
-  rc = ak::launch_gemm(ak::make_gemm(0, 0, b, a, a, grad_scale, T, dA, Ainv, dA, 0.f, G, dA), 1, s);
+  rc = ak::launch_gemm(g2, 1, s);
   if (rc != AK_OK) return rc;
   if (bias != nullptr) {
     float* tb = T + dB * dA;

@@ -37,6 +37,7 @@ struct GemmParams {
   int kmode, tile_mode;
   const int* active;        // optional per-batch flags: batch z runs only if active[z*active_stride] != 0
   int active_stride;
+  int split;                // 0: fp32 MFMA; 2 / 3: bf16 MFMA on operands split into that many bf16 pieces (gemm_x3.hpp)
 };
 
 constexpr int GBT = 128, GBK = 16;     // GBT: granularity of the triangular contraction ranges (both tile sizes)
@@ -192,8 +193,20 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
     }
 }
 
+}  // namespace ak
+
+#include "gemm_x3.hpp"
+
+namespace ak {
+
 inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return AK_OK;
+  if (p.split >= 2 && p.M >= 256 && p.N >= 256 && p.K >= 128 && gemm_x3_ok(p)) {
+    dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
+    if (p.split == 2) hipLaunchKernelGGL(gemm_x3_kernel<2>, grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(gemm_x3_kernel<3>, grid, dim3(256), 0, stream, p);
+    return check_launch();
+  }
   // 128 x 128 tiles when they alone fill the 256 CUs twice over, else 64 x 64 tiles (four times the work groups)
   const int64_t tiles128 = static_cast<int64_t>((p.N + 127) / 128) * ((p.M + 127) / 128) * batch;
   const bool lower = p.tile_mode != TILE_ALL;
@@ -218,6 +231,7 @@ inline GemmParams make_gemm(int transA, int transB, int M, int N, int K, float a
   p.alpha = alpha; p.beta = beta;
   p.kmode = K_FULL; p.tile_mode = TILE_ALL;
   p.active = nullptr; p.active_stride = 0;
+  p.split = 0;
   return p;
 }
 

@@ -1,0 +1,234 @@
+// fp32 GEMM on the bf16 matrix cores: every fp32 operand element is split exactly into three bf16 pieces
+// (8 + 8 + 8 mantissa bits, by truncation, so hi + mid + lo == x), and the product is accumulated in fp32 from
+// the six piece products that matter:
+//   x*y ~= hi*hi' + hi*mid' + mid*hi' + hi*lo' + lo*hi' + mid*mid'      (dropped terms are below 2^-24 |x y|),
+// i.e. the accuracy of an fp32 multiply at 6/16 of the cost of the fp32 MFMA.  With NSPLIT = 2 only hi and mid
+// are kept (16 mantissa bits, 3 products) for callers whose tolerance allows it.
+//
+// Same interface as gemm_f32_kernel (GemmParams: transposes, triangular contraction ranges, lower-triangle tile
+// modes, batches).  One work group = 4 waves (2x2) = one 128x128 tile, k-tiles of 32.  The fp32 panels are
+// fetched into registers one k-tile ahead, split and written to the LDS as bf16 planes after the MFMAs of the
+// current k-tile.  An operand whose contraction index is contiguous in memory is kept as [row][32 k] with the
+// 16-byte chunks of a row XOR-swizzled by (row/4)%4, so that the ds_read_b128 of 16 consecutive rows hits 64
+// different banks; one whose row/column index is contiguous is kept as [32 columns][32 k-rows][64 B] blocks
+// and read with ds_read_b64_tr_b16 (no bank conflicts, no transposed copies).
+#pragma once
+#include <type_traits>
+#include "common.hpp"
+
+namespace ak {
+
+#define AK_LDS3 __attribute__((address_space(3)))
+typedef uint32_t x3_u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int X3_BT = 128, X3_BK = 32;
+constexpr int X3_PLANE = X3_BT * X3_BK * 2;      // bytes of one bf16 plane of one operand panel
+
+struct X3Fetch {
+  floatx4 v[4];
+};
+
+// Loads this thread's four float4 of a 128 x 32 operand panel.  kcontig: memory rows are the 128 tile rows and
+// hold 32 consecutive k; else memory rows are the 32 k values and hold 128 consecutive tile rows.
+template <bool INTERIOR>
+__device__ __forceinline__ void x3_fetch(X3Fetch& r, const float* __restrict__ P, int64_t ld, bool kcontig, int r0,
+                                         int r_end, int k0, int k_end, int tid) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int f = tid + 256 * u;
+    int outer, inner, o_end, i_end;
+    if (kcontig) { outer = r0 + (f >> 3); inner = k0 + 4 * (f & 7); o_end = r_end; i_end = k_end; }
+    else { outer = k0 + (f >> 5); inner = r0 + 4 * (f & 31); o_end = k_end; i_end = r_end; }
+    if (INTERIOR) {
+      r.v[u] = *reinterpret_cast<const floatx4*>(P + static_cast<int64_t>(outer) * ld + inner);
+    } else {
+      // no branch around the load: an invalid chunk reads the first chunk of the matrix and is zeroed afterwards
+      const bool ok = outer < o_end && inner < i_end;        // inner and i_end are multiples of 4
+      const float* src = ok ? P + static_cast<int64_t>(outer) * ld + inner : P;
+      const floatx4 w = *reinterpret_cast<const floatx4*>(src);
+      const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+      r.v[u] = ok ? w : z;
+    }
+  }
+}
+
+__device__ __forceinline__ uint32_t x3_pack_hi16(uint32_t lo_word, uint32_t hi_word) {
+  // bf16 (top halves) of two fp32 bit patterns into one dword: element 0 in the low half
+  return __builtin_amdgcn_perm(hi_word, lo_word, 0x07060302u);
+}
+
+// Splits the fetched panel into NSPLIT bf16 planes and writes them to the LDS.
+template <int NSPLIT>
+__device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char* panel, bool kcontig, int tid) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int f = tid + 256 * u;
+    uint32_t off;
+    if (kcontig) {
+      const int row = f >> 3, c4 = f & 7;
+      off = row * 64 + 16 * ((c4 >> 1) ^ ((row >> 2) & 3)) + 8 * (c4 & 1);
+    } else {
+      const int krow = f >> 5, c4 = f & 31;
+      off = (c4 >> 3) * 2048 + krow * 64 + (c4 & 7) * 8;
+    }
+    uint32_t piece[NSPLIT][4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float rem = r.v[u][e];
+#pragma unroll
+      for (int s = 0; s < NSPLIT; ++s) {
+        const uint32_t top = __builtin_bit_cast(uint32_t, rem) & 0xffff0000u;     // truncation: exact piece
+        piece[s][e] = top;
+        if (s + 1 < NSPLIT) rem -= __builtin_bit_cast(float, top);                // exact
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < NSPLIT; ++s) {
+      x3_u32x2 w;
+      w[0] = x3_pack_hi16(piece[s][0], piece[s][1]);
+      w[1] = x3_pack_hi16(piece[s][2], piece[s][3]);
+      *reinterpret_cast<AK_LDS3 x3_u32x2*>(panel + s * X3_PLANE + off) = w;
+    }
+  }
+}
+
+// The 8 k values (16*h + 8*g ...) of tile row `row` for this lane, as an MFMA operand.
+__device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bool kcontig, int row, int h, int lane) {
+  if (kcontig) {
+    const int g = lane >> 5;
+    return *reinterpret_cast<AK_LDS3 const bf16x8*>(plane + row * 64 + 16 * ((2 * h + g) ^ ((row >> 2) & 3)));
+  }
+  // row = 32*cb + (lane % 32): the transposing read serves 16 columns per half-wave group
+  const int g = lane >> 5, hl = (lane >> 4) & 1, j16 = lane & 15;
+  AK_LDS3 const unsigned char* q = plane + (row >> 5) * 2048 + (16 * h + 8 * g + (j16 >> 2)) * 64 + hl * 32 + (j16 & 3) * 8;
+  const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AK_LDS3 short4v*)(q));
+  const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AK_LDS3 short4v*)(q + 256));
+  return pack_bf16x8(lo, hi);
+}
+
+template <int NSPLIT>
+static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
+  constexpr int BT = X3_BT, BK = X3_BK;
+  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
+  AK_LDS3 unsigned char* lds = (AK_LDS3 unsigned char*)x3_smem;
+  AK_LDS3 unsigned char* panelA = lds;
+  AK_LDS3 unsigned char* panelB = lds + NSPLIT * X3_PLANE;
+  const int z = blockIdx.z;
+  if (p.active != nullptr && p.active[static_cast<int64_t>(z) * p.active_stride] == 0) return;
+  const int tj = blockIdx.x, ti = blockIdx.y;
+  if (p.tile_mode != TILE_ALL && ti < tj) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave >> 1, wc = wave & 1, g = lane >> 5, l32 = lane & 31;
+
+  int kbeg = 0, kend = p.K;
+  switch (p.kmode) {     // ranges rounded outwards to multiples of the tile; the operands are zero outside their triangle
+    case K_LE_J: kend = min(p.K, (tj + 1) * BT); break;
+    case K_GE_J: kbeg = tj * BT; break;
+    case K_LE_I: kend = min(p.K, (ti + 1) * BT); break;
+    case K_GE_MAXIJ: kbeg = max(ti, tj) * BT; break;
+    default: break;
+  }
+  const float* __restrict__ A = p.A + static_cast<int64_t>(z) * p.sA;
+  const float* __restrict__ B = p.B + static_cast<int64_t>(z) * p.sB;
+  float* __restrict__ C = p.C_list != nullptr ? p.C_list[z] : p.C + static_cast<int64_t>(z) * p.sC;
+  const bool a_kc = (p.transA == 0), b_kc = (p.transB != 0);
+  const int i0 = ti * BT, j0 = tj * BT;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  const int nk = kbeg < kend ? (kend - kbeg + BK - 1) / BK : 0;
+  const bool interior = i0 + BT <= p.M && j0 + BT <= p.N && (kend - kbeg) % BK == 0;
+
+  auto mainloop = [&](auto interior_tag) {
+    constexpr bool INTERIOR = decltype(interior_tag)::value;
+    X3Fetch ra, rb;
+    if (nk > 0) {
+      x3_fetch<INTERIOR>(ra, A, p.lda, a_kc, i0, p.M, kbeg, kend, tid);
+      x3_fetch<INTERIOR>(rb, B, p.ldb, b_kc, j0, p.N, kbeg, kend, tid);
+      x3_stash<NSPLIT>(ra, panelA, a_kc, tid);
+      x3_stash<NSPLIT>(rb, panelB, b_kc, tid);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+      if (kt + 1 < nk) {                    // next k-tile's global loads fly during this one's MFMAs
+        const int k0 = kbeg + (kt + 1) * BK;
+        x3_fetch<INTERIOR>(ra, A, p.lda, a_kc, i0, p.M, k0, kend, tid);
+        x3_fetch<INTERIOR>(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, tid);
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        bf16x8 fa[2][NSPLIT], fb[2][NSPLIT];
+#pragma unroll
+        for (int s = 0; s < NSPLIT; ++s) {
+#pragma unroll
+          for (int a = 0; a < 2; ++a) fa[a][s] = x3_frag(panelA + s * X3_PLANE, a_kc, 64 * wr + 32 * a + l32, h, lane);
+#pragma unroll
+          for (int b = 0; b < 2; ++b) fb[b][s] = x3_frag(panelB + s * X3_PLANE, b_kc, 64 * wc + 32 * b + l32, h, lane);
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            // smallest terms first
+            if (NSPLIT >= 3) {
+              acc[a][b] = mfma_bf16(fa[a][1], fb[b][1], acc[a][b]);
+              acc[a][b] = mfma_bf16(fa[a][0], fb[b][2], acc[a][b]);
+              acc[a][b] = mfma_bf16(fa[a][2], fb[b][0], acc[a][b]);
+            }
+            if (NSPLIT >= 2) {
+              acc[a][b] = mfma_bf16(fa[a][0], fb[b][1], acc[a][b]);
+              acc[a][b] = mfma_bf16(fa[a][1], fb[b][0], acc[a][b]);
+            }
+            acc[a][b] = mfma_bf16(fa[a][0], fb[b][0], acc[a][b]);
+          }
+      }
+      __syncthreads();                      // everybody is done reading this k-tile
+      if (kt + 1 < nk) {
+        x3_stash<NSPLIT>(ra, panelA, a_kc, tid);
+        x3_stash<NSPLIT>(rb, panelB, b_kc, tid);
+      }
+      __syncthreads();
+    }
+  };
+  if (interior) mainloop(std::true_type{});
+  else mainloop(std::false_type{});
+  (void)g;
+
+  // the partial products of (i, j) and (j, i) are summed in different orders, so a mirrored result takes both
+  // triangles of a diagonal tile from the lower one
+  const bool mirror = (p.tile_mode == TILE_LOWER_MIRROR);
+  const bool lower_only = (p.tile_mode == TILE_LOWER) || (mirror && ti == tj);
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int gj = j0 + 64 * wc + 32 * b + l32;
+      if (gj >= p.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gi = i0 + 64 * wr + 32 * a + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (gi >= p.M) continue;
+        if (lower_only && gi < gj) continue;
+        float v = p.alpha * acc[a][b][r];
+        float* dst = C + static_cast<int64_t>(gi) * p.ldc + gj;
+        if (p.beta != 0.f) v += p.beta * *dst;
+        *dst = v;
+        if (mirror && gi != gj) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
+      }
+    }
+}
+
+// The split kernel takes operands whose 16-byte chunks never straddle the end of a row.
+inline bool gemm_x3_ok(const GemmParams& p) {
+  const int innerA = p.transA == 0 ? p.K : p.M, innerB = p.transB != 0 ? p.K : p.N;
+  return p.lda % 4 == 0 && p.ldb % 4 == 0 && p.sA % 4 == 0 && p.sB % 4 == 0 && innerA % 4 == 0 && innerB % 4 == 0 &&
+         (reinterpret_cast<uintptr_t>(p.A) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.B) & 15) == 0;
+}
+
+}  // namespace ak

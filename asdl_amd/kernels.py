@@ -265,8 +265,9 @@ def cholesky_inv(X, damping=1e-7):
 
 
 # ------------------------------------------------------------------------------ products
-def gemm(A, B, out=None, transA=False, transB=False, alpha=1.0, beta=0.0):
-    """out <- alpha * op(A) op(B) + beta * out for float32 matrices with contiguous rows."""
+def gemm(A, B, out=None, transA=False, transB=False, alpha=1.0, beta=0.0, pieces=0):
+    """out <- alpha * op(A) op(B) + beta * out for float32 matrices with contiguous rows.  pieces = 3 / 2:
+    on the bf16 matrix cores after an exact 3- / 2-way split of the operands (0: fp32 MFMA)."""
     _require_gpu(A, B, out)
     for t in (A, B):
         if t.dtype != torch.float32 or t.ndim != 2 or t.stride(1) != 1:
@@ -282,11 +283,11 @@ def gemm(A, B, out=None, transA=False, transB=False, alpha=1.0, beta=0.0):
         beta = 0.0
     if out.data_ptr() in (A.data_ptr(), B.data_ptr()):
         raise ValueError('gemm cannot run in place')
-    rc = _lib.load().ak_gemm_f32(int(transA), int(transB), M, N, K, alpha, ctypes.c_void_p(A.data_ptr()),
-                                 max(A.stride(0), A.shape[1]), ctypes.c_void_p(B.data_ptr()),
-                                 max(B.stride(0), B.shape[1]), beta, ctypes.c_void_p(out.data_ptr()),
-                                 max(out.stride(0), N), 1, 0, 0, 0, _stream())
-    _lib.check(rc, 'ak_gemm_f32')
+    rc = _lib.load().ak_gemm_f32_split(int(pieces), int(transA), int(transB), M, N, K, alpha,
+                                       ctypes.c_void_p(A.data_ptr()), max(A.stride(0), A.shape[1]),
+                                       ctypes.c_void_p(B.data_ptr()), max(B.stride(0), B.shape[1]), beta,
+                                       ctypes.c_void_p(out.data_ptr()), max(out.stride(0), N), 1, 0, 0, 0, _stream())
+    _lib.check(rc, 'ak_gemm_f32_split')
     return out
 
 

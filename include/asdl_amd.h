@@ -126,6 +126,16 @@ int ak_gemm_f32(int transA, int transB, int64_t M, int64_t N, int64_t K, float a
                 float* C, int64_t ldc, int batch, int64_t strideA, int64_t strideB, int64_t strideC,
                 ak_stream_t stream);
 
+/* The same product on the bf16 matrix cores: each fp32 operand element is split exactly into `pieces`
+ * bf16 values (3: all 24 mantissa bits, six partial products, error of the order of an fp32 multiply;
+ * 2: 16 bits, three partial products) and accumulated in fp32.  pieces = 0 is ak_gemm_f32.  Operands that
+ * the split kernel cannot take (leading dimensions or inner extents not multiples of 4, small shapes)
+ * are multiplied by the fp32 MFMA kernel.  Same reference call sites as ak_gemm_f32. */
+int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, int64_t K, float alpha,
+                const float* A, int64_t lda, const float* B, int64_t ldb, float beta,
+                float* C, int64_t ldc, int batch, int64_t strideA, int64_t strideB, int64_t strideC,
+                ak_stream_t stream);
+
 /* G <- grad_scale * Binv G Ainv (G = [dB, dA] in place), bias <- grad_scale * Binv bias when
  * bias != NULL.  ws holds the [dB, dA] intermediate.  Replaces Kron.mvp(use_inv, inplace)
  * (asdl/symmatrix.py:536-548) and the grad_scale pre-multiply of

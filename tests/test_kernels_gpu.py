@@ -293,6 +293,30 @@ def test_gemm_matches_fp64(K, tA, tB, M, N, K_):
     assert relerr(out, ref) < 1e-5
 
 
+@pytest.mark.parametrize('pieces,tol', [(3, 2e-6), (2, 3e-5)])
+@pytest.mark.parametrize('tA', [False, True])
+@pytest.mark.parametrize('tB', [False, True])
+@pytest.mark.parametrize('M,N,K_', [(256, 256, 128), (384, 640, 1000), (1100, 520, 516)])
+def test_gemm_split_matches_fp64(K, pieces, tol, tA, tB, M, N, K_):
+    """fp32 product on the bf16 matrix cores: 3 pieces have to be as good as the fp32 MFMA kernel."""
+    torch.manual_seed(M + N)
+    A = torch.randn((K_, M) if tA else (M, K_)) * torch.logspace(-3, 3, K_ if not tA else M)[None, :]
+    B = torch.randn((N, K_) if tB else (K_, N))
+    ref = (A.T if tA else A).double() @ (B.T if tB else B).double()
+    print(f'gemm split pieces={pieces} tA={tA} tB={tB} M={M} N={N} K={K_}', flush=True)
+    out = K.gemm(A.cuda(), B.cuda(), transA=tA, transB=tB, pieces=pieces)
+    out32 = K.gemm(A.cuda(), B.cuda(), transA=tA, transB=tB)
+    torch.cuda.synchronize()
+    e, e32 = relerr(out, ref), relerr(out32, ref)
+    assert e < tol, (e, e32)
+    if pieces == 3:
+        assert e < 4 * e32 + 1e-7, (e, e32)
+    # accumulate form
+    C0 = torch.randn(M, N)
+    out2 = K.gemm(A.cuda(), B.cuda(), out=C0.cuda().clone(), transA=tA, transB=tB, alpha=0.5, beta=-2.0, pieces=pieces)
+    assert relerr(out2, 0.5 * ref - 2.0 * C0.double()) < tol
+
+
 @pytest.mark.parametrize('dB,dA,bias', [(4, 5, True), (10, 784, True), (512, 512, True), (64, 147, False),
                                         (300, 1152, False)])
 def test_kron_precond_matches_oracle(K, dB, dA, bias):
