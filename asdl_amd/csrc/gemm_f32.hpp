@@ -201,16 +201,19 @@ namespace ak {
 
 inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return AK_OK;
-  if (p.split >= 2 && p.M >= 256 && p.N >= 256 && p.K >= 128 && gemm_x3_ok(p)) {
+  const int64_t tiles128 = static_cast<int64_t>((p.N + 127) / 128) * ((p.M + 127) / 128) * batch;
+  const bool lower = p.tile_mode != TILE_ALL;
+  const int64_t work_groups = lower ? tiles128 / 2 : tiles128;
+  // The split kernel (128 x 128 tiles, a pipeline that needs a few k-tiles to fill) pays off once its tiles
+  // fill most of the device; below that the 64 x 64 tiles of the fp32 kernel spread the work better.
+  if (p.split >= 2 && work_groups >= 200 && p.K >= 256 && gemm_x3_ok(p)) {
     dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
     if (p.split == 2) hipLaunchKernelGGL(gemm_x3_kernel<2>, grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL(gemm_x3_kernel<3>, grid, dim3(256), 0, stream, p);
     return check_launch();
   }
   // 128 x 128 tiles when they alone fill the 256 CUs twice over, else 64 x 64 tiles (four times the work groups)
-  const int64_t tiles128 = static_cast<int64_t>((p.N + 127) / 128) * ((p.M + 127) / 128) * batch;
-  const bool lower = p.tile_mode != TILE_ALL;
-  if ((lower ? tiles128 / 2 : tiles128) >= 512) {
+  if (work_groups >= 512) {
     dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
     hipLaunchKernelGGL(gemm_f32_kernel<2>, grid, dim3(256), 0, stream, p);
   } else {
