@@ -17,13 +17,32 @@ __all__ = ['extend', 'no_centered_cov', 'module_wise_assignments', 'modules_to_a
 
 
 @contextmanager
-def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, stream=None) -> OperationContext:
+def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, stream=None,
+           factor_stream=None) -> OperationContext:
+    """``stream``: as in the reference, the hook operations run under ``torch.cuda.stream(stream)``.
+    ``factor_stream``: the hook operations run on that stream, ordered after the kernels that produced their
+    inputs (the producing stream is waited for, the inputs are kept alive with record_stream), so that the
+    statistics kernels overlap the forward / backward kernels that follow; OperationContext.join_factor_stream()
+    orders the consumers after them."""
     handles = []
     cxt = OperationContext(vectors=vectors)
     use_stream = torch.cuda.is_available() and stream is not None
+    cxt.factor_stream = factor_stream if torch.cuda.is_available() else None
 
     def stream_cxt():
         return torch.cuda.stream(stream) if use_stream else nullcontext()
+
+    def run_hook(fn, *tensors):
+        fs = cxt.factor_stream
+        if fs is None or not tensors[0].is_cuda:
+            with stream_cxt():
+                fn()
+            return
+        fs.wait_stream(torch.cuda.current_stream(tensors[0].device))
+        with torch.cuda.stream(fs):
+            fn()
+        for t in tensors:
+            t.record_stream(fs)
 
     try:
         for module, names in module_wise_assignments(model, *op_names, ignore_modules=ignore_modules, map_rule=map_rule):
@@ -40,14 +59,14 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
                 continue
 
             def forward_hook(_module, in_data, out_data, _has_bwd=has_bwd):
-                with stream_cxt():
-                    cxt.call_operations_in_forward(_module, in_data[0].detach(), out_data.detach())
+                x, y = in_data[0].detach(), out_data.detach()
+                run_hook(lambda: cxt.call_operations_in_forward(_module, x, y), x, y)
                 if _has_bwd and out_data.requires_grad:
                     def grad_hook(grad, _m=_module):
                         if not cxt.is_operation_registered(_m):
                             return None          # context already closed
-                        with stream_cxt():
-                            cxt.call_operations_in_backward(_m, grad.detach())
+                        g = grad.detach()
+                        run_hook(lambda: cxt.call_operations_in_backward(_m, g), g)
                         return None
                     handles.append(out_data.register_hook(grad_hook))
             handles.append(module.register_forward_hook(forward_hook))
@@ -61,7 +80,7 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
 
 
 def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, vectors=None, stream=None,
-                    calc_inv=False) -> OperationContext:
+                    calc_inv=False, factor_stream=None) -> OperationContext:
     """Maps Fisher shapes to operations (asdl/core.py:83-97); only SHAPE_KRON has kernels here."""
     if cvp:
         raise NotImplementedError('covariance-vector products are not on this path')
@@ -72,7 +91,8 @@ def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, ve
         raise NotImplementedError(
             f'Fisher shape "{shape}" has no MI355X kernel in this build; only "{SHAPE_KRON}" is supported. '
             'Exclude such modules with PreconditioningConfig(ignore_modules=[...]).')
-    return extend(model, *shapes, ignore_modules=ignore_modules, map_rule=map_rule, vectors=vectors, stream=stream)
+    return extend(model, *shapes, ignore_modules=ignore_modules, map_rule=map_rule, vectors=vectors, stream=stream,
+                  factor_stream=factor_stream)
 
 
 def named_supported_modules(model):

@@ -20,6 +20,7 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
+FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (costs more host time per hook than the overlap gains)
 EAGER_INVERSE = False       # start the bulk of the inverses during a single sampled / empirical backward pass (no gain while the GPU is throughput-bound)
 
 
@@ -54,6 +55,19 @@ class FisherMaker(GradientMaker):
         for module in self.model.modules():
             if hasattr(module, attr):
                 delattr(module, attr)
+
+    def _factor_stream(self):
+        """Side stream (default priority) for the statistics kernels of the hooks, one per maker."""
+        if not FACTOR_SIDE_STREAM or not torch.cuda.is_available():
+            return None
+        p = next(self.model.parameters(), None)
+        if p is None or not p.is_cuda:
+            return None
+        fs = getattr(self, '_factor_stream_obj', None)
+        if fs is None or fs.device != p.device:
+            fs = torch.cuda.Stream(device=p.device)
+            self._factor_stream_obj = fs
+        return fs
 
     @property
     def single_backward_pass(self):
@@ -102,7 +116,7 @@ class FisherMaker(GradientMaker):
         inv_after_fisher = calc_inv and self.do_local_accumulate
 
         with no_centered_cov(model, fisher_shapes, ignore_modules=config.ignore_modules,
-                             calc_inv=inv_with_fisher) as cxt:
+                             calc_inv=inv_with_fisher, factor_stream=self._factor_stream()) as cxt:
             if accumulate:
                 self._register_fisher(cxt, accumulate_prescale)
             if damping is not None:
@@ -127,6 +141,7 @@ class FisherMaker(GradientMaker):
                 closure(lambda: loss)
             else:
                 self._fisher_loop(closure)
+            cxt.join_factor_stream()
             cxt.finish_registered()
             # The inverses only need the factors: enqueue them now (side streams) and, when a loss backward
             # pass follows, let that pass run on the main stream meanwhile; the flags are read afterwards.
@@ -223,7 +238,9 @@ class FisherMCCrossEntropy(FisherMaker):
         n_mc_samples = self.config.n_mc_samples
         probs = F.softmax(logits, dim=-1)
         log_probs = F.log_softmax(logits, dim=-1)
-        dist = torch.distributions.Categorical(probs)
+        # validate_args=False: the check of the simplex constraint would synchronise the host with the forward
+        # pass; the draw itself (normalisation + multinomial) is unchanged
+        dist = torch.distributions.Categorical(probs, validate_args=False)
         for i in range(n_mc_samples):
             with torch.no_grad():
                 targets = self.sample_targets(dist, i)
@@ -262,7 +279,7 @@ class FisherMCMSE(FisherMaker):
     def _fisher_loop(self, closure):
         logits = self._logits
         n_mc_samples = self.config.n_mc_samples
-        dist = torch.distributions.normal.Normal(logits, scale=np.sqrt(self.config.var))
+        dist = torch.distributions.normal.Normal(logits, scale=np.sqrt(self.config.var), validate_args=False)
         for i in range(n_mc_samples):
             with torch.no_grad():
                 targets = dist.sample()

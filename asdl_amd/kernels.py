@@ -51,8 +51,34 @@ def _require_gpu(*tensors):
                                f'{t.device}. There is no CPU fallback.')
 
 
-def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
+def _stream_handle(device=None):
+    """The calling thread's current HIP stream on ``device`` as an integer handle."""
+    if _raw_stream is not None:
+        idx = device.index if device is not None and device.index is not None else torch.cuda.current_device()
+        return _raw_stream(idx)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _stream(device=None):
+    return ctypes.c_void_p(_stream_handle(device))
+
+
+_size_cache = {}
+
+
+def _ws_need(fn_name, *args):
+    """Cached ak_*_ws_bytes query (pure functions of the shape)."""
+    key = (fn_name, args)
+    need = _size_cache.get(key)
+    if need is None:
+        need = getattr(_lib.load(), fn_name)(*args)
+        if len(_size_cache) > 8192:
+            _size_cache.clear()
+        _size_cache[key] = need
+    return need
 
 
 def _dtype_code(t):
@@ -68,8 +94,7 @@ def workspace(nbytes, device):
     Kernels on one stream run in order, so consecutive calls may share it."""
     if nbytes <= 0:
         return None, 0
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream().cuda_stream)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream_handle(device))
     with _ws_lock:
         buf = _workspaces.get(key)
         if buf is None or buf.numel() < nbytes:
@@ -139,7 +164,7 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
         raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
     lib = _lib.load()
-    need = lib.ak_syrk_tn_ws_bytes(M, d)
+    need = _ws_need('ak_syrk_tn_ws_bytes', M, d)
     ws, ws_bytes, keep = _ws_args(need, x.device)
     with _Timed('syrk_tn', M * d * (d + 1)):
         rc = lib.ak_syrk_tn(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), M, d, ldx, alpha, beta,
@@ -178,7 +203,7 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     if x.dtype == torch.bfloat16 and C % 8 == 0 and _is_channels_last(x):
         if (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0):
             return syrk_tn(x.permute(0, 2, 3, 1).reshape(N * H * W, C), out=out, alpha=alpha, beta=beta)
-        need = lib.ak_conv_syrk_nhwc_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)
+        need = _ws_need('ak_conv_syrk_nhwc_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
         ws, ws_bytes, keep = _ws_args(need, x.device)
         with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
             rc = lib.ak_conv_syrk_nhwc(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw,
@@ -188,7 +213,7 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
             _lib.check(rc, 'ak_conv_syrk_nhwc')
             return out
     x = x.contiguous()
-    need = lib.ak_conv_syrk_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)
+    need = _ws_need('ak_conv_syrk_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
     ws, ws_bytes, keep = _ws_args(need, x.device)
     with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
         rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw, ph, pw,
@@ -239,7 +264,7 @@ def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1
     if info is None:
         info = torch.empty(batch, dtype=torch.int32, device=dev)
     lib = _lib.load()
-    need = lib.ak_chol_inv_ws_bytes(d, batch)
+    need = _ws_need('ak_chol_inv_ws_bytes', d, batch)
     ws, ws_bytes, keep = _ws_args(need, dev)
     pa, po = device_ptr_array(mats), device_ptr_array(outs)
     rc = lib.ak_chol_inv_batched(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(po.data_ptr()), d, batch,
@@ -301,7 +326,7 @@ def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
     if grad_b is not None and (grad_b.numel() != dB or not grad_b.is_contiguous() or grad_b.dtype != torch.float32):
         raise ValueError('grad_b has to be a contiguous float32 vector with dB elements')
     lib = _lib.load()
-    ws, ws_bytes, keep = _ws_args(lib.ak_kron_precond_ws_bytes(dB, dA), grad_w.device)
+    ws, ws_bytes, keep = _ws_args(_ws_need('ak_kron_precond_ws_bytes', dB, dA), grad_w.device)
     rc = lib.ak_kron_precond(ctypes.c_void_p(B_inv.data_ptr()), ctypes.c_void_p(A_inv.data_ptr()),
                              ctypes.c_void_p(grad_w.data_ptr()), dB, dA,
                              ctypes.c_void_p(grad_b.data_ptr()) if grad_b is not None else ctypes.c_void_p(0),
@@ -331,7 +356,7 @@ def inv_root_newton(S, p, ridge_eps, v0, out=None, max_power_iter=100, power_tol
         raise ValueError('out has to be float32 [batch, n, n] with dense matrices')
     stats = torch.empty(batch, 4, dtype=torch.float32, device=S.device)
     lib = _lib.load()
-    ws, ws_bytes, keep = _ws_args(lib.ak_inv_root_ws_bytes(n, batch), S.device)
+    ws, ws_bytes, keep = _ws_args(_ws_need('ak_inv_root_ws_bytes', n, batch), S.device)
     strideS = S3.stride(0) if batch > 1 else n * n
     strideO = out3.stride(0) if batch > 1 else n * n
     rc = lib.ak_inv_root_newton(ctypes.c_void_p(S3.data_ptr()), n, batch, strideS, int(p), float(ridge_eps),

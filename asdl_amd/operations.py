@@ -293,6 +293,7 @@ class OperationContext:
         self._vectors = vectors
         self._pending_inverse = []
         self._inverse_chunks = []
+        self.factor_stream = None
         self._eager_total = 0.0
         self._eager_done = False
         self._inverse_cost = 0.0
@@ -340,6 +341,11 @@ class OperationContext:
 
     def calc_full_cov(self, model, scale=1., calc_inv=False, damping=1e-7):
         pass  # only needed for the full (non layer-wise) shape
+
+    def join_factor_stream(self):
+        """Orders the current stream after the statistics kernels that ran on the factor stream."""
+        if self.factor_stream is not None:
+            torch.cuda.current_stream(self.factor_stream.device).wait_stream(self.factor_stream)
 
     # ---- deferred, batched inverses
     def set_eager_inverse(self, total_cost):
