@@ -167,7 +167,8 @@ def test_resnet18_cifar_fp32_small_batch():
     print(f'ResNet-18: worst grad err {g:.2e}, worst inverse err {i:.2e}', flush=True)
 
 
-def test_small_cnn_bf16_autocast():
+@pytest.mark.parametrize('channels_last', [False, True])
+def test_small_cnn_bf16_autocast(channels_last):
     # bf16 forward/backward through autocast, fp32 factors accumulated from the bf16 activations.  CPU and GPU
     # bf16 convolutions round differently, so the oracle is fed the very activations / output gradients the GPU
     # run produced (captured with extra hooks) and the GPU's raw gradients: same inputs, same formulas.
@@ -176,6 +177,10 @@ def test_small_cnn_bf16_autocast():
                           nn.Conv2d(32, 32, 1), nn.ReLU(), nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
     bs, damping = 16, 1e-2
     x, t = torch.randn(bs, 3, 16, 16).cuda(), torch.randint(0, 10, (bs,)).cuda()
+    if channels_last:
+        # NHWC activations: conv factors are gathered in place (16 and 32 channels), output gradients stay 4-D
+        model = model.to(memory_format=torch.channels_last)
+        x = x.contiguous(memory_format=torch.channels_last)
 
     def fwd(inp):
         with torch.autocast('cuda', dtype=torch.bfloat16):
@@ -196,6 +201,9 @@ def test_small_cnn_bf16_autocast():
     for h in handles:
         h.remove()
     assert saw_bf16, 'autocast should hand bf16 activations to the hooks'
+    if channels_last:
+        assert any(v.ndim == 4 and not v.is_contiguous() and v.is_contiguous(memory_format=torch.channels_last)
+                   for v in ins.values()), 'the hooks should see channels-last activations'
 
     gm = KfacGradientMaker(model, PreconditioningConfig(data_size=bs, damping=damping), fisher_type=FISHER_EMP)
     model.zero_grad(set_to_none=True)
@@ -215,6 +223,111 @@ def test_small_cnn_bf16_autocast():
         w, b = R.kron_mvp(A_inv, B_inv, raw[name + '.weight'].cpu(), raw[name + '.bias'].cpu())
         assert relerr(m.weight.grad, w) < 1e-2, (name, relerr(m.weight.grad, w))
         assert relerr(m.bias.grad, b) < 1e-2
+
+
+def test_config2_linear_4096_batch8192_bf16_ema():
+    """BASELINE config 2 at full size: Linear(4096, 4096), 8192 rows, bf16 activations, fp32 factors with EMA.
+    The factors are compared with fp64 products of the same rounded values, the inverses through the identity
+    (A + lam I) A_inv = I, the preconditioned gradient with B_inv G A_inv in fp64."""
+    torch.manual_seed(5)
+    M, d, damping, ema = 8192, 4096, 1e-3, 0.05
+    a = torch.randn(M, d).to(torch.bfloat16)
+    lin = nn.Linear(d, d).cuda()
+    model = nn.Sequential(lin)
+    t = torch.randn(M, d).cuda() * 0.01
+    config = PreconditioningConfig(data_size=M, damping=damping, ema_decay=ema)
+    gm = KfacGradientMaker(model, config, fisher_type=FISHER_EMP, loss_type='mse')
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    model.zero_grad(set_to_none=True)
+    gm.setup_loss_call(F.mse_loss, gm.setup_model_call(fwd, a.cuda()), t)
+    gm.forward_and_backward()
+    kron = lin.fisher.kron
+    a64 = a.cuda().double()                        # fp64 products on the device: torch's GEMM as independent reference
+    A_ref = ema * (a64.T @ a64) / M                # first EMA update: (1 - ema) * 0 + ema * statistic
+    assert relerr(kron.A, A_ref) < 1e-5
+    assert torch.equal(kron.A, kron.A.T)
+    assert abs(float(kron.A.diagonal().sum().double()) - ema * float((a64 ** 2).sum() / M)) < 1e-4 * float(A_ref.trace())
+    for which in ('A', 'B'):
+        F_, inv = getattr(kron, which).double(), getattr(kron, which + '_inv').double()
+        trA, trB = float(kron.A.diagonal().sum()), float(kron.B.diagonal().sum())
+        pi = (trA / trB) ** 0.5                    # dA == dB
+        lam = damping ** 0.5 * pi if which == 'A' else damping ** 0.5 / pi
+        lam = max(lam, 1e-7)
+        eye = torch.eye(d, dtype=torch.float64, device='cuda')
+        resid = (F_ + lam * eye) @ inv - eye
+        assert float(resid.norm()) / d ** 0.5 < 1e-3, (which, float(resid.norm()) / d ** 0.5)
+        assert torch.equal(getattr(kron, which + '_inv'), getattr(kron, which + '_inv').T)
+
+
+def test_resnet50_batch64_channels_last_properties():
+    """BASELINE's benchmark configuration at full size, checked through properties that do not need a CPU run of
+    the model: every conv A factor against an fp64 product of the unfolded input the GPU produced, every inverse
+    through its defining identity, and the preconditioned gradients against B_inv G A_inv recomputed in fp64 from
+    the stored inverses (sampled layers, to keep the host time down)."""
+    torch.manual_seed(6)
+    bs, damping, ema = 64, 1e-3, 0.5
+    model = bench_models.resnet50().cuda().to(memory_format=torch.channels_last)
+    x = torch.randn(bs, 3, 224, 224).cuda().contiguous(memory_format=torch.channels_last)
+    t = torch.randint(0, 1000, (bs,)).cuda()
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    picks = ['conv1', 'layer1.0.conv2', 'layer2.0.conv2', 'layer3.1.conv1', 'layer4.0.downsample.0', 'layer4.2.conv2', 'fc']
+    mods = dict(model.named_modules())
+    ins, gouts, handles = {}, {}, []
+    for name in picks:
+        def fhook(mod, inp, out, name=name):
+            ins[name] = inp[0].detach()
+            out.register_hook(lambda g, name=name: gouts.__setitem__(name, g.detach()))
+        handles.append(mods[name].register_forward_hook(fhook))
+    raw = {}
+    handles.append(mods['layer4.2.conv2'].weight.register_hook(lambda g: raw.__setitem__('g', g.detach().clone())))
+    config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema, ignore_modules=[nn.BatchNorm2d])
+    gm = KfacGradientMaker(model, config, fisher_type=FISHER_EMP)
+    model.zero_grad(set_to_none=True)
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
+    gm.forward_and_backward()
+    for h in handles:
+        h.remove()
+    for name in picks:
+        m = mods[name]
+        kron = m.fisher.kron
+        a = ins[name].float()
+        g = gouts[name].float()              # summed loss inside the maker: these are the K-FAC out-grads
+        if isinstance(m, nn.Conv2d):
+            u = F.unfold(a.contiguous().double(), m.kernel_size, padding=m.padding, stride=m.stride)   # [n, d, hw]
+            hw = u.shape[-1]
+            U = u.permute(1, 0, 2).reshape(u.shape[1], -1)
+            A_ref = ema * (U @ U.T) / hw / bs
+            del u, U
+            g2 = g.permute(0, 2, 3, 1).reshape(-1, g.shape[1]).double()
+        else:
+            A_ref = ema * a.double().T @ a.double() / bs
+            g2 = g.double()
+        B_ref = ema * g2.T @ g2 / bs
+        assert relerr(kron.A, A_ref) < 1e-5, (name, 'A', relerr(kron.A, A_ref))
+        assert relerr(kron.B, B_ref) < 1e-5, (name, 'B', relerr(kron.B, B_ref))
+        assert torch.equal(kron.A, kron.A.T) and torch.equal(kron.B, kron.B.T)
+        dA, dB = kron.A.shape[0], kron.B.shape[0]
+        trA, trB = float(kron.A.diagonal().sum().double()), float(kron.B.diagonal().sum().double())
+        pi = ((trA / dA) / (trB / dB)) ** 0.5
+        for which, lam, dim in (('A', max(damping ** 0.5 * pi, 1e-7), dA), ('B', max(damping ** 0.5 / pi, 1e-7), dB)):
+            F_, inv = getattr(kron, which).double(), getattr(kron, which + '_inv').double()
+            resid = (F_ + lam * torch.eye(dim, dtype=torch.float64, device='cuda')) @ inv - \
+                torch.eye(dim, dtype=torch.float64, device='cuda')
+            assert float(resid.norm()) / dim ** 0.5 < 2e-3, (name, which, float(resid.norm()) / dim ** 0.5)
+    # preconditioned gradient of a large layer: B_inv G A_inv in fp64 on the raw gradient of the same backward pass
+    m = mods['layer4.2.conv2']
+    G = raw['g'].double().reshape(m.weight.shape[0], -1) / bs
+    ref = m.fisher.kron.B_inv.double() @ G @ m.fisher.kron.A_inv.double()
+    got = m.weight.grad.detach().double().reshape(m.weight.shape[0], -1)
+    assert relerr(got, ref) < 1e-3, relerr(got, ref)
 
 
 def test_fisher_attributes_and_steps_without_curvature_update():
