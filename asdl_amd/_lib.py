@@ -33,6 +33,11 @@ _SIGNATURES = {
     'ak_kron_damping': (c_int, [c_ptr, c_ptr, c_ptr, c_int, c_f32, c_f32, c_ptr, c_ptr, c_ptr]),
     'ak_chol_inv_ws_bytes': (c_size, [c_i64, c_int]),
     'ak_chol_inv_batched': (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_size, c_ptr]),
+    'ak_unit_wise_ws_bytes': (c_size, [c_i64, c_i64, c_i64]),
+    'ak_unit_wise_stats': (c_int, [c_ptr, c_int, c_i64, c_i64, c_i64, c_ptr, c_int, c_i64, c_i64, c_i64, c_ptr, c_ptr,
+                                   c_i64, c_i64, c_i64, c_f32, c_f32, c_ptr, c_ptr, c_size, c_ptr]),
+    'ak_unit_wise_inv': (c_int, [c_ptr, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
+    'ak_unit_wise_mvp': (c_int, [c_ptr, c_i64, c_ptr, c_ptr, c_f32, c_ptr]),
     'ak_gemm_f32': (c_int, [c_int, c_int, c_i64, c_i64, c_i64, c_f32, c_ptr, c_i64, c_ptr, c_i64, c_f32,
                             c_ptr, c_i64, c_int, c_i64, c_i64, c_i64, c_ptr]),
     'ak_gemm_f32_split': (c_int, [c_int, c_int, c_int, c_i64, c_i64, c_i64, c_f32, c_ptr, c_i64, c_ptr, c_i64, c_f32,

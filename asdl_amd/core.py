@@ -11,7 +11,7 @@ from .operations import *
 from .operations import FWD_OPS, BWD_OPS
 from .utils import record_original_requires_grad
 
-_supported_module_classes = (nn.Linear, nn.Conv2d)
+_supported_module_classes = (nn.Linear, nn.Conv2d, nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 
 __all__ = ['extend', 'no_centered_cov', 'module_wise_assignments', 'modules_to_assign']
 
@@ -88,8 +88,11 @@ def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, ve
     def map_rule(shape):
         if shape == SHAPE_KRON:
             return OP_COV_KRON_INV if calc_inv else OP_COV_KRON
+        if shape == SHAPE_UNIT_WISE:
+            return OP_COV_UNIT_WISE_INV if calc_inv else OP_COV_UNIT_WISE
         raise NotImplementedError(
-            f'Fisher shape "{shape}" has no MI355X kernel in this build; only "{SHAPE_KRON}" is supported. '
+            f'Fisher shape "{shape}" has no MI355X kernel in this build; only "{SHAPE_KRON}" and '
+            f'"{SHAPE_UNIT_WISE}" are supported. '
             'Exclude such modules with PreconditioningConfig(ignore_modules=[...]).')
     return extend(model, *shapes, ignore_modules=ignore_modules, map_rule=map_rule, vectors=vectors, stream=stream,
                   factor_stream=factor_stream)

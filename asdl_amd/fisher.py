@@ -185,6 +185,8 @@ class FisherMaker(GradientMaker):
             fisher: SymMatrix = getattr(module, attr, None)
             if fisher is not None and fisher.has_kron:
                 krons.append(fisher.kron)
+            if fisher is not None and fisher.has_unit:
+                fisher.unit.update_inv(damping, replace=True)
         batched_update_inv(krons, damping=damping, replace=True)
 
     def _fisher_loop(self, closure):

@@ -231,6 +231,85 @@ def syrk_nt(x, out=None, alpha=1.0, beta=0.0):
     return conv_syrk(x.unsqueeze(2), (1, 1), (1, 1), (0, 0), out=out, alpha=alpha, beta=beta)
 
 
+# ------------------------------------------------------------------------------ unit-wise blocks
+def unit_wise_stats(y, g, weight, bias, out=None, alpha=1.0, beta=0.0):
+    """out[f] <- beta*out[f] + alpha * sum_n [[gw^2, gw*gb], [gw*gb, gb^2]] with the per-sample gradients
+    gw = sum_s (y - bias)/weight * g, gb = sum_s g.  y, g: [n, f], [n, f, *spatial] (any strides, e.g. channels
+    last) or [rows, *normalized_shape] for LayerNorm (pass them flattened to [rows, f])."""
+    _require_gpu(y, g, weight, bias, out)
+    if y.shape != g.shape:
+        raise ValueError(f'shapes differ: {tuple(y.shape)} vs {tuple(g.shape)}')
+    N, F = y.shape[0], y.shape[1]
+
+    def strides(t):
+        if t.ndim == 2:
+            return t.stride(0), t.stride(1), 1, 1
+        sp = t.shape[2:]
+        S = 1
+        for d in sp:
+            S *= d
+        # the positions have to be addressable with one stride
+        st = t.stride(-1)
+        expect = st
+        for d, s_ in zip(reversed(sp), reversed(t.stride()[2:])):
+            if d != 1 and s_ != expect:
+                return None
+            expect *= d
+        return t.stride(0), t.stride(1), st, S
+
+    sy, sg = strides(y), strides(g)
+    if sy is None:
+        y = y.contiguous()
+        sy = strides(y)
+    if sg is None:
+        g = g.contiguous()
+        sg = strides(g)
+    S = sy[3]
+    weight = weight.detach().float().contiguous()
+    bias = bias.detach().float().contiguous()
+    if out is None:
+        out = torch.empty(F, 2, 2, dtype=torch.float32, device=y.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or out.shape != (F, 2, 2) or not out.is_contiguous():
+        raise ValueError('out has to be a contiguous float32 [f, 2, 2] tensor')
+    need = _ws_need('ak_unit_wise_ws_bytes', N, F, S)
+    ws, ws_bytes, keep = _ws_args(need, y.device)
+    rc = _lib.load().ak_unit_wise_stats(ctypes.c_void_p(y.data_ptr()), _dtype_code(y), sy[0], sy[1], sy[2],
+                                        ctypes.c_void_p(g.data_ptr()), _dtype_code(g), sg[0], sg[1], sg[2],
+                                        ctypes.c_void_p(weight.data_ptr()), ctypes.c_void_p(bias.data_ptr()), N, F, S,
+                                        alpha, beta, ctypes.c_void_p(out.data_ptr()), ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_unit_wise_stats')
+    return out
+
+
+def unit_wise_inv(blocks, damping, out=None):
+    """(out, flags): out[f] = (blocks[f] + damping I)^-1; flags is a device int32[2] = (any non-zero entry,
+    1-based index of the first singular block or 0x7fffffff)."""
+    _require_gpu(blocks, out)
+    if blocks.dtype != torch.float32 or blocks.ndim != 3 or blocks.shape[1:] != (2, 2) or not blocks.is_contiguous():
+        raise ValueError('blocks has to be a contiguous float32 [f, 2, 2] tensor')
+    if out is None:
+        out = torch.empty_like(blocks)
+    flags = torch.empty(2, dtype=torch.int32, device=blocks.device)
+    rc = _lib.load().ak_unit_wise_inv(ctypes.c_void_p(blocks.data_ptr()), blocks.shape[0], float(damping),
+                                      ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(flags.data_ptr()), _stream())
+    _lib.check(rc, 'ak_unit_wise_inv')
+    return out, flags
+
+
+def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
+    """[vec_weight, vec_bias][f] <- mat[f] @ (scale * [vec_weight, vec_bias][f]) in place."""
+    _require_gpu(mat, vec_weight, vec_bias)
+    F = mat.shape[0]
+    for v in (vec_weight, vec_bias):
+        if v.dtype != torch.float32 or v.numel() != F or not v.is_contiguous():
+            raise ValueError('vectors have to be contiguous float32 tensors with one entry per block')
+    rc = _lib.load().ak_unit_wise_mvp(ctypes.c_void_p(mat.data_ptr()), F, ctypes.c_void_p(vec_weight.data_ptr()),
+                                      ctypes.c_void_p(vec_bias.data_ptr()), float(scale), _stream())
+    _lib.check(rc, 'ak_unit_wise_mvp')
+    return vec_weight, vec_bias
+
+
 # ------------------------------------------------------------------------------ damping / inverse
 def kron_damping(A_list, B_list, damping, eps=1e-7):
     """Returns (lam [batch, 2] float32, nonzero [batch, 2] int32), both on the device."""

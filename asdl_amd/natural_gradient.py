@@ -21,7 +21,8 @@ from .symmatrix import SymMatrix, batched_update_inv
 
 _invalid_ema_decay = -1
 _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KFE, SHAPE_UNIT_WISE, SHAPE_DIAG]
-_kernel_shapes = [SHAPE_KRON]
+_kernel_shapes = [SHAPE_KRON, SHAPE_UNIT_WISE]
+_norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 
 __all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
 
@@ -48,13 +49,13 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         if not self.do_accumulate and config.curvature_upd_ratio is not None:
             raise ValueError('curvature_upd_ratio cannot be specified when no curvature accumulation is performed.')
 
-        unsupported = [m for m in self.module_dict.values() if not isinstance(m, (nn.Linear, nn.Conv2d))]
+        unsupported = [m for m in self.module_dict.values() if not isinstance(m, (nn.Linear, nn.Conv2d) + _norm_classes)]
         if unsupported:
             kinds = sorted({type(m).__name__ for m in unsupported})
             raise NotImplementedError(
-                f'{kinds} modules would get a unit-wise / diagonal Fisher in the reference; this build has kernels '
-                f'for the Kronecker-factored shape of Linear and Conv2d only. Pass '
-                f'PreconditioningConfig(ignore_modules=[...]) to leave them un-preconditioned.')
+                f'{kinds} modules have no kernels in this build (Linear / Conv2d: Kronecker-factored, BatchNorm / '
+                f'LayerNorm: unit-wise). Pass PreconditioningConfig(ignore_modules=[...]) to leave them '
+                f'un-preconditioned.')
 
         self.named_modules_for_curvature = []
         self.modules_for_curvature = []
@@ -65,6 +66,8 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                                  f'{name} is assigned {len(shapes)} shapes.')
             if shapes[0] not in _kernel_shapes:
                 raise NotImplementedError(f'Fisher shape "{shapes[0]}" (module {name}) is not on this path.')
+            if shapes[0] == SHAPE_UNIT_WISE and not isinstance(module, _norm_classes):
+                raise NotImplementedError(f'the unit-wise shape is built for BatchNorm / LayerNorm only (module {name}).')
             self.modules_for_curvature.append(module)
             self.named_modules_for_curvature.append((name, module))
             self.shape_for[module] = shapes[0]
@@ -108,6 +111,8 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             return None
         if shape in [SHAPE_KRON, SHAPE_SWIFT_KRON]:
             return fisher.kron
+        if shape == SHAPE_UNIT_WISE:
+            return fisher.unit
         raise ValueError(f'Invalid shape: {shape}.')
 
     @property
@@ -134,7 +139,7 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             kron = ['A', 'B']
         if damping is None:
             damping = self.config.damping
-        matrices = []
+        matrices, units = [], []
         for shape in _kernel_shapes:
             for name, module in self.named_modules_for(shape):
                 if module_name is not None and name != module_name:
@@ -143,8 +148,12 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                     continue
                 matrix = self._get_module_symmatrix(module, shape)
                 if matrix is not None:
-                    matrices.append(matrix)
+                    (units if shape == SHAPE_UNIT_WISE else matrices).append(matrix)
         batched_update_inv(matrices, damping, calc_A_inv='A' in kron, calc_B_inv='B' in kron)
+        for unit in units:
+            unit.update_inv(damping)
+            if zero_curvature:
+                unit.mul_(0)
         if zero_curvature:
             with torch.no_grad():
                 for matrix in matrices:
@@ -216,13 +225,15 @@ class KfacGradientMaker(NaturalGradientMaker):
     """K-FAC (https://arxiv.org/abs/1503.05671) behind the GradientMaker interface; same constructor
     arguments as asdl/precondition/natural_gradient.py:883-900.
 
-    BatchNorm / LayerNorm modules (unit-wise Fisher in the reference) and ``swift=True`` have no
-    kernels in this build: exclude such modules through ``config.ignore_modules``."""
+    BatchNorm1d/2d and LayerNorm modules get the unit-wise shape, as in the reference.  ``swift=True`` and
+    Embedding modules have no kernels in this build (exclude the latter through ``config.ignore_modules``)."""
 
     def __init__(self, model, config: PreconditioningConfig, fisher_type: str = FISHER_MC,
                  loss_type: str = LOSS_CROSS_ENTROPY, scale: float = 1, grad_scale: float = 1, n_mc_samples: int = 1,
                  var: float = 1., seed: int = None, swift=False):
         if swift:
             raise NotImplementedError('swift=True (SKFAC) is not on this path')
-        super().__init__(model, config, fisher_type=fisher_type, fisher_shape=[SHAPE_KRON], loss_type=loss_type,
+        fisher_shape = [SHAPE_KRON, (nn.BatchNorm1d, SHAPE_UNIT_WISE), (nn.BatchNorm2d, SHAPE_UNIT_WISE),
+                        (nn.LayerNorm, SHAPE_UNIT_WISE)]
+        super().__init__(model, config, fisher_type=fisher_type, fisher_shape=fisher_shape, loss_type=loss_type,
                          scale=scale, grad_scale=grad_scale, n_mc_samples=n_mc_samples, var=var, seed=seed)

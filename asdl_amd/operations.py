@@ -19,27 +19,32 @@ import torch
 import torch.nn as nn
 
 from . import kernels
-from .symmatrix import Kron, SymMatrix, batched_update_inv
-from .utils import UnfoldedInput, im2col_2d
+from .symmatrix import Kron, SymMatrix, UnitWise, batched_update_inv
+from .utils import UnfoldedInput, im2col_2d, original_requires_grad
 
 OP_COV_KRON = 'cov_kron'
 OP_COV_KRON_INV = 'cov_kron_inv'
+OP_COV_UNIT_WISE = 'cov_unit_wise'
+OP_COV_UNIT_WISE_INV = 'cov_unit_wise_inv'
 OP_SAVE_INPUTS = 'save_inputs'
 OP_SAVE_OUTPUTS = 'save_outputs'
 OP_SAVE_OUTGRADS = 'save_outgrads'
 
-ALL_OPS = [OP_COV_KRON, OP_COV_KRON_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS]
-FWD_OPS = [OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_COV_KRON, OP_COV_KRON_INV]
-BWD_OPS = [OP_SAVE_OUTGRADS, OP_COV_KRON, OP_COV_KRON_INV]
+ALL_OPS = [OP_COV_KRON, OP_COV_KRON_INV, OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS,
+           OP_SAVE_OUTGRADS]
+BWD_OPS_WITH_INPUTS = [OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV]     # the forward hook has to keep the output
+FWD_OPS = [OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_COV_KRON, OP_COV_KRON_INV] + BWD_OPS_WITH_INPUTS
+BWD_OPS = [OP_SAVE_OUTGRADS, OP_COV_KRON, OP_COV_KRON_INV, OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV]
 
-__all__ = ['Operation', 'Linear', 'Conv2d', 'OperationContext', 'get_op_class', 'ALL_OPS', 'FWD_OPS', 'BWD_OPS',
-           'OP_COV_KRON', 'OP_COV_KRON_INV', 'OP_SAVE_INPUTS', 'OP_SAVE_OUTPUTS', 'OP_SAVE_OUTGRADS']
+__all__ = ['Operation', 'Linear', 'Conv2d', 'BatchNorm', 'LayerNorm', 'OperationContext', 'get_op_class', 'ALL_OPS',
+           'FWD_OPS', 'BWD_OPS', 'OP_COV_KRON', 'OP_COV_KRON_INV', 'OP_COV_UNIT_WISE', 'OP_COV_UNIT_WISE_INV',
+           'OP_SAVE_INPUTS', 'OP_SAVE_OUTPUTS', 'OP_SAVE_OUTGRADS']
 
 _FACTOR_CACHE_ATTR = '_asdl_amd_factor_cache'
 
 
 class Operation:
-    supported_operations = set(ALL_OPS)
+    supported_operations = {OP_COV_KRON, OP_COV_KRON_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS}
 
     def __init__(self, module, op_names, model_for_kernel=None):
         if hasattr(module, 'weight'):
@@ -250,6 +255,88 @@ class Conv2d(Operation):
         return kernels.syrk_nt(out_grads, out=out, alpha=alpha, beta=beta)    # c_out x c_out
 
 
+class _NormOperation(Operation):
+    """Unit-wise Fisher of modules with one (weight, bias) pair per feature: 2 x 2 blocks of the per-sample
+    gradients (asdl/operations/batchnorm.py:8-108, asdl/operations/layernorm.py:7-84, and the unit-wise branch of
+    Operation.backward_pre_process, asdl/operations/operation.py:230-235, 308-321).  As in the reference the
+    normalised input is recovered from the module's output, which the forward hook keeps by reference: an
+    in-place activation behind the module changes what the backward hook sees there, too."""
+    supported_operations = {OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS}
+
+    def forward_post_process(self, in_data, out_data):
+        op_names = self._op_names
+        if OP_SAVE_INPUTS in op_names:
+            self.accumulate_result([in_data], OP_SAVE_INPUTS, extend=True)
+        if OP_SAVE_OUTPUTS in op_names:
+            self.accumulate_result([out_data], OP_SAVE_OUTPUTS, extend=True)
+        if any(n in BWD_OPS_WITH_INPUTS for n in op_names):
+            self._op_results['_out_data'] = out_data
+
+    @staticmethod
+    def as_samples(module, tensor):
+        """[samples, features, *positions] view of an output / output-gradient tensor."""
+        return tensor
+
+    def backward_pre_process(self, out_grads, vector=None):
+        module = self._module
+        op_names = self._op_names
+        if OP_SAVE_OUTGRADS in op_names:
+            self.accumulate_result([out_grads], OP_SAVE_OUTGRADS, extend=True)
+        if not any(n in BWD_OPS_WITH_INPUTS for n in op_names):
+            return
+        if not (original_requires_grad(module, 'weight') and original_requires_grad(module, 'bias')):
+            raise ValueError(f'Both weight and bias have to require grad for {OP_COV_UNIT_WISE} (module: {module}).')
+        out_data = self._op_results.get('_out_data')
+        if out_data is None:
+            raise RuntimeError(f'{OP_COV_UNIT_WISE}: the forward hook did not run (module: {module})')
+        y, g = self.as_samples(module, out_data), self.as_samples(module, out_grads)
+        weight, bias = module.weight.detach().flatten(), module.bias.detach().flatten()
+        if OP_COV_UNIT_WISE in op_names:
+            store = self._op_results.setdefault(OP_COV_UNIT_WISE, {})
+            existing = store.get('data')
+            if existing is None:
+                store['data'] = kernels.unit_wise_stats(y, g, weight, bias, alpha=self._cov_scale)
+            else:
+                beta = self._first_beta.pop('data', 1.0)
+                kernels.unit_wise_stats(y, g, weight, bias, out=existing, alpha=self._cov_scale, beta=beta)
+        else:
+            first = '_unit_tmp' not in self._op_results
+            cache = getattr(module, _FACTOR_CACHE_ATTR, None)
+            if cache is None:
+                cache = {}
+                setattr(module, _FACTOR_CACHE_ATTR, cache)
+            buf = cache.get('unit')
+            if buf is None or buf.shape[0] != weight.numel() or buf.device != weight.device:
+                buf = torch.empty(weight.numel(), 2, 2, dtype=torch.float32, device=weight.device)
+                cache['unit'] = buf
+            kernels.unit_wise_stats(y, g, weight, bias, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
+            self._op_results['_unit_tmp'] = buf
+            self._n_backward += 1
+            if self._context is not None:
+                self._context.queue_unit_inverse(self)
+
+    def finish_registered(self):
+        unit = self._op_results.get(OP_COV_UNIT_WISE)
+        beta = self._first_beta.pop('data', 1.0)
+        if unit is not None and unit.get('data') is not None and beta != 1.0:
+            unit['data'].mul_(beta)
+        self._first_beta = {}
+
+
+class BatchNorm(_NormOperation):
+    """BatchNorm1d: [n, f]; BatchNorm2d: [n, c, h, w] in any memory format."""
+
+
+class LayerNorm(_NormOperation):
+    """[n, *, normalized_shape]: every leading index is a sample, the normalized shape is flattened to the
+    features (asdl/operations/layernorm.py:20-42)."""
+
+    @staticmethod
+    def as_samples(module, tensor):
+        f = module.weight.numel()
+        return tensor.reshape(-1, f)
+
+
 EAGER_COST_FRACTION = 0.6
 
 
@@ -259,10 +346,13 @@ class DeferredInverses:
     and removes from ``module.<attr>.kron`` the inverse of any all-zero factor (which the reference never
     computes)."""
 
-    def __init__(self, chunks):
+    def __init__(self, chunks, context=None):
         self._chunks = chunks            # [(PendingInverses, [(module, kron), ...]), ...]
+        self._context = context
 
     def finish(self, attr):
+        if self._context is not None:
+            self._context.check_unit_flags()
         for pending, _ in self._chunks:
             pending.join()               # all waits first, then the flag reads
         for pending, targets in self._chunks:
@@ -283,6 +373,10 @@ def get_op_class(module):
         return Linear
     elif isinstance(module, nn.Conv2d):
         return Conv2d
+    elif isinstance(module, (nn.BatchNorm1d, nn.BatchNorm2d)):
+        return BatchNorm
+    elif isinstance(module, nn.LayerNorm):
+        return LayerNorm
     warnings.warn(f'Failed to lookup operations for Module {module}.')
     return None
 
@@ -293,6 +387,8 @@ class OperationContext:
         self._vectors = vectors
         self._pending_inverse = []
         self._inverse_chunks = []
+        self._pending_unit = []
+        self._unit_flags = []
         self.factor_stream = None
         self._eager_total = 0.0
         self._eager_done = False
@@ -315,6 +411,7 @@ class OperationContext:
         self._operations.clear()
         self._pending_inverse = []
         self._inverse_chunks = []
+        self._pending_unit = []
 
     def call_operations_in_forward(self, module, in_data, out_data):
         self.get_operation(module).forward_post_process(in_data, out_data)
@@ -375,6 +472,38 @@ class OperationContext:
             self._eager_done = True
             self._enqueue_pending()
 
+    def queue_unit_inverse(self, operation):
+        if operation not in self._pending_unit:
+            self._pending_unit.append(operation)
+
+    def _invert_units(self):
+        """Damped inverses of the queued unit-wise blocks (one small launch each); their singularity flags are
+        read together in check_unit_flags()."""
+        ops = self._pending_unit
+        self._pending_unit = []
+        for op in ops:
+            blocks = op._op_results.pop('_unit_tmp', None)
+            if blocks is None:
+                continue
+            store = op._op_results.setdefault(OP_COV_UNIT_WISE, {})
+            prev = store.get('inv')
+            reuse = prev is not None and prev.shape == blocks.shape
+            inv, flags = kernels.unit_wise_inv(blocks, op._damping, out=prev if reuse else None)
+            store['inv'] = inv
+            self._unit_flags.append((op._module, flags))
+
+    def check_unit_flags(self):
+        """torch.inverse raises for a singular block (asdl/operations/operation.py:317-320); here the flags of all
+        modules are read with one copy."""
+        pending = self._unit_flags
+        self._unit_flags = []
+        if not pending:
+            return
+        host = torch.stack([f for _, f in pending]).cpu().tolist()
+        for (module, _), (nonzero, bad) in zip(pending, host):
+            if bad != 0x7fffffff:
+                raise torch.linalg.LinAlgError(f'unit-wise block {bad - 1} of {module} + damping is singular')
+
     def _enqueue_pending(self):
         """Starts the batched inverse of every queued pair (side streams, worker threads) and places the
         output tensors in the result store; their flags are read by DeferredInverses.finish()."""
@@ -404,13 +533,16 @@ class OperationContext:
         enqueued: the result store receives the output tensors right away and the returned object's
         finish() must be called before they are used (it reads the zero / not-positive-definite flags)."""
         self._enqueue_pending()
+        self._invert_units()
         chunks = self._inverse_chunks
         self._inverse_chunks = []
         if not chunks:
+            self.check_unit_flags()
             return None
-        deferred = DeferredInverses(chunks)
+        deferred = DeferredInverses(chunks, self)
         if defer:
             return deferred
+        self.check_unit_flags()
         for pending, _ in chunks:
             pending.join()
         for pending, targets in chunks:
@@ -426,10 +558,13 @@ class OperationContext:
     def cov_symmatrix(self, module, pop=False):
         self.flush_inverses()       # no-op when the caller has already flushed (possibly deferred)
         cov_kron = self.get_result(module, OP_COV_KRON, pop=pop)
-        if cov_kron is None:
-            return None
-        kwargs = dict(kron_A=cov_kron.pop('A', None), kron_B=cov_kron.pop('B', None),
-                      kron_A_inv=cov_kron.pop('A_inv', None), kron_B_inv=cov_kron.pop('B_inv', None))
+        cov_unit = self.get_result(module, OP_COV_UNIT_WISE, pop=pop)
+        kwargs = {}
+        if cov_kron is not None:
+            kwargs = dict(kron_A=cov_kron.pop('A', None), kron_B=cov_kron.pop('B', None),
+                          kron_A_inv=cov_kron.pop('A_inv', None), kron_B_inv=cov_kron.pop('B_inv', None))
+        if cov_unit is not None and not all(v is None for v in cov_unit.values()):
+            kwargs['unit'] = UnitWise(data=cov_unit.pop('data', None), inv=cov_unit.pop('inv', None))
         if all(v is None for v in kwargs.values()):
             return None
         return SymMatrix(**kwargs)
@@ -445,6 +580,9 @@ class OperationContext:
             if matrix.kron.has_B:
                 operation.accumulate_result(matrix.kron.B, OP_COV_KRON, 'B')
                 operation._first_beta['B'] = first_beta
+        if matrix.has_unit and matrix.unit.has_data:
+            operation.accumulate_result(matrix.unit.data, OP_COV_UNIT_WISE, 'data')
+            operation._first_beta['data'] = first_beta
 
     def finish_registered(self):
         for operation in self._operations.values():

@@ -294,6 +294,76 @@ class Kron:
         return w
 
 
+class UnitWise:
+    """[f, 2, 2] blocks of a BatchNorm / LayerNorm module (asdl/symmatrix.py:617-719)."""
+
+    def __init__(self, data=None, inv=None):
+        self.data = data.contiguous() if isinstance(data, torch.Tensor) else data
+        self.inv = inv
+
+    def __add__(self, other):
+        if not other.has_data:
+            return self
+        return UnitWise(data=self.data.add(other.data) if self.has_data else other.data)
+
+    def __iadd__(self, other):
+        if not other.has_data:
+            return self
+        if self.has_data:
+            self.data.add_(other.data)
+        else:
+            self.data = other.data
+        return self
+
+    @property
+    def has_data(self):
+        return self.data is not None
+
+    @property
+    def has_inv(self):
+        return self.inv is not None
+
+    def mul_(self, value):
+        if self.has_data:
+            self.data.mul_(value)
+        return self
+
+    def trace(self):
+        return float(torch.diagonal(self.data, dim1=1, dim2=2).sum())
+
+    def update_inv(self, damping=_default_damping, replace=False):
+        """asdl/symmatrix.py:687-699: an all-zero tensor keeps its old inverse (none)."""
+        if not self.has_data:
+            raise ValueError('data do not exist.')
+        inv, flags = kernels.unit_wise_inv(self.data, float(damping))
+        nonzero, bad = flags.cpu().tolist()
+        if not nonzero:
+            return
+        if bad != 0x7fffffff:
+            raise torch.linalg.LinAlgError(f'unit-wise block {bad - 1} + damping is singular')
+        self.inv = inv
+        if replace:
+            self.data = None
+
+    def mvp(self, vec_weight, vec_bias, use_inv=False, inplace=False):
+        """asdl/symmatrix.py:701-719 for modules with one (weight, bias) pair per block."""
+        mat = self.inv if use_inv else self.data
+        if mat is None:
+            raise ValueError('inv does not exist.' if use_inv else 'data do not exist.')
+        if vec_bias is None or vec_weight.shape != vec_bias.shape or mat.ndim != 3 or mat.shape[1:] != (2, 2):
+            raise NotImplementedError('unit-wise blocks larger than 2 x 2 (Linear / Conv2d) are not on this path')
+        if not inplace:
+            vec_weight, vec_bias = vec_weight.clone(), vec_bias.clone()
+        w = vec_weight if vec_weight.is_contiguous() else vec_weight.contiguous()
+        b = vec_bias if vec_bias.is_contiguous() else vec_bias.contiguous()
+        kernels.unit_wise_mvp(mat, w.view(-1), b.view(-1))
+        if w is not vec_weight:
+            vec_weight.copy_(w)
+        if b is not vec_bias:
+            vec_bias.copy_(b)
+        return vec_weight, vec_bias
+
+
 class SymMatrix:
     def __init__(self, data=None, inv=None, kron=None, kfe=None, diag=None, unit=None,
                  kron_A=None, kron_B=None, kron_A_inv=None, kron_B_inv=None):
@@ -314,6 +384,11 @@ class SymMatrix:
                 v = getattr(self.kron, key)
                 if v is not None:
                     parts.append(f'kron.{key} {tuple(v.shape)}')
+        if self.has_unit:
+            for key in ('data', 'inv'):
+                v = getattr(self.unit, key)
+                if v is not None:
+                    parts.append(f'unit.{key} {tuple(v.shape)}')
         return 'SymMatrix(' + ', '.join(parts) + ')'
 
     @property
@@ -337,8 +412,8 @@ class SymMatrix:
         return self.unit is not None
 
     def _only_kron(self, what):
-        if self.has_data or self.has_kfe or self.has_diag or self.has_unit:
-            raise NotImplementedError(f'{what}: only the Kronecker-factored shape is on this path')
+        if self.has_data or self.has_kfe or self.has_diag:
+            raise NotImplementedError(f'{what}: only the Kronecker-factored and unit-wise shapes are on this path')
 
     def __iadd__(self, other):
         self._only_kron('__iadd__')
@@ -347,18 +422,27 @@ class SymMatrix:
                 self.kron += other.kron
             else:
                 self.kron = other.kron
+        if other.unit is not None:
+            if self.unit is not None:
+                self.unit += other.unit
+            else:
+                self.unit = other.unit
         return self
 
     def mul_(self, value):
         self._only_kron('mul_')
         if self.has_kron:
             self.kron.mul_(value)
+        if self.has_unit:
+            self.unit.mul_(value)
         return self
 
     def update_inv(self, damping=_default_damping, replace=False):
         self._only_kron('update_inv')
         if self.has_kron:
             self.kron.update_inv(damping, replace=replace)
+        if self.has_unit:
+            self.unit.update_inv(damping, replace=replace)
 
     def mvp(self, vectors=None, vec_weight=None, vec_bias=None, use_inv=False, inplace=False):
         raise NotImplementedError('SymMatrix.mvp with a full / layer-wise matrix is not on this path; '

@@ -114,6 +114,35 @@ int ak_chol_inv_batched(const float* const* A_list, float* const* out_list, int6
                         const float* lam, int lam_stride, const int* skip_flags, int skip_stride,
                         int* info, void* ws, size_t ws_bytes, ak_stream_t stream);
 
+/* ---- unit-wise blocks (BatchNorm / LayerNorm) ------------------------------------- */
+
+/* blocks[f] <- beta*blocks[f] + alpha * sum_n [[gw^2, gw*gb], [gw*gb, gb^2]] for f < F, blocks = [F, 2, 2] fp32,
+ * with gw[n,f] = sum_s (y[n,f,s] - bias[f]) / weight[f] * g[n,f,s] and gb[n,f] = sum_s g[n,f,s].
+ * y is the module's output, g the gradient with respect to it; both fp32 or bf16, addressed through element
+ * strides for (sample n, feature f, position s), so NCHW, channels-last and [rows, features] (S = 1) layouts
+ * are read in place.  Replaces _BatchNormNd.preprocess_in_data + cov_unit_wise
+ * (asdl/operations/batchnorm.py:11-21, 28-55, 95-108), LayerNorm.preprocess_in_data + cov_unit_wise
+ * (asdl/operations/layernorm.py:20-31, 75-84) and the .mul_(cov_scale) / accumulate of
+ * asdl/operations/operation.py:308-316. */
+size_t ak_unit_wise_ws_bytes(int64_t N, int64_t F, int64_t S);
+int ak_unit_wise_stats(const void* y, int y_dtype, int64_t ysn, int64_t ysf, int64_t yss,
+                       const void* g, int g_dtype, int64_t gsn, int64_t gsf, int64_t gss,
+                       const float* weight, const float* bias, int64_t N, int64_t F, int64_t S,
+                       float alpha, float beta, float* blocks,
+                       void* ws, size_t ws_bytes, ak_stream_t stream);
+
+/* inv[f] <- (blocks[f] + damping I)^-1 for the F 2x2 blocks.  flags: device int[2]; flags[0] = 1 when blocks has a
+ * non-zero entry (the reference skips the inverse of an all-zero tensor), flags[1] = 1-based index of the first
+ * singular block or 0x7fffffff.  Replaces UnitWise.update_inv (asdl/symmatrix.py:687-699) and the inverse of
+ * asdl/operations/operation.py:317-321. */
+int ak_unit_wise_inv(const float* blocks, int64_t F, float damping, float* inv, int* flags, ak_stream_t stream);
+
+/* [vec_weight[f], vec_bias[f]] <- mat[f] @ (scale * [vec_weight[f], vec_bias[f]]) in place, mat = [F, 2, 2].
+ * Replaces UnitWise.mvp for BatchNorm / LayerNorm (asdl/symmatrix.py:701-709, 716-719) and the grad_scale
+ * pre-multiply of asdl/precondition/natural_gradient.py:535-538. */
+int ak_unit_wise_mvp(const float* mat, int64_t F, float* vec_weight, float* vec_bias, float scale,
+                     ak_stream_t stream);
+
 /* ---- dense fp32 products ---------------------------------------------------------- */
 
 /* C <- alpha * op(A) op(B) + beta * C, fp32 MFMA, row-major; op = identity (0) or transpose (1);

@@ -21,6 +21,13 @@ reference checkout).  How each function is pinned (tests/test_oracle.py):
   cholesky_inv          (X + damping I) @ inv == I, fp64 torch.linalg.inv
   kron_mvp              (B^-1 kron A^-1) vec(G) identity  -- the reference has no
                         test that calls precondition(); pinned by mathematics
+  norm_cov_unit_wise    per-example gradients of (weight, bias) taken one sample at a
+                        time by autograd: block f == sum_n g_n g_n^T with
+                        g_n = (dL_n/dw_f, dL_n/db_f) (brute force), for BatchNorm1d/2d
+                        in eval mode and LayerNorm; golden default-K-FAC runs of a
+                        BatchNorm CNN written from the reference
+  unit_wise_inv / mvp   (block + damping I) @ inv == I per block; block-diagonal
+                        matrix-vector product against an explicit dense matrix
   power_iter            eigvalsh lambda_max (converged limit only)
   compute_power         fp64 eigh closed form (S + rI)^(-1/p), X^p (S + rI) == I;
                         golden trajectories written from the reference
@@ -37,6 +44,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 __all__ = [
+    'norm_restore_input', 'norm_cov_unit_wise', 'unit_wise_inv', 'unit_wise_mvp',
     'linear_cov_kron_A', 'linear_cov_kron_B', 'im2col_2d', 'conv_cov_kron_A', 'conv_cov_kron_B',
     'ema_accumulate', 'kron_damping', 'cholesky_inv', 'kron_update_inv', 'kron_mvp',
     'power_iter', 'mat_power', 'compute_power', 'shampoo_statistics', 'shampoo_precondition',
@@ -236,6 +244,52 @@ def _update_by_interval(step, interval, warmup=0):
     return step < warmup or (step - warmup) % interval == 0
 
 
+def norm_restore_input(module, out_data):
+    """Normalised input of a BatchNorm / LayerNorm module recovered from its output
+    (asdl/operations/batchnorm.py:11-21, asdl/operations/layernorm.py:20-31)."""
+    if isinstance(module, nn.LayerNorm):
+        x = (out_data - module.bias).div(module.weight)
+        k = len(module.weight.shape)
+        if k < x.ndim - 1:
+            x = x.flatten(end_dim=-k - 1)
+        return x
+    shape = (1, module.num_features) + (1,) * (out_data.ndim - 2)
+    return (out_data - module.bias.view(shape)).div(module.weight.view(shape))
+
+
+def norm_cov_unit_wise(module, out_data, out_grads):
+    """[f, 2, 2] blocks sum_n [[gw^2, gw gb], [gw gb, gb^2]] of the per-sample gradients of (weight, bias)
+    (asdl/operations/batchnorm.py:28-55, 95-108; asdl/operations/layernorm.py:33-84)."""
+    x = norm_restore_input(module, out_data)
+    if isinstance(module, nn.LayerNorm):
+        k = len(module.weight.shape)
+        g = out_grads.flatten(end_dim=-k - 1) if k < out_grads.ndim - 1 else out_grads
+        gw, gb = x.mul(g).flatten(start_dim=1), g.flatten(start_dim=1)
+    else:
+        gw, gb = x.mul(out_grads), out_grads
+        if gw.ndim > 2:
+            dims = tuple(range(2, gw.ndim))
+            gw, gb = gw.sum(dim=dims), gb.sum(dim=dims)
+    f = gw.shape[1]
+    ww, bb, wb = (gw ** 2).sum(0), (gb ** 2).sum(0), (gw * gb).sum(0)
+    return torch.vstack([ww, wb, wb, bb]).reshape(2, 2, f).transpose(0, 2).contiguous()
+
+
+def unit_wise_inv(blocks, damping):
+    """(blocks + damping I)^-1 per block; None for an all-zero tensor (asdl/symmatrix.py:687-699)."""
+    if torch.all(blocks == 0):
+        return None
+    eye = torch.eye(blocks.shape[-1], dtype=blocks.dtype)
+    return torch.inverse(blocks + damping * eye)
+
+
+def unit_wise_mvp(mat, vec_weight, vec_bias):
+    """asdl/symmatrix.py:701-709: [w, b][f] <- mat[f] @ [w, b][f]."""
+    v = torch.stack([vec_weight.flatten(), vec_bias.flatten()], dim=1).unsqueeze(2)
+    out = torch.matmul(mat, v).squeeze(2)
+    return out[:, 0].view_as(vec_weight), out[:, 1].view_as(vec_bias)
+
+
 class KfacOracle:
     """Restatement of KfacGradientMaker.forward_and_backward for Linear / Conv2d layers
     (BatchNorm / LayerNorm ignored, as in the reference's training script,
@@ -252,7 +306,7 @@ class KfacOracle:
 
     def __init__(self, model, data_size, damping=1e-7, ema_decay=-1, fisher_type='fisher_emp',
                  scale=1., grad_scale=1., seed=None, curvature_upd_interval=None,
-                 preconditioner_upd_interval=1, factor_dtype=None):
+                 preconditioner_upd_interval=1, factor_dtype=None, unit_wise_norm=False):
         self.model = model
         self.data_size = data_size
         self.damping = damping
@@ -268,10 +322,16 @@ class KfacOracle:
         self.layers = [(n, m) for n, m in model.named_modules()
                        if isinstance(m, (nn.Linear, nn.Conv2d))
                        and any(p.requires_grad for p in m.parameters())]
+        # unit_wise_norm: BatchNorm1d/2d and LayerNorm get the unit-wise shape, as in the default
+        # KfacGradientMaker (asdl/precondition/natural_gradient.py:886-889); else they are ignored
+        self.norm_layers = [(n, m) for n, m in model.named_modules()
+                            if unit_wise_norm and isinstance(m, (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm))]
         self.A = {}
         self.B = {}
         self.A_inv = {}
         self.B_inv = {}
+        self.unit = {}
+        self.unit_inv = {}
         self.last_mc_targets = None
 
     # -- schedule (prec_grad_maker.py:174-187)
@@ -308,8 +368,16 @@ class KfacOracle:
             if accumulate:
                 scale = scale * self.ema_decay      # the (1 - ema_decay) pre-scale is in ema_accumulate
             cov_scale = scale / N
-            saved_in, saved_g = {}, {}
+            saved_in, saved_g, saved_out = {}, {}, {}
             handles = []
+            for name, m in self.norm_layers:
+                # a hook on the output tensor, not a module backward hook: the latter forbids the in-place
+                # activations that commonly follow a normalisation layer
+                def norm_hook(mod, inp, out, name=name):
+                    saved_out[name] = out.detach()
+                    if out.requires_grad:
+                        out.register_hook(lambda g, name=name: saved_g.__setitem__(name, g.detach()))
+                handles.append(m.register_forward_hook(norm_hook))
             for name, m in self.layers:
                 handles.append(m.register_forward_hook(
                     lambda mod, inp, out, name=name: saved_in.__setitem__(name, inp[0].detach())))
@@ -345,6 +413,13 @@ class KfacOracle:
                     self.B[name] = ema_accumulate(self.B.get(name), B, self.ema_decay)
                 else:
                     self.A_inv[name], self.B_inv[name] = kron_update_inv(A, B, self.damping)
+            for name, m in self.norm_layers:
+                blocks = norm_cov_unit_wise(m, saved_out[name].float(), saved_g[name].float()) * cov_scale
+                if accumulate:
+                    self.unit[name] = ema_accumulate(self.unit.get(name), blocks, self.ema_decay)
+                else:
+                    # asdl/operations/operation.py:317-321: inverted in the hook, no all-zero test
+                    self.unit_inv[name] = torch.inverse(blocks + self.damping * torch.eye(2))
             if self.fisher_type != 'fisher_emp':
                 loss.backward()
             for p in model.parameters():
@@ -355,6 +430,20 @@ class KfacOracle:
             for name, _ in self.layers:
                 if name in self.A:
                     self.A_inv[name], self.B_inv[name] = kron_update_inv(self.A[name], self.B[name], self.damping)
+            for name, _ in self.norm_layers:
+                if name in self.unit:
+                    inv = unit_wise_inv(self.unit[name], self.damping)
+                    if inv is not None:
+                        self.unit_inv[name] = inv
+        for name, m in self.norm_layers:
+            if self.unit_inv.get(name) is None:
+                continue
+            if self.grad_scale != 1:
+                m.weight.grad.mul_(self.grad_scale)
+                m.bias.grad.mul_(self.grad_scale)
+            w, b = unit_wise_mvp(self.unit_inv[name], m.weight.grad, m.bias.grad)
+            m.weight.grad.copy_(w)
+            m.bias.grad.copy_(b)
         for name, m in self.layers:
             if self.A_inv.get(name) is None or self.B_inv.get(name) is None:
                 continue

@@ -81,8 +81,40 @@ def gemm(A, B, out=None, transA=False, transB=False, alpha=1.0, beta=0.0):
     return out
 
 
+def unit_wise_stats(y, g, weight, bias, out=None, alpha=1.0, beta=0.0):
+    f = weight.numel()
+    shape = (1, f) + (1,) * (y.ndim - 2)
+    x = (y.float() - bias.view(shape)) / weight.view(shape)
+    gw, gb = x * g.float(), g.float()
+    if gw.ndim > 2:
+        dims = tuple(range(2, gw.ndim))
+        gw, gb = gw.sum(dims), gb.sum(dims)
+    ww, bb, wb = (gw ** 2).sum(0), (gb ** 2).sum(0), (gw * gb).sum(0)
+    val = alpha * torch.stack([ww, wb, wb, bb], dim=1).reshape(f, 2, 2)
+    if out is None:
+        return val
+    out.copy_(val if beta == 0 else beta * out + val)
+    return out
+
+
+def unit_wise_inv(blocks, damping, out=None):
+    flags = torch.tensor([int(bool((blocks != 0).any())), 0x7fffffff], dtype=torch.int32)
+    inv = torch.inverse(blocks + damping * torch.eye(2))
+    if out is not None:
+        out.copy_(inv)
+        inv = out
+    return inv, flags
+
+
+def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
+    w, b = R.unit_wise_mvp(mat, vec_weight * scale, vec_bias * scale)
+    vec_weight.copy_(w)
+    vec_bias.copy_(b)
+    return vec_weight, vec_bias
+
+
 def install(monkeypatch):
     from asdl_amd import kernels
     for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'cholesky_inv',
-                 'kron_precond', 'gemm']:
+                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_mvp']:
         monkeypatch.setattr(kernels, name, globals()[name])

@@ -4,7 +4,8 @@ Run once as ``python tests/golden/make_golden.py`` with the reference checkout a
 /root/reference.  It covers only what closed forms cannot pin:
 
   * kfac_*.npz     multi-step KfacGradientMaker runs (orchestration, EMA state, MC sampling
-                   under a fixed seed) on the tiny MLP / CNN of the reference's test/conftest.py
+                   under a fixed seed) on the tiny MLP / CNN of the reference's test/conftest.py and
+                   on a CNN with BatchNorm / LayerNorm (unit-wise blocks of the default K-FAC)
   * shampoo_*.npz  multi-step ShampooGradientMaker run (in-place ridge accumulation,
                    power-iteration start vectors under a fixed seed)
   * power_*.npz    ComputePower outputs for well- and ill-conditioned inputs
@@ -42,6 +43,14 @@ def get_cnn2(in_dim=3, hid=6, out=5):
                          nn.Conv2d(hid, 8, 1, 2, 0, bias=False), nn.ReLU(), nn.Flatten(), nn.Linear(8 * 2 * 2, out))
 
 
+def get_cnn_bn(in_dim=3, hid=8, out=5):
+    # BatchNorm2d behind an in-place ReLU, BatchNorm1d and LayerNorm: unit-wise shapes of the default K-FAC
+    return nn.Sequential(nn.Conv2d(in_dim, hid, 3, 1, 1), nn.BatchNorm2d(hid), nn.ReLU(inplace=True),
+                         nn.Conv2d(hid, hid, 3, 2, 1), nn.BatchNorm2d(hid), nn.ReLU(), nn.Flatten(),
+                         nn.Linear(hid * 4 * 4, 12), nn.BatchNorm1d(12), nn.ReLU(), nn.Linear(12, 10),
+                         nn.LayerNorm(10), nn.Linear(10, out))
+
+
 def state_arrays(model, prefix):
     return {f'{prefix}{k}': v.detach().numpy().copy() for k, v in model.state_dict().items()}
 
@@ -72,6 +81,14 @@ def run_kfac(tag, model, xs, ts, fisher_type, ema_decay, damping, seed=None, cur
                 v = getattr(fisher.kron, key)
                 if v is not None:
                     out[f'step{step}/kron/{name}/{key}'] = v.detach().numpy().copy()
+        for name, m in model.named_modules():
+            fisher = getattr(m, 'fisher', None)
+            if fisher is None or fisher.unit is None:
+                continue
+            for key in ['data', 'inv']:
+                v = getattr(fisher.unit, key)
+                if v is not None:
+                    out[f'step{step}/unit/{name}/{key}'] = v.detach().numpy().copy()
         opt.step()
     np.savez_compressed(os.path.join(HERE, f'kfac_{tag}.npz'), **out)
     print('wrote', tag, len(out))
@@ -134,7 +151,23 @@ def run_power():
     print('wrote power', len(out))
 
 
+def main_bn():
+    torch.manual_seed(5)
+    bs = 8
+    xs = [torch.randn(bs, 3, 8, 8) for _ in range(3)]
+    ts = [torch.randint(5, (bs,)) for _ in range(3)]
+    torch.manual_seed(17)
+    run_kfac('cnnbn_fisher_emp_ema-1', get_cnn_bn(), xs, ts, 'fisher_emp', -1, 1e-2)
+    torch.manual_seed(18)
+    run_kfac('cnnbn_fisher_emp_ema0.4', get_cnn_bn(), xs, ts, 'fisher_emp', 0.4, 1e-2)
+    torch.manual_seed(19)
+    run_kfac('cnnbn_fisher_mc_ema-1', get_cnn_bn(), xs, ts, 'fisher_mc', -1, 1e-2, seed=3)
+
+
 def main():
+    if len(sys.argv) > 1 and sys.argv[1] == 'bn':
+        return main_bn()
+    main_bn()
     torch.manual_seed(0)
     bs = 8
     xs = [torch.randn(bs, 5) for _ in range(3)]

@@ -17,6 +17,14 @@ def get_cnn2(in_dim=3, hid=6, out=5):
                          nn.Conv2d(hid, 8, 1, 2, 0, bias=False), nn.ReLU(), nn.Flatten(), nn.Linear(8 * 2 * 2, out))
 
 
+def get_cnn_bn(in_dim=3, hid=8, out=5):
+    # BatchNorm2d behind an in-place ReLU, BatchNorm1d and LayerNorm: unit-wise shapes of the default K-FAC
+    return nn.Sequential(nn.Conv2d(in_dim, hid, 3, 1, 1), nn.BatchNorm2d(hid), nn.ReLU(inplace=True),
+                         nn.Conv2d(hid, hid, 3, 2, 1), nn.BatchNorm2d(hid), nn.ReLU(), nn.Flatten(),
+                         nn.Linear(hid * 4 * 4, 12), nn.BatchNorm1d(12), nn.ReLU(), nn.Linear(12, 10),
+                         nn.LayerNorm(10), nn.Linear(10, out))
+
+
 GOLDEN_KFAC = {
     # tag: (model factory, fisher_type, ema_decay, damping, seed, curvature interval, preconditioner interval)
     'mlp_fisher_emp_ema-1': (get_mlp, 'fisher_emp', -1, 1e-2, None, None, 1),
@@ -27,6 +35,9 @@ GOLDEN_KFAC = {
     'cnn_fisher_mc_ema-1': (get_cnn, 'fisher_mc', -1, 1e-2, 1, None, 1),
     'cnn2_fisher_emp_ema0.5_int2': (get_cnn2, 'fisher_emp', 0.5, 1e-3, None, 1, 2),
     'cnn2_fisher_emp_ema-1_int2': (get_cnn2, 'fisher_emp', -1, 1e-3, None, None, 2),
+    'cnnbn_fisher_emp_ema-1': (get_cnn_bn, 'fisher_emp', -1, 1e-2, None, None, 1),
+    'cnnbn_fisher_emp_ema0.4': (get_cnn_bn, 'fisher_emp', 0.4, 1e-2, None, None, 1),
+    'cnnbn_fisher_mc_ema-1': (get_cnn_bn, 'fisher_mc', -1, 1e-2, 3, None, 1),
 }
 
 GOLDEN_SHAMPOO = {

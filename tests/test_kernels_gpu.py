@@ -8,6 +8,7 @@ an fp64 inverse; preconditioned gradients 1e-3.
 """
 import pytest
 import torch
+import torch.nn as nn
 
 from oracle import cpu_ref as R
 
@@ -343,3 +344,56 @@ def test_kron_precond_matches_oracle(K, dB, dA, bias):
         G4 = G.view(dB, dA // 9, 3, 3).contiguous().cuda()
         K.kron_precond(Bi.cuda(), Ai.cuda(), G4, None, grad_scale=0.5)
         assert relerr(G4.view(dB, dA), 0.5 * rw) < 1e-5
+
+
+# ------------------------------------------------------------------ unit-wise blocks (BatchNorm / LayerNorm)
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('kind,shape', [('bn2d', (6, 16, 7, 5)), ('bn2d_cl', (6, 16, 7, 5)), ('bn2d', (3, 70, 14, 14)),
+                                        ('bn2d_cl', (3, 70, 14, 14)), ('bn2d_cl', (2, 8, 33, 40)), ('bn1d', (300, 12)),
+                                        ('ln', (5, 37, 48)), ('ln', (200, 768))])
+def test_unit_wise_stats_matches_oracle(K, dtype, kind, shape):
+    torch.manual_seed(len(shape) + shape[1])
+    if kind.startswith('bn2d'):
+        m = nn.BatchNorm2d(shape[1])
+    elif kind == 'bn1d':
+        m = nn.BatchNorm1d(shape[1])
+    else:
+        m = nn.LayerNorm(shape[-1])
+    with torch.no_grad():
+        m.weight.uniform_(0.5, 1.5)
+        m.bias.uniform_(-0.5, 0.5)
+    y = _inputs(shape, dtype, seed=1)
+    g = _inputs(shape, dtype, seed=2) * 0.1
+    ref = R.norm_cov_unit_wise(m.double(), y.float().double(), g.float().double())
+    yg, gg = y.cuda(), g.cuda()
+    if kind == 'bn2d_cl':
+        yg = yg.contiguous(memory_format=torch.channels_last)
+        gg = gg.contiguous(memory_format=torch.channels_last)
+    if kind == 'ln':
+        yg, gg = yg.reshape(-1, shape[-1]), gg.reshape(-1, shape[-1])
+    print(f'unit_wise_stats {kind} {shape} {dtype}', flush=True)
+    w, b = m.weight.detach().float().cuda(), m.bias.detach().float().cuda()
+    out = K.unit_wise_stats(yg, gg, w, b, alpha=0.25)
+    torch.cuda.synchronize()
+    assert relerr(out, 0.25 * ref) < 1e-5
+    # accumulate form
+    out2 = K.unit_wise_stats(yg, gg, w, b, out=out.clone(), alpha=0.5, beta=2.0)
+    assert relerr(out2, 1.0 * ref) < 1e-5
+
+
+def test_unit_wise_inv_and_mvp_match_oracle(K):
+    torch.manual_seed(3)
+    v = torch.randn(1000, 2, 3)
+    blocks = v @ v.transpose(1, 2)
+    inv, flags = K.unit_wise_inv(blocks.cuda(), 0.05)
+    ref = R.unit_wise_inv(blocks.double(), 0.05)
+    assert relerr(inv, ref) < 1e-5
+    assert flags.cpu().tolist() == [1, 0x7fffffff]
+    _, flags0 = K.unit_wise_inv(torch.zeros(5, 2, 2).cuda(), 0.05)
+    assert flags0.cpu().tolist()[0] == 0
+    _, flags_bad = K.unit_wise_inv(torch.zeros(5, 2, 2).cuda(), 0.0)
+    assert flags_bad.cpu().tolist()[1] == 1                           # first singular block, 1-based
+    w, b = torch.randn(1000), torch.randn(1000)
+    rw, rb = R.unit_wise_mvp(ref, w.double(), b.double())
+    gw, gb = K.unit_wise_mvp(inv, w.cuda(), b.cuda(), scale=2.0)
+    assert relerr(gw, 2 * rw) < 1e-5 and relerr(gb, 2 * rb) < 1e-5

@@ -17,6 +17,16 @@ def relerr(a, b):
     return float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-300))
 
 
+def grad_close(got, ref, tol):
+    """Relative error below tol, or both essentially zero (a bias in front of a normalisation layer has an
+    exactly zero gradient; what is left of it in fp32 is rounding noise)."""
+    ref = ref.double()
+    got = got.detach().double().cpu()
+    if float(ref.norm()) < 1e-6:
+        return float((got - ref).norm()) < 1e-5
+    return float((got - ref).norm() / ref.norm()) < tol
+
+
 # ----------------------------------------------------------------- factors
 def test_linear_factors_closed_form():
     torch.manual_seed(0)
@@ -231,7 +241,8 @@ def test_kfac_oracle_matches_reference_golden(tag):
     n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
     x0 = torch.from_numpy(z['step0/x'])
     orc = R.KfacOracle(model, data_size=x0.shape[0], damping=damping, ema_decay=ema, fisher_type=fisher_type,
-                       seed=seed, curvature_upd_interval=ci, preconditioner_upd_interval=pi)
+                       seed=seed, curvature_upd_interval=ci, preconditioner_upd_interval=pi,
+                       unit_wise_norm=True)        # the fixtures come from the default KfacGradientMaker
     opt = torch.optim.SGD(model.parameters(), lr=0.05)
     for step in range(n_steps):
         opt.zero_grad(set_to_none=True)
@@ -241,7 +252,7 @@ def test_kfac_oracle_matches_reference_golden(tag):
         torch.testing.assert_close(loss, torch.from_numpy(z[f'step{step}/loss']), rtol=1e-5, atol=1e-6)
         for name, p in model.named_parameters():
             ref = torch.from_numpy(z[f'step{step}/grad/{name}'])
-            assert relerr(p.grad, ref) < 2e-4, (tag, step, name, relerr(p.grad, ref))
+            assert grad_close(p.grad, ref, 2e-4), (tag, step, name, relerr(p.grad, ref))
         for key in z.files:
             if not key.startswith(f'step{step}/kron/'):
                 continue
@@ -249,6 +260,13 @@ def test_kfac_oracle_matches_reference_golden(tag):
             got = getattr(orc, which).get(mname)
             assert got is not None, key
             assert relerr(got, torch.from_numpy(z[key])) < 2e-4, (tag, key)
+        for key in z.files:
+            if not key.startswith(f'step{step}/unit/'):
+                continue
+            _, _, mname, which = key.split('/')
+            got = (orc.unit if which == 'data' else orc.unit_inv).get(mname)
+            assert got is not None, key
+            assert relerr(got, torch.from_numpy(z[key])) < 2e-4, (tag, key, relerr(got, torch.from_numpy(z[key])))
         opt.step()
 
 
@@ -275,3 +293,67 @@ def test_shampoo_oracle_matches_reference_golden(tag):
         for name, p in model.named_parameters():
             assert relerr(p.grad, torch.from_numpy(z[f'step{step}/grad/{name}'])) < 1e-4, (tag, step, name)
         opt.step()
+
+
+# ------------------------------------------------------------------ unit-wise blocks (BatchNorm / LayerNorm)
+def _per_sample_blocks(module, x, G, sample_of_row=None):
+    """Brute force: gradient of sum(y_n * G_n) with respect to (weight, bias), one sample at a time by autograd."""
+    y = module(x)
+    n = x.shape[0]
+    f = module.weight.numel()
+    blocks = torch.zeros(f, 2, 2, dtype=torch.float64)
+    rows = y.reshape(n, -1) if sample_of_row is None else None
+    if sample_of_row is None:
+        groups = [[i] for i in range(n)]
+        yr, Gr = y, G
+    else:
+        yr, Gr = y.reshape(-1, f), G.reshape(-1, f)
+        groups = [[i] for i in range(yr.shape[0])]
+    for idx in groups:
+        gw, gb = torch.autograd.grad((yr[idx] * Gr[idx]).sum(), [module.weight, module.bias], retain_graph=True)
+        v = torch.stack([gw.flatten().double(), gb.flatten().double()], dim=1)      # [f, 2]
+        blocks += v.unsqueeze(2) * v.unsqueeze(1)
+    return blocks, y.detach()
+
+
+@pytest.mark.parametrize('kind', ['bn1d', 'bn2d', 'ln', 'ln_seq'])
+def test_norm_cov_unit_wise_matches_per_sample_autograd(kind):
+    torch.manual_seed(11)
+    if kind == 'bn1d':
+        m, x = nn.BatchNorm1d(5), torch.randn(7, 5)
+    elif kind == 'bn2d':
+        m, x = nn.BatchNorm2d(4), torch.randn(6, 4, 3, 5)
+    elif kind == 'ln':
+        m, x = nn.LayerNorm(6), torch.randn(9, 6)
+    else:
+        m, x = nn.LayerNorm(6), torch.randn(3, 4, 6)
+    with torch.no_grad():
+        m.weight.uniform_(0.5, 1.5)
+        m.bias.uniform_(-0.5, 0.5)
+    if isinstance(m, (nn.BatchNorm1d, nn.BatchNorm2d)):
+        m.running_mean.normal_()
+        m.running_var.uniform_(0.5, 2.0)
+        m.eval()                          # samples are independent, so per-sample gradients are well defined
+    x = x.double()
+    m = m.double()
+    G = torch.randn_like(x)
+    ref, y = _per_sample_blocks(m, x, G, sample_of_row=True if kind.startswith('ln') else None)
+    got = R.norm_cov_unit_wise(m, y, G)
+    assert got.shape == ref.shape
+    assert relerr(got, ref) < 1e-10
+    assert torch.equal(got[:, 0, 1], got[:, 1, 0])
+
+
+def test_unit_wise_inv_and_mvp():
+    torch.manual_seed(12)
+    v = torch.randn(9, 2, 3, dtype=torch.float64)
+    blocks = v @ v.transpose(1, 2)
+    inv = R.unit_wise_inv(blocks, 0.1)
+    eye = torch.eye(2, dtype=torch.float64)
+    assert relerr((blocks + 0.1 * eye) @ inv, eye.expand(9, 2, 2)) < 1e-12
+    assert R.unit_wise_inv(torch.zeros(3, 2, 2), 0.1) is None
+    w, b = torch.randn(9, dtype=torch.float64), torch.randn(9, dtype=torch.float64)
+    dense = torch.block_diag(*inv)                                  # [18, 18], (w_f, b_f) interleaved
+    ref = dense @ torch.stack([w, b], dim=1).flatten()
+    mw, mb = R.unit_wise_mvp(inv, w, b)
+    assert relerr(torch.stack([mw, mb], dim=1).flatten(), ref) < 1e-12
