@@ -82,6 +82,64 @@ static __global__ __launch_bounds__(256) void uw_cols_kernel(UwParams p) {
   }
 }
 
+// feature-contiguous, 16-byte loads: grid (ceil(F/FT), N, chunks of positions), 256 threads = 8 feature groups of VEC
+// consecutive features x 32 position lanes.  part[((n * CH + ch) * F + f) * 2 + {0, 1}] = partial (gw, gb).
+template <typename T>
+static __global__ __launch_bounds__(256) void uw_cols_vec_kernel(UwParams p, int64_t pos_per_chunk) {
+  constexpr int VEC = 16 / sizeof(T), FT = 8 * VEC;
+  __shared__ float red[2][32][FT + 1];
+  const int fg = threadIdx.x & 7, sl = threadIdx.x >> 3;
+  const int64_t f0 = static_cast<int64_t>(blockIdx.x) * FT + fg * VEC, n = blockIdx.y, ch = blockIdx.z;
+  const int64_t s_begin = ch * pos_per_chunk;
+  const int64_t s_end = s_begin + pos_per_chunk < p.S ? s_begin + pos_per_chunk : p.S;
+  float sw[VEC], sb[VEC], wf[VEC], bf[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) { sw[e] = sb[e] = 0.f; wf[e] = 1.f; bf[e] = 0.f; }
+  const bool live = f0 < p.F;               // F is a multiple of VEC
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) { wf[e] = 1.f / p.w[f0 + e]; bf[e] = p.b[f0 + e]; }
+    const T* yp = static_cast<const T*>(p.y) + n * p.ysn + f0;
+    const T* gp = static_cast<const T*>(p.g) + n * p.gsn + f0;
+    for (int64_t s = s_begin + sl; s < s_end; s += 32) {
+      const uint4 yv = *reinterpret_cast<const uint4*>(yp + s * p.yss);
+      const uint4 gv = *reinterpret_cast<const uint4*>(gp + s * p.gss);
+      const uint32_t yw[4] = {yv.x, yv.y, yv.z, yv.w}, gw4[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float ye, ge;
+        if (sizeof(T) == 2) {
+          const uint32_t ys = (e & 1) ? (yw[e >> 1] & 0xffff0000u) : (yw[e >> 1] << 16);
+          const uint32_t gs = (e & 1) ? (gw4[e >> 1] & 0xffff0000u) : (gw4[e >> 1] << 16);
+          ye = __builtin_bit_cast(float, ys);
+          ge = __builtin_bit_cast(float, gs);
+        } else {
+          ye = __builtin_bit_cast(float, yw[e]);
+          ge = __builtin_bit_cast(float, gw4[e]);
+        }
+        sw[e] += (ye - bf[e]) * wf[e] * ge;
+        sb[e] += ge;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    red[0][sl][fg * VEC + e] = sw[e];
+    red[1][sl][fg * VEC + e] = sb[e];
+  }
+  __syncthreads();
+  if (threadIdx.x < 2 * FT) {
+    const int which = threadIdx.x / FT, fl = threadIdx.x % FT;
+    const int64_t f = static_cast<int64_t>(blockIdx.x) * FT + fl;
+    if (f < p.F) {
+      float acc = 0.f;
+#pragma unroll
+      for (int l = 0; l < 32; ++l) acc += red[which][l][fl];
+      p.part[((n * gridDim.z + ch) * p.F + f) * 2 + which] = acc;
+    }
+  }
+}
+
 // feature-contiguous, one position (LayerNorm rows, BatchNorm1d): grid (ceil(F/256), chunks); the three product
 // sums of a chunk of samples
 static __global__ __launch_bounds__(256) void uw_cols_single_kernel(UwParams p) {
@@ -104,31 +162,48 @@ static __global__ __launch_bounds__(256) void uw_cols_single_kernel(UwParams p) 
   dst[0] = ww; dst[1] = wb; dst[2] = bb;
 }
 
-// blocks[f] = beta*blocks[f] + alpha * sum over the partial rows; `width` 2: per-sample (gw, gb), 3: product sums
-static __global__ __launch_bounds__(256) void uw_finalize_kernel(const float* __restrict__ part, int64_t rows, int64_t F,
-                                                                 int width, float alpha, float beta,
-                                                                 float* __restrict__ blocks) {
-  const int64_t f = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (f >= F) return;
+// blocks[f] = beta*blocks[f] + alpha * sum over the partial rows; `width` 2: per-sample (gw, gb) in `chunks` pieces,
+// 3: product sums.  grid ceil(F/64), 1024 threads = 64 features x 16 row lanes; fixed summation order.
+static __global__ __launch_bounds__(1024) void uw_finalize_kernel(const float* __restrict__ part, int64_t rows, int64_t F,
+                                                                  int width, int chunks, float alpha, float beta,
+                                                                  float* __restrict__ blocks) {
+  __shared__ float red[3][16][65];
+  const int fl = threadIdx.x & 63, lane = threadIdx.x >> 6;
+  const int64_t f = static_cast<int64_t>(blockIdx.x) * 64 + fl;
   float ww = 0.f, wb = 0.f, bb = 0.f;
-  if (width == 2) {
-    for (int64_t n = 0; n < rows; ++n) {
-      const float gw = part[(n * F + f) * 2], gv = part[(n * F + f) * 2 + 1];
-      ww += gw * gw;
-      wb += gw * gv;
-      bb += gv * gv;
-    }
-  } else {
-    for (int64_t n = 0; n < rows; ++n) {
-      ww += part[(n * F + f) * 3];
-      wb += part[(n * F + f) * 3 + 1];
-      bb += part[(n * F + f) * 3 + 2];
+  if (f < F) {
+    if (width == 2) {
+      for (int64_t n = lane; n < rows; n += 16) {
+        float gw = 0.f, gv = 0.f;
+        for (int c = 0; c < chunks; ++c) {          // per-sample sums first: the positions were split over chunks
+          gw += part[((n * chunks + c) * F + f) * 2];
+          gv += part[((n * chunks + c) * F + f) * 2 + 1];
+        }
+        ww += gw * gw;
+        wb += gw * gv;
+        bb += gv * gv;
+      }
+    } else {
+      for (int64_t n = lane; n < rows; n += 16) {
+        ww += part[(n * F + f) * 3];
+        wb += part[(n * F + f) * 3 + 1];
+        bb += part[(n * F + f) * 3 + 2];
+      }
     }
   }
-  float* dst = blocks + f * 4;
-  float o0 = alpha * ww, o1 = alpha * wb, o3 = alpha * bb;
-  if (beta != 0.f) { o0 += beta * dst[0]; o1 += beta * dst[1]; o3 += beta * dst[3]; }
-  dst[0] = o0; dst[1] = o1; dst[2] = o1; dst[3] = o3;
+  red[0][lane][fl] = ww;
+  red[1][lane][fl] = wb;
+  red[2][lane][fl] = bb;
+  __syncthreads();
+  if (lane == 0 && f < F) {
+    ww = wb = bb = 0.f;
+#pragma unroll
+    for (int l = 0; l < 16; ++l) { ww += red[0][l][fl]; wb += red[1][l][fl]; bb += red[2][l][fl]; }
+    float* dst = blocks + f * 4;
+    float o0 = alpha * ww, o1 = alpha * wb, o3 = alpha * bb;
+    if (beta != 0.f) { o0 += beta * dst[0]; o1 += beta * dst[1]; o3 += beta * dst[3]; }
+    dst[0] = o0; dst[1] = o1; dst[2] = o1; dst[3] = o3;
+  }
 }
 
 // inv[f] = (blocks[f] + damping I)^-1; info = 1-based index of the first singular block (0: none)
@@ -170,12 +245,23 @@ static __global__ __launch_bounds__(256) void uw_mvp_kernel(const float* __restr
 
 constexpr int64_t kUwChunkRows = 64;
 
+// Chunks of positions per (sample, feature tile) for the vector kernel: enough work groups to fill the device.
+static int uw_chunks(int64_t N, int64_t F, int64_t S, int ft) {
+  const int64_t tiles = N * ((F + ft - 1) / ft);
+  int64_t ch = (2048 + tiles - 1) / tiles;
+  const int64_t max_ch = (S + 127) / 128;         // at least 128 positions per chunk
+  if (ch > max_ch) ch = max_ch;
+  if (ch < 1) ch = 1;
+  if (ch > 64) ch = 64;
+  return static_cast<int>(ch);
+}
+
 }  // namespace ak
 
 extern "C" size_t ak_unit_wise_ws_bytes(int64_t N, int64_t F, int64_t S) {
   if (N <= 0 || F <= 0 || S <= 0) return 0;
   if (S == 1) return static_cast<size_t>((N + ak::kUwChunkRows - 1) / ak::kUwChunkRows) * F * 3 * sizeof(float);
-  return static_cast<size_t>(N) * F * 2 * sizeof(float);
+  return static_cast<size_t>(N) * F * 2 * sizeof(float) * ak::uw_chunks(N, F, S, 32);    // upper bound over both layouts
 }
 
 extern "C" int ak_unit_wise_stats(const void* y, int y_dtype, int64_t ysn, int64_t ysf, int64_t yss, const void* g,
@@ -197,7 +283,7 @@ extern "C" int ak_unit_wise_stats(const void* y, int y_dtype, int64_t ysn, int64
   p.part = static_cast<float*>(ws);
   p.rows_per_chunk = kUwChunkRows;
   int64_t rows;
-  int width;
+  int width, chunks = 1;
   if (S == 1) {
     rows = (N + kUwChunkRows - 1) / kUwChunkRows;
     width = 3;
@@ -207,16 +293,27 @@ extern "C" int ak_unit_wise_stats(const void* y, int y_dtype, int64_t ysn, int64
   } else {
     rows = N;
     width = 2;
+    const int vec = y_dtype == AK_BF16 ? 8 : 4;
+    const bool vec_ok = ysf == 1 && gsf == 1 && y_dtype == g_dtype && F % vec == 0 && ysn % vec == 0 && gsn % vec == 0 &&
+                        yss % vec == 0 && gss % vec == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+                        (reinterpret_cast<uintptr_t>(g) & 15) == 0;
     if (yss == 1 && gss == 1) {
       if (F > 0x7fffffff) return AK_ERR_UNSUPPORTED;
       hipLaunchKernelGGL(uw_rows_kernel, dim3(static_cast<unsigned>(F), static_cast<unsigned>(N)), dim3(64), 0, s, p);
+    } else if (vec_ok) {
+      const int ft = 8 * vec;
+      chunks = uw_chunks(N, F, S, ft);
+      const int64_t per = (S + chunks - 1) / chunks;
+      dim3 grid(static_cast<unsigned>((F + ft - 1) / ft), static_cast<unsigned>(N), static_cast<unsigned>(chunks));
+      if (y_dtype == AK_BF16) hipLaunchKernelGGL(uw_cols_vec_kernel<uint16_t>, grid, dim3(256), 0, s, p, per);
+      else hipLaunchKernelGGL(uw_cols_vec_kernel<float>, grid, dim3(256), 0, s, p, per);
     } else {
       hipLaunchKernelGGL(uw_cols_kernel, dim3(static_cast<unsigned>((F + 63) / 64), static_cast<unsigned>(N)), dim3(256),
                          0, s, p);
     }
   }
-  hipLaunchKernelGGL(uw_finalize_kernel, dim3(static_cast<unsigned>((F + 255) / 256)), dim3(256), 0, s, p.part, rows, F,
-                     width, alpha, beta, blocks);
+  hipLaunchKernelGGL(uw_finalize_kernel, dim3(static_cast<unsigned>((F + 63) / 64)), dim3(1024), 0, s, p.part, rows, F,
+                     width, chunks, alpha, beta, blocks);
   return check_launch();
 }
 

@@ -35,6 +35,9 @@ def parse():
     ap.add_argument('--damping', type=float, default=1e-3)
     ap.add_argument('--memory-format', default='channels_last', choices=['channels_last', 'contiguous'],
                     help='layout of activations and conv weights; the K-FAC step is the same either way')
+    ap.add_argument('--with-batchnorm', action='store_true',
+                    help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
+                         '(the headline configuration ignores them, as the reference training script does)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-batch', type=int, default=16,
                     help='batch of the CPU baseline sample (its time is scaled to the full batch)')
@@ -108,7 +111,8 @@ def main():
         model = model.to(memory_format=torch.channels_last)
         x = x.contiguous(memory_format=torch.channels_last)
     t = torch.randint(0, 1000, (bs,)).to(dev)
-    config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=[nn.BatchNorm2d])
+    ignore = [] if args.with_batchnorm else [nn.BatchNorm2d]
+    config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=ignore)
     gm = KfacGradientMaker(model, config, fisher_type=args.fisher)
     opt = torch.optim.SGD(model.parameters(), lr=1e-4)
 
@@ -152,7 +156,7 @@ def main():
         'config': {'workload': f'K-FAC step (factors + pi-damped Cholesky inverses + precondition every step, '
                                f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
-                               f'BatchNorm ignored, {args.memory_format} activations and weights',
+                               f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights',
                    'batch': bs},
     }
     if sink:
