@@ -310,6 +310,37 @@ def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
     return vec_weight, vec_bias
 
 
+# ------------------------------------------------------------------------------ saved factors
+def tril_pack(mat):
+    """1-D lower triangle (row direction) of a float32 square matrix with contiguous rows."""
+    _require_gpu(mat)
+    if mat.ndim != 2:
+        raise ValueError(f'mat.ndim has to be 2. Got {mat.ndim}.')
+    if mat.shape[0] != mat.shape[1] or mat.dtype != torch.float32 or mat.stride(1) != 1:
+        raise ValueError('mat has to be a square float32 matrix with contiguous rows')
+    d = mat.shape[0]
+    out = torch.empty(d * (d + 1) // 2, dtype=torch.float32, device=mat.device)
+    rc = _lib.load().ak_tril_pack(ctypes.c_void_p(mat.data_ptr()), d, mat.stride(0), ctypes.c_void_p(out.data_ptr()),
+                                  _stream())
+    _lib.check(rc, 'ak_tril_pack')
+    return out
+
+
+def tril_unpack(tril, n_cols):
+    """Full symmetric [n_cols, n_cols] matrix from its packed lower triangle."""
+    _require_gpu(tril)
+    if tril.ndim != 1:
+        raise ValueError(f'tril.ndim has to be 1. Got {tril.ndim}.')
+    if tril.dtype != torch.float32 or tril.numel() != n_cols * (n_cols + 1) // 2:
+        raise ValueError('tril has to hold n_cols*(n_cols+1)/2 float32 values')
+    tril = tril.contiguous()
+    out = torch.empty(n_cols, n_cols, dtype=torch.float32, device=tril.device)
+    rc = _lib.load().ak_tril_unpack(ctypes.c_void_p(tril.data_ptr()), n_cols, ctypes.c_void_p(out.data_ptr()), n_cols,
+                                    _stream())
+    _lib.check(rc, 'ak_tril_unpack')
+    return out
+
+
 # ------------------------------------------------------------------------------ damping / inverse
 def kron_damping(A_list, B_list, damping, eps=1e-7):
     """Returns (lam [batch, 2] float32, nonzero [batch, 2] int32), both on the device."""

@@ -5,16 +5,63 @@ the arithmetic runs in the HIP kernels.  Only the Kronecker-factored shape is on
 full / layer-wise / KFE / unit-wise / diagonal containers are accepted as opaque attributes but
 have no kernels here.
 """
+import os
 from collections import defaultdict
 
+import numpy as np
 import torch
 from torch import Tensor
 
 from . import kernels
 
-__all__ = ['SymMatrix', 'Kron', 'batched_update_inv', 'PendingInverses']
+__all__ = ['SymMatrix', 'Kron', 'UnitWise', 'batched_update_inv', 'PendingInverses', 'matrix_to_tril', 'tril_to_matrix',
+           'get_n_cols_by_tril']
 
 _default_damping = 1e-5
+
+
+def matrix_to_tril(mat: Tensor):
+    """Lower triangle of a square matrix as a 1-D tensor, row direction: [[1,x,x],[2,3,x],[4,5,6]] ->
+    [1,2,3,4,5,6] (asdl/symmatrix.py:25-38).  The matrix has to be on the GPU."""
+    if mat.ndim != 2:
+        raise ValueError(f'mat.ndim has to be 2. Got {mat.ndim}.')
+    if mat.dtype != torch.float32 or mat.stride(1) != 1:
+        mat = mat.float().contiguous()
+    return kernels.tril_pack(mat)
+
+
+def get_n_cols_by_tril(tril: Tensor):
+    """n with n(n+1)/2 == tril.numel() (asdl/symmatrix.py:57-67)."""
+    if tril.ndim != 1:
+        raise ValueError(f'tril.ndim has to be 1. Got {tril.ndim}.')
+    return int(np.sqrt(2 * tril.numel() + 0.25) - 0.5)
+
+
+def tril_to_matrix(tril: Tensor):
+    """Full symmetric matrix of a packed lower triangle (asdl/symmatrix.py:41-54).  On the GPU."""
+    if tril.ndim != 1:
+        raise ValueError(f'tril.ndim has to be 1. Got {tril.ndim}.')
+    n_cols = get_n_cols_by_tril(tril)
+    if n_cols * (n_cols + 1) // 2 != tril.numel():
+        raise ValueError(f'{tril.numel()} values are not the lower triangle of a square matrix.')
+    return kernels.tril_unpack(tril.float(), n_cols)
+
+
+def _save_as_numpy(path, tensor):
+    """float32 .npy file, directories created on the way (asdl/symmatrix.py:74-78)."""
+    dirname = os.path.dirname(path)
+    if dirname and not os.path.isdir(dirname):
+        os.makedirs(dirname)
+    np.save(path, tensor.detach().cpu().numpy().astype('float32'))
+
+
+def _load_from_numpy(path, device=None):
+    """The matrices of this build live on the GPU: ``device`` None means the current one, a CPU device is an
+    error rather than a silent host path (the reference defaults to 'cpu', asdl/symmatrix.py:81-83)."""
+    device = torch.device('cuda' if device is None else device)
+    if device.type != 'cuda':
+        raise RuntimeError(f'factors are loaded onto a GPU in this build, got device {device}')
+    return torch.from_numpy(np.load(path)).to(device)
 
 
 _side_stream_cache = {}
@@ -294,6 +341,27 @@ class Kron:
         return w
 
 
+    def save(self, root, relative_dir):
+        """Writes <root>/<relative_dir>/kron/{A,B}_tril.npy and returns their relative paths under the keys
+        'A_tril' / 'B_tril' (asdl/symmatrix.py:471-485)."""
+        relative_paths = {}
+        for name in ['A', 'B']:
+            mat = getattr(self, name, None)
+            if mat is None:
+                continue
+            tril_name = f'{name}_tril'
+            relative_path = os.path.join(relative_dir, 'kron', f'{tril_name}.npy')
+            _save_as_numpy(os.path.join(root, relative_path), matrix_to_tril(mat))
+            relative_paths[tril_name] = relative_path
+        return relative_paths
+
+    def load(self, A_path, B_path, device=None):
+        """asdl/symmatrix.py:487-491."""
+        self.A = tril_to_matrix(_load_from_numpy(A_path, device))
+        self.B = tril_to_matrix(_load_from_numpy(B_path, device))
+        self._A_dim = self._B_dim = None
+
+
 class UnitWise:
     """[f, 2, 2] blocks of a BatchNorm / LayerNorm module (asdl/symmatrix.py:617-719)."""
 
@@ -330,6 +398,17 @@ class UnitWise:
 
     def trace(self):
         return float(torch.diagonal(self.data, dim1=1, dim2=2).sum())
+
+    def save(self, root, relative_dir):
+        """Writes the [f, 2, 2] blocks whole to <root>/<relative_dir>/unit_wise.npy (asdl/symmatrix.py:672-676)."""
+        relative_path = os.path.join(relative_dir, 'unit_wise.npy')
+        _save_as_numpy(os.path.join(root, relative_path), self.data)
+        return relative_path
+
+    def load(self, path=None, device=None):
+        """asdl/symmatrix.py:678-680."""
+        if path:
+            self.data = _load_from_numpy(path, device).contiguous()
 
     def update_inv(self, damping=_default_damping, replace=False):
         """asdl/symmatrix.py:687-699: an all-zero tensor keeps its old inverse (none)."""
@@ -443,6 +522,38 @@ class SymMatrix:
             self.kron.update_inv(damping, replace=replace)
         if self.has_unit:
             self.unit.update_inv(damping, replace=replace)
+
+    def save(self, root, relative_dir):
+        """Saves what the matrix holds below <root>/<relative_dir> and returns the relative paths, keyed as in
+        asdl/symmatrix.py:226-244: 'tril' (full matrix, packed lower triangle), 'kron' ({'A_tril', 'B_tril'}),
+        'unit_wise'.  A diagonal part is not on this path."""
+        if self.has_diag:
+            raise NotImplementedError('save: the diagonal shape is not on this path')
+        relative_paths = {}
+        if self.has_data:
+            relative_path = os.path.join(relative_dir, 'tril.npy')
+            _save_as_numpy(os.path.join(root, relative_path), matrix_to_tril(self.data))
+            relative_paths['tril'] = relative_path
+        if self.has_kron:
+            relative_paths['kron'] = self.kron.save(root, relative_dir)
+        if self.has_unit:
+            relative_paths['unit_wise'] = self.unit.save(root, relative_dir)
+        return relative_paths
+
+    def load(self, path=None, kron_path=None, diag_path=None, unit_path=None, device=None):
+        """asdl/symmatrix.py:246-269; ``device`` None is the current GPU."""
+        if diag_path is not None:
+            raise NotImplementedError('load: the diagonal shape is not on this path')
+        if path:
+            self.data = tril_to_matrix(_load_from_numpy(path, device))
+        if kron_path is not None:
+            if not self.has_kron:
+                self.kron = Kron(A=None, B=None)
+            self.kron.load(A_path=kron_path['A_tril'], B_path=kron_path['B_tril'], device=device)
+        if unit_path is not None:
+            if not self.has_unit:
+                self.unit = UnitWise()
+            self.unit.load(path=unit_path, device=device)
 
     def mvp(self, vectors=None, vec_weight=None, vec_bias=None, use_inv=False, inplace=False):
         raise NotImplementedError('SymMatrix.mvp with a full / layer-wise matrix is not on this path; '

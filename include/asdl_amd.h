@@ -143,6 +143,15 @@ int ak_unit_wise_inv(const float* blocks, int64_t F, float damping, float* inv, 
 int ak_unit_wise_mvp(const float* mat, int64_t F, float* vec_weight, float* vec_bias, float scale,
                      ak_stream_t stream);
 
+/* ---- saved factors ----------------------------------------------------------------- */
+
+/* tril[i*(i+1)/2 + j] = mat[i][j] for j <= i (row direction), the 1-D form in which factors are saved as
+ * float32 .npy files; and the inverse, which fills both triangles.  d <= 65535.
+ * Replaces matrix_to_tril / tril_to_matrix (asdl/symmatrix.py:25-54) as used by SymMatrix.save / load and
+ * Kron.save / load (asdl/symmatrix.py:226-269, 471-492). */
+int ak_tril_pack(const float* mat, int64_t d, int64_t ld, float* tril, ak_stream_t stream);
+int ak_tril_unpack(const float* tril, int64_t d, float* mat, int64_t ld, ak_stream_t stream);
+
 /* ---- dense fp32 products ---------------------------------------------------------- */
 
 /* C <- alpha * op(A) op(B) + beta * C, fp32 MFMA, row-major; op = identity (0) or transpose (1);

@@ -28,6 +28,8 @@ reference checkout).  How each function is pinned (tests/test_oracle.py):
                         BatchNorm CNN written from the reference
   unit_wise_inv / mvp   (block + damping I) @ inv == I per block; block-diagonal
                         matrix-vector product against an explicit dense matrix
+  matrix_to_tril /      the worked 3x3 example in the docstrings of asdl/symmatrix.py:25-54,
+  tril_to_matrix        numpy.tril_indices (library routine), pack(unpack(t)) == t
   power_iter            eigvalsh lambda_max (converged limit only)
   compute_power         fp64 eigh closed form (S + rI)^(-1/p), X^p (S + rI) == I;
                         golden trajectories written from the reference
@@ -48,7 +50,7 @@ __all__ = [
     'linear_cov_kron_A', 'linear_cov_kron_B', 'im2col_2d', 'conv_cov_kron_A', 'conv_cov_kron_B',
     'ema_accumulate', 'kron_damping', 'cholesky_inv', 'kron_update_inv', 'kron_mvp',
     'power_iter', 'mat_power', 'compute_power', 'shampoo_statistics', 'shampoo_precondition',
-    'KfacOracle', 'ShampooOracle',
+    'matrix_to_tril', 'tril_to_matrix', 'KfacOracle', 'ShampooOracle',
 ]
 
 
@@ -288,6 +290,23 @@ def unit_wise_mvp(mat, vec_weight, vec_bias):
     v = torch.stack([vec_weight.flatten(), vec_bias.flatten()], dim=1).unsqueeze(2)
     out = torch.matmul(mat, v).squeeze(2)
     return out[:, 0].view_as(vec_weight), out[:, 1].view_as(vec_bias)
+
+
+def matrix_to_tril(mat):
+    # asdl/symmatrix.py:25-38: rows of the lower triangle one after the other
+    return torch.cat([mat[i, :i + 1] for i in range(mat.shape[0])])
+
+
+def tril_to_matrix(tril):
+    # asdl/symmatrix.py:41-54 (n from asdl/symmatrix.py:57-67: n^2 + n = 2 numel)
+    n = int(math.sqrt(2 * tril.numel() + 0.25) - 0.5)
+    out = torch.zeros(n, n, dtype=tril.dtype)
+    k = 0
+    for i in range(n):
+        out[i, :i + 1] = tril[k:k + i + 1]
+        out[:i + 1, i] = tril[k:k + i + 1]
+        k += i + 1
+    return out
 
 
 class KfacOracle:

@@ -397,3 +397,69 @@ def test_unit_wise_inv_and_mvp_match_oracle(K):
     rw, rb = R.unit_wise_mvp(ref, w.double(), b.double())
     gw, gb = K.unit_wise_mvp(inv, w.cuda(), b.cuda(), scale=2.0)
     assert relerr(gw, 2 * rw) < 1e-5 and relerr(gb, 2 * rb) < 1e-5
+
+
+# ------------------------------------------------------------------------------ saved factors (bit-exact)
+@pytest.mark.parametrize('d', [1, 3, 64, 257, 1000, 4608])
+def test_tril_pack_unpack_bit_exact(K, d):
+    import numpy as np
+    g = torch.Generator().manual_seed(d)
+    mat = torch.randn(d, d, generator=g)
+    packed = K.tril_pack(mat.cuda())
+    rows, cols = np.tril_indices(d)
+    assert np.array_equal(packed.cpu().numpy(), mat.numpy()[rows, cols])
+    if d <= 257:
+        assert torch.equal(packed.cpu(), R.matrix_to_tril(mat))
+        assert torch.equal(K.tril_unpack(packed, d).cpu(), R.tril_to_matrix(R.matrix_to_tril(mat)))
+    full = K.tril_unpack(packed, d).cpu()
+    assert torch.equal(full, full.T) and torch.equal(torch.tril(full), torch.tril(mat))
+    # a row stride larger than d (a view of a wider buffer)
+    wide = torch.zeros(d, d + 5)
+    wide[:, :d] = mat
+    assert torch.equal(K.tril_pack(wide.cuda()[:, :d]), packed)
+
+
+def test_symmatrix_save_load_files(K, tmp_path):
+    """File names, dictionary keys and contents as written by asdl/symmatrix.py:226-269, 471-491, 672-680: float32
+    .npy, Kronecker factors as packed lower triangles, unit-wise blocks whole."""
+    import numpy as np
+    from asdl_amd.symmatrix import Kron, SymMatrix, UnitWise, matrix_to_tril, tril_to_matrix
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(40, 23, generator=g)
+    b = torch.randn(40, 7, generator=g)
+    A, B = a.T @ a, b.T @ b
+    A, B = (A + A.T) / 2, (B + B.T) / 2     # bit-exact symmetry, so that equality below is exact
+    unit = torch.randn(9, 2, 2, generator=g)
+    full = torch.randn(11, 11, generator=g)
+    full = full + full.T
+    sm = SymMatrix(data=full.cuda(), kron=Kron(A.cuda(), B.cuda()), unit=UnitWise(data=unit.cuda()))
+    paths = sm.save(str(tmp_path), 'fisher_emp/layer1')
+    assert paths == {'tril': 'fisher_emp/layer1/tril.npy',
+                     'kron': {'A_tril': 'fisher_emp/layer1/kron/A_tril.npy',
+                              'B_tril': 'fisher_emp/layer1/kron/B_tril.npy'},
+                     'unit_wise': 'fisher_emp/layer1/unit_wise.npy'}
+    on_disk = np.load(tmp_path / paths['kron']['A_tril'])
+    assert on_disk.dtype == np.float32 and on_disk.ndim == 1
+    assert np.array_equal(on_disk, A.numpy()[np.tril_indices(23)])
+    assert np.array_equal(np.load(tmp_path / paths['unit_wise']), unit.numpy())
+    assert np.array_equal(np.load(tmp_path / paths['tril']), R.matrix_to_tril(full).numpy())
+
+    back = SymMatrix()
+    back.load(path=str(tmp_path / paths['tril']),
+              kron_path={k: str(tmp_path / v) for k, v in paths['kron'].items()},
+              unit_path=str(tmp_path / paths['unit_wise']))
+    assert back.kron.A.is_cuda and torch.equal(back.kron.A.cpu(), A) and torch.equal(back.kron.B.cpu(), B)
+    assert torch.equal(back.unit.data.cpu(), unit) and torch.equal(back.data.cpu(), full)
+    assert back.kron.A_dim == 23 and back.kron.B_dim == 7
+
+    # a file written the reference's way (numpy only) loads to the same factor
+    ref_file = tmp_path / 'ref_A_tril.npy'
+    np.save(ref_file, R.matrix_to_tril(A).numpy().astype('float32'))
+    k2 = Kron(None, None)
+    k2.load(str(ref_file), str(ref_file))
+    assert torch.equal(k2.A.cpu(), A)
+    assert torch.equal(tril_to_matrix(matrix_to_tril(B.cuda())).cpu(), B)
+    with pytest.raises(RuntimeError):
+        k2.load(str(ref_file), str(ref_file), device='cpu')
+    with pytest.raises(ValueError):
+        matrix_to_tril(torch.zeros(3, device='cuda'))

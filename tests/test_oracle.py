@@ -357,3 +357,20 @@ def test_unit_wise_inv_and_mvp():
     ref = dense @ torch.stack([w, b], dim=1).flatten()
     mw, mb = R.unit_wise_mvp(inv, w, b)
     assert relerr(torch.stack([mw, mb], dim=1).flatten(), ref) < 1e-12
+
+
+def test_tril_packing_matches_docstring_example_and_numpy():
+    # the worked example of asdl/symmatrix.py:25-54
+    mat = torch.tensor([[1., 9., 9.], [2., 3., 9.], [4., 5., 6.]])
+    tril = R.matrix_to_tril(mat)
+    assert tril.tolist() == [1., 2., 3., 4., 5., 6.]
+    assert R.tril_to_matrix(tril).tolist() == [[1., 2., 4.], [2., 3., 5.], [4., 5., 6.]]
+    # numpy's row-major lower-triangle indices on a larger, non-symmetric input; round trip
+    g = torch.Generator().manual_seed(0)
+    big = torch.randn(37, 37, generator=g)
+    rows, cols = np.tril_indices(37)
+    packed = R.matrix_to_tril(big)
+    assert np.array_equal(packed.numpy(), big.numpy()[rows, cols])
+    full = R.tril_to_matrix(packed)
+    assert torch.equal(full, full.T) and torch.equal(torch.tril(full), torch.tril(big))
+    assert torch.equal(R.matrix_to_tril(full), packed)
