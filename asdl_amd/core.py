@@ -5,6 +5,7 @@ from contextlib import contextmanager, nullcontext
 
 import torch
 import torch.nn as nn
+from torch.autograd.graph import GradientEdge
 
 from .matrices import *
 from .operations import *
@@ -69,7 +70,11 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
                         run_hook(lambda: cxt.call_operations_in_backward(_m, g), g)
                         return None
                     handles.append(out_data.register_hook(grad_hook))
+                    # the graph edge the hook sits on: a backward pass restricted to these edges still fires
+                    # every hook, without the weight-gradient kernels of the layers
+                    cxt.grad_edges.append(GradientEdge(out_data.grad_fn, out_data.output_nr))
             handles.append(module.register_forward_hook(forward_hook))
+        handles.append(model.register_forward_pre_hook(lambda *_: cxt.grad_edges.clear()))
         if not cxt.is_operation_registered(model):
             cxt.register_operation(model, Operation(model, []))
         yield cxt

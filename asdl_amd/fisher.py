@@ -21,6 +21,7 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
 FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (costs more host time per hook than the overlap gains)
+PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
 EAGER_INVERSE = False       # start the bulk of the inverses during a single sampled / empirical backward pass (no gain while the GPU is throughput-bound)
 
 
@@ -134,8 +135,15 @@ class FisherMaker(GradientMaker):
                 loss = self._loss
 
             def closure(nll_expr, retain_graph=False):
+                keep = retain_graph or loss_grad_after_fisher
                 with skip_param_grad(model, disable=loss_grad_with_fisher):
-                    nll_expr().backward(retain_graph=retain_graph or loss_grad_after_fisher)
+                    if loss_grad_with_fisher or not PRUNED_FISHER_BACKWARD or not cxt.grad_edges:
+                        nll_expr().backward(retain_graph=keep)
+                    else:
+                        # No parameter takes a gradient from this pass: differentiate with respect to the
+                        # hooked module outputs only.  Every hook fires as in a full pass; the autograd
+                        # engine leaves out the weight-gradient kernels, whose results would be dropped.
+                        torch.autograd.grad(nll_expr(), list(cxt.grad_edges), retain_graph=keep, allow_unused=True)
 
             if self.is_fisher_emp:
                 closure(lambda: loss)

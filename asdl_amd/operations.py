@@ -390,6 +390,7 @@ class OperationContext:
         self._pending_unit = []
         self._unit_flags = []
         self.factor_stream = None
+        self.grad_edges = []       # autograd edges of the hooked module outputs of the latest forward pass
         self._eager_total = 0.0
         self._eager_done = False
         self._inverse_cost = 0.0

@@ -270,3 +270,41 @@ def test_fisher_maker_invariants(network, fisher_type, loss_type, monkeypatch):
     for m, (Ai, Bi) in zip(mods, inv1):
         torch.testing.assert_close(m.fisher.kron.A_inv, Ai * N)
         torch.testing.assert_close(m.fisher.kron.B_inv, Bi * N)
+
+
+@pytest.mark.parametrize('fisher_type', [FISHER_MC, FISHER_EXACT])
+def test_pruned_fisher_backward_equals_full_backward(fisher_type, monkeypatch):
+    """The sampled / exact passes differentiate with respect to the hooked module outputs only; every hook must
+    still fire and see the same gradients, also when the first trainable module is a BatchNorm whose output an
+    in-place ReLU overwrites, and the loss gradient that follows must be untouched."""
+    import asdl_amd.fisher as fisher_mod
+    cpu_backend.install(monkeypatch)
+
+    def run(pruned):
+        monkeypatch.setattr(fisher_mod, 'PRUNED_FISHER_BACKWARD', pruned)
+        torch.manual_seed(3)
+        model = nn.Sequential(nn.BatchNorm2d(5), nn.ReLU(inplace=True), nn.Conv2d(5, 6, 3, padding=1, bias=False),
+                              nn.BatchNorm2d(6), nn.ReLU(inplace=True), nn.Conv2d(6, 4, 2), nn.Flatten(),
+                              nn.Linear(4 * 3 * 3, 4))
+        x, t = torch.randn(6, 5, 4, 4), torch.randint(4, (6,))
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=6, damping=1e-2, ema_decay=0.5),
+                               fisher_type=fisher_type, seed=11)
+        gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+        gm.forward_and_backward()
+        out = {}
+        for name, m in model.named_modules():
+            f = getattr(m, 'fisher', None)
+            if f is None:
+                continue
+            if f.has_kron:
+                out[name + '.A'], out[name + '.B'] = f.kron.A.clone(), f.kron.B.clone()
+            if f.has_unit:
+                out[name + '.unit'] = f.unit.data.clone()
+        for name, p in model.named_parameters():
+            out['grad.' + name] = p.grad.clone()
+        return out
+
+    full, pruned = run(False), run(True)
+    assert full.keys() == pruned.keys() and any(k.endswith('.unit') for k in full)
+    for key in full:
+        assert torch.equal(full[key], pruned[key]), key
