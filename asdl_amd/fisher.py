@@ -165,9 +165,9 @@ class FisherMaker(GradientMaker):
             deferred.finish(config.fisher_attr)
         if calc_loss_grad:
             # the loss was summed over the batch: divide gradients and loss by the data size
-            for p in model.parameters():
-                if p.grad is not None:
-                    p.grad.div_(data_size)
+            grads = [p.grad for p in model.parameters() if p.grad is not None]
+            if grads:
+                torch._foreach_div_(grads, data_size)     # one launch for all parameters
             loss.div_(data_size)
         return self._model_output, loss
 
