@@ -180,6 +180,14 @@ size_t syrk_dtl_plain_ws_bytes(int64_t M, int64_t d, int64_t ldx);
 int syrk_dtl_plain(const void* X, int64_t M, int64_t d, int64_t ldx, float alpha, float beta, float* C, int64_t ldc,
                    void* ws, size_t ws_bytes, hipStream_t stream);
 
+// Input factor of a convolution with d = C*kh*kw <= 160 from an LDS-resident input window (conv_patch.hip); x has
+// element strides (sn, sc, sh_el, sw_el).  The workspace query answers 0, the launcher AK_ERR_UNSUPPORTED, for
+// other layers.
+size_t conv_patch_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw);
+int conv_patch_syrk(const void* x, int dtype, int64_t sn, int64_t sc, int64_t sh_el, int64_t sw_el, int64_t N, int64_t C,
+                    int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw, float alpha, float beta,
+                    float* A, int64_t lda, void* ws, size_t ws_bytes, hipStream_t stream);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_ERR_LAUNCH; }
 
 // Split-K factor shared by the SYRK front ends: enough work groups to fill 256 CUs twice over

@@ -582,6 +582,8 @@ static int launch_conv_syrk(ConvPlan& plan, hipStream_t stream) {
 extern "C" size_t ak_conv_syrk_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw,
                                         int ph, int pw) {
   if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 || ph < 0 || pw < 0) return 0;
+  const size_t patch = ak::conv_patch_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw);
+  if (patch > 0) return patch;
   ak::ConvPlan a, b;
   size_t need = 0;
   if (ak::make_plan(a, 2, N, C, H, W, kh, kw, sh, sw, ph, pw)) need = a.ws_need;
@@ -596,6 +598,11 @@ extern "C" int ak_conv_syrk(const void* x, int dtype, int64_t N, int64_t C, int6
       sw <= 0 || ph < 0 || pw < 0)
     return AK_ERR_ARG;
   if (dtype != AK_BF16 && dtype != AK_F32) return AK_ERR_ARG;
+  {  // few input channels: the window kernel
+    const int rc = ak::conv_patch_syrk(x, dtype, C * H * W, H * W, W, 1, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,
+                                       A, lda, ws, ws_bytes, static_cast<hipStream_t>(stream));
+    if (rc != AK_ERR_UNSUPPORTED) return rc;
+  }
   ak::ConvPlan plan;
   if (!ak::make_plan(plan, dtype == AK_BF16 ? 2 : 4, N, C, H, W, kh, kw, sh, sw, ph, pw)) return AK_ERR_UNSUPPORTED;
   if (lda < plan.p.d) return AK_ERR_ARG;

@@ -83,3 +83,10 @@ extern "C" int ak_kron_precond(const float* Binv, const float* Ainv, float* G, i
   }
   return ak::check_launch();
 }
+
+// Tuning hook, not part of the interface: the smallest grid (in 128 x 128 tiles) and contraction length from which
+// products that ask for the split-bf16 kernel get it.
+extern "C" void ak_debug_set_gemm_split_threshold(int min_groups, int min_k) {
+  ak::g_x3_min_groups = min_groups;
+  ak::g_x3_min_k = min_k;
+}

@@ -199,6 +199,8 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
 
 namespace ak {
 
+inline int g_x3_min_groups = 100, g_x3_min_k = 256;   // tuning hook (ak_debug_set_gemm_split_threshold)
+
 inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return AK_OK;
   const int64_t tiles128 = static_cast<int64_t>((p.N + 127) / 128) * ((p.M + 127) / 128) * batch;
@@ -206,7 +208,7 @@ inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   const int64_t work_groups = lower ? tiles128 / 2 : tiles128;
   // The split kernel (128 x 128 tiles, a pipeline that needs a few k-tiles to fill) pays off once its tiles
   // fill most of the device; below that the 64 x 64 tiles of the fp32 kernel spread the work better.
-  if (p.split >= 2 && work_groups >= 200 && p.K >= 256 && gemm_x3_ok(p)) {
+  if (p.split >= 2 && work_groups >= g_x3_min_groups && p.K >= g_x3_min_k && gemm_x3_ok(p)) {
     dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
     if (p.split == 2) hipLaunchKernelGGL(gemm_x3_kernel<2>, grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL(gemm_x3_kernel<3>, grid, dim3(256), 0, stream, p);

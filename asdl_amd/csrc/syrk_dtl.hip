@@ -392,6 +392,7 @@ struct DtlPlan {
   size_t ws_bytes;
 };
 
+static int g_force_group = 0;            // tuning hook (ak_debug_force_gather_group); 0: the built-in choice
 static int g_force_bt = 0, g_force_ns = 0;   // tuning hook (ak_debug_force_syrk_plan); 0: use the model
 
 // Tile size and split-K factor from a small cost model (microseconds, constants measured on MI355X): the
@@ -536,6 +537,9 @@ static bool nhwc_ok(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, i
 
 }  // namespace ak
 
+// Not part of the public interface: pins the channel group size of the gathered column order (0: built-in choice).
+extern "C" void ak_debug_force_gather_group(int group) { ak::g_force_group = group; }
+
 // Not part of the public interface: pins the tile size (64/128/256) and split-K factor of the direct-to-LDS
 // SYRK for tuning runs; (0, 0) restores the cost model.
 extern "C" void ak_debug_force_syrk_plan(int bt, int nsplit) {
@@ -547,6 +551,8 @@ extern "C" size_t ak_conv_syrk_nhwc_ws_bytes(int64_t N, int64_t C, int64_t H, in
                                              int sw, int ph, int pw) {
   int64_t Ho, Wo;
   if (!ak::nhwc_ok(reinterpret_cast<const void*>(16), N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return 0;
+  const size_t patch = ak::conv_patch_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw);
+  if (patch > 0) return patch;
   return ak::dtl_plan(N * Ho * Wo, C * kh * kw, INT64_MAX, true).ws_bytes;
 }
 
@@ -557,6 +563,12 @@ extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C,
   if (A == nullptr || !ak::nhwc_ok(x, N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return AK_ERR_ARG;
   const int64_t d = C * kh * kw, M = N * Ho * Wo;
   if (lda < d) return AK_ERR_ARG;
+  if (dtype != AK_BF16 && dtype != AK_F32) return AK_ERR_ARG;
+  {  // few input channels: the window kernel, any dtype and channel count
+    const int rc = ak::conv_patch_syrk(x, dtype, H * W * C, 1, W * C, C, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,
+                                       A, lda, ws, ws_bytes, static_cast<hipStream_t>(stream));
+    if (rc != AK_ERR_UNSUPPORTED) return rc;
+  }
   if (dtype != AK_BF16) return AK_ERR_UNSUPPORTED;
   // 16-byte chunks must not straddle taps, offsets must fit the 32-bit buffer range, and the magic
   // divisions by Wo, Ho, C and kw must be exact over their operand ranges
@@ -570,7 +582,7 @@ extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C,
   p.kw = kw; p.KK = kh * kw; p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw;
   p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
   p.mWo = ak::make_magic(p.Wo); p.mHo = ak::make_magic(p.Ho); p.mKw = ak::make_magic(kw);
-  p.G = d >= 3456 ? 8 : p.Cin;
+  p.G = ak::g_force_group > 0 && p.Cin % ak::g_force_group == 0 ? ak::g_force_group : (d >= 3456 ? 8 : (p.Cin % 128 == 0 ? 128 : p.Cin));
   p.mBlk = ak::make_magic(p.G * p.KK); p.mG = ak::make_magic(p.G);
   const ak::DtlPlan pl = ak::dtl_plan(M, d, INT64_MAX, true);
   return ak::dtl_launch<true>(p, pl, ws, ws_bytes, static_cast<hipStream_t>(stream));

@@ -200,7 +200,8 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
         raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
     lib = _lib.load()
     h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
-    if x.dtype == torch.bfloat16 and C % 8 == 0 and _is_channels_last(x):
+    few_channels = d <= 160 and kh * kw > 1 and x.dtype in (torch.bfloat16, torch.float32)   # the LDS-window kernel
+    if _is_channels_last(x) and ((x.dtype == torch.bfloat16 and C % 8 == 0) or few_channels):
         if (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0):
             return syrk_tn(x.permute(0, 2, 3, 1).reshape(N * H * W, C), out=out, alpha=alpha, beta=beta)
         need = _ws_need('ak_conv_syrk_nhwc_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)

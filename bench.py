@@ -42,6 +42,10 @@ def parse():
     ap.add_argument('--cpu-batch', type=int, default=16,
                     help='batch of the CPU baseline sample (its time is scaled to the full batch)')
     ap.add_argument('--no-factor-timing', action='store_true')
+    ap.add_argument('--traffic-calibration-mib', type=int, default=0,
+                    help='before the warm-up, launch one plain copy kernel (ak::debug_copy_kernel) of this many MiB: '
+                         'the known traffic against which a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this '
+                         'command is scaled')
     return ap.parse_args()
 
 
@@ -126,6 +130,19 @@ def main():
         gm.setup_loss_call(F.cross_entropy, dummy_y, t)
         gm.forward_and_backward()
         opt.step()
+
+    if args.traffic_calibration_mib > 0:
+        import ctypes
+        from asdl_amd import _lib
+        n = args.traffic_calibration_mib << 20
+        src = torch.ones(n // 4, device=dev)
+        dst = torch.empty_like(src)
+        lib = _lib.load()
+        lib.ak_debug_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        torch.cuda.synchronize()
+        _lib.check(lib.ak_debug_copy(src.data_ptr(), dst.data_ptr(), n, None), 'ak_debug_copy')
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

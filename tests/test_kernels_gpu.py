@@ -114,6 +114,44 @@ def test_conv_syrk_matches_oracle(K, dtype, case):
     assert torch.equal(out, out.T)
 
 
+WINDOW_CASES = [
+    # N, C, H, W, kernel, stride, padding: layers with C*kh*kw <= 160, taken by the LDS-window kernel
+    (2, 3, 64, 64, (7, 7), (2, 2), (3, 3)),        # ImageNet stem geometry, d = 147 (15 tiles, two per wave)
+    (3, 3, 37, 29, (7, 7), (2, 2), (3, 3)),        # odd sizes: last strip shorter than the others
+    (2, 40, 9, 9, (2, 2), (1, 1), (0, 0)),         # d = 160: the largest it takes
+    (2, 1, 28, 28, (5, 5), (1, 1), (2, 2)),        # one channel, d = 25: one tile, eight position slices
+    (2, 7, 12, 10, (3, 3), (1, 1), (1, 1)),        # d = 63: three tiles, two position slices
+    (2, 10, 12, 10, (3, 3), (2, 1), (1, 0)),       # d = 90: six tiles
+    (2, 13, 8, 8, (3, 3), (1, 1), (1, 1)),         # d = 117: ten tiles, idle waves
+    (700, 3, 6, 6, (3, 3), (1, 1), (1, 1)),        # more strips than work groups
+    (2, 3, 8, 40, (3, 5), (1, 8), (1, 2)),         # stride wider than the kernel, few output columns
+    (1, 2, 5, 3, (5, 3), (1, 1), (0, 0)),          # a single output position
+]
+
+
+@pytest.mark.parametrize('layout', ['nchw', 'channels_last'])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('case', WINDOW_CASES, ids=[str(c) for c in WINDOW_CASES])
+def test_conv_syrk_window_kernel_matches_oracle(K, dtype, layout, case):
+    N, C, H, W, k, s, p = case
+    x = _inputs((N, C, H, W), dtype, seed=N + 10 * C + H)
+    out_size = ((H + 2 * p[0] - k[0]) // s[0] + 1) * ((W + 2 * p[1] - k[1]) // s[1] + 1)
+    ref = R.conv_cov_kron_A(x.float().double(), k, s, p) * out_size      # the plain sum over positions
+    print(f'conv_syrk window dtype={dtype} layout={layout} case={case}', flush=True)
+    xg = x.cuda()
+    if layout == 'channels_last':
+        xg = xg.contiguous(memory_format=torch.channels_last)
+    out = K.conv_syrk(xg, k, s, p, alpha=0.5)
+    torch.cuda.synchronize()
+    assert relerr(out, 0.5 * ref) < 1e-5
+    assert torch.equal(out, out.T)
+    # accumulation: out <- beta * out + alpha * stat
+    K.conv_syrk(xg, k, s, p, out=out, alpha=0.25, beta=2.0)
+    torch.cuda.synchronize()
+    assert relerr(out, 1.25 * ref) < 1e-5
+    assert torch.equal(out, out.T)
+
+
 NHWC_CASES = [
     # N, C, H, W, kernel, stride, padding
     (2, 8, 6, 6, (3, 3), (1, 1), (1, 1)),          # smallest channel count the gather path takes
