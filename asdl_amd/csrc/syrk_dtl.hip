@@ -137,10 +137,21 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = wave / WC, wc = wave % WC;
   int ti, tj;
-  decode_upper_tile(blockIdx.x, p.T, ti, tj);
+  // Work groups go to the 8 XCDs round-robin by their linear index, and each XCD has its own L2.  Renumber them so
+  // that one XCD gets a contiguous range of (split, tile) pairs: the tiles of one split then share the rows they
+  // read through one L2 instead of fetching them once per XCD.
+  uint32_t tile_id, split_id;
+  {
+    const uint32_t nwg = gridDim.x * gridDim.y, wgid = blockIdx.x + blockIdx.y * gridDim.x;
+    const uint32_t xcd = wgid & 7, local = wgid >> 3, q = nwg >> 3, rem = nwg & 7;
+    const uint32_t logical = xcd * q + (xcd < rem ? xcd : rem) + local;
+    split_id = logical / gridDim.x;
+    tile_id = logical - split_id * gridDim.x;
+  }
+  decode_upper_tile(tile_id, p.T, ti, tj);
   const bool diag = (ti == tj);
   const int64_t i0 = static_cast<int64_t>(ti) * BT, j0 = static_cast<int64_t>(tj) * BT;
-  const int64_t k_begin = static_cast<int64_t>(blockIdx.y) * p.rows_per_split;
+  const int64_t k_begin = static_cast<int64_t>(split_id) * p.rows_per_split;
   int64_t k_end = k_begin + p.rows_per_split;
   if (k_end > p.M) k_end = p.M;
   const int rows = k_begin < k_end ? static_cast<int>(k_end - k_begin) : 0;
@@ -307,7 +318,7 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
   } else {
     // partial tile in accumulator order: [(a,b,q)][thread] float4
     floatx4* dst = reinterpret_cast<floatx4*>(p.ws) +
-                   (static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * (BT * BT / 4);
+                   (static_cast<size_t>(split_id) * gridDim.x + tile_id) * (BT * BT / 4);
 #pragma unroll
     for (int a = 0; a < FR; ++a)
 #pragma unroll
