@@ -23,6 +23,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0
+# Device-memory bytes per factor call (fetched + written, average over the 108 calls of a step) of the default
+# workload, from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) of this script scaled by a plain copy kernel of
+# known size (--traffic-calibration-mib); counters cannot be read from inside the timed run, so the figure is recorded
+# here and reported only for the configuration it was measured on.  Algorithmic bytes of the same calls: 31.7e6.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 74.7e6
 
 
 def parse():
@@ -180,10 +185,13 @@ def main():
         flops = sum(s[1] for s in sink)
         secs = sum(s[2].elapsed_time(s[3]) for s in sink) * 1e-3
         achieved = flops / secs / 1e12
+        default_workload = (bs == 64 and args.fisher == 'fisher_mc' and args.memory_format == 'channels_last'
+                            and not args.with_batchnorm)
+        traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None
         out['roofline'] = {'bound': 'mfma', 'achieved': achieved, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
-                           'frac': achieved / BF16_MFMA_PEAK_TFLOPS, 'traffic': None,
-                           'kernel': 'factor statistics (syrk_dtl_kernel; conv_syrk_kernel for the 3-channel stem), '
-                                     'SYRK FLOP M*d*(d+1)',
+                           'frac': achieved / BF16_MFMA_PEAK_TFLOPS, 'traffic': traffic,
+                           'kernel': 'factor statistics (syrk_dtl_kernel; conv_patch_syrk_kernel for the 3-channel '
+                                     'stem), SYRK FLOP M*d*(d+1)',
                            'launches_per_step': len(sink) // args.steps,
                            'factor_ms_per_step': secs / args.steps * 1e3,
                            'gemm_equiv_tflops': 2 * achieved}
