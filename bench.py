@@ -43,6 +43,10 @@ def parse():
     ap.add_argument('--with-batchnorm', action='store_true',
                     help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
                          '(the headline configuration ignores them, as the reference training script does)')
+    ap.add_argument('--no-conv-autotune', action='store_true',
+                    help='leave torch.backends.cudnn.benchmark off (it is on by default, as in the reference training '
+                         'script examples/arxiv_results/train.py:227: MIOpen then times its convolution kernels once '
+                         'per layer shape during the warm-up and keeps the fastest)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-batch', type=int, default=16,
                     help='batch of the CPU baseline sample (its time is scaled to the full batch)')
@@ -112,6 +116,7 @@ def main():
         print('bench.py needs a ROCm GPU.', file=sys.stderr)
         sys.exit(2)
     dev = torch.device('cuda:0')
+    torch.backends.cudnn.benchmark = not args.no_conv_autotune
     torch.manual_seed(0)
     model = bench_models.resnet50().to(dev)
     bs = args.batch
@@ -178,7 +183,8 @@ def main():
         'config': {'workload': f'K-FAC step (factors + pi-damped Cholesky inverses + precondition every step, '
                                f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
-                               f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights',
+                               f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights, '
+                               f'cudnn.benchmark {"off" if args.no_conv_autotune else "on"}',
                    'batch': bs},
     }
     if sink:
