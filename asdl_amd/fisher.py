@@ -22,7 +22,7 @@ _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
 FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (costs more host time per hook than the overlap gains)
 PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
-EAGER_INVERSE = False       # start the bulk of the inverses during a single sampled / empirical backward pass (no gain while the GPU is throughput-bound)
+EAGER_INVERSE = True        # start the bulk of the inverses during a single sampled / empirical backward pass: the longest chains get a head start
 
 
 @dataclass

@@ -345,6 +345,37 @@ def test_resnet50_batch64_channels_last_properties():
     assert relerr(got, ref) < 1e-3, relerr(got, ref)
 
 
+@pytest.mark.parametrize('fisher_type', ['fisher_emp', 'fisher_mc'])
+def test_early_start_of_inverses_gives_the_same_result(fisher_type, monkeypatch):
+    """fisher.EAGER_INVERSE starts the inverse of the layers whose factors are final while the backward pass still
+    runs (from the second step on, when the total cost is known); the results must be those of the single batch
+    after the pass (up to the run-to-run differences of the backward kernels underneath, which use atomics)."""
+    import asdl_amd.fisher as fisher_mod
+
+    def run(eager):
+        monkeypatch.setattr(fisher_mod, 'EAGER_INVERSE', eager)
+        torch.manual_seed(7)
+        model = bench_models.resnet18_cifar().cuda()
+        x, t = torch.randn(4, 3, 32, 32).cuda(), torch.randint(0, 10, (4,)).cuda()
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=4, damping=1e-2), fisher_type=fisher_type, seed=3)
+        out = {}
+        for step in range(3):
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+            gm.forward_and_backward()
+            for name, m in model.named_modules():
+                if isinstance(m, (nn.Linear, nn.Conv2d)):
+                    out[(step, name, 'A_inv')] = m.fisher.kron.A_inv.clone()
+                    out[(step, name, 'B_inv')] = m.fisher.kron.B_inv.clone()
+                    out[(step, name, 'grad')] = m.weight.grad.clone()
+        return out
+
+    lazy, eager = run(False), run(True)
+    assert lazy.keys() == eager.keys()
+    for key in lazy:
+        assert relerr(eager[key], lazy[key]) < (1e-3 if key[2] == 'grad' else 1e-4), key
+
+
 def test_fisher_attributes_and_steps_without_curvature_update():
     torch.manual_seed(4)
     model = bench_models.mlp(20, 16, 5).cuda()
