@@ -93,10 +93,12 @@ def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, ve
     def map_rule(shape):
         if shape == SHAPE_KRON:
             return OP_COV_KRON_INV if calc_inv else OP_COV_KRON
+        if shape == SHAPE_SWIFT_KRON:
+            return OP_COV_SWIFT_KRON_INV if calc_inv else OP_COV_SWIFT_KRON
         if shape == SHAPE_UNIT_WISE:
             return OP_COV_UNIT_WISE_INV if calc_inv else OP_COV_UNIT_WISE
         raise NotImplementedError(
-            f'Fisher shape "{shape}" has no MI355X kernel in this build; only "{SHAPE_KRON}" and '
+            f'Fisher shape "{shape}" has no MI355X kernel in this build; only "{SHAPE_KRON}", "{SHAPE_SWIFT_KRON}" and '
             f'"{SHAPE_UNIT_WISE}" are supported. '
             'Exclude such modules with PreconditioningConfig(ignore_modules=[...]).')
     return extend(model, *shapes, ignore_modules=ignore_modules, map_rule=map_rule, vectors=vectors, stream=stream,

@@ -343,23 +343,96 @@ def tril_unpack(tril, n_cols):
 
 
 # ------------------------------------------------------------------------------ damping / inverse
-def kron_damping(A_list, B_list, damping, eps=1e-7):
-    """Returns (lam [batch, 2] float32, nonzero [batch, 2] int32), both on the device."""
+def kron_damping(A_list, B_list, damping, eps=1e-7, eig_scale=None):
+    """Returns (lam [batch, 2] float32, nonzero [batch, 2] int32), both on the device.  A factor is a square
+    [d, d] matrix or, for the low-rank (swift) factors, an [n, d] matrix with n < d rows; ``eig_scale``: optional
+    per-pair (sA, sB) multiplied into the eigenvalue means before the pi split."""
     _require_gpu(*A_list, *B_list)
     dev = A_list[0].device
     batch = len(A_list)
+    swift = eig_scale is not None
     for t in list(A_list) + list(B_list):
-        if t.dtype != torch.float32 or not t.is_contiguous() or t.ndim != 2 or t.shape[0] != t.shape[1]:
-            raise ValueError('factors have to be contiguous square float32 matrices')
-    dims = device_ints(tuple((a.shape[0], b.shape[0]) for a, b in zip(A_list, B_list)), dev)
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.ndim != 2:
+            raise ValueError('factors have to be contiguous float32 matrices')
+        if t.shape[0] > t.shape[1]:
+            raise ValueError('a factor has to be square or have fewer rows than columns')
+        swift = swift or t.shape[0] != t.shape[1]
     lam = torch.empty(batch, 2, dtype=torch.float32, device=dev)
     nonzero = torch.empty(batch, 2, dtype=torch.int32, device=dev)
     pa, pb = device_ptr_array(A_list), device_ptr_array(B_list)
-    rc = _lib.load().ak_kron_damping(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(pb.data_ptr()),
-                                     ctypes.c_void_p(dims.data_ptr()), batch, damping, eps,
-                                     ctypes.c_void_p(lam.data_ptr()), ctypes.c_void_p(nonzero.data_ptr()), _stream())
-    _lib.check(rc, 'ak_kron_damping')
+    if not swift:
+        dims = device_ints(tuple((a.shape[0], b.shape[0]) for a, b in zip(A_list, B_list)), dev)
+        rc = _lib.load().ak_kron_damping(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(pb.data_ptr()),
+                                         ctypes.c_void_p(dims.data_ptr()), batch, damping, eps,
+                                         ctypes.c_void_p(lam.data_ptr()), ctypes.c_void_p(nonzero.data_ptr()), _stream())
+        _lib.check(rc, 'ak_kron_damping')
+        return lam, nonzero
+
+    def rows(t):
+        return 0 if t.shape[0] == t.shape[1] else t.shape[0]
+    dims = device_ints(tuple((rows(a), a.shape[1], rows(b), b.shape[1]) for a, b in zip(A_list, B_list)), dev)
+    scale = None
+    if eig_scale is not None:
+        scale = device_ints(tuple((float(sa), float(sb)) for sa, sb in eig_scale), dev, dtype=torch.float32)
+    rc = _lib.load().ak_kron_damping_swift(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(pb.data_ptr()),
+                                           ctypes.c_void_p(dims.data_ptr()),
+                                           ctypes.c_void_p(scale.data_ptr()) if scale is not None else ctypes.c_void_p(0),
+                                           batch, damping, eps, ctypes.c_void_p(lam.data_ptr()),
+                                           ctypes.c_void_p(nonzero.data_ptr()), _stream())
+    _lib.check(rc, 'ak_kron_damping_swift')
     return lam, nonzero
+
+
+# ------------------------------------------------------------------------------ low-rank (swift) factors
+def conv_patch_sum(x, kernel_size=(1, 1), stride=(1, 1), padding=(0, 0), out=None, alpha=1.0, beta=0.0):
+    """out[n, (c, ky, kx)] <- beta*out + alpha * sum over output positions of the patch element, for x = [N, C, H, W]
+    in any memory format ([N, C, L] and [N, C] are taken as W = L, H = 1 and H = W = 1): the [n, d] matrix the swift
+    factors keep.  kernel 1x1: the sum over positions; [N, C]: a scaled float32 copy."""
+    _require_gpu(x, out)
+    if x.ndim == 2:
+        x = x[:, :, None, None]
+    elif x.ndim == 3:
+        x = x[:, :, None, :]
+    if x.ndim != 4:
+        raise ValueError(f'x.ndim has to be 2, 3 or 4. Got {x.ndim}.')
+    if x.dtype not in (torch.float32, torch.bfloat16):
+        x = x.float()
+    N, C, H, W = x.shape
+    kh, kw = kernel_size
+    sh, sw = stride
+    ph, pw = padding
+    d = C * kh * kw
+    if out is None:
+        out = torch.empty(N, d, dtype=torch.float32, device=x.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or out.shape != (N, d) or out.stride(1) != 1:
+        raise ValueError('out has to be a float32 [N, C*kh*kw] tensor with contiguous rows')
+    sn, sc, sy, sx = x.stride()
+    rc = _lib.load().ak_conv_patch_sum(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), sn, sc, sy, sx, N, C, H, W,
+                                       kh, kw, sh, sw, ph, pw, alpha, beta, ctypes.c_void_p(out.data_ptr()),
+                                       out.stride(0), _stream())
+    _lib.check(rc, 'ak_conv_patch_sum')
+    return out
+
+
+def smw_inv(x, lam, out=None, info=None):
+    """(x^T x / n + lam I)^-1 for an [n, d] float32 matrix with n < d through the n x n Gram matrix
+    (Sherman-Morrison-Woodbury): (I - x^T (x x^T + n lam I)^-1 x) / lam.  ``lam``: one-element float32 device tensor.
+    Returns (inverse [d, d], info) with the Cholesky info word of the Gram matrix."""
+    _require_gpu(x, lam, out)
+    if x.ndim != 2 or x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError('x has to be a contiguous float32 matrix')
+    n, d = x.shape
+    lam = lam.reshape(1)
+    gram = syrk_nt(x)                                            # x x^T, [n, n]
+    gram_inv = torch.empty_like(gram)
+    info = chol_inv_batched([gram], [gram_inv], lam * float(n), info=info)
+    y = gemm(gram_inv, x)                                        # [n, d]
+    z = gemm(x, y, out=out, transA=True)                         # x^T G^-1 x, [d, d]
+    rc = _lib.load().ak_smw_finish(ctypes.c_void_p(z.data_ptr()), d, z.stride(0), ctypes.c_void_p(lam.data_ptr()),
+                                   _stream())
+    _lib.check(rc, 'ak_smw_finish')
+    return z, info
 
 
 def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1, info=None):

@@ -21,7 +21,7 @@ from .symmatrix import SymMatrix, batched_update_inv
 
 _invalid_ema_decay = -1
 _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KFE, SHAPE_UNIT_WISE, SHAPE_DIAG]
-_kernel_shapes = [SHAPE_KRON, SHAPE_UNIT_WISE]
+_kernel_shapes = [SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_UNIT_WISE]
 _norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 
 __all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
@@ -225,15 +225,14 @@ class KfacGradientMaker(NaturalGradientMaker):
     """K-FAC (https://arxiv.org/abs/1503.05671) behind the GradientMaker interface; same constructor
     arguments as asdl/precondition/natural_gradient.py:883-900.
 
-    BatchNorm1d/2d and LayerNorm modules get the unit-wise shape, as in the reference.  ``swift=True`` and
-    Embedding modules have no kernels in this build (exclude the latter through ``config.ignore_modules``)."""
+    BatchNorm1d/2d and LayerNorm modules get the unit-wise shape, as in the reference; ``swift=True`` keeps the
+    factors of layers that see fewer samples than they have columns as row matrices (SKFAC).  Embedding modules
+    have no kernels in this build (exclude them through ``config.ignore_modules``)."""
 
     def __init__(self, model, config: PreconditioningConfig, fisher_type: str = FISHER_MC,
                  loss_type: str = LOSS_CROSS_ENTROPY, scale: float = 1, grad_scale: float = 1, n_mc_samples: int = 1,
                  var: float = 1., seed: int = None, swift=False):
-        if swift:
-            raise NotImplementedError('swift=True (SKFAC) is not on this path')
-        fisher_shape = [SHAPE_KRON, (nn.BatchNorm1d, SHAPE_UNIT_WISE), (nn.BatchNorm2d, SHAPE_UNIT_WISE),
+        fisher_shape = [SHAPE_SWIFT_KRON if swift else SHAPE_KRON, (nn.BatchNorm1d, SHAPE_UNIT_WISE), (nn.BatchNorm2d, SHAPE_UNIT_WISE),
                         (nn.LayerNorm, SHAPE_UNIT_WISE)]
         super().__init__(model, config, fisher_type=fisher_type, fisher_shape=fisher_shape, loss_type=loss_type,
                          scale=scale, grad_scale=grad_scale, n_mc_samples=n_mc_samples, var=var, seed=seed)

@@ -24,27 +24,33 @@ from .utils import UnfoldedInput, im2col_2d, original_requires_grad
 
 OP_COV_KRON = 'cov_kron'
 OP_COV_KRON_INV = 'cov_kron_inv'
+OP_COV_SWIFT_KRON = 'cov_swift_kron'            # Kronecker factors kept as n x d row matrices where n < d (SKFAC)
+OP_COV_SWIFT_KRON_INV = 'cov_swift_kron_inv'
 OP_COV_UNIT_WISE = 'cov_unit_wise'
 OP_COV_UNIT_WISE_INV = 'cov_unit_wise_inv'
 OP_SAVE_INPUTS = 'save_inputs'
 OP_SAVE_OUTPUTS = 'save_outputs'
 OP_SAVE_OUTGRADS = 'save_outgrads'
 
-ALL_OPS = [OP_COV_KRON, OP_COV_KRON_INV, OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS,
-           OP_SAVE_OUTGRADS]
+ALL_OPS = [OP_COV_KRON, OP_COV_KRON_INV, OP_COV_SWIFT_KRON, OP_COV_SWIFT_KRON_INV, OP_COV_UNIT_WISE,
+           OP_COV_UNIT_WISE_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS]
 BWD_OPS_WITH_INPUTS = [OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV]     # the forward hook has to keep the output
-FWD_OPS = [OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_COV_KRON, OP_COV_KRON_INV] + BWD_OPS_WITH_INPUTS
-BWD_OPS = [OP_SAVE_OUTGRADS, OP_COV_KRON, OP_COV_KRON_INV, OP_COV_UNIT_WISE, OP_COV_UNIT_WISE_INV]
+FWD_OPS = [OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_COV_KRON, OP_COV_KRON_INV, OP_COV_SWIFT_KRON,
+           OP_COV_SWIFT_KRON_INV] + BWD_OPS_WITH_INPUTS
+BWD_OPS = [OP_SAVE_OUTGRADS, OP_COV_KRON, OP_COV_KRON_INV, OP_COV_SWIFT_KRON, OP_COV_SWIFT_KRON_INV, OP_COV_UNIT_WISE,
+           OP_COV_UNIT_WISE_INV]
 
 __all__ = ['Operation', 'Linear', 'Conv2d', 'BatchNorm', 'LayerNorm', 'OperationContext', 'get_op_class', 'ALL_OPS',
-           'FWD_OPS', 'BWD_OPS', 'OP_COV_KRON', 'OP_COV_KRON_INV', 'OP_COV_UNIT_WISE', 'OP_COV_UNIT_WISE_INV',
+           'FWD_OPS', 'BWD_OPS', 'OP_COV_KRON', 'OP_COV_KRON_INV', 'OP_COV_SWIFT_KRON', 'OP_COV_SWIFT_KRON_INV',
+           'OP_COV_UNIT_WISE', 'OP_COV_UNIT_WISE_INV',
            'OP_SAVE_INPUTS', 'OP_SAVE_OUTPUTS', 'OP_SAVE_OUTGRADS']
 
 _FACTOR_CACHE_ATTR = '_asdl_amd_factor_cache'
 
 
 class Operation:
-    supported_operations = {OP_COV_KRON, OP_COV_KRON_INV, OP_SAVE_INPUTS, OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS}
+    supported_operations = {OP_COV_KRON, OP_COV_KRON_INV, OP_COV_SWIFT_KRON, OP_COV_SWIFT_KRON_INV, OP_SAVE_INPUTS,
+                            OP_SAVE_OUTPUTS, OP_SAVE_OUTGRADS}
 
     def __init__(self, module, op_names, model_for_kernel=None):
         if hasattr(module, 'weight'):
@@ -118,17 +124,36 @@ class Operation:
             compute(existing, self._cov_scale, beta)
         self._touched.add(key)
 
-    def _scratch_factor(self, key, dim, device):
-        """Reusable buffer for a factor that only lives until it has been inverted."""
+    def _scratch_factor(self, key, dim, device, rows=None):
+        """Reusable buffer for a factor that only lives until it has been inverted: [dim, dim], or [rows, dim]
+        for a low-rank factor."""
         cache = getattr(self._module, _FACTOR_CACHE_ATTR, None)
         if cache is None:
             cache = {}
             setattr(self._module, _FACTOR_CACHE_ATTR, cache)
+        shape = (dim if rows is None else rows, dim)
         buf = cache.get(key)
-        if buf is None or buf.shape[0] != dim or buf.device != device:
-            buf = torch.empty(dim, dim, dtype=torch.float32, device=device)
+        if buf is None or tuple(buf.shape) != shape or buf.device != device:
+            buf = torch.empty(*shape, dtype=torch.float32, device=device)
             cache[key] = buf
         return buf
+
+    def _factor_inv_mode(self, key, tmp_key, data, swift, square_fn, low_rank_fn, device):
+        """One contribution to the scratch factor of the *_INV operations.  Swift (asdl/operations/operation.py:
+        282-299): a factor with fewer samples than columns is the unscaled [n, d] row matrix; a square one is
+        scaled by cov_scale only after the damping has been taken from the unscaled factors, which the damping
+        kernel reproduces by un-scaling its eigenvalue mean."""
+        n, dim = self.swift_rows_cols(data)
+        first = tmp_key not in self._op_results
+        if swift and n < dim:
+            buf = self._scratch_factor(key, dim, device, rows=n)
+            low_rank_fn(buf, 1.0, 0.0 if first else 1.0)
+            self._op_results['_eig_scale_' + key] = 1.0
+        else:
+            buf = self._scratch_factor(key, dim, device)
+            square_fn(buf, self._cov_scale, 0.0 if first else 1.0)
+            self._op_results['_eig_scale_' + key] = 1.0 / self._cov_scale if swift else 1.0
+        self._op_results[tmp_key] = buf
 
     def forward_post_process(self, in_data: torch.Tensor, out_data: torch.Tensor):
         module = self._module
@@ -140,13 +165,18 @@ class Operation:
         if OP_COV_KRON in op_names:
             data = self.preprocess_in_data(module, in_data, out_data)
             self._update_factor('A', lambda out, alpha, beta: self.cov_kron_A(module, data, out=out, alpha=alpha, beta=beta))
-        elif OP_COV_KRON_INV in op_names:
+        elif OP_COV_SWIFT_KRON in op_names:
             data = self.preprocess_in_data(module, in_data, out_data)
-            dim = data.shape[1]
-            first = '_A_tmp' not in self._op_results
-            buf = self._scratch_factor('A', dim, in_data.device)
-            self.cov_kron_A(module, data, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
-            self._op_results['_A_tmp'] = buf
+            n, dim = self.swift_rows_cols(data)
+            fn = self.cov_swift_kron_A if n < dim else self.cov_kron_A
+            self._update_factor('A', lambda out, alpha, beta: fn(module, data, out=out, alpha=alpha, beta=beta))
+        elif OP_COV_KRON_INV in op_names or OP_COV_SWIFT_KRON_INV in op_names:
+            data = self.preprocess_in_data(module, in_data, out_data)
+            self._factor_inv_mode(
+                'A', '_A_tmp', data, OP_COV_SWIFT_KRON_INV in op_names,
+                lambda out, alpha, beta: self.cov_kron_A(module, data, out=out, alpha=alpha, beta=beta),
+                lambda out, alpha, beta: self.cov_swift_kron_A(module, data, out=out, alpha=alpha, beta=beta),
+                in_data.device)
             self._n_forward += 1
 
     def backward_pre_process(self, out_grads, vector: torch.Tensor = None):
@@ -159,11 +189,16 @@ class Operation:
             self.accumulate_result([grads], OP_SAVE_OUTGRADS, extend=True)
         if OP_COV_KRON in op_names:
             self._update_factor('B', lambda out, alpha, beta: self.cov_kron_B(module, grads, out=out, alpha=alpha, beta=beta))
-        elif OP_COV_KRON_INV in op_names:
-            first = '_B_tmp' not in self._op_results
-            buf = self._scratch_factor('B', grads.shape[1], grads.device)
-            self.cov_kron_B(module, grads, out=buf, alpha=self._cov_scale, beta=0.0 if first else 1.0)
-            self._op_results['_B_tmp'] = buf
+        elif OP_COV_SWIFT_KRON in op_names:
+            n, dim = self.swift_rows_cols(grads)
+            fn = self.cov_swift_kron_B if n < dim else self.cov_kron_B
+            self._update_factor('B', lambda out, alpha, beta: fn(module, grads, out=out, alpha=alpha, beta=beta))
+        elif OP_COV_KRON_INV in op_names or OP_COV_SWIFT_KRON_INV in op_names:
+            self._factor_inv_mode(
+                'B', '_B_tmp', grads, OP_COV_SWIFT_KRON_INV in op_names,
+                lambda out, alpha, beta: self.cov_kron_B(module, grads, out=out, alpha=alpha, beta=beta),
+                lambda out, alpha, beta: self.cov_swift_kron_B(module, grads, out=out, alpha=alpha, beta=beta),
+                grads.device)
             self._n_backward += 1
             # a module called several times in the forward pass is complete after as many backward hooks
             if self._context is not None and self._n_backward % max(self._n_forward, 1) == 0:
@@ -193,6 +228,20 @@ class Operation:
     def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
         raise NotImplementedError
 
+    @staticmethod
+    def swift_rows_cols(data):
+        """(samples, columns) of a preprocessed input / output gradient: the swift factors keep the row matrix
+        when there are fewer samples than columns."""
+        return data.shape[0], data.shape[1]
+
+    @staticmethod
+    def cov_swift_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
+        raise NotImplementedError
+
+    @staticmethod
+    def cov_swift_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        raise NotImplementedError
+
 
 class Linear(Operation):
     """module.weight: f_out x f_in; in_data: n x f_in; out_grads: n x f_out
@@ -217,6 +266,16 @@ class Linear(Operation):
     @staticmethod
     def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
         return kernels.syrk_tn(out_grads, out=out, alpha=alpha, beta=beta)    # f_out x f_out
+
+    @staticmethod
+    def cov_swift_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
+        """The inputs themselves, n x f_in with n < f_in (asdl/operations/linear.py:79-85)."""
+        return kernels.conv_patch_sum(in_data, out=out, alpha=alpha, beta=beta)
+
+    @staticmethod
+    def cov_swift_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        """n x f_out with n < f_out (asdl/operations/linear.py:91-97)."""
+        return kernels.conv_patch_sum(out_grads, out=out, alpha=alpha, beta=beta)
 
 
 class Conv2d(Operation):
@@ -253,6 +312,20 @@ class Conv2d(Operation):
             rows = out_grads.permute(0, 2, 3, 1).reshape(n * h * w, c)        # a view
             return kernels.syrk_tn(rows, out=out, alpha=alpha, beta=beta)
         return kernels.syrk_nt(out_grads, out=out, alpha=alpha, beta=beta)    # c_out x c_out
+
+    @staticmethod
+    def cov_swift_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
+        """Per-sample sums of the patches over the output positions, n x (c_in k_h k_w): `in_data.sum(dim=-1)` of the
+        unfolded input (asdl/operations/conv.py:90-97), taken straight from the activation."""
+        if not isinstance(in_data, UnfoldedInput):
+            return kernels.conv_patch_sum(in_data, out=out, alpha=alpha, beta=beta)      # [n, d, out_size] patches
+        return kernels.conv_patch_sum(in_data.x, in_data.kernel_size, in_data.stride, in_data.padding, out=out,
+                                      alpha=alpha, beta=beta)
+
+    @staticmethod
+    def cov_swift_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
+        """`out_grads.sum(dim=-1)`, n x c_out (asdl/operations/conv.py:105-111)."""
+        return kernels.conv_patch_sum(out_grads, out=out, alpha=alpha, beta=beta)
 
 
 class _NormOperation(Operation):
@@ -519,7 +592,11 @@ class OperationContext:
             if A is None or B is None:
                 raise RuntimeError('cov_kron_inv: the forward and backward hooks did not both run')
             prev = op._op_results.get(OP_COV_KRON) or {}
-            krons.append(Kron(A, B, prev.get('A_inv'), prev.get('B_inv')))
+            kron = Kron(A, B, prev.get('A_inv'), prev.get('B_inv'))
+            scales = (op._op_results.pop('_eig_scale_A', 1.0), op._op_results.pop('_eig_scale_B', 1.0))
+            if scales != (1.0, 1.0):
+                kron._eig_scale = scales          # swift: the damping is taken from the unscaled factors
+            krons.append(kron)
         # every operation in one context shares the damping value
         pending = batched_update_inv(krons, damping=ops[0]._damping, replace=False, defer=True)
         outs = {(id(k), which): out for _, k, which, out in pending._records}

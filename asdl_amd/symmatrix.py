@@ -159,26 +159,32 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         if calc_B_inv and not k.has_B:
             raise ValueError('B does not exist.')
         for m in (k.A, k.B):
-            if m is not None and (m.ndim != 2 or m.shape[0] != m.shape[1]):
-                raise NotImplementedError('non-square (swift) Kronecker factors are not on this path')
+            if m is not None and (m.ndim != 2 or m.shape[0] > m.shape[1]):
+                raise ValueError('a Kronecker factor is a square matrix or an [n, d] row matrix with n < d')
     dev = (krons[0].A if krons[0].has_A else krons[0].B).device
     mats_on_gpu = dev.type == 'cuda'
     A_list = [k.A if k.has_A else k.B for k in krons]
     B_list = [k.B if k.has_B else k.A for k in krons]
     A_list = [a if a.is_contiguous() else a.contiguous() for a in A_list]
     B_list = [b if b.is_contiguous() else b.contiguous() for b in B_list]
-    lam, nonzero = kernels.kron_damping(A_list, B_list, float(damping), float(eps))
+    eig_scale = None
+    if any(getattr(k, '_eig_scale', None) is not None for k in krons):
+        eig_scale = [getattr(k, '_eig_scale', None) or (1.0, 1.0) for k in krons]
+    lam, nonzero = kernels.kron_damping(A_list, B_list, float(damping), float(eps), eig_scale=eig_scale)
     single = [i for i, k in enumerate(krons) if not (k.has_A and k.has_B)]
     if single:
         lam[kernels.device_ints(tuple(single), dev)] = float(damping)      # no pi split without both factors
     lam_flat, nz_flat = lam.view(-1), nonzero.view(-1)
 
     groups = defaultdict(list)   # d -> [(flat index, matrix, kron, 'A'|'B')]
+    low_rank = []                # the same entries for [n, d] row matrices (n < d), inverted through their Gram matrix
     for i, k in enumerate(krons):
         if calc_A_inv:
-            groups[A_list[i].shape[0]].append((2 * i, A_list[i], k, 'A'))
+            entry = (2 * i, A_list[i], k, 'A')
+            (groups[A_list[i].shape[0]] if A_list[i].shape[0] == A_list[i].shape[1] else low_rank).append(entry)
         if calc_B_inv:
-            groups[B_list[i].shape[0]].append((2 * i + 1, B_list[i], k, 'B'))
+            entry = (2 * i + 1, B_list[i], k, 'B')
+            (groups[B_list[i].shape[0]] if B_list[i].shape[0] == B_list[i].shape[1] else low_rank).append(entry)
     # Each size group is an independent chain of small launches: spread the groups over a few side streams
     # (default priority) so that their launch latencies overlap; everything joins the caller's stream again.
     order = sorted(groups, key=lambda d: d ** 3 * len(groups[d]), reverse=True)
@@ -227,6 +233,14 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
     for entries, outs, lam_g, act_g, info in prepared:
         infos.append(info)
         records.extend((e[0], e[2], e[3], out) for e, out in zip(entries, outs))
+    for flat, mat, k, which in low_rank:
+        # (x^T x / n + lam I)^-1 by Sherman-Morrison-Woodbury (smw_inv, asdl/utils.py:107-115), on the caller's stream
+        d = mat.shape[1]
+        old = getattr(k, which + '_inv')
+        reuse = old is not None and tuple(old.shape) == (d, d) and old.is_contiguous() and old.dtype == mat.dtype
+        out, info = kernels.smw_inv(mat, lam_flat[flat:flat + 1], out=old if reuse else None)
+        infos.append(info)
+        records.append((flat, k, which, out))
     pending = PendingInverses(records, infos, nz_flat, events, replace,
                               keep_alive=(prepared, lam, nonzero, A_list, B_list), futures=futures)
     if defer:
@@ -306,6 +320,14 @@ class Kron:
             else:
                 raise ValueError('B nor B_inv has not been set.')
         return self._B_dim
+
+    @property
+    def A_is_square(self):
+        return self.A is not None and self.A.shape[0] == self.A.shape[1]
+
+    @property
+    def B_is_square(self):
+        return self.B is not None and self.B.shape[0] == self.B.shape[1]
 
     def mul_(self, value):
         if self.has_A:

@@ -98,6 +98,32 @@ int ak_kron_damping(const float* const* A_list, const float* const* B_list, cons
                     int batch, float damping, float eps, float* lam_out, int* nonzero_out,
                     ak_stream_t stream);
 
+/* ---- low-rank ("swift") Kronecker factors --------------------------------------------- */
+
+/* X[n][(c,ky,kx)] <- beta*X + alpha * sum over output positions of the patch element of sample n, read straight
+ * from the activation x[n][c][iy][ix] with element strides (sn, sc, sh_el, sw_el): the n x d matrix SKFAC keeps
+ * in place of a d x d factor when n < d.  With kh = kw = 1 it is the sum over positions (of an output gradient),
+ * with H = W = 1 a scaled fp32 copy (Linear).  X = [N, ldo] fp32.
+ * Replaces Conv2d.cov_swift_kron_A / _B (asdl/operations/conv.py:90-111: `in_data.sum(dim=-1)` of the unfolded
+ * input, `out_grads.sum(dim=-1)`) and Linear.cov_swift_kron_A / _B (asdl/operations/linear.py:79-97). */
+int ak_conv_patch_sum(const void* x, int dtype, int64_t sn, int64_t sc, int64_t sh_el, int64_t sw_el,
+                      int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw,
+                      float alpha, float beta, float* out, int64_t ldo, ak_stream_t stream);
+
+/* ak_kron_damping for pairs whose factors may be n x d row matrices: dims = device int64 [batch,4]
+ * (rows_A, d_A, rows_B, d_B; rows = 0: square d x d factor, eigenvalue mean trace/d; rows > 0: sum(x^2)/d),
+ * eig_scale = device float [batch,2] multiplied into the eigenvalue means (may be null).
+ * Replaces Operation.cov_kron_damping (asdl/operations/operation.py:457-466) and the head of Kron.update_inv
+ * (asdl/symmatrix.py:499-510) for non-square factors. */
+int ak_kron_damping_swift(const float* const* A_list, const float* const* B_list, const int64_t* dims,
+                          const float* eig_scale, int batch, float damping, float eps, float* lam_out,
+                          int* nonzero_out, ak_stream_t stream);
+
+/* Z <- (I - Z) / lam[0], Z = [d, d] fp32 with row stride ld, lam in device memory: the last step of
+ * smw_inv (asdl/utils.py:107-115), whose products run in ak_conv_syrk (x x^T), ak_chol_inv_batched and
+ * ak_gemm_f32. */
+int ak_smw_finish(float* Z, int64_t d, int64_t ld, const float* lam, ak_stream_t stream);
+
 /* ---- damped inverse --------------------------------------------------------------- */
 
 /* out_b <- (A_b + lam_b I)^-1 for b < batch; all matrices d x d fp32 dense (ld = d); A_b is not

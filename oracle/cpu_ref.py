@@ -30,6 +30,10 @@ reference checkout).  How each function is pinned (tests/test_oracle.py):
                         matrix-vector product against an explicit dense matrix
   matrix_to_tril /      the worked 3x3 example in the docstrings of asdl/symmatrix.py:25-54,
   tril_to_matrix        numpy.tril_indices (library routine), pack(unpack(t)) == t
+  smw_inv               fp64 inverse of x^T x / n + damping I formed densely (the identity it
+                        implements); golden SKFAC runs written from the reference
+  *_cov_swift_*         the row sums of F.unfold / of the output gradient (library routines);
+                        golden SKFAC runs (swift=True) written from the reference
   power_iter            eigvalsh lambda_max (converged limit only)
   compute_power         fp64 eigh closed form (S + rI)^(-1/p), X^p (S + rI) == I;
                         golden trajectories written from the reference
@@ -51,6 +55,7 @@ __all__ = [
     'ema_accumulate', 'kron_damping', 'cholesky_inv', 'kron_update_inv', 'kron_mvp',
     'power_iter', 'mat_power', 'compute_power', 'shampoo_statistics', 'shampoo_precondition',
     'matrix_to_tril', 'tril_to_matrix', 'KfacOracle', 'ShampooOracle',
+    'linear_cov_swift', 'conv_cov_swift_kron_A', 'conv_cov_swift_kron_B', 'swift_kron_damping', 'smw_inv', 'swift_inv',
 ]
 
 
@@ -139,6 +144,55 @@ def kron_update_inv(A, B, damping, eps=1e-7):
     A_inv = None if bool(torch.all(A == 0)) else cholesky_inv(A, dA)
     B_inv = None if bool(torch.all(B == 0)) else cholesky_inv(B, dB)
     return A_inv, B_inv
+
+
+# --------------------------------------------------------------------------- low-rank ("swift") factors
+def linear_cov_swift(data):
+    """n x f rows themselves when n < f, else the f x f factor (asdl/operations/linear.py:79-97)."""
+    data = _flatten_rows(data)
+    n, f = data.shape
+    return data.clone() if n < f else data.T @ data
+
+
+def conv_cov_swift_kron_A(x, kernel_size, stride, padding):
+    """asdl/operations/conv.py:90-97: per-sample sum of the patches over the output positions when n < c_in k_h k_w
+    (not divided by the output size), else the ordinary factor."""
+    col = im2col_2d(x, kernel_size, stride, padding)
+    n, d, _ = col.shape
+    return col.sum(dim=-1) if n < d else conv_cov_kron_A(x, kernel_size, stride, padding)
+
+
+def conv_cov_swift_kron_B(out_grads):
+    """asdl/operations/conv.py:105-111."""
+    g = out_grads.flatten(start_dim=2)
+    n, c, _ = g.shape
+    return g.sum(dim=-1) if n < c else conv_cov_kron_B(out_grads)
+
+
+def swift_kron_damping(A, B, damping, eps=1e-7):
+    """asdl/operations/operation.py:457-466, asdl/symmatrix.py:499-510: the eigenvalue mean of an n x d row matrix
+    is sum(x^2) / d."""
+    def mean(M):
+        return (M.trace() if M.shape[0] == M.shape[1] else (M ** 2).sum()) / M.shape[-1]
+    pi = torch.sqrt(mean(A) / mean(B))
+    pi_v = float(pi)
+    if pi_v != 0 and pi_v != float('inf'):
+        r = damping ** 0.5
+        return max(float(r * pi), eps), max(float(r / pi), eps)
+    return damping, damping
+
+
+def smw_inv(x, damping=1e-7):
+    """(x^T x / n + damping I)^-1 of an n x d matrix through its n x n Gram matrix (asdl/utils.py:107-115)."""
+    n, d = x.shape
+    G = x @ x.T
+    G = G + damping * n * torch.eye(n, dtype=x.dtype)
+    Ginv_x = torch.linalg.solve(G, x)
+    return (torch.eye(d, dtype=x.dtype) - x.T @ Ginv_x) / damping
+
+
+def swift_inv(M, damping):
+    return cholesky_inv(M, damping) if M.shape[0] == M.shape[1] else smw_inv(M, damping)
 
 
 def kron_mvp(A_inv, B_inv, grad_w, grad_b=None):
@@ -325,7 +379,7 @@ class KfacOracle:
 
     def __init__(self, model, data_size, damping=1e-7, ema_decay=-1, fisher_type='fisher_emp',
                  scale=1., grad_scale=1., seed=None, curvature_upd_interval=None,
-                 preconditioner_upd_interval=1, factor_dtype=None, unit_wise_norm=False):
+                 preconditioner_upd_interval=1, factor_dtype=None, unit_wise_norm=False, swift=False):
         self.model = model
         self.data_size = data_size
         self.damping = damping
@@ -337,6 +391,7 @@ class KfacOracle:
         self.curv_interval = curvature_upd_interval
         self.prec_interval = preconditioner_upd_interval
         self.factor_dtype = factor_dtype
+        self.swift = swift        # KfacGradientMaker(swift=True), asdl/precondition/natural_gradient.py:886-887
         self.step = 0
         self.layers = [(n, m) for n, m in model.named_modules()
                        if isinstance(m, (nn.Linear, nn.Conv2d))
@@ -371,6 +426,21 @@ class KfacOracle:
             A = linear_cov_kron_A(cast(in_data))
             B = linear_cov_kron_B(cast(out_grads))
         return A * cov_scale, B * cov_scale
+
+    def _swift_factor(self, module, in_data, out_grads):
+        """Unscaled swift factors (asdl/operations/operation.py:201-204, 279-285)."""
+        cast = (lambda t: t.to(self.factor_dtype)) if self.factor_dtype is not None else (lambda t: t)
+        if isinstance(module, nn.Conv2d):
+            return (conv_cov_swift_kron_A(cast(in_data), module.kernel_size, module.stride, module.padding),
+                    conv_cov_swift_kron_B(cast(out_grads)))
+        return linear_cov_swift(cast(in_data)), linear_cov_swift(cast(out_grads))
+
+    def _swift_update_inv(self, A, B):
+        """Kron.update_inv with non-square factors (asdl/symmatrix.py:499-534)."""
+        dA, dB = swift_kron_damping(A, B, self.damping)
+        A_inv = None if bool(torch.all(A == 0)) else swift_inv(A, dA)
+        B_inv = None if bool(torch.all(B == 0)) else swift_inv(B, dB)
+        return A_inv, B_inv
 
     def forward_and_backward(self, x, t, loss_fn=F.cross_entropy, mc_targets=None):
         model = self.model
@@ -426,6 +496,18 @@ class KfacOracle:
             for h in handles:
                 h.remove()
             for name, m in self.layers:
+                if self.swift:
+                    A, B = self._swift_factor(m, saved_in[name], saved_g[name])
+                    if accumulate:        # OP_COV_SWIFT_KRON: every factor, square or not, times cov_scale
+                        self.A[name] = ema_accumulate(self.A.get(name), A * cov_scale, self.ema_decay)
+                        self.B[name] = ema_accumulate(self.B.get(name), B * cov_scale, self.ema_decay)
+                    else:
+                        # OP_COV_SWIFT_KRON_INV (asdl/operations/operation.py:282-299): damping from the unscaled
+                        # factors; only the square ones are scaled before the inverse
+                        dA, dB = swift_kron_damping(A, B, self.damping)
+                        self.A_inv[name] = cholesky_inv(A * cov_scale, dA) if A.shape[0] == A.shape[1] else smw_inv(A, dA)
+                        self.B_inv[name] = cholesky_inv(B * cov_scale, dB) if B.shape[0] == B.shape[1] else smw_inv(B, dB)
+                    continue
                 A, B = self._factor(m, saved_in[name], saved_g[name], cov_scale)
                 if accumulate:
                     self.A[name] = ema_accumulate(self.A.get(name), A, self.ema_decay)
@@ -448,7 +530,8 @@ class KfacOracle:
         if accumulate and self._do_update_preconditioner(step):
             for name, _ in self.layers:
                 if name in self.A:
-                    self.A_inv[name], self.B_inv[name] = kron_update_inv(self.A[name], self.B[name], self.damping)
+                    update = self._swift_update_inv if self.swift else (lambda A, B: kron_update_inv(A, B, self.damping))
+                    self.A_inv[name], self.B_inv[name] = update(self.A[name], self.B[name])
             for name, _ in self.norm_layers:
                 if name in self.unit:
                     inv = unit_wise_inv(self.unit[name], self.damping)

@@ -35,11 +35,15 @@ def syrk_nt(x, out=None, alpha=1.0, beta=0.0):
     return out
 
 
-def kron_damping(A_list, B_list, damping, eps=1e-7):
+def kron_damping(A_list, B_list, damping, eps=1e-7, eig_scale=None):
     lam = torch.empty(len(A_list), 2)
     nz = torch.empty(len(A_list), 2, dtype=torch.int32)
     for i, (A, B) in enumerate(zip(A_list, B_list)):
-        lam[i, 0], lam[i, 1] = R.kron_damping(A, B, damping, eps)
+        sa, sb = eig_scale[i] if eig_scale is not None else (1.0, 1.0)
+        # a scale on an eigenvalue mean is a scale on the matrix (square) or on its square root (row matrix)
+        As = A * sa if A.shape[0] == A.shape[1] else A * sa ** 0.5
+        Bs = B * sb if B.shape[0] == B.shape[1] else B * sb ** 0.5
+        lam[i, 0], lam[i, 1] = R.swift_kron_damping(As, Bs, damping, eps)
         nz[i, 0] = int(not bool(torch.all(A == 0)))
         nz[i, 1] = int(not bool(torch.all(B == 0)))
     return lam, nz
@@ -61,6 +65,32 @@ def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1
 
 def cholesky_inv(X, damping=1e-7):
     return R.cholesky_inv(X, damping)
+
+
+def conv_patch_sum(x, kernel_size=(1, 1), stride=(1, 1), padding=(0, 0), out=None, alpha=1.0, beta=0.0):
+    x = x.float()
+    if x.ndim == 2:
+        val = x
+    elif x.ndim == 3:
+        val = x.sum(-1)
+    else:
+        val = R.im2col_2d(x, kernel_size, stride, padding).sum(-1)
+    val = alpha * val
+    if out is None:
+        return val.clone()
+    out.copy_(val if beta == 0 else beta * out + val)
+    return out
+
+
+def smw_inv(x, lam, out=None, info=None):
+    val = R.smw_inv(x, float(lam.reshape(-1)[0]))
+    if out is not None:
+        out.copy_(val)
+        val = out
+    if info is None:
+        info = torch.zeros(1, dtype=torch.int32)
+    info.zero_()
+    return val, info
 
 
 def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
@@ -116,5 +146,5 @@ def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
 def install(monkeypatch):
     from asdl_amd import kernels
     for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'cholesky_inv',
-                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_mvp']:
+                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_mvp', 'conv_patch_sum', 'smw_inv']:
         monkeypatch.setattr(kernels, name, globals()[name])

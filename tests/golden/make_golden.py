@@ -55,12 +55,13 @@ def state_arrays(model, prefix):
     return {f'{prefix}{k}': v.detach().numpy().copy() for k, v in model.state_dict().items()}
 
 
-def run_kfac(tag, model, xs, ts, fisher_type, ema_decay, damping, seed=None, curv_interval=None, prec_interval=1):
+def run_kfac(tag, model, xs, ts, fisher_type, ema_decay, damping, seed=None, curv_interval=None, prec_interval=1,
+             swift=False):
     out = {}
     out.update(state_arrays(model, 'init/'))
     config = PreconditioningConfig(data_size=xs[0].shape[0], damping=damping, ema_decay=ema_decay,
                                    curvature_upd_interval=curv_interval, preconditioner_upd_interval=prec_interval)
-    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed)
+    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed, swift=swift)
     opt = torch.optim.SGD(model.parameters(), lr=0.05)
     for step, (x, t) in enumerate(zip(xs, ts)):
         opt.zero_grad(set_to_none=True)
@@ -164,10 +165,44 @@ def main_bn():
     run_kfac('cnnbn_fisher_mc_ema-1', get_cnn_bn(), xs, ts, 'fisher_mc', -1, 1e-2, seed=3)
 
 
+def get_mlp_wide():
+    # more columns than samples (batch 8) in the first two layers, on both sides
+    return get_mlp(in_dim=12, hid=10, out=4)
+
+
+def get_cnn3(in_dim=3, hid=6, out=5):
+    # convolutions with more patch elements than samples, a Linear layer with fewer
+    return nn.Sequential(nn.Conv2d(in_dim, hid, 3, 1, 1), nn.ReLU(), nn.Conv2d(hid, hid, 3, 2, 1), nn.ReLU(),
+                         nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(hid, out))
+
+
+def main_swift():
+    # KfacGradientMaker(swift=True): factors of layers with fewer samples than columns stay n x d row matrices
+    bs = 8
+    torch.manual_seed(23)
+    xs = [torch.randn(bs, 3, 8, 8) for _ in range(3)]
+    ts = [torch.randint(5, (bs,)) for _ in range(3)]
+    torch.manual_seed(24)
+    run_kfac('swift_cnn2_fisher_emp_ema-1', get_cnn2(), xs, ts, 'fisher_emp', -1, 1e-2, swift=True)
+    torch.manual_seed(25)
+    run_kfac('swift_cnn2_fisher_mc_ema-1', get_cnn2(), xs, ts, 'fisher_mc', -1, 1e-3, seed=4, swift=True)
+    # accumulation (EMA) of row matrices: only for layers whose row matrix is a fresh tensor (convolutions); for a
+    # Linear layer the reference scales the live activation in place in this mode
+    torch.manual_seed(26)
+    run_kfac('swift_cnn3_fisher_emp_ema0.5', get_cnn3(), xs, ts, 'fisher_emp', 0.5, 1e-2, swift=True)
+    xs = [torch.randn(bs, 12) for _ in range(3)]
+    ts = [torch.randint(4, (bs,)) for _ in range(3)]
+    torch.manual_seed(27)
+    run_kfac('swift_mlpw_fisher_emp_ema-1', get_mlp_wide(), xs, ts, 'fisher_emp', -1, 1e-2, swift=True)
+
+
 def main():
     if len(sys.argv) > 1 and sys.argv[1] == 'bn':
         return main_bn()
+    if len(sys.argv) > 1 and sys.argv[1] == 'swift':
+        return main_swift()
     main_bn()
+    main_swift()
     torch.manual_seed(0)
     bs = 8
     xs = [torch.randn(bs, 5) for _ in range(3)]

@@ -25,6 +25,17 @@ def get_cnn_bn(in_dim=3, hid=8, out=5):
                          nn.LayerNorm(10), nn.Linear(10, out))
 
 
+def get_mlp_wide():
+    # more columns than samples (batch 8) in the first two layers, on both sides
+    return get_mlp(in_dim=12, hid=10, out=4)
+
+
+def get_cnn3(in_dim=3, hid=6, out=5):
+    # convolutions with more patch elements than samples, a Linear layer with fewer
+    return nn.Sequential(nn.Conv2d(in_dim, hid, 3, 1, 1), nn.ReLU(), nn.Conv2d(hid, hid, 3, 2, 1), nn.ReLU(),
+                         nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(hid, out))
+
+
 GOLDEN_KFAC = {
     # tag: (model factory, fisher_type, ema_decay, damping, seed, curvature interval, preconditioner interval)
     'mlp_fisher_emp_ema-1': (get_mlp, 'fisher_emp', -1, 1e-2, None, None, 1),
@@ -38,6 +49,11 @@ GOLDEN_KFAC = {
     'cnnbn_fisher_emp_ema-1': (get_cnn_bn, 'fisher_emp', -1, 1e-2, None, None, 1),
     'cnnbn_fisher_emp_ema0.4': (get_cnn_bn, 'fisher_emp', 0.4, 1e-2, None, None, 1),
     'cnnbn_fisher_mc_ema-1': (get_cnn_bn, 'fisher_mc', -1, 1e-2, 3, None, 1),
+    # tags that start with 'swift_': KfacGradientMaker(swift=True)
+    'swift_cnn2_fisher_emp_ema-1': (get_cnn2, 'fisher_emp', -1, 1e-2, None, None, 1),
+    'swift_cnn2_fisher_mc_ema-1': (get_cnn2, 'fisher_mc', -1, 1e-3, 4, None, 1),
+    'swift_cnn3_fisher_emp_ema0.5': (get_cnn3, 'fisher_emp', 0.5, 1e-2, None, None, 1),
+    'swift_mlpw_fisher_emp_ema-1': (get_mlp_wide, 'fisher_emp', -1, 1e-2, None, None, 1),
 }
 
 GOLDEN_SHAMPOO = {

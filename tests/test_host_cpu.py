@@ -183,7 +183,7 @@ def test_kfac_host_logic_matches_reference_golden(tag, monkeypatch):
     bs = z['step0/x'].shape[0]
     config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema, curvature_upd_interval=ci,
                                    preconditioner_upd_interval=pi)
-    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed)
+    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed, swift=tag.startswith('swift_'))
     opt = torch.optim.SGD(model.parameters(), lr=0.05)
     n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
     for step in range(n_steps):

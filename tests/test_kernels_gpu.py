@@ -501,3 +501,60 @@ def test_symmatrix_save_load_files(K, tmp_path):
         k2.load(str(ref_file), str(ref_file), device='cpu')
     with pytest.raises(ValueError):
         matrix_to_tril(torch.zeros(3, device='cuda'))
+
+
+# ------------------------------------------------------------------------------ low-rank (swift) factors
+@pytest.mark.parametrize('layout', ['nchw', 'channels_last'])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('case', [(3, 4, 6, 5, (3, 3), (2, 1), (1, 0)), (5, 70, 9, 9, (3, 3), (1, 1), (1, 1)),
+                                  (2, 3, 20, 20, (7, 7), (2, 2), (3, 3)), (4, 130, 7, 7, (1, 1), (1, 1), (0, 0))])
+def test_conv_patch_sum_matches_oracle(K, dtype, layout, case):
+    N, C, H, W, k, s, p = case
+    x = _inputs((N, C, H, W), dtype, seed=N + C)
+    want = torch.nn.functional.unfold(x.double(), k, padding=p, stride=s).sum(-1)
+    xg = x.cuda()
+    if layout == 'channels_last':
+        xg = xg.contiguous(memory_format=torch.channels_last)
+    print(f'conv_patch_sum dtype={dtype} layout={layout} case={case}', flush=True)
+    out = K.conv_patch_sum(xg, k, s, p, alpha=0.5)
+    torch.cuda.synchronize()
+    assert out.shape == (N, C * k[0] * k[1]) and relerr(out, 0.5 * want) < 1e-5
+    K.conv_patch_sum(xg, k, s, p, out=out, alpha=0.25, beta=2.0)
+    assert relerr(out, 1.25 * want) < 1e-5
+
+
+def test_patch_sum_of_rows_and_positions(K):
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(7, 300, generator=g).to(torch.bfloat16)
+    assert torch.equal(K.conv_patch_sum(a.cuda(), alpha=1.0).cpu(), a.float())          # Linear: a float32 copy
+    gr = torch.randn(5, 33, 49, generator=g)                                              # [n, c, positions]
+    assert relerr(K.conv_patch_sum(gr.cuda()), gr.double().sum(-1)) < 1e-6
+
+
+@pytest.mark.parametrize('n,d,lam', [(8, 27, 1e-2), (64, 576, 3e-2), (3, 300, 0.5), (16, 1100, 1e-1)])
+def test_smw_inv_matches_oracle(K, n, d, lam):
+    g = torch.Generator().manual_seed(n + d)
+    x = torch.randn(n, d, generator=g)
+    dense = torch.linalg.inv(x.double().T @ x.double() / n + lam * torch.eye(d, dtype=torch.float64))
+    out, info = K.smw_inv(x.cuda(), torch.tensor([lam], device='cuda'))
+    assert int(info[0]) == 0
+    assert relerr(out, dense) < TOL_INV and relerr(out, R.smw_inv(x, lam)) < TOL_INV
+
+
+def test_kron_damping_with_row_matrices(K):
+    g = torch.Generator().manual_seed(9)
+    a_rows, b_sq = torch.randn(6, 40, generator=g), torch.randn(30, 12, generator=g)
+    b_sq = b_sq.T @ b_sq
+    a_sq = torch.randn(50, 9, generator=g)
+    a_sq = a_sq.T @ a_sq
+    b_rows = torch.randn(4, 21, generator=g)
+    zero = torch.zeros(3, 17)
+    pairs = [(a_rows, b_sq), (a_sq, b_rows), (a_rows, b_rows), (zero, b_sq)]
+    lam, nz = K.kron_damping([p[0].cuda() for p in pairs], [p[1].cuda() for p in pairs], 1e-2,
+                             eig_scale=[(1.0, 4.0), (0.25, 1.0), (1.0, 1.0), (1.0, 1.0)])
+    lam, nz = lam.cpu(), nz.cpu()
+    for i, ((A, B), (sa, sb)) in enumerate(zip(pairs, [(1.0, 4.0), (0.25, 1.0), (1.0, 1.0), (1.0, 1.0)])):
+        want = R.swift_kron_damping(A * (sa if A.shape[0] == A.shape[1] else sa ** 0.5),
+                                    B * (sb if B.shape[0] == B.shape[1] else sb ** 0.5), 1e-2)
+        assert abs(float(lam[i, 0]) - want[0]) < 1e-5 * want[0] and abs(float(lam[i, 1]) - want[1]) < 1e-5 * want[1]
+    assert nz.tolist() == [[1, 1], [1, 1], [1, 1], [0, 1]]

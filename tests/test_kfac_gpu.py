@@ -51,13 +51,14 @@ def test_kfac_gpu_matches_reference_golden(tag):
         # the sampled targets depend on the CPU RNG stream: draw them with the oracle and replay them
         cpu_model = copy.deepcopy(model)
         orc = R.KfacOracle(cpu_model, data_size=bs, damping=damping, ema_decay=ema, fisher_type=fisher_type, seed=seed,
-                           curvature_upd_interval=ci, preconditioner_upd_interval=pi, unit_wise_norm=True)
+                           curvature_upd_interval=ci, preconditioner_upd_interval=pi, unit_wise_norm=True,
+                           swift=tag.startswith('swift_'))
         cpu_opt = torch.optim.SGD(cpu_model.parameters(), lr=0.05)
         replay = []
     model = model.cuda()
     config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema, curvature_upd_interval=ci,
                                    preconditioner_upd_interval=pi)
-    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed)
+    gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed, swift=tag.startswith('swift_'))
     opt = torch.optim.SGD(model.parameters(), lr=0.05)
     n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
     for step in range(n_steps):
@@ -345,19 +346,26 @@ def test_resnet50_batch64_channels_last_properties():
     assert relerr(got, ref) < 1e-3, relerr(got, ref)
 
 
-@pytest.mark.parametrize('fisher_type', ['fisher_emp', 'fisher_mc'])
-def test_early_start_of_inverses_gives_the_same_result(fisher_type, monkeypatch):
+@pytest.mark.parametrize('network', ['mlp', 'resnet18'])
+def test_early_start_of_inverses_gives_the_same_result(network, monkeypatch):
     """fisher.EAGER_INVERSE starts the inverse of the layers whose factors are final while the backward pass still
     runs (from the second step on, when the total cost is known); the results must be those of the single batch
-    after the pass (up to the run-to-run differences of the backward kernels underneath, which use atomics)."""
+    after the pass: bit for bit on an MLP, whose kernels are deterministic, and up to the run-to-run differences of
+    the convolution backward kernels (atomics; the most upstream inverses amplify them most) on a ResNet."""
     import asdl_amd.fisher as fisher_mod
+    import asdl_amd.operations as ops_mod
+    monkeypatch.setattr(ops_mod, 'EAGER_COST_FRACTION', 0.3)
 
     def run(eager):
         monkeypatch.setattr(fisher_mod, 'EAGER_INVERSE', eager)
         torch.manual_seed(7)
-        model = bench_models.resnet18_cifar().cuda()
-        x, t = torch.randn(4, 3, 32, 32).cuda(), torch.randint(0, 10, (4,)).cuda()
-        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=4, damping=1e-2), fisher_type=fisher_type, seed=3)
+        if network == 'mlp':
+            model = bench_models.mlp().cuda()
+            x, t = torch.randn(32, 784).cuda(), torch.randint(0, 10, (32,)).cuda()
+        else:
+            model = bench_models.resnet18_cifar().cuda()
+            x, t = torch.randn(4, 3, 32, 32).cuda(), torch.randint(0, 10, (4,)).cuda()
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=x.shape[0], damping=1e-2), fisher_type='fisher_emp')
         out = {}
         for step in range(3):
             model.zero_grad(set_to_none=True)
@@ -373,7 +381,10 @@ def test_early_start_of_inverses_gives_the_same_result(fisher_type, monkeypatch)
     lazy, eager = run(False), run(True)
     assert lazy.keys() == eager.keys()
     for key in lazy:
-        assert relerr(eager[key], lazy[key]) < (1e-3 if key[2] == 'grad' else 1e-4), key
+        if network == 'mlp':
+            assert torch.equal(eager[key], lazy[key]), key
+        else:
+            assert relerr(eager[key], lazy[key]) < 3e-3, key
 
 
 def test_fisher_attributes_and_steps_without_curvature_update():

@@ -242,7 +242,8 @@ def test_kfac_oracle_matches_reference_golden(tag):
     x0 = torch.from_numpy(z['step0/x'])
     orc = R.KfacOracle(model, data_size=x0.shape[0], damping=damping, ema_decay=ema, fisher_type=fisher_type,
                        seed=seed, curvature_upd_interval=ci, preconditioner_upd_interval=pi,
-                       unit_wise_norm=True)        # the fixtures come from the default KfacGradientMaker
+                       unit_wise_norm=True,        # the fixtures come from the default KfacGradientMaker
+                       swift=tag.startswith('swift_'))
     opt = torch.optim.SGD(model.parameters(), lr=0.05)
     for step in range(n_steps):
         opt.zero_grad(set_to_none=True)
@@ -374,3 +375,32 @@ def test_tril_packing_matches_docstring_example_and_numpy():
     full = R.tril_to_matrix(packed)
     assert torch.equal(full, full.T) and torch.equal(torch.tril(full), torch.tril(big))
     assert torch.equal(R.matrix_to_tril(full), packed)
+
+
+def test_smw_inv_is_the_inverse_of_the_damped_gram_form():
+    # asdl/utils.py:107-115 implements (x^T x / n + damping I)^-1 through the n x n Gram matrix
+    g = torch.Generator().manual_seed(3)
+    for n, d, lam in [(4, 9, 1e-2), (8, 27, 0.3), (1, 5, 1e-3)]:
+        x = torch.randn(n, d, generator=g, dtype=torch.float64)
+        dense = torch.linalg.inv(x.T @ x / n + lam * torch.eye(d, dtype=torch.float64))
+        assert relerr(R.smw_inv(x, lam), dense) < 1e-9
+        assert relerr(R.smw_inv(x.float(), lam), dense) < 1e-3        # fp32: cond ~ |x|^2 / (n lam)
+
+
+def test_swift_factors_are_row_sums_or_the_ordinary_factors():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(3, 4, 6, 5, generator=g)                   # n = 3 < d = 4*3*3 = 36
+    got = R.conv_cov_swift_kron_A(x, (3, 3), (2, 1), (1, 0))
+    want = F.unfold(x, (3, 3), padding=(1, 0), stride=(2, 1)).sum(-1)
+    assert got.shape == (3, 36) and relerr(got, want) < 1e-6
+    x = torch.randn(40, 4, 6, 5, generator=g)                  # n = 40 >= 36: the ordinary factor
+    assert relerr(R.conv_cov_swift_kron_A(x, (3, 3), (2, 1), (1, 0)), R.conv_cov_kron_A(x, (3, 3), (2, 1), (1, 0))) == 0
+    gr = torch.randn(3, 7, 4, 4, generator=g)
+    assert relerr(R.conv_cov_swift_kron_B(gr), gr.sum((2, 3))) < 1e-6
+    assert R.conv_cov_swift_kron_B(torch.randn(9, 7, 2, 2, generator=g)).shape == (7, 7)
+    a = torch.randn(3, 8, generator=g)
+    assert torch.equal(R.linear_cov_swift(a), a) and R.linear_cov_swift(torch.randn(8, 3, generator=g)).shape == (3, 3)
+    # eigenvalue mean of a row matrix: trace of its Gram form over the column count
+    la, lb = R.swift_kron_damping(a, torch.eye(5) * 2.0, 1e-2)
+    pi = ((a ** 2).sum() / 8 / 2.0) ** 0.5
+    assert abs(la - 0.1 * float(pi)) < 1e-6 and abs(lb - 0.1 / float(pi)) < 1e-6
