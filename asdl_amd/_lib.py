@@ -41,6 +41,8 @@ _SIGNATURES = {
     'ak_conv_patch_sum': (c_int, [c_ptr, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_f32, c_f32, c_ptr, c_i64, c_ptr]),
     'ak_kron_damping_swift': (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_f32, c_f32, c_ptr, c_ptr, c_ptr]),
+    'ak_smw_inv_ws_bytes': (c_size, [c_i64, c_i64]),
+    'ak_smw_inv': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
     'ak_smw_finish': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     'ak_tril_pack': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     'ak_tril_unpack': (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_ptr]),

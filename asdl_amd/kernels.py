@@ -424,14 +424,18 @@ def smw_inv(x, lam, out=None, info=None):
         raise ValueError('x has to be a contiguous float32 matrix')
     n, d = x.shape
     lam = lam.reshape(1)
-    gram = syrk_nt(x)                                            # x x^T, [n, n]
-    gram_inv = torch.empty_like(gram)
-    info = chol_inv_batched([gram], [gram_inv], lam * float(n), info=info)
-    y = gemm(gram_inv, x)                                        # [n, d]
-    z = gemm(x, y, out=out, transA=True)                         # x^T G^-1 x, [d, d]
-    rc = _lib.load().ak_smw_finish(ctypes.c_void_p(z.data_ptr()), d, z.stride(0), ctypes.c_void_p(lam.data_ptr()),
-                                   _stream())
-    _lib.check(rc, 'ak_smw_finish')
+    if out is None:
+        out = torch.empty(d, d, dtype=torch.float32, device=x.device)
+    if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
+        raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
+    if info is None:
+        info = torch.empty(1, dtype=torch.int32, device=x.device)
+    ws, ws_bytes, keep = _ws_args(_ws_need('ak_smw_inv_ws_bytes', n, d), x.device)
+    rc = _lib.load().ak_smw_inv(ctypes.c_void_p(x.data_ptr()), n, d, ctypes.c_void_p(lam.data_ptr()),
+                                ctypes.c_void_p(out.data_ptr()), out.stride(0), ctypes.c_void_p(info.data_ptr()),
+                                ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_smw_inv')
+    z = out
     return z, info
 
 

@@ -199,12 +199,24 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             outs.append(old if reuse else torch.empty_like(mat))
         info = torch.empty(len(entries), dtype=torch.int32, device=dev)
         prepared.append((entries, outs, lam_flat[idx], nz_flat[idx].contiguous(), info))
+    for flat, mat, k, which in low_rank:
+        # (x^T x / n + lam I)^-1 by Sherman-Morrison-Woodbury (smw_inv, asdl/utils.py:107-115): a group of its own
+        d = mat.shape[1]
+        old = getattr(k, which + '_inv')
+        reuse = old is not None and tuple(old.shape) == (d, d) and old.is_contiguous() and old.dtype == mat.dtype
+        out = old if reuse else torch.empty(d, d, dtype=mat.dtype, device=dev)
+        info = torch.empty(1, dtype=torch.int32, device=dev)
+        prepared.append(([(flat, mat, k, which)], [out], lam_flat[flat:flat + 1], None, info))
+    prepared.sort(key=lambda g: -sum(e[1].shape[0] * e[1].shape[1] ** 2 for e in g[0]))
     infos, records, events, futures = [], [], [], []
     use_streams = mats_on_gpu and (len(prepared) > 1 or defer)
 
     def run_group(group):
         entries, outs, lam_g, act_g, info = group
-        kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
+        if act_g is None:          # a low-rank factor
+            kernels.smw_inv(entries[0][1], lam_g, out=outs[0], info=info)
+        else:
+            kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
 
     if use_streams:
         main = torch.cuda.current_stream()
@@ -233,14 +245,6 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
     for entries, outs, lam_g, act_g, info in prepared:
         infos.append(info)
         records.extend((e[0], e[2], e[3], out) for e, out in zip(entries, outs))
-    for flat, mat, k, which in low_rank:
-        # (x^T x / n + lam I)^-1 by Sherman-Morrison-Woodbury (smw_inv, asdl/utils.py:107-115), on the caller's stream
-        d = mat.shape[1]
-        old = getattr(k, which + '_inv')
-        reuse = old is not None and tuple(old.shape) == (d, d) and old.is_contiguous() and old.dtype == mat.dtype
-        out, info = kernels.smw_inv(mat, lam_flat[flat:flat + 1], out=old if reuse else None)
-        infos.append(info)
-        records.append((flat, k, which, out))
     pending = PendingInverses(records, infos, nz_flat, events, replace,
                               keep_alive=(prepared, lam, nonzero, A_list, B_list), futures=futures)
     if defer:

@@ -43,6 +43,9 @@ def parse():
     ap.add_argument('--with-batchnorm', action='store_true',
                     help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
                          '(the headline configuration ignores them, as the reference training script does)')
+    ap.add_argument('--swift', action='store_true',
+                    help='KfacGradientMaker(swift=True): factors of layers with fewer samples than columns are kept as '
+                         'row matrices (SKFAC); not the headline configuration')
     ap.add_argument('--no-conv-autotune', action='store_true',
                     help='leave torch.backends.cudnn.benchmark off (it is on by default, as in the reference training '
                          'script examples/arxiv_results/train.py:227: MIOpen then times its convolution kernels once '
@@ -127,7 +130,7 @@ def main():
     t = torch.randint(0, 1000, (bs,)).to(dev)
     ignore = [] if args.with_batchnorm else [nn.BatchNorm2d]
     config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=ignore)
-    gm = KfacGradientMaker(model, config, fisher_type=args.fisher)
+    gm = KfacGradientMaker(model, config, fisher_type=args.fisher, swift=args.swift)
     opt = torch.optim.SGD(model.parameters(), lr=1e-4)
 
     def fwd(inp):
@@ -184,7 +187,7 @@ def main():
                                f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
                                f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights, '
-                               f'cudnn.benchmark {"off" if args.no_conv_autotune else "on"}',
+                               f'cudnn.benchmark {"off" if args.no_conv_autotune else "on"}' + (', swift (SKFAC) factors' if args.swift else ''),
                    'batch': bs},
     }
     if sink:
@@ -192,7 +195,7 @@ def main():
         secs = sum(s[2].elapsed_time(s[3]) for s in sink) * 1e-3
         achieved = flops / secs / 1e12
         default_workload = (bs == 64 and args.fisher == 'fisher_mc' and args.memory_format == 'channels_last'
-                            and not args.with_batchnorm)
+                            and not args.with_batchnorm and not args.swift)
         traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None
         out['roofline'] = {'bound': 'mfma', 'achieved': achieved, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
                            'frac': achieved / BF16_MFMA_PEAK_TFLOPS, 'traffic': traffic,

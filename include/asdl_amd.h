@@ -124,6 +124,14 @@ int ak_kron_damping_swift(const float* const* A_list, const float* const* B_list
  * ak_gemm_f32. */
 int ak_smw_finish(float* Z, int64_t d, int64_t ld, const float* lam, ak_stream_t stream);
 
+/* out <- (x^T x / n + lam[0] I)^-1 for x = [n, d] fp32 dense (n < d), lam in device memory: the whole of smw_inv
+ * (asdl/utils.py:107-115) in one call -- Gram matrix x x^T + n lam I, its Cholesky inverse (info[0] as in
+ * ak_chol_inv_batched), G^-1 x, x^T G^-1 x and the final (I - .) / lam, all enqueued on `stream`.
+ * ws: 256-byte aligned, ak_smw_inv_ws_bytes(n, d) bytes. */
+size_t ak_smw_inv_ws_bytes(int64_t n, int64_t d);
+int ak_smw_inv(const float* x, int64_t n, int64_t d, const float* lam, float* out, int64_t ldo, int* info,
+               void* ws, size_t ws_bytes, ak_stream_t stream);
+
 /* ---- damped inverse --------------------------------------------------------------- */
 
 /* out_b <- (A_b + lam_b I)^-1 for b < batch; all matrices d x d fp32 dense (ld = d); A_b is not
