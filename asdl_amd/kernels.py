@@ -19,11 +19,31 @@ _ptr_cache = {}
 _timing_sink = None      # when set to a list, factor launches append (name, flops, start event, end event)
 
 
-def set_timing_sink(sink):
+_event_pool = []         # pre-created timing events: creating one costs more host time than recording it
+
+
+def set_timing_sink(sink, n_events=0):
     """Benchmark instrumentation: with a list as sink every factor-statistics launch is bracketed by
-    two events on the launching stream and recorded with its algorithmic FLOP count M*d*(d+1)."""
+    two events on the launching stream and recorded with its algorithmic FLOP count M*d*(d+1).
+    ``n_events`` events are created up front so that the timed region only records them."""
     global _timing_sink
     _timing_sink = sink
+    del _event_pool[:]
+    if sink is not None:
+        _event_pool.extend(torch.cuda.Event(enable_timing=True) for _ in range(n_events))
+
+
+def enable_timing(flag):
+    """Switches the recording into the sink set by set_timing_sink() on or off (to sample a subset of steps)."""
+    global _timing_on
+    _timing_on = bool(flag)
+
+
+_timing_on = True
+
+
+def _timing_event():
+    return _event_pool.pop() if _event_pool else torch.cuda.Event(enable_timing=True)
 
 
 class _Timed:
@@ -31,14 +51,15 @@ class _Timed:
         self.name, self.flops = name, flops
 
     def __enter__(self):
-        if _timing_sink is not None:
-            self.start = torch.cuda.Event(enable_timing=True)
+        self.timed = _timing_sink is not None and _timing_on
+        if self.timed:
+            self.start = _timing_event()
             self.start.record()
         return self
 
     def __exit__(self, *exc):
-        if _timing_sink is not None:
-            end = torch.cuda.Event(enable_timing=True)
+        if self.timed:
+            end = _timing_event()
             end.record()
             _timing_sink.append((self.name, self.flops, self.start, end))
         return False

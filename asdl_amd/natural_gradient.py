@@ -23,6 +23,7 @@ _invalid_ema_decay = -1
 _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KFE, SHAPE_UNIT_WISE, SHAPE_DIAG]
 _kernel_shapes = [SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_UNIT_WISE]
 _norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
+PRECONDITION_STREAMS = 6      # side streams over which precondition() spreads the layers
 
 __all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
 
@@ -179,7 +180,7 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         from .symmatrix import _side_streams
         dev = grads[0].device
         main = torch.cuda.current_stream(dev)
-        side = _side_streams(dev, 4)
+        side = _side_streams(dev, PRECONDITION_STREAMS)
         start = torch.cuda.Event()
         start.record(main)
         work.sort(key=lambda mw: -(mw[0].weight.numel() * (mw[0].weight.shape[0] + mw[0].weight[0].numel())))
