@@ -6,6 +6,7 @@ MI355X-first host layout: every statistic of one size n (and one root exponent p
 convergence tests run on the device; Preconditioner.statistics / .preconditioners hold views into
 these groups.
 """
+import itertools
 from collections import defaultdict
 
 import torch
@@ -14,7 +15,7 @@ import torch.distributed as dist
 from . import kernels
 from .prec_grad_maker import PreconditionedGradientMaker, PreconditioningConfig
 
-__all__ = ['ShampooGradientMaker', 'Preconditioner', 'compute_power']
+__all__ = ['ShampooGradientMaker', 'Preconditioner', 'BlockPartitioner', 'compute_power']
 
 _invalid = -1
 
@@ -35,59 +36,160 @@ def compute_power(mat_g, p, iter_count=100, error_tolerance=1e-6, ridge_epsilon=
     return out
 
 
-class Preconditioner:
-    """Statistics and preconditioners of one parameter (asdl/precondition/shampoo.py:300-367)."""
+def _merge_small_dims(shape_to_merge, max_dim):
+    """Collapses runs of neighbouring dimensions whose product stays within ``max_dim``
+    (asdl/precondition/shampoo.py:370-395): [1, 2, 512, 1, 2048, 1, 3, 4] -> [1024, 2048, 12] for max_dim 1024."""
+    merged, run = [], 1
+    for d in shape_to_merge:
+        if run * d <= max_dim:
+            run *= d
+            continue
+        if run > 1:
+            merged.append(run)
+        run = d
+    if run > 1:
+        merged.append(run)
+    return merged
 
-    def __init__(self, param, config: PreconditioningConfig, statistics, preconditioners, inverse_exponent=_invalid):
-        if param.ndim <= 1:
-            raise ValueError(f'len(self._transformed_shape) has to be > 1. Got {param.ndim}.')
+
+class BlockPartitioner:
+    """Cuts a tensor into blocks of at most ``block_size`` along every axis that is longer than that
+    (asdl/precondition/shampoo.py:398-462).  Blocks are ordered with the first axis slowest; each block has one
+    square statistic per axis."""
+
+    def __init__(self, shape, block_size=_invalid):
+        self._shape = tuple(shape)
+        self._ranges = []          # per axis: [(start, stop), ...]
+        for d in self._shape:
+            if block_size != _invalid and d > block_size:
+                starts = list(range(0, d, block_size))
+                self._ranges.append([(a, min(a + block_size, d)) for a in starts])
+            else:
+                self._ranges.append([(0, d)])
+        self._blocks = list(itertools.product(*self._ranges))      # one tuple of (start, stop) per block
+
+    def kronecker_factor_shapes(self):
+        return [[b - a, b - a] for block in self._blocks for a, b in block]
+
+    def num_splits(self):
+        """Statistics per block (= number of axes)."""
+        return len(self._shape)
+
+    def partition(self, tensor):
+        if tuple(tensor.shape) != self._shape:
+            raise ValueError(f'tensor shape ({tensor.shape}) does not match self._shape ({self._shape}).')
+        return [tensor[tuple(slice(a, b) for a, b in block)] for block in self._blocks]
+
+    def merge_partitions(self, partitions):
+        if len(partitions) != len(self._blocks):
+            raise ValueError(f'len(partitions) has to be {len(self._blocks)}. Got {len(partitions)}.')
+        out = torch.empty(self._shape, dtype=partitions[0].dtype, device=partitions[0].device)
+        for block, part in zip(self._blocks, partitions):
+            out[tuple(slice(a, b) for a, b in block)] = part
+        return out
+
+
+def _axis_statistic(grad, axis, out, alpha, beta):
+    """out <- beta*out + alpha * (grad contracted with itself over every axis but ``axis``)."""
+    ndim = grad.ndim
+    if axis == ndim - 1:
+        kernels.syrk_tn(grad.reshape(-1, grad.shape[-1]), out=out, alpha=alpha, beta=beta)
+    elif axis == 0:
+        kernels.syrk_nt(grad.reshape(grad.shape[0], -1), out=out, alpha=alpha, beta=beta)
+    else:
+        kernels.syrk_nt(grad.movedim(axis, 0).reshape(grad.shape[axis], -1).contiguous(), out=out, alpha=alpha, beta=beta)
+
+
+def _precondition_block(grad, preconditioners):
+    """tensordot(grad, P_j, [[0], [0]]) for every axis in turn (asdl/precondition/shampoo.py:358-364)."""
+    cur = grad
+    for j in range(grad.ndim):
+        x2d = cur.reshape(cur.shape[0], -1)
+        cur = kernels.gemm(x2d, preconditioners[j], transA=True).view(*cur.shape[1:], cur.shape[0])
+    return cur
+
+
+class Preconditioner:
+    """Statistics and preconditioners of one parameter; constructor arguments of
+    asdl/precondition/shampoo.py:300-323.  ``statistics`` / ``preconditioners`` (keyword only) let
+    ShampooGradientMaker hand in views into its per-size groups, whose roots it takes in batched calls."""
+
+    def __init__(self, param, config: PreconditioningConfig, block_size: int = _invalid, inverse_exponent: int = _invalid,
+                 best_effort_shape_interpretation: bool = False, init_scale: float = 1e-12, *, statistics=None,
+                 preconditioners=None):
         self.config = config
         self.param = param
-        self.statistics = statistics            # views into the per-size groups
+        self._transformed_shape = tuple(param.shape)
+        if best_effort_shape_interpretation:
+            self._transformed_shape = tuple(_merge_small_dims(param.shape, block_size))
+        if len(self._transformed_shape) <= 1:
+            raise ValueError(f'len(self._transformed_shape) has to be > 1. Got {len(self._transformed_shape)}.')
+        if not param.is_cuda:
+            raise RuntimeError('asdl_amd kernels run on a ROCm device only; move the model to the GPU first. '
+                               'There is no CPU fallback.')
+        self._partitioner = BlockPartitioner(self._transformed_shape, block_size)
+        shapes = self._partitioner.kronecker_factor_shapes()
+        if statistics is None:
+            statistics = [init_scale * torch.eye(s[0], device=param.device) for s in shapes]
+            preconditioners = [torch.eye(s[0], device=param.device) for s in shapes]
+        if len(statistics) != len(shapes) or len(preconditioners) != len(shapes):
+            raise ValueError(f'{len(shapes)} statistics and preconditioners are needed.')
+        self.statistics = statistics
         self.preconditioners = preconditioners
         self.inverse_exponent = inverse_exponent
+        self.start_vector_fn = None     # optional: n -> [n] start vector of the power iteration
 
     @property
     def exponent(self):
-        return 2 * self.param.ndim if self.inverse_exponent == _invalid else self.inverse_exponent
+        return 2 * len(self._transformed_shape) if self.inverse_exponent == _invalid else self.inverse_exponent
 
-    def update_statistics(self):
+    def _blocks_of_grad(self):
         grad = self.param.grad
         if grad.dtype != torch.float32:
             raise TypeError('Shampoo statistics are float32: keep parameters (and so their gradients) in float32')
+        return self._partitioner.partition(grad.detach().reshape(self._transformed_shape))
+
+    def update_statistics(self):
         ema_decay = self.config.ema_decay
         alpha, beta = (1.0, 1.0) if ema_decay == _invalid else (float(ema_decay), 1.0 - float(ema_decay))
-        ndim = grad.ndim
-        for i in range(ndim):
-            stat = self.statistics[i]
-            if i == ndim - 1:
-                kernels.syrk_tn(grad.reshape(-1, grad.shape[-1]), out=stat, alpha=alpha, beta=beta)
-            elif i == 0:
-                kernels.syrk_nt(grad.reshape(grad.shape[0], -1), out=stat, alpha=alpha, beta=beta)
+        ndim = len(self._transformed_shape)
+        for j, block in enumerate(self._blocks_of_grad()):
+            block = block if block.is_contiguous() else block.contiguous()
+            for i in range(ndim):
+                _axis_statistic(block, i, self.statistics[j * ndim + i], alpha, beta)
+
+    def update_preconditioners(self):
+        """L^(-1/exponent) of every statistic, one at a time (asdl/precondition/shampoo.py:341-349); the gradient
+        maker takes the roots of its grouped statistics in batched calls instead."""
+        for i, stat in enumerate(self.statistics):
+            v0 = self.start_vector_fn(stat.shape[0]) if self.start_vector_fn is not None else None
+            root = compute_power(stat, self.exponent, ridge_epsilon=self.config.damping, start_vector=v0)
+            if isinstance(self.preconditioners[i], torch.Tensor) and self.preconditioners[i].shape == root.shape:
+                self.preconditioners[i].copy_(root)
             else:
-                kernels.syrk_nt(grad.movedim(i, 0).reshape(grad.shape[i], -1).contiguous(), out=stat, alpha=alpha, beta=beta)
+                self.preconditioners[i] = root
 
     def precondition(self):
-        grad = self.param.grad
-        cur = grad.detach()
-        for j in range(grad.ndim):
-            x2d = cur.reshape(cur.shape[0], -1)
-            cur = kernels.gemm(x2d, self.preconditioners[j], transA=True).view(*cur.shape[1:], cur.shape[0])
-        self.param.grad.data.copy_(cur.reshape(self.param.shape))
+        ndim = len(self._transformed_shape)
+        out = []
+        for j, block in enumerate(self._blocks_of_grad()):
+            block = block if block.is_contiguous() else block.contiguous()
+            out.append(_precondition_block(block, self.preconditioners[j * ndim:(j + 1) * ndim]))
+        merged = out[0] if len(out) == 1 else self._partitioner.merge_partitions(out)
+        self.param.grad.data.copy_(merged.reshape(self.param.shape))
 
 
 class ShampooGradientMaker(PreconditionedGradientMaker):
     """Shampoo (https://arxiv.org/abs/1802.09568) behind the GradientMaker interface; constructor of
-    asdl/precondition/shampoo.py:34-35.  ``block_size`` other than -1 is not supported (the reference
-    never forwards it to its Preconditioner either)."""
+    asdl/precondition/shampoo.py:34-35.  As in the reference, ``block_size`` is kept but not forwarded to the
+    Preconditioner objects (asdl/precondition/shampoo.py:53): there it only enters the cost model of the multi-GPU layer
+    assignment.  Preconditioner itself takes ``block_size`` / ``best_effort_shape_interpretation``."""
 
     def __init__(self, model: torch.nn.Module, config: PreconditioningConfig, block_size: int = _invalid,
                  sync_group=None, init_scale: float = 1e-12):
         super().__init__(model, config)
         if dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1:
             raise NotImplementedError('this build runs on one GPU')
-        if block_size != _invalid:
-            raise NotImplementedError('block partitioning is not on this path')
         self.sync_group = sync_group
         self.block_size = block_size
         self.world_rank, self.world_size = 0, 1
@@ -112,8 +214,8 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
                 views[(pi, axis)] = (stats[k], precs[k])
         self.preconditioners = []
         for pi, p in enumerate(params):
-            self.preconditioners.append(Preconditioner(p, config, [views[(pi, a)][0] for a in range(p.ndim)],
-                                                       [views[(pi, a)][1] for a in range(p.ndim)]))
+            self.preconditioners.append(Preconditioner(p, config, statistics=[views[(pi, a)][0] for a in range(p.ndim)],
+                                                       preconditioners=[views[(pi, a)][1] for a in range(p.ndim)]))
         self.start_vector_fn = None     # optional: (count, n, device) -> [count, n] start vectors
         self.last_root_stats = {}
 

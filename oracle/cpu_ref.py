@@ -34,6 +34,9 @@ reference checkout).  How each function is pinned (tests/test_oracle.py):
                         implements); golden SKFAC runs written from the reference
   *_cov_swift_*         the row sums of F.unfold / of the output gradient (library routines);
                         golden SKFAC runs (swift=True) written from the reference
+  merge_small_dims /    the two worked examples in the docstring of asdl/precondition/shampoo.py:370-384;
+  block_slices /        partition + merge round trip, block statistics against tensordot on slices; golden
+  PartitionedShampoo..  runs of the reference's Preconditioner with block_size and dimension merging
   power_iter            eigvalsh lambda_max (converged limit only)
   compute_power         fp64 eigh closed form (S + rI)^(-1/p), X^p (S + rI) == I;
                         golden trajectories written from the reference
@@ -55,6 +58,7 @@ __all__ = [
     'ema_accumulate', 'kron_damping', 'cholesky_inv', 'kron_update_inv', 'kron_mvp',
     'power_iter', 'mat_power', 'compute_power', 'shampoo_statistics', 'shampoo_precondition',
     'matrix_to_tril', 'tril_to_matrix', 'KfacOracle', 'ShampooOracle',
+    'merge_small_dims', 'block_slices', 'PartitionedShampooOracle',
     'linear_cov_swift', 'conv_cov_swift_kron_A', 'conv_cov_swift_kron_B', 'swift_kron_damping', 'smw_inv', 'swift_inv',
 ]
 
@@ -292,6 +296,67 @@ def shampoo_precondition(grad, preconditioners):
     for P in preconditioners:
         out = torch.tensordot(out, P, [[0], [0]])
     return out
+
+
+def merge_small_dims(shape, max_dim):
+    """asdl/precondition/shampoo.py:370-395."""
+    out, prod = [], 1
+    for d in shape:
+        if prod * d <= max_dim:
+            prod *= d
+        else:
+            if prod > 1:
+                out.append(prod)
+            prod = d
+    if prod > 1:
+        out.append(prod)
+    return out
+
+
+def block_slices(shape, block_size):
+    """Index ranges of the blocks of BlockPartitioner (asdl/precondition/shampoo.py:405-447), first axis slowest."""
+    import itertools
+    per_axis = []
+    for d in shape:
+        if block_size != -1 and d > block_size:
+            per_axis.append([slice(a, min(a + block_size, d)) for a in range(0, d, block_size)])
+        else:
+            per_axis.append([slice(0, d)])
+    return list(itertools.product(*per_axis))
+
+
+class PartitionedShampooOracle:
+    """One parameter's Preconditioner with block partitioning and dimension merging
+    (asdl/precondition/shampoo.py:300-367)."""
+
+    def __init__(self, shape, block_size=-1, merge=False, damping=1e-7, ema_decay=-1, init_scale=1e-12):
+        self.shape = tuple(shape)
+        self.tshape = tuple(merge_small_dims(shape, block_size)) if merge else tuple(shape)
+        self.blocks = block_slices(self.tshape, block_size)
+        self.damping, self.ema_decay = damping, ema_decay
+        self.statistics = [init_scale * torch.eye(s.stop - s.start) for blk in self.blocks for s in blk]
+        self.preconditioners = [torch.eye(s.stop - s.start) for blk in self.blocks for s in blk]
+
+    def update_statistics(self, grad):
+        g = grad.reshape(self.tshape)
+        nd = len(self.tshape)
+        for j, blk in enumerate(self.blocks):
+            shampoo_statistics(g[blk], self.statistics[j * nd:(j + 1) * nd], self.ema_decay)
+
+    def update_preconditioners(self, start_vectors):
+        exp = 2 * len(self.tshape)
+        for i, stat in enumerate(self.statistics):
+            n = stat.shape[0]
+            self.preconditioners[i] = compute_power(stat, exp, start_vectors(n), ridge_epsilon=self.damping)[0] \
+                if n > 1 else torch.eye(1)
+
+    def precondition(self, grad):
+        g = grad.reshape(self.tshape)
+        nd = len(self.tshape)
+        out = torch.empty(self.tshape)
+        for j, blk in enumerate(self.blocks):
+            out[blk] = shampoo_precondition(g[blk], self.preconditioners[j * nd:(j + 1) * nd])
+        return out.reshape(self.shape)
 
 
 # --------------------------------------------------------------------------- end-to-end K-FAC

@@ -196,13 +196,54 @@ def main_swift():
     run_kfac('swift_mlpw_fisher_emp_ema-1', get_mlp_wide(), xs, ts, 'fisher_emp', -1, 1e-2, swift=True)
 
 
+def run_partitioned(tag, shape, block_size, merge, damping, ema_decay, seed):
+    """The reference's Preconditioner driven directly (ShampooGradientMaker never passes it a block size)."""
+    from asdl.precondition.shampoo import Preconditioner
+    out = {}
+    g = torch.Generator().manual_seed(seed)
+    param = torch.nn.Parameter(torch.randn(*shape, generator=g))
+    config = PreconditioningConfig(damping=damping, ema_decay=ema_decay)
+    prec = Preconditioner(param, config, block_size=block_size, best_effort_shape_interpretation=merge)
+    out['shape'] = np.array(shape)
+    out['block_size'] = np.array(block_size)
+    out['merge'] = np.array(int(merge))
+    out['damping'] = np.array(damping)
+    out['ema_decay'] = np.array(ema_decay)
+    out['seed'] = np.array(seed)
+    for step in range(3):
+        grad = torch.randn(*shape, generator=g)
+        param.grad = grad.clone()
+        out[f'step{step}/grad_in'] = grad.numpy().copy()
+        prec.update_statistics()
+        torch.manual_seed(1000 * seed + step)          # the start vectors of the power iterations
+        prec.update_preconditioners()
+        prec.precondition()
+        out[f'step{step}/grad_out'] = param.grad.detach().numpy().copy()
+        for i, (st, pm) in enumerate(zip(prec.statistics, prec.preconditioners)):
+            out[f'step{step}/stat/{i}'] = st.numpy().copy()
+            out[f'step{step}/prec/{i}'] = pm.numpy().copy()
+    np.savez_compressed(os.path.join(HERE, f'shampoo_blocks_{tag}.npz'), **out)
+    print('wrote shampoo blocks', tag, len(out))
+
+
+def main_blocks():
+    run_partitioned('mat_10x6_b4', (10, 6), 4, False, 1e-6, -1, 31)
+    # best_effort_shape_interpretation=True cannot be recorded: the reference compares torch.Size with the merged
+    # list in BlockPartitioner.partition and raises ValueError for every input
+    run_partitioned('mat_9x13_b5_ema', (9, 13), 5, False, 1e-5, 0.2, 32)
+    run_partitioned('conv_5x4x3x3_b4', (5, 4, 3, 3), 4, False, 1e-6, -1, 33)
+
+
 def main():
+    if len(sys.argv) > 1 and sys.argv[1] == 'blocks':
+        return main_blocks()
     if len(sys.argv) > 1 and sys.argv[1] == 'bn':
         return main_bn()
     if len(sys.argv) > 1 and sys.argv[1] == 'swift':
         return main_swift()
     main_bn()
     main_swift()
+    main_blocks()
     torch.manual_seed(0)
     bs = 8
     xs = [torch.randn(bs, 5) for _ in range(3)]

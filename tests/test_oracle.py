@@ -404,3 +404,40 @@ def test_swift_factors_are_row_sums_or_the_ordinary_factors():
     la, lb = R.swift_kron_damping(a, torch.eye(5) * 2.0, 1e-2)
     pi = ((a ** 2).sum() / 8 / 2.0) ** 0.5
     assert abs(la - 0.1 * float(pi)) < 1e-6 and abs(lb - 0.1 / float(pi)) < 1e-6
+
+
+def test_merge_small_dims_and_block_partition():
+    # the worked examples of asdl/precondition/shampoo.py:370-384
+    assert R.merge_small_dims([1, 2, 512, 1, 2048, 1, 3, 4], 1024) == [1024, 2048, 12]
+    assert R.merge_small_dims([1, 2, 768, 1, 2048], 1024) == [2, 768, 2048]
+    # the example of the class docstring (:398-404): (4096, 512) with blocks of 1024 -> four (1024, 512) tensors
+    blocks = R.block_slices((4096, 512), 1024)
+    assert [(b[0].stop - b[0].start, b[1].stop - b[1].start) for b in blocks] == [(1024, 512)] * 4
+    # ragged last block, first axis slowest, every element in exactly one block
+    blocks = R.block_slices((10, 6), 4)
+    assert [(b[0].start, b[0].stop, b[1].start, b[1].stop) for b in blocks] == \
+        [(0, 4, 0, 4), (0, 4, 4, 6), (4, 8, 0, 4), (4, 8, 4, 6), (8, 10, 0, 4), (8, 10, 4, 6)]
+    count = torch.zeros(10, 6)
+    for b in blocks:
+        count[b] += 1
+    assert bool((count == 1).all())
+    assert R.block_slices((3, 5), -1) == [(slice(0, 3), slice(0, 5))]
+
+
+@pytest.mark.parametrize('tag', ['mat_10x6_b4', 'mat_9x13_b5_ema', 'conv_5x4x3x3_b4'])
+def test_partitioned_shampoo_oracle_matches_reference_golden(tag):
+    z = np.load(os.path.join(GOLDEN, f'shampoo_blocks_{tag}.npz'))
+    orc = R.PartitionedShampooOracle(tuple(int(v) for v in z['shape']), int(z['block_size']), bool(int(z['merge'])),
+                                     float(z['damping']), float(z['ema_decay']))
+    n_stats = len(orc.statistics)
+    assert n_stats == len([k for k in z.files if k.startswith('step0/stat/')])
+    for step in range(3):
+        grad = torch.from_numpy(z[f'step{step}/grad_in'])
+        orc.update_statistics(grad)
+        torch.manual_seed(1000 * int(z['seed']) + step)
+        orc.update_preconditioners(lambda n: torch.rand(n) * 2 - 1)
+        out = orc.precondition(grad)
+        for i in range(n_stats):
+            torch.testing.assert_close(orc.statistics[i], torch.from_numpy(z[f'step{step}/stat/{i}']), rtol=1e-5, atol=1e-12)
+            assert relerr(orc.preconditioners[i], torch.from_numpy(z[f'step{step}/prec/{i}'])) < 1e-4, (tag, step, i)
+        assert relerr(out, torch.from_numpy(z[f'step{step}/grad_out'])) < 1e-4, (tag, step)

@@ -184,3 +184,67 @@ def test_shampoo_gpt2_shaped_mini_vs_oracle():
                 continue
             e = relerr(p_gpu.grad, p_cpu.grad)
             assert e < 5e-3, (step, name, e)
+
+
+@pytest.mark.parametrize('tag', ['mat_10x6_b4', 'mat_9x13_b5_ema', 'conv_5x4x3x3_b4'])
+def test_block_partitioned_preconditioner_matches_reference_golden(tag):
+    """Preconditioner(param, config, block_size=...) driven directly, as recorded from the reference
+    (asdl/precondition/shampoo.py:300-367, 398-462)."""
+    from asdl_amd.shampoo import Preconditioner
+    z = np.load(os.path.join(GOLDEN, f'shampoo_blocks_{tag}.npz'))
+    shape = tuple(int(v) for v in z['shape'])
+    param = nn.Parameter(torch.zeros(*shape).cuda())
+    config = PreconditioningConfig(damping=float(z['damping']), ema_decay=float(z['ema_decay']))
+    prec = Preconditioner(param, config, block_size=int(z['block_size']))
+    exp = 2 * len(shape)
+    for step in range(3):
+        grad = torch.from_numpy(z[f'step{step}/grad_in'])
+        param.grad = grad.clone().cuda()
+        print(f'shampoo blocks {tag} step {step}', flush=True)
+        prec.update_statistics()
+        gen = torch.Generator().manual_seed(1000 * int(z['seed']) + step)
+        prec.start_vector_fn = lambda n, _g=gen: (torch.rand(n, generator=_g) * 2 - 1).cuda()
+        prec.update_preconditioners()
+        prec.precondition()
+        worst_ref = 0.0
+        for i, (st, pm) in enumerate(zip(prec.statistics, prec.preconditioners)):
+            after = torch.from_numpy(z[f'step{step}/stat/{i}'])
+            torch.testing.assert_close(st.cpu(), after, rtol=1e-4, atol=1e-12)
+            if after.shape[0] > 1:
+                worst_ref = max(worst_ref, _check_root(pm, torch.from_numpy(z[f'step{step}/prec/{i}']), after, exp,
+                                                       (tag, step, i)) or 0.0)
+        assert relerr(param.grad, torch.from_numpy(z[f'step{step}/grad_out'])) < max(1e-3, 8 * worst_ref), (tag, step)
+
+
+def test_block_partitioner_and_dimension_merging():
+    from asdl_amd.shampoo import BlockPartitioner, Preconditioner, _merge_small_dims
+    assert _merge_small_dims([1, 2, 512, 1, 2048, 1, 3, 4], 1024) == [1024, 2048, 12]
+    assert _merge_small_dims([1, 2, 768, 1, 2048], 1024) == [2, 768, 2048]
+    g = torch.Generator().manual_seed(1)
+    t = torch.randn(10, 6, 7, generator=g).cuda()
+    bp = BlockPartitioner(t.shape, 4)
+    parts = bp.partition(t)
+    want = [t[b] for b in R.block_slices((10, 6, 7), 4)]
+    assert len(parts) == len(want) == 12 and all(torch.equal(a, b) for a, b in zip(parts, want))
+    assert bp.kronecker_factor_shapes()[:3] == [[4, 4], [4, 4], [4, 4]] and bp.num_splits() == 3
+    assert torch.equal(bp.merge_partitions(parts), t)
+    # merged dimensions: a (6, 3, 2, 2) weight with max_dim 8 is preconditioned as (6, 6, 2), against the oracle
+    param = nn.Parameter(torch.zeros(6, 3, 2, 2).cuda())
+    prec = Preconditioner(param, PreconditioningConfig(damping=1e-4, ema_decay=-1), block_size=8,
+                          best_effort_shape_interpretation=True)
+    orc = R.PartitionedShampooOracle((6, 3, 2, 2), 8, True, damping=1e-4)
+    assert [tuple(s.shape) for s in prec.statistics] == [(6, 6), (6, 6), (2, 2)]
+    for step in range(2):
+        grad = torch.randn(6, 3, 2, 2, generator=g)
+        param.grad = grad.clone().cuda()
+        prec.update_statistics()
+        orc.update_statistics(grad)
+        vecs = [torch.rand(n, generator=g) * 2 - 1 for n in (6, 6, 2)]
+        it_a, it_b = iter(vecs), iter(vecs)
+        prec.start_vector_fn = lambda n: next(it_a).cuda()
+        prec.update_preconditioners()
+        orc.update_preconditioners(lambda n: next(it_b))
+        prec.precondition()
+        for a, b in zip(prec.statistics, orc.statistics):
+            assert relerr(a, b) < 1e-5
+        assert relerr(param.grad, orc.precondition(grad)) < 1e-3
