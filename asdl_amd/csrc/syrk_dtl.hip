@@ -21,6 +21,9 @@
 // outside the image) are given a byte offset beyond the buffer range, for which the hardware returns
 // zeros, so the main loop has no masks and no branches.
 #include <cmath>
+#include <initializer_list>
+#include <mutex>
+#include <unordered_map>
 #include <type_traits>
 #include "common.hpp"
 
@@ -409,7 +412,7 @@ static int g_force_bt = 0, g_force_ns = 0;   // tuning hook (ak_debug_force_syrk
 // Tile size and split-K factor from a small cost model (microseconds, constants measured on MI355X): the
 // k-tiles of one split times the k-tile time of the most loaded CU, a fixed charge per work group, the
 // partial-tile traffic and the reduction passes.
-static DtlPlan dtl_plan(int64_t M, int64_t d, int64_t max_rows_per_split, bool gather) {
+static DtlPlan dtl_plan_search(int64_t M, int64_t d, int64_t max_rows_per_split, bool gather) {
   struct Cand { int bt; int occ; double t_alone, t_shared, t_fix; };
   // t_alone: k-tile time of a work group that has its CU to itself, t_shared: with `occ` of them on the CU
   const Cand cands[3] = {{64, 4, 0.20, 0.20, 3.0},
@@ -466,6 +469,37 @@ static DtlPlan dtl_plan(int64_t M, int64_t d, int64_t max_rows_per_split, bool g
   }
   best.ws_bytes = parts * best.ntiles * best.bt * best.bt * sizeof(float);
   return best;
+}
+
+// The search above walks over up to 3 x 1024 candidates (tens of microseconds on the host): the same few shapes
+// recur every step, so the plans are memoised.  Entry points may be called from several host threads.
+static DtlPlan dtl_plan(int64_t M, int64_t d, int64_t max_rows_per_split, bool gather) {
+  struct Key {
+    int64_t M, d, rows;
+    int gather, bt, ns;
+    bool operator==(const Key& o) const {
+      return M == o.M && d == o.d && rows == o.rows && gather == o.gather && bt == o.bt && ns == o.ns;
+    }
+  };
+  struct Hash {
+    size_t operator()(const Key& k) const {
+      uint64_t h = 0x9e3779b97f4a7c15ull;
+      for (uint64_t v : {static_cast<uint64_t>(k.M), static_cast<uint64_t>(k.d), static_cast<uint64_t>(k.rows),
+                         static_cast<uint64_t>(k.gather), static_cast<uint64_t>(k.bt), static_cast<uint64_t>(k.ns)})
+        h = (h ^ v) * 0xff51afd7ed558ccdull + (h >> 29);
+      return static_cast<size_t>(h);
+    }
+  };
+  static std::unordered_map<Key, DtlPlan, Hash> cache;
+  static std::mutex lock;
+  const Key key{M, d, max_rows_per_split, gather ? 1 : 0, g_force_bt, g_force_ns};
+  std::lock_guard<std::mutex> guard(lock);
+  auto it = cache.find(key);
+  if (it != cache.end()) return it->second;
+  if (cache.size() > 4096) cache.clear();
+  const DtlPlan plan = dtl_plan_search(M, d, max_rows_per_split, gather);
+  cache.emplace(key, plan);
+  return plan;
 }
 
 template <int WR, int WC, int FR, int FC, bool GATHER>
