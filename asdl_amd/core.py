@@ -86,7 +86,8 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
 
 def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, vectors=None, stream=None,
                     calc_inv=False, factor_stream=None) -> OperationContext:
-    """Maps Fisher shapes to operations (asdl/core.py:83-97); only SHAPE_KRON has kernels here."""
+    """Maps Fisher shapes to operations (asdl/core.py:83-97): the Kronecker-factored, swift Kronecker-factored and
+    unit-wise shapes have kernels here."""
     if cvp:
         raise NotImplementedError('covariance-vector products are not on this path')
 

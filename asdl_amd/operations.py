@@ -1,9 +1,9 @@
 """Per-layer operations of the K-FAC path and the context that stores their results.
 
 Mirrors the operator seam of the reference (asdl/operations/operation.py:87-548 for Operation,
-:551-964 for OperationContext, asdl/operations/linear.py and conv.py for the layer classes) for the
-two operations on this path, OP_COV_KRON and OP_COV_KRON_INV.  Differences that come from running
-on the GPU kernels:
+:551-964 for OperationContext, asdl/operations/linear.py, conv.py, batchnorm.py and layernorm.py for the layer
+classes) for the operations on this path: OP_COV_KRON(_INV), OP_COV_SWIFT_KRON(_INV) and OP_COV_UNIT_WISE(_INV).
+Differences that come from running on the GPU kernels:
 
 * cov_kron_A / cov_kron_B take optional ``out``, ``alpha``, ``beta`` and compute
   ``out <- beta*out + alpha*factor`` in one launch, so the reference's separate

@@ -1,9 +1,9 @@
-"""Containers of the curvature matrices on the K-FAC path: SymMatrix and its Kronecker part.
+"""Containers of the curvature matrices on the K-FAC path: SymMatrix, its Kronecker part (square factors or the
+row matrices of the swift variant) and the unit-wise 2 x 2 blocks, with their packed on-disk form.
 
-Same attributes and call signatures as asdl/symmatrix.py (SymMatrix :94-358, Kron :361-548);
-the arithmetic runs in the HIP kernels.  Only the Kronecker-factored shape is on this path:
-full / layer-wise / KFE / unit-wise / diagonal containers are accepted as opaque attributes but
-have no kernels here.
+Same attributes and call signatures as asdl/symmatrix.py (SymMatrix :94-358, Kron :361-548, UnitWise :617-719,
+save / load :25-87, 226-269, 471-492); the arithmetic runs in the HIP kernels.  Full / layer-wise matrices can be
+saved and loaded; KFE and diagonal containers are accepted as opaque attributes but have no kernels here.
 """
 import os
 from collections import defaultdict
