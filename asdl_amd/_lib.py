@@ -44,6 +44,11 @@ _SIGNATURES = {
     'ak_smw_inv_ws_bytes': (c_size, [c_i64, c_i64]),
     'ak_smw_inv': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
     'ak_smw_finish': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
+    'ak_event_create': (c_int, [ctypes.POINTER(ctypes.c_void_p), c_int]),
+    'ak_event_destroy': (c_int, [c_ptr]),
+    'ak_event_record': (c_int, [c_ptr, c_ptr]),
+    'ak_stream_order': (c_int, [c_ptr, c_ptr, c_ptr]),
+    'ak_event_elapsed_ms': (c_int, [c_ptr, c_ptr, ctypes.POINTER(ctypes.c_float)]),
     'ak_tril_pack': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     'ak_tril_unpack': (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_ptr]),
     'ak_gemm_f32': (c_int, [c_int, c_int, c_i64, c_i64, c_i64, c_f32, c_ptr, c_i64, c_ptr, c_i64, c_f32,

@@ -21,10 +21,9 @@ __all__ = ['extend', 'no_centered_cov', 'module_wise_assignments', 'modules_to_a
 def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, stream=None,
            factor_stream=None) -> OperationContext:
     """``stream``: as in the reference, the hook operations run under ``torch.cuda.stream(stream)``.
-    ``factor_stream``: the hook operations run on that stream, ordered after the kernels that produced their
-    inputs (the producing stream is waited for, the inputs are kept alive with record_stream), so that the
-    statistics kernels overlap the forward / backward kernels that follow; OperationContext.join_factor_stream()
-    orders the consumers after them."""
+    ``factor_stream``: a kernels.FactorStream; the hook operations launch on its side stream, ordered after the
+    kernels that produced their inputs, so that the statistics kernels overlap the forward / backward kernels that
+    follow; OperationContext.join_factor_stream() orders the consumers after them."""
     handles = []
     cxt = OperationContext(vectors=vectors)
     use_stream = torch.cuda.is_available() and stream is not None
@@ -39,11 +38,7 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
             with stream_cxt():
                 fn()
             return
-        fs.wait_stream(torch.cuda.current_stream(tensors[0].device))
-        with torch.cuda.stream(fs):
-            fn()
-        for t in tensors:
-            t.record_stream(fs)
+        fs.run(fn, *tensors)
 
     try:
         for module, names in module_wise_assignments(model, *op_names, ignore_modules=ignore_modules, map_rule=map_rule):

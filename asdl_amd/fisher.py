@@ -20,7 +20,7 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
-FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (costs more host time per hook than the overlap gains)
+FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (ordering the two streams costs ~30 us of host time per hook: more than the overlap gains)
 PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
 EAGER_INVERSE = True        # start the bulk of the inverses during a single sampled / empirical backward pass: the longest chains get a head start
 
@@ -66,7 +66,8 @@ class FisherMaker(GradientMaker):
             return None
         fs = getattr(self, '_factor_stream_obj', None)
         if fs is None or fs.device != p.device:
-            fs = torch.cuda.Stream(device=p.device)
+            from .kernels import FactorStream
+            fs = FactorStream(p.device)
             self._factor_stream_obj = fs
         return fs
 

@@ -4,6 +4,7 @@ Every function takes tensors that live on a ROCm device, passes raw device point
 calling thread's current HIP stream to libasdl_amd.so, and returns without synchronising.
 There is no CPU path: a CPU tensor raises.
 """
+import contextlib
 import ctypes
 import threading
 
@@ -22,6 +23,30 @@ _timing_sink = None      # when set to a list, factor launches append (name, flo
 _event_pool = []         # pre-created timing events: creating one costs more host time than recording it
 
 
+class _RawEvent:
+    """Timing event of the HIP runtime recorded on an explicit stream handle (torch.cuda.Event only sees torch's
+    current stream, not the side stream a FactorStream launches on)."""
+
+    def __init__(self):
+        handle = ctypes.c_void_p()
+        _lib.check(_lib.load().ak_event_create(ctypes.byref(handle), 1), 'ak_event_create')
+        self.handle = handle
+
+    def record(self):
+        _lib.check(_lib.load().ak_event_record(self.handle, _stream()), 'ak_event_record')
+
+    def elapsed_time(self, other):
+        ms = ctypes.c_float()
+        _lib.check(_lib.load().ak_event_elapsed_ms(self.handle, other.handle, ctypes.byref(ms)), 'ak_event_elapsed_ms')
+        return ms.value
+
+    def __del__(self):
+        try:
+            _lib.load().ak_event_destroy(self.handle)
+        except Exception:
+            pass
+
+
 def set_timing_sink(sink, n_events=0):
     """Benchmark instrumentation: with a list as sink every factor-statistics launch is bracketed by
     two events on the launching stream and recorded with its algorithmic FLOP count M*d*(d+1).
@@ -30,7 +55,7 @@ def set_timing_sink(sink, n_events=0):
     _timing_sink = sink
     del _event_pool[:]
     if sink is not None:
-        _event_pool.extend(torch.cuda.Event(enable_timing=True) for _ in range(n_events))
+        _event_pool.extend(_RawEvent() for _ in range(n_events))
 
 
 def enable_timing(flag):
@@ -43,7 +68,7 @@ _timing_on = True
 
 
 def _timing_event():
-    return _event_pool.pop() if _event_pool else torch.cuda.Event(enable_timing=True)
+    return _event_pool.pop() if _event_pool else _RawEvent()
 
 
 class _Timed:
@@ -75,8 +100,15 @@ def _require_gpu(*tensors):
 _raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
 
 
+_override = threading.local()      # .handle: stream the calling thread's kernel launches go to instead of the current one
+
+
 def _stream_handle(device=None):
-    """The calling thread's current HIP stream on ``device`` as an integer handle."""
+    """The calling thread's current HIP stream on ``device`` as an integer handle (or the side stream a
+    FactorStream has switched this thread to)."""
+    forced = getattr(_override, 'handle', None)
+    if forced is not None:
+        return forced
     if _raw_stream is not None:
         idx = device.index if device is not None and device.index is not None else torch.cuda.current_device()
         return _raw_stream(idx)
@@ -166,6 +198,83 @@ def device_ints(values, device, dtype=torch.int64):
     return t
 
 
+class main_stream_launches:
+    """Context: inside FactorStream.run(), kernel launches of this thread go to its current stream again."""
+
+    def __enter__(self):
+        self._saved = (getattr(_override, 'handle', None), getattr(_override, 'stream', None))
+        _override.handle = _override.stream = None
+
+    def __exit__(self, *exc):
+        _override.handle, _override.stream = self._saved
+        return False
+
+
+def _on_launch_stream():
+    """Context for the few framework ops (copies to a contiguous layout, casts) that feed a kernel: they have to run
+    on the stream the kernel is launched on."""
+    st = getattr(_override, 'stream', None)
+    return torch.cuda.stream(st) if st is not None else contextlib.nullcontext()
+
+
+def _contiguous(x):
+    if x.is_contiguous():
+        return x
+    with _on_launch_stream():
+        return x.contiguous()
+
+
+class FactorStream:
+    """A side stream (default priority) for the statistics kernels of the hooks.  ``run(fn, *tensors)`` orders the
+    side stream after everything the calling thread's current stream holds, runs ``fn`` with this thread's kernel
+    launches redirected to the side stream, and keeps ``tensors`` alive until ``join()`` makes the current stream
+    wait for the side stream (the caching allocator would otherwise hand a freed gradient buffer to the next kernel
+    of the main stream while the side stream still reads it)."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.stream = torch.cuda.Stream(device=self.device)
+        self.handle = self.stream.cuda_stream
+        lib = _lib.load()
+        self._events = []
+        for _ in range(8):
+            ev = ctypes.c_void_p()
+            _lib.check(lib.ak_event_create(ctypes.byref(ev), 0), 'ak_event_create')
+            self._events.append(ev)
+        self._next = 0
+        self._keep = []
+
+    def _event(self):
+        ev = self._events[self._next]
+        self._next = (self._next + 1) % len(self._events)
+        return ev
+
+    def run(self, fn, *tensors):
+        main = _stream_handle(self.device)
+        _lib.check(_lib.load().ak_stream_order(ctypes.c_void_p(main), ctypes.c_void_p(self.handle), self._event()),
+                   'ak_stream_order')
+        self._keep.append(tensors)
+        _override.handle, _override.stream = self.handle, self.stream
+        try:
+            fn()
+        finally:
+            _override.handle = _override.stream = None
+
+    def join(self):
+        main = _stream_handle(self.device)
+        _lib.check(_lib.load().ak_stream_order(ctypes.c_void_p(self.handle), ctypes.c_void_p(main), self._event()),
+                   'ak_stream_order')
+        keep, self._keep = self._keep, []
+        return keep          # the caller may drop these once work enqueued after the join has been issued
+
+    def __del__(self):
+        try:
+            for ev in self._events:
+                _lib.load().ak_event_destroy(ev)
+        except Exception:
+            pass
+
+
 # ------------------------------------------------------------------------------ factors
 def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     """out <- beta*out + alpha * x^T x for x = [M, d] (rows may be strided, columns contiguous)."""
@@ -173,11 +282,11 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     if x.ndim != 2:
         raise ValueError(f'x.ndim has to be 2. Got {x.ndim}.')
     if x.stride(1) != 1 and x.shape[1] > 1:
-        x = x.contiguous()
+        x = _contiguous(x)
     M, d = x.shape
     ldx = x.stride(0) if M > 1 else max(d, x.stride(0))
     if ldx < d:
-        x = x.contiguous()
+        x = _contiguous(x)
         ldx = d
     if out is None:
         out = torch.empty(d, d, dtype=torch.float32, device=x.device)
@@ -234,7 +343,7 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
         if rc != AK_ERR_UNSUPPORTED:
             _lib.check(rc, 'ak_conv_syrk_nhwc')
             return out
-    x = x.contiguous()
+    x = _contiguous(x)
     need = _ws_need('ak_conv_syrk_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
     ws, ws_bytes, keep = _ws_args(need, x.device)
     with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
@@ -281,14 +390,15 @@ def unit_wise_stats(y, g, weight, bias, out=None, alpha=1.0, beta=0.0):
 
     sy, sg = strides(y), strides(g)
     if sy is None:
-        y = y.contiguous()
+        y = _contiguous(y)
         sy = strides(y)
     if sg is None:
-        g = g.contiguous()
+        g = _contiguous(g)
         sg = strides(g)
     S = sy[3]
-    weight = weight.detach().float().contiguous()
-    bias = bias.detach().float().contiguous()
+    with _on_launch_stream():
+        weight = weight.detach().float().contiguous()
+        bias = bias.detach().float().contiguous()
     if out is None:
         out = torch.empty(F, 2, 2, dtype=torch.float32, device=y.device)
         beta = 0.0
@@ -417,7 +527,8 @@ def conv_patch_sum(x, kernel_size=(1, 1), stride=(1, 1), padding=(0, 0), out=Non
     if x.ndim != 4:
         raise ValueError(f'x.ndim has to be 2, 3 or 4. Got {x.ndim}.')
     if x.dtype not in (torch.float32, torch.bfloat16):
-        x = x.float()
+        with _on_launch_stream():
+            x = x.float()
     N, C, H, W = x.shape
     kh, kw = kernel_size
     sh, sw = stride

@@ -516,7 +516,7 @@ class OperationContext:
     def join_factor_stream(self):
         """Orders the current stream after the statistics kernels that ran on the factor stream."""
         if self.factor_stream is not None:
-            torch.cuda.current_stream(self.factor_stream.device).wait_stream(self.factor_stream)
+            self.factor_stream.join()
 
     # ---- deferred, batched inverses
     def set_eager_inverse(self, total_cost):
@@ -544,7 +544,11 @@ class OperationContext:
         if self._eager_total > 0 and not self._eager_done and \
                 self._inverse_cost >= EAGER_COST_FRACTION * self._eager_total:
             self._eager_done = True
-            self._enqueue_pending()
+            # this runs inside a backward hook: with a factor stream the hook's launches are redirected to it, and
+            # the factors queued so far were computed there
+            with kernels.main_stream_launches():
+                self.join_factor_stream()
+                self._enqueue_pending()
 
     def queue_unit_inverse(self, operation):
         if operation not in self._pending_unit:

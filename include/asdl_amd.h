@@ -232,6 +232,16 @@ int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, f
                        float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
                        ak_stream_t stream);
 
+/* ---- stream helpers (no counterpart in the reference) ------------------------------------ */
+
+/* For hosts that run the statistics kernels on a side stream: events of the HIP runtime this library is linked
+ * against, and `after` waits for what `before` holds so far (two runtime calls).  The caller owns the events. */
+int ak_event_create(void** event, int timing);
+int ak_event_destroy(void* event);
+int ak_event_record(void* event, ak_stream_t stream);
+int ak_stream_order(ak_stream_t before, ak_stream_t after, void* event);
+int ak_event_elapsed_ms(void* start, void* stop, float* ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -389,6 +389,15 @@ def test_early_start_of_inverses_gives_the_same_result(network, monkeypatch):
             assert relerr(eager[key], lazy[key]) < 3e-2, key
 
 
+@pytest.mark.parametrize('tag', ['cnn2_fisher_emp_ema0.5_int2', 'cnn_fisher_mc_ema-1', 'cnnbn_fisher_emp_ema-1'])
+def test_factor_side_stream_gives_the_golden_results(tag, monkeypatch):
+    """fisher.FACTOR_SIDE_STREAM (off by default: ordering the side stream costs more host time per hook than the
+    overlap gains on this runtime) runs the statistics kernels of the hooks on a side stream."""
+    import asdl_amd.fisher as fisher_mod
+    monkeypatch.setattr(fisher_mod, 'FACTOR_SIDE_STREAM', True)
+    test_kfac_gpu_matches_reference_golden(tag)
+
+
 def test_fisher_attributes_and_steps_without_curvature_update():
     torch.manual_seed(4)
     model = bench_models.mlp(20, 16, 5).cuda()
