@@ -120,7 +120,9 @@ def main():
         print('bench.py needs a ROCm GPU.', file=sys.stderr)
         sys.exit(2)
     dev = torch.device('cuda:0')
-    torch.backends.cudnn.benchmark = not args.no_conv_autotune
+    # MIOpen's search over NCHW bf16 solvers takes many minutes on a fresh machine: only the default layout is tuned
+    autotune = not args.no_conv_autotune and args.memory_format == 'channels_last'
+    torch.backends.cudnn.benchmark = autotune
     torch.manual_seed(0)
     model = bench_models.resnet50().to(dev)
     bs = args.batch
@@ -158,8 +160,11 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
+    for i in range(args.warmup):
         step()
+        if i == 0:
+            torch.cuda.synchronize()
+            print('bench.py: first warm-up step done (kernel selection, workspaces)', file=sys.stderr, flush=True)
     sink = None if args.no_factor_timing else []
     kernels.set_timing_sink(sink, n_events=2 * 110 * args.steps)     # two events per factor call, made up front
     torch.cuda.synchronize()
@@ -192,7 +197,7 @@ def main():
                                f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
                                f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights, '
-                               f'cudnn.benchmark {"off" if args.no_conv_autotune else "on"}' + (', swift (SKFAC) factors' if args.swift else ''),
+                               f'cudnn.benchmark {"on" if autotune else "off"}' + (', swift (SKFAC) factors' if args.swift else ''),
                    'batch': bs},
     }
     if sink:
