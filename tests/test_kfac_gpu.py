@@ -346,6 +346,60 @@ def test_resnet50_batch64_channels_last_properties():
     assert relerr(got, ref) < 1e-3, relerr(got, ref)
 
 
+def test_resnet18_cifar_batch128_fp32_properties():
+    """BASELINE's third configuration at full size (fp32, NCHW, batch 128, Conv2d factors up to 4608 x 4608), checked
+    through the same size-independent properties as the ResNet-50 test."""
+    torch.manual_seed(8)
+    bs, damping, ema = 128, 1e-3, 0.5
+    model = bench_models.resnet18_cifar().cuda()
+    x, t = torch.randn(bs, 3, 32, 32).cuda(), torch.randint(0, 10, (bs,)).cuda()
+    picks = ['conv1', 'layer1.0.conv2', 'layer2.0.conv1', 'layer3.0.shortcut.0', 'layer4.1.conv2', 'linear']
+    mods = dict(model.named_modules())
+    ins, gouts, handles = {}, {}, []
+    for name in picks:
+        def fhook(mod, inp, out, name=name):
+            ins[name] = inp[0].detach()
+            out.register_hook(lambda g, name=name: gouts.__setitem__(name, g.detach()))
+        handles.append(mods[name].register_forward_hook(fhook))
+    raw = {}
+    handles.append(mods['layer4.1.conv2'].weight.register_hook(lambda g: raw.__setitem__('g', g.detach().clone())))
+    config = PreconditioningConfig(data_size=bs, damping=damping, ema_decay=ema,
+                                   ignore_modules=[nn.BatchNorm2d, nn.BatchNorm1d])
+    gm = KfacGradientMaker(model, config, fisher_type=FISHER_EMP)
+    model.zero_grad(set_to_none=True)
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+    gm.forward_and_backward()
+    for h in handles:
+        h.remove()
+    for name in picks:
+        m = mods[name]
+        kron = m.fisher.kron
+        a, g = ins[name].double(), gouts[name].double()
+        if isinstance(m, nn.Conv2d):
+            u = F.unfold(a, m.kernel_size, padding=m.padding, stride=m.stride)
+            U = u.permute(1, 0, 2).reshape(u.shape[1], -1)
+            A_ref = ema * (U @ U.T) / u.shape[-1] / bs
+            del u, U
+            g2 = g.permute(0, 2, 3, 1).reshape(-1, g.shape[1])
+        else:
+            A_ref, g2 = ema * a.T @ a / bs, g
+        B_ref = ema * g2.T @ g2 / bs
+        assert relerr(kron.A, A_ref) < 1e-5, (name, 'A', relerr(kron.A, A_ref))
+        assert relerr(kron.B, B_ref) < 1e-5, (name, 'B', relerr(kron.B, B_ref))
+        assert torch.equal(kron.A, kron.A.T) and torch.equal(kron.B, kron.B.T)
+        dA, dB = kron.A.shape[0], kron.B.shape[0]
+        pi = ((float(kron.A.diagonal().sum().double()) / dA) / (float(kron.B.diagonal().sum().double()) / dB)) ** 0.5
+        for which, lam, dim in (('A', max(damping ** 0.5 * pi, 1e-7), dA), ('B', max(damping ** 0.5 / pi, 1e-7), dB)):
+            F_, inv = getattr(kron, which).double(), getattr(kron, which + '_inv').double()
+            eye = torch.eye(dim, dtype=torch.float64, device='cuda')
+            resid = (F_ + lam * eye) @ inv - eye
+            assert float(resid.norm()) / dim ** 0.5 < 2e-3, (name, which, float(resid.norm()) / dim ** 0.5)
+    m = mods['layer4.1.conv2']
+    G = raw['g'].double().reshape(m.weight.shape[0], -1) / bs
+    ref = m.fisher.kron.B_inv.double() @ G @ m.fisher.kron.A_inv.double()
+    assert relerr(m.weight.grad.detach().double().reshape(m.weight.shape[0], -1), ref) < 1e-3
+
+
 @pytest.mark.parametrize('network', ['mlp', 'resnet18'])
 def test_early_start_of_inverses_gives_the_same_result(network, monkeypatch):
     """fisher.EAGER_INVERSE starts the inverse of the layers whose factors are final while the backward pass still

@@ -248,3 +248,41 @@ def test_block_partitioner_and_dimension_merging():
         for a, b in zip(prec.statistics, orc.statistics):
             assert relerr(a, b) < 1e-5
         assert relerr(param.grad, orc.precondition(grad)) < 1e-3
+
+
+def test_shampoo_gpt2_small_weight_shapes_full_size():
+    """BASELINE's fifth configuration at the real weight shapes of one decoder block (768 x 2304 attention input,
+    768 x 768 attention output, 768 x 3072 and 3072 x 768 MLP): statistics against fp64 products of the very
+    gradients, inverse fourth roots through the closed form of the ridged statistic, and the preconditioned
+    gradient against P_L^T G P_R recomputed in fp64 from the stored roots."""
+    torch.manual_seed(9)
+    shapes = [(2304, 768), (768, 768), (3072, 768), (768, 3072)]
+    model = nn.Sequential(*[nn.Linear(i, o, bias=False) for o, i in shapes]).cuda()
+    params = [m.weight for m in model]
+    gm = ShampooGradientMaker(model, PreconditioningConfig(damping=1e-6, ema_decay=-1))
+    # statistics accumulated over five gradients, as in training: every statistic has full rank (a single gradient
+    # leaves the larger side of each weight rank deficient, cond = 1e6 after the ridge, where no fp32 root is accurate)
+    sums = [[torch.zeros(s[0], s[0], dtype=torch.float64, device='cuda'),
+             torch.zeros(s[1], s[1], dtype=torch.float64, device='cuda')] for s in shapes]
+    for _ in range(5):
+        grads = [torch.randn(*s).cuda() * 1e-2 for s in shapes]
+        for p, g, acc in zip(params, grads, sums):
+            p.grad = g.clone()
+            acc[0] += g.double() @ g.double().T
+            acc[1] += g.double().T @ g.double()
+        gm.update_curvature()
+    for prec, acc in zip(gm.preconditioners, sums):
+        for stat, ref in zip(prec.statistics, acc):
+            assert relerr(stat, ref) < 1e-5, relerr(stat, ref)
+    gm.update_preconditioner()
+    for prec, acc in zip(gm.preconditioners, sums):
+        for stat, root, ref in zip(prec.statistics, prec.preconditioners, acc):
+            lam_max = float(torch.linalg.eigvalsh(ref)[-1])
+            ridge = float((stat.double() - ref).diagonal().mean())      # the root computation leaves its ridge behind
+            assert abs(ridge - 1e-6 * lam_max) < 0.1 * 1e-6 * lam_max
+            exact = _closed_form_root(stat, 4)
+            assert exact is not None and relerr(root, exact) < 5e-3, relerr(root, exact)
+    gm.precondition()
+    for prec, g, p in zip(gm.preconditioners, grads, params):
+        ref = prec.preconditioners[0].double().T @ g.double() @ prec.preconditioners[1].double()
+        assert relerr(p.grad, ref) < 1e-4
