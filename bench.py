@@ -44,6 +44,10 @@ def parse():
     ap.add_argument('--with-batchnorm', action='store_true',
                     help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
                          '(the headline configuration ignores them, as the reference training script does)')
+    ap.add_argument('--workload', default='resnet50', choices=['resnet50', 'linear4096'],
+                    help="resnet50: the headline benchmark.  linear4096: BASELINE's second configuration, a single "
+                         'Linear 4096x4096 with bias on 8192 bf16 rows, EMA 0.95 (factor + inverse + precondition of one '
+                         'large layer; its own metric name, not the headline)')
     ap.add_argument('--swift', action='store_true',
                     help='KfacGradientMaker(swift=True): factors of layers with fewer samples than columns are kept as '
                          'row matrices (SKFAC); not the headline configuration')
@@ -124,15 +128,22 @@ def main():
     autotune = not args.no_conv_autotune and args.memory_format == 'channels_last'
     torch.backends.cudnn.benchmark = autotune
     torch.manual_seed(0)
-    model = bench_models.resnet50().to(dev)
-    bs = args.batch
-    x = torch.randn(bs, 3, 224, 224).to(dev)
-    if args.memory_format == 'channels_last':
-        model = model.to(memory_format=torch.channels_last)
-        x = x.contiguous(memory_format=torch.channels_last)
-    t = torch.randint(0, 1000, (bs,)).to(dev)
-    ignore = [] if args.with_batchnorm else [nn.BatchNorm2d]
-    config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=ignore)
+    if args.workload == 'linear4096':
+        model = nn.Sequential(nn.Linear(4096, 4096, bias=True)).to(dev)
+        bs = 8192
+        x = torch.randn(bs, 4096).to(dev).to(torch.bfloat16)
+        t = torch.randint(0, 4096, (bs,)).to(dev)
+        config = PreconditioningConfig(data_size=bs, damping=args.damping, ema_decay=0.95)
+    else:
+        model = bench_models.resnet50().to(dev)
+        bs = args.batch
+        x = torch.randn(bs, 3, 224, 224).to(dev)
+        if args.memory_format == 'channels_last':
+            model = model.to(memory_format=torch.channels_last)
+            x = x.contiguous(memory_format=torch.channels_last)
+        t = torch.randint(0, 1000, (bs,)).to(dev)
+        ignore = [] if args.with_batchnorm else [nn.BatchNorm2d]
+        config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=ignore)
     gm = KfacGradientMaker(model, config, fisher_type=args.fisher, swift=args.swift)
     opt = torch.optim.SGD(model.parameters(), lr=1e-4)
 
@@ -216,7 +227,15 @@ def main():
                            'factor_ms_per_step': secs / timed_steps * 1e3,
                            'timed_steps': timed_steps,
                            'gemm_equiv_tflops': 2 * achieved}
-    if not args.no_cpu_baseline:
+    if args.workload == 'linear4096':
+        out['metric'] = 'K-FAC steps/s Linear 4096x4096, 8192 rows'
+        out['config'] = {'workload': f'K-FAC step (factors with EMA 0.95 + pi-damped Cholesky inverses + precondition every '
+                                     f'step, {args.fisher}) on one Linear 4096x4096 with bias, 8192 N(0,1) rows, bf16 '
+                                     f'autocast, fp32 factors/inverses, damping {args.damping}', 'batch': bs}
+        if 'roofline' in out:
+            out['roofline']['traffic'] = None
+            out['roofline']['kernel'] = 'factor statistics (syrk_dtl_kernel, 8192 x 4096 bf16 operands), SYRK FLOP M*d*(d+1)'
+    elif not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(args)
     print(json.dumps(out))
 
