@@ -55,6 +55,10 @@ _SIGNATURES = {
                             c_ptr, c_i64, c_int, c_i64, c_i64, c_i64, c_ptr]),
     'ak_gemm_f32_split': (c_int, [c_int, c_int, c_int, c_i64, c_i64, c_i64, c_f32, c_ptr, c_i64, c_ptr, c_i64, c_f32,
                                   c_ptr, c_i64, c_int, c_i64, c_i64, c_i64, c_ptr]),
+    'ak_gemm_f32_grouped': (c_int, [c_int, c_ptr, c_int, c_i64, c_ptr]),
+    'ak_gemv_f32_grouped': (c_int, [c_ptr, c_int, c_i64, c_f32, c_ptr]),
+    'ak_weight_layout_max_row': (c_i64, []),
+    'ak_weight_layout_grouped': (c_int, [c_ptr, c_int, c_i64, c_int, c_ptr]),
     'ak_kron_precond_ws_bytes': (c_size, [c_i64, c_i64]),
     'ak_kron_precond': (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr, c_size, c_ptr]),
     'ak_inv_root_ws_bytes': (c_size, [c_i64, c_int]),

@@ -17,6 +17,65 @@ static __global__ __launch_bounds__(256) void gemv_kernel(const float* __restric
   if (lane == 0) y[row] = scale * s;
 }
 
+// The same for many matrices in one launch.  `table`: one row of 5 int64 per product: M, x, y, n, first block
+// (blocks of 4 rows, numbered in table order); y must not alias x.
+static __global__ __launch_bounds__(256) void gemv_grouped_kernel(const int64_t* __restrict__ table, int count,
+                                                                  float scale) {
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[static_cast<int64_t>(mid) * 5 + 4] <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * 5;
+  const float* __restrict__ M = reinterpret_cast<const float*>(r[0]);
+  const float* __restrict__ x = reinterpret_cast<const float*>(r[1]);
+  float* __restrict__ y = reinterpret_cast<float*>(r[2]);
+  const int64_t n = r[3];
+  const int64_t row = static_cast<int64_t>(w - r[4]) * 4 + (threadIdx.x >> 6);
+  if (row >= n) return;
+  const int lane = threadIdx.x & 63;
+  float s = 0.f;
+  for (int64_t k = lane; k < n; k += 64) s += M[row * n + k] * x[k];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if (lane == 0) y[row] = scale * s;
+}
+
+// Convolution weight gradients between the channels-last layout [Cout][kh*kw][Cin] and the contiguous layout
+// [Cout][Cin][kh*kw] the Kronecker factors are indexed by, for many modules in one launch: one work group per
+// output channel stages the row in the LDS, so both the read and the write are coalesced.  `table`: one row of
+// 5 int64 per module: channels-last address, contiguous address, Cin, kh*kw, first row (running sum of Cout).
+constexpr int LAYOUT_MAX_ROW = 12288;       // floats of one weight row (Cin * kh * kw) the staging buffer holds
+
+static __global__ __launch_bounds__(256) void weight_layout_grouped_kernel(const int64_t* __restrict__ table, int count,
+                                                                           int to_contiguous) {
+  __shared__ float row[LAYOUT_MAX_ROW];
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[static_cast<int64_t>(mid) * 5 + 4] <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * 5;
+  const int cin = static_cast<int>(r[2]), kk = static_cast<int>(r[3]);
+  const int len = cin * kk;
+  const int64_t off = static_cast<int64_t>(w - r[4]) * len;
+  float* nhwc = reinterpret_cast<float*>(r[0]) + off;
+  float* nchw = reinterpret_cast<float*>(r[1]) + off;
+  const float* __restrict__ src = to_contiguous ? nhwc : nchw;
+  float* __restrict__ dst = to_contiguous ? nchw : nhwc;
+  for (int i = threadIdx.x; i < len; i += 256) row[i] = src[i];
+  __syncthreads();
+  if (to_contiguous) {
+    for (int n = threadIdx.x; n < len; n += 256) dst[n] = row[(n % kk) * cin + n / kk];      // n = ci * kk + k
+  } else {
+    for (int j = threadIdx.x; j < len; j += 256) dst[j] = row[(j % cin) * kk + j / cin];     // j = k * cin + ci
+  }
+}
+
 static __global__ void copy_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t n) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = src[i];
@@ -81,6 +140,41 @@ extern "C" int ak_kron_precond(const float* Binv, const float* Ainv, float* G, i
                        grad_scale);
     hipLaunchKernelGGL(ak::copy_kernel, dim3(static_cast<unsigned>((dB + 255) / 256)), dim3(256), 0, s, tb, bias, dB);
   }
+  return ak::check_launch();
+}
+
+extern "C" int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t total_tiles,
+                                   ak_stream_t stream) {
+  if (pieces != 2 && pieces != 3) return AK_ERR_ARG;
+  if (count < 0 || total_tiles < 0 || total_tiles > (1ll << 30)) return AK_ERR_ARG;
+  if (count == 0 || total_tiles == 0) return AK_OK;
+  if (table == nullptr) return AK_ERR_ARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(total_tiles));
+  if (pieces == 2) hipLaunchKernelGGL(ak::gemm_x3_grouped_kernel<2>, grid, dim3(256), 0, s, table, count);
+  else hipLaunchKernelGGL(ak::gemm_x3_grouped_kernel<3>, grid, dim3(256), 0, s, table, count);
+  return ak::check_launch();
+}
+
+extern "C" int ak_gemv_f32_grouped(const int64_t* table, int count, int64_t total_blocks, float alpha,
+                                   ak_stream_t stream) {
+  if (count < 0 || total_blocks < 0 || total_blocks > (1ll << 30)) return AK_ERR_ARG;
+  if (count == 0 || total_blocks == 0) return AK_OK;
+  if (table == nullptr) return AK_ERR_ARG;
+  hipLaunchKernelGGL(ak::gemv_grouped_kernel, dim3(static_cast<unsigned>(total_blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), table, count, alpha);
+  return ak::check_launch();
+}
+
+extern "C" int64_t ak_weight_layout_max_row(void) { return ak::LAYOUT_MAX_ROW; }
+
+extern "C" int ak_weight_layout_grouped(const int64_t* table, int count, int64_t total_rows, int to_contiguous,
+                                        ak_stream_t stream) {
+  if (count < 0 || total_rows < 0 || total_rows > (1ll << 30)) return AK_ERR_ARG;
+  if (count == 0 || total_rows == 0) return AK_OK;
+  if (table == nullptr) return AK_ERR_ARG;
+  hipLaunchKernelGGL(ak::weight_layout_grouped_kernel, dim3(static_cast<unsigned>(total_rows)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), table, count, to_contiguous != 0 ? 1 : 0);
   return ak::check_launch();
 }
 

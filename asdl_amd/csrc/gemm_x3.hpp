@@ -3,7 +3,7 @@
 // the six piece products that matter:
 //   x*y ~= hi*hi' + hi*mid' + mid*hi' + hi*lo' + lo*hi' + mid*mid'      (dropped terms are below 2^-24 |x y|),
 // i.e. the accuracy of an fp32 multiply at 6/16 of the cost of the fp32 MFMA.  With NSPLIT = 2 only hi and mid
-// are kept (16 mantissa bits, 3 products) for callers whose tolerance allows it.
+// are kept (16 mantissa bits, mid rounded to nearest; 3 products) for callers whose tolerance allows it.
 //
 // Same interface as gemm_f32_kernel (GemmParams: transposes, triangular contraction ranges, lower-triangle tile
 // modes, batches).  One work group = 4 waves (2x2) = one 128x128 tile, k-tiles of 32.  The fp32 panels are
@@ -77,7 +77,11 @@ __device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char
       float rem = r.v[u][e];
 #pragma unroll
       for (int s = 0; s < NSPLIT; ++s) {
-        const uint32_t top = __builtin_bit_cast(uint32_t, rem) & 0xffff0000u;     // truncation: exact piece
+        uint32_t bits = __builtin_bit_cast(uint32_t, rem);
+        // the last of two pieces is rounded to nearest even (halves the error and removes its bias); every
+        // other piece is cut off, which keeps the remainder exact (the third piece has no bits left to lose)
+        if (NSPLIT == 2 && s == 1) bits += 0x7fffu + ((bits >> 16) & 1u);
+        const uint32_t top = bits & 0xffff0000u;
         piece[s][e] = top;
         if (s + 1 < NSPLIT) rem -= __builtin_bit_cast(float, top);                // exact
       }
@@ -106,16 +110,13 @@ __device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bo
   return pack_bf16x8(lo, hi);
 }
 
+// One 128 x 128 tile (ti, tj) of batch entry z of the product described by p.
 template <int NSPLIT>
-static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
+__device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj, int z, AK_LDS3 unsigned char* lds) {
   constexpr int BT = X3_BT, BK = X3_BK;
-  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
-  AK_LDS3 unsigned char* lds = (AK_LDS3 unsigned char*)x3_smem;
   AK_LDS3 unsigned char* panelA = lds;
   AK_LDS3 unsigned char* panelB = lds + NSPLIT * X3_PLANE;
-  const int z = blockIdx.z;
   if (p.active != nullptr && p.active[static_cast<int64_t>(z) * p.active_stride] == 0) return;
-  const int tj = blockIdx.x, ti = blockIdx.y;
   if (p.tile_mode != TILE_ALL && ti < tj) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave >> 1, wc = wave & 1, g = lane >> 5, l32 = lane & 31;
@@ -176,12 +177,12 @@ static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
             // smallest terms first
-            if (NSPLIT >= 3) {
+            if constexpr (NSPLIT >= 3) {
               acc[a][b] = mfma_bf16(fa[a][1], fb[b][1], acc[a][b]);
               acc[a][b] = mfma_bf16(fa[a][0], fb[b][2], acc[a][b]);
               acc[a][b] = mfma_bf16(fa[a][2], fb[b][0], acc[a][b]);
             }
-            if (NSPLIT >= 2) {
+            if constexpr (NSPLIT >= 2) {
               acc[a][b] = mfma_bf16(fa[a][0], fb[b][1], acc[a][b]);
               acc[a][b] = mfma_bf16(fa[a][1], fb[b][0], acc[a][b]);
             }
@@ -222,6 +223,51 @@ static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
         if (mirror && gi != gj) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
       }
     }
+}
+
+template <int NSPLIT>
+static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
+  gemm_x3_tile<NSPLIT>(p, blockIdx.y, blockIdx.x, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
+}
+
+// Grouped products: many independent C_i <- alpha_i * op(A_i) op(B_i) of different sizes in one launch, so that
+// products too small to fill the device share it and nothing waits on the host between them.  `table` holds one
+// row of GROUPED_ROW int64 per product: A, B, C, lda, ldb, ldc, M, N, K, transA | transB << 1, alpha (float bits in
+// the low word), first tile.  Tiles are numbered row-major inside a product, products in table order (longest
+// contraction first gives the best balance); work group w looks its product up by bisection on `first tile`.
+constexpr int GROUPED_ROW = 12;
+
+template <int NSPLIT>
+static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
+  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[static_cast<int64_t>(mid) * GROUPED_ROW + 11] <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * GROUPED_ROW;
+  GemmParams p;
+  p.A = reinterpret_cast<const float*>(r[0]);
+  p.B = reinterpret_cast<const float*>(r[1]);
+  p.C = reinterpret_cast<float*>(r[2]);
+  p.C_list = nullptr;
+  p.lda = r[3]; p.ldb = r[4]; p.ldc = r[5];
+  p.sA = p.sB = p.sC = 0;
+  p.M = static_cast<int>(r[6]); p.N = static_cast<int>(r[7]); p.K = static_cast<int>(r[8]);
+  p.transA = static_cast<int>(r[9] & 1); p.transB = static_cast<int>((r[9] >> 1) & 1);
+  p.alpha = __builtin_bit_cast(float, static_cast<uint32_t>(r[10]));
+  p.beta = 0.f;
+  p.kmode = K_FULL; p.tile_mode = TILE_ALL;
+  p.active = nullptr; p.active_stride = 0;
+  p.split = NSPLIT;
+  const int local = w - static_cast<int>(r[11]);
+  const int tn = (p.N + X3_BT - 1) / X3_BT;
+  const int ti = local / tn, tj = local - ti * tn;
+  if (ti * X3_BT >= p.M) return;            // a table whose tile count overstates this product
+  gemm_x3_tile<NSPLIT>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // The split kernel takes operands whose 16-byte chunks never straddle the end of a row.

@@ -356,7 +356,8 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
           float* dst = buf[sq];
           if (power == base) {      // keep the value `power` points at alive
             float* keep = buf[pw];
-            hipMemcpyAsync(keep, base, sizeof(float) * batch * nn, hipMemcpyDeviceToDevice, s);
+            if (hipMemcpyAsync(keep, base, sizeof(float) * batch * nn, hipMemcpyDeviceToDevice, s) != hipSuccess)
+              return AK_ERR_LAUNCH;
             power = keep;
             pw = (pw == 2) ? 3 : 2;
           }

@@ -6,6 +6,7 @@ There is no CPU path: a CPU tensor raises.
 """
 import contextlib
 import ctypes
+import struct
 import threading
 
 import torch
@@ -194,6 +195,22 @@ def device_ints(values, device, dtype=torch.int64):
         if len(_int_cache) > 8192:
             _int_cache.clear()
         t = torch.tensor(values, dtype=dtype).to(dev)
+        _int_cache[key] = t
+    return t
+
+
+def device_table(rows, device):
+    """device_ints for tables that hold addresses, which may change from call to call: a miss is staged through
+    pinned memory and copied asynchronously on the launch stream, so the host never waits for the device."""
+    dev = torch.device(device)
+    key = (dev.index, 'table', rows)
+    t = _int_cache.get(key)
+    if t is None:
+        if len(_int_cache) > 8192:
+            _int_cache.clear()
+        host = torch.tensor(rows, dtype=torch.int64).pin_memory()
+        with _on_launch_stream():
+            t = host.to(dev, non_blocking=True)
         _int_cache[key] = t
     return t
 
@@ -653,6 +670,136 @@ def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
                              grad_scale, ws, ws_bytes, _stream())
     _lib.check(rc, 'ak_kron_precond')
     return grad_w, grad_b
+
+
+def _float_bits(value):
+    return struct.unpack('<I', struct.pack('<f', float(value)))[0]
+
+
+def _grouped_operand_ok(ptr, ld, contiguous_extent):
+    return ptr % 16 == 0 and ld % 4 == 0 and contiguous_extent % 4 == 0
+
+
+def gemm_grouped_raw(specs, device, pieces=3):
+    """One launch for many products C_i <- alpha_i * op(A_i) op(B_i).  specs: tuples (a_ptr, lda, b_ptr, ldb, c_ptr,
+    ldc, M, N, K, transA, transB, alpha) of device addresses of float32 matrices with contiguous rows."""
+    rows, first = [], 0
+    for a, lda, b, ldb, c, ldc, M, N, K, tA, tB, alpha in sorted(specs, key=lambda sp: -sp[8]):
+        if M <= 0 or N <= 0 or K <= 0:
+            continue
+        if not (_grouped_operand_ok(a, lda, M if tA else K) and _grouped_operand_ok(b, ldb, K if tB else N)):
+            raise ValueError('grouped products need 16-byte aligned operands whose leading dimension and '
+                             'contiguous extent are multiples of 4')
+        if lda < (M if tA else K) or ldb < (K if tB else N) or ldc < N:
+            raise ValueError('leading dimension smaller than the row length')
+        rows.append((a, b, c, lda, ldb, ldc, M, N, K, int(bool(tA)) | (int(bool(tB)) << 1), _float_bits(alpha), first))
+        first += ((M + 127) // 128) * ((N + 127) // 128)
+    if not rows:
+        return
+    table = device_table(tuple(rows), device)
+    rc = _lib.load().ak_gemm_f32_grouped(int(pieces), ctypes.c_void_p(table.data_ptr()), len(rows), first, _stream())
+    _lib.check(rc, 'ak_gemm_f32_grouped')
+
+
+def gemm_grouped(problems, pieces=3):
+    """problems: (A, B, C, transA, transB, alpha) with 2-D float32 tensors whose rows are contiguous;
+    C <- alpha * op(A) @ op(B) for all of them in one launch."""
+    if not problems:
+        return
+    specs = []
+    for A, B, C, tA, tB, alpha in problems:
+        _require_gpu(A, B, C)
+        for t in (A, B, C):
+            if t.dtype != torch.float32 or t.ndim != 2 or (t.stride(1) != 1 and t.shape[1] > 1):
+                raise ValueError('operands have to be float32 matrices with contiguous rows')
+        M, K = (A.shape[1], A.shape[0]) if tA else A.shape
+        K2, N = (B.shape[1], B.shape[0]) if tB else B.shape
+        if K != K2 or tuple(C.shape) != (M, N):
+            raise ValueError('shapes do not match')
+        specs.append((A.data_ptr(), A.stride(0), B.data_ptr(), B.stride(0), C.data_ptr(), C.stride(0), M, N, K,
+                      tA, tB, alpha))
+    gemm_grouped_raw(specs, problems[0][0].device, pieces)
+
+
+def _channels_last_weight(g):
+    """A 4-D gradient stored as [Cout][kh][kw][Cin] (and not at the same time as [Cout][Cin][kh][kw])."""
+    return g.ndim == 4 and not g.is_contiguous() and g.is_contiguous(memory_format=torch.channels_last)
+
+
+def kron_precond_groupable(B_inv, A_inv, grad_w, grad_b=None):
+    """Whether kron_precond_grouped takes this module (else: kron_precond)."""
+    small = [B_inv, A_inv] + ([grad_b] if grad_b is not None else [])
+    if any(t is None or not t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous() for t in small):
+        return False
+    if grad_w is None or not grad_w.is_cuda or grad_w.dtype != torch.float32:
+        return False
+    if B_inv.ndim != 2 or A_inv.ndim != 2 or B_inv.shape[0] != B_inv.shape[1] or A_inv.shape[0] != A_inv.shape[1]:
+        return False
+    dB, dA = B_inv.shape[0], A_inv.shape[0]
+    if grad_w.numel() != dB * dA or (grad_b is not None and grad_b.numel() != dB):
+        return False
+    if not grad_w.is_contiguous():
+        if not _channels_last_weight(grad_w) or grad_w.shape[0] != dB or dA > _lib.load().ak_weight_layout_max_row():
+            return False
+    return dB % 4 == 0 and dA % 4 == 0 and all(t.data_ptr() % 16 == 0 for t in (B_inv, A_inv, grad_w))
+
+
+def kron_precond_grouped(items, grad_scale=1.0):
+    """kron_precond for many modules in a handful of launches: all B_inv @ G, then all (.) @ A_inv, then all
+    B_inv @ bias; channels-last convolution gradients are gathered into the contiguous layout before and
+    scattered back after, one launch each.  items: (B_inv, A_inv, grad_w, grad_b or None), each accepted by
+    kron_precond_groupable; in place."""
+    if not items:
+        return
+    lib = _lib.load()
+    dev = items[0][0].device
+    n_w = sum(it[2].numel() for it in items)
+    n_cl = sum(it[2].numel() for it in items if not it[2].is_contiguous())
+    n_b = sum(it[0].shape[0] for it in items if it[3] is not None)
+    buf, _ = workspace(4 * (n_w + n_cl + n_b), dev)
+    base = buf.data_ptr()
+    first, second, layout, layout_rows, off = [], [], [], 0, 0
+    for B_inv, A_inv, g, _ in items:
+        dB, dA = B_inv.shape[0], A_inv.shape[0]
+        t = base + 4 * off
+        off += dB * dA
+        g_ptr = g.data_ptr()
+        if not g.is_contiguous():
+            g_ptr = base + 4 * off
+            off += dB * dA
+            layout.append((g.data_ptr(), g_ptr, g.shape[1], g.shape[2] * g.shape[3], layout_rows))
+            layout_rows += dB
+        first.append((B_inv.data_ptr(), dB, g_ptr, dA, t, dA, dB, dA, dB, 0, 0, 1.0))
+        # the inverses are symmetric: reading A_inv as its transpose makes both operands contiguous along k
+        second.append((t, dA, A_inv.data_ptr(), dA, g_ptr, dA, dB, dA, dA, 0, 1, grad_scale))
+    layout_table = device_table(tuple(layout), dev) if layout else None
+    if layout:
+        rc = lib.ak_weight_layout_grouped(ctypes.c_void_p(layout_table.data_ptr()), len(layout), layout_rows, 1, _stream())
+        _lib.check(rc, 'ak_weight_layout_grouped')
+    # all 24 mantissa bits: the terms of these sums cancel (entries of the inverses reach 1/damping), and what a
+    # shorter split loses relative to the terms shows up magnified in the result
+    gemm_grouped_raw(first, dev, pieces=3)
+    gemm_grouped_raw(second, dev, pieces=3)
+    if layout:
+        rc = lib.ak_weight_layout_grouped(ctypes.c_void_p(layout_table.data_ptr()), len(layout), layout_rows, 0, _stream())
+        _lib.check(rc, 'ak_weight_layout_grouped')
+    rows, blocks, tmps, biases = [], 0, [], []
+    flat = buf[:4 * (n_w + n_cl + n_b)].view(torch.float32)
+    for B_inv, _, _, b in items:
+        if b is None:
+            continue
+        dB = B_inv.shape[0]
+        rows.append((B_inv.data_ptr(), b.data_ptr(), base + 4 * off, dB, blocks))
+        tmps.append(flat[off:off + dB])
+        biases.append(b.view(-1))
+        blocks += (dB + 3) // 4
+        off += dB
+    if rows:
+        table = device_table(tuple(rows), dev)
+        rc = lib.ak_gemv_f32_grouped(ctypes.c_void_p(table.data_ptr()), len(rows), blocks, float(grad_scale), _stream())
+        _lib.check(rc, 'ak_gemv_f32_grouped')
+        with _on_launch_stream():
+            torch._foreach_copy_(biases, tmps)
 
 
 # ------------------------------------------------------------------------------ Shampoo inverse root

@@ -12,6 +12,7 @@ import torch
 import torch.distributed as dist
 from torch import nn
 
+from . import kernels
 from .core import module_wise_assignments, modules_to_assign
 from .fisher import FisherConfig, get_fisher_maker
 from .grad_maker import LOSS_CROSS_ENTROPY
@@ -24,6 +25,7 @@ _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KF
 _kernel_shapes = [SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_UNIT_WISE]
 _norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 PRECONDITION_STREAMS = 6      # side streams over which precondition() spreads the layers
+GROUPED_PRECONDITION = True      # all Kronecker-factored modules in three launches instead of one stream-juggled chain per module
 
 __all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
 
@@ -170,6 +172,8 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             grad_scale = self.grad_scale
         work = [(module, shape) for shape in _kernel_shapes for module in self.modules_for(shape)
                 if module in self.modules_for_curvature]
+        if use_inv and GROUPED_PRECONDITION:
+            work = self._precondition_grouped(work, grad_scale)
         grads = [m.weight.grad for m, _ in work if getattr(m, 'weight', None) is not None and m.weight.grad is not None]
         if len(work) < 4 or not grads or not grads[0].is_cuda:
             for module, shape in work:
@@ -193,6 +197,33 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             done = torch.cuda.Event()
             done.record(st)
             main.wait_event(done)
+
+    def _precondition_grouped(self, work, grad_scale):
+        """Preconditions every Kronecker-factored module whose operands the grouped kernels take, all in the same
+        three launches (B_inv G for every module, (.) A_inv for every module, B_inv bias), and returns the rest of
+        ``work`` for the per-module path.  Same arithmetic per module as Kron.mvp(use_inv=True, inplace=True)."""
+        items, rest = [], []
+        for module, shape in work:
+            kron = self._get_module_symmatrix(module, shape) if shape in (SHAPE_KRON, SHAPE_SWIFT_KRON) else None
+            weight = getattr(module, 'weight', None)
+            item = None
+            if kron is not None and kron.has_inv and weight is not None and weight.requires_grad \
+                    and weight.grad is not None:
+                grad_b = None
+                has_bias = _bias_requires_grad(module)
+                if has_bias:
+                    grad_b = module.bias.grad
+                if not has_bias or grad_b is not None:
+                    if kernels.kron_precond_groupable(kron.B_inv, kron.A_inv, weight.grad, grad_b):
+                        item = (kron.B_inv, kron.A_inv, weight.grad.data, None if grad_b is None else grad_b.data)
+            if item is None:
+                rest.append((module, shape))
+            else:
+                items.append(item)
+        if len(items) < 2:
+            return work
+        kernels.kron_precond_grouped(items, grad_scale)
+        return rest
 
     def _precondition_module(self, module, shape=None, vectors=None, vec_weight=None, vec_bias=None,
                              grad_scale=None, use_inv=True):

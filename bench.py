@@ -45,7 +45,7 @@ def parse():
                     help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
                          '(the headline configuration ignores them, as the reference training script does)')
     ap.add_argument('--workload', default='resnet50', choices=['resnet50', 'linear4096'],
-                    help="resnet50: the headline benchmark.  linear4096: BASELINE's second configuration, a single "
+                    help="resnet50: the headline benchmark.  linear4096: the large single-layer configuration, a single "
                          'Linear 4096x4096 with bias on 8192 bf16 rows, EMA 0.95 (factor + inverse + precondition of one '
                          'large layer; its own metric name, not the headline)')
     ap.add_argument('--swift', action='store_true',

@@ -208,6 +208,33 @@ int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, 
                 float* C, int64_t ldc, int batch, int64_t strideA, int64_t strideB, int64_t strideC,
                 ak_stream_t stream);
 
+/* Many products of different sizes in one launch: C_i <- alpha_i * op(A_i) op(B_i) on the bf16 matrix cores
+ * (pieces = 2 or 3 as in ak_gemm_f32_split).  `table` is DEVICE memory, `count` rows of 12 int64:
+ *   A, B, C (addresses), lda, ldb, ldc, M, N, K, transA | transB << 1, alpha (float bit pattern in the low
+ *   32 bits), first_tile
+ * with first_tile the running sum of ceil(M/128) * ceil(N/128) over the rows before, and total_tiles that sum
+ * over all rows.  Every operand has to satisfy what the split kernel needs (16-byte aligned addresses, leading
+ * dimensions and the contiguous extents of both operands multiples of 4); the table cannot be checked from the
+ * host.  Rows sorted by descending K balance best.  Replaces the per-module loop around Kron.mvp of
+ * NaturalGradientMaker.precondition (asdl/precondition/natural_gradient.py:481-486, asdl/symmatrix.py:536-548):
+ * one call computes Binv_i G_i for every module, a second one (.) Ainv_i. */
+int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t total_tiles, ak_stream_t stream);
+
+/* y_i <- alpha * M_i x_i for dense row-major [n_i, n_i] fp32 matrices, one launch.  `table` is DEVICE memory,
+ * `count` rows of 5 int64: M, x, y (addresses, y not aliasing x), n, first_block, with first_block the running
+ * sum of ceil(n/4).  The bias half of Kron.mvp (asdl/symmatrix.py:543-546) for all modules at once. */
+int ak_gemv_f32_grouped(const int64_t* table, int count, int64_t total_blocks, float alpha, ak_stream_t stream);
+
+/* Convolution weight gradients of many modules between the channels-last layout [Cout][kh*kw][Cin] and the
+ * contiguous [Cout][Cin][kh*kw] that the Kronecker factors index (to_contiguous != 0: channels-last -> contiguous,
+ * else back), one launch.  `table` is DEVICE memory, `count` rows of 5 int64: channels-last address, contiguous
+ * address, Cin, kh*kw, first_row (running sum of Cout); total_rows the sum of Cout; Cin*kh*kw at most
+ * ak_weight_layout_max_row().  Replaces the .view(B.shape[0], -1) of Kron.mvp (asdl/symmatrix.py:539), which
+ * for a channels-last parameter gradient has to gather first. */
+int64_t ak_weight_layout_max_row(void);
+int ak_weight_layout_grouped(const int64_t* table, int count, int64_t total_rows, int to_contiguous,
+                             ak_stream_t stream);
+
 /* G <- grad_scale * Binv G Ainv (G = [dB, dA] in place), bias <- grad_scale * Binv bias when
  * bias != NULL.  ws holds the [dB, dA] intermediate.  Replaces Kron.mvp(use_inv, inplace)
  * (asdl/symmatrix.py:536-548) and the grad_scale pre-multiply of

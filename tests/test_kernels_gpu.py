@@ -356,6 +356,69 @@ def test_gemm_split_matches_fp64(K, pieces, tol, tA, tB, M, N, K_):
     assert relerr(out2, 0.5 * ref - 2.0 * C0.double()) < tol
 
 
+def test_gemm_grouped_matches_fp64(K):
+    """Products of very different sizes in one launch, each against its fp64 product; edge tiles, transposes,
+    strided rows, a scale per product."""
+    torch.manual_seed(5)
+    shapes = [(64, 576, 64, False, False), (512, 4608, 512, False, False), (512, 4608, 4608, False, True),
+              (1000, 2048, 1000, False, False), (132, 260, 516, True, False), (256, 64, 2048, True, True),
+              (4, 8, 12, False, False)]
+    for pieces, tol in [(3, 2e-6), (2, 3e-5)]:
+        problems, refs = [], []
+        for i, (M, N, K_, tA, tB) in enumerate(shapes):
+            A = torch.randn((K_, M) if tA else (M, K_), device='cuda')
+            B = torch.randn(N, K_ + 8, device='cuda')[:, :K_] if tB else torch.randn(K_, N, device='cuda')   # strided rows
+            C = torch.full((M, N), float('nan'), device='cuda')
+            alpha = 0.25 * (i + 1)
+            problems.append((A, B, C, tA, tB, alpha))
+            refs.append(alpha * (A.T if tA else A).double() @ (B.T if tB else B).double())
+        print(f'grouped gemm pieces={pieces}', flush=True)
+        K.gemm_grouped(problems, pieces=pieces)
+        torch.cuda.synchronize()
+        for (A, B, C, tA, tB, alpha), ref in zip(problems, refs):
+            assert relerr(C, ref) < tol, (tuple(C.shape), A.shape, relerr(C, ref))
+    with pytest.raises(ValueError):
+        K.gemm_grouped([(torch.randn(6, 6, device='cuda'), torch.randn(6, 6, device='cuda'),
+                         torch.empty(6, 6, device='cuda'), False, False, 1.0)])       # extents not multiples of 4
+
+
+def test_kron_precond_grouped_matches_fp64(K):
+    """All modules in three launches: against B_inv G A_inv and B_inv b in fp64, and against the per-module kernel."""
+    torch.manual_seed(6)
+    dims = [(64, 576, False), (512, 4608, False), (1000, 2048, True), (64, 64, True), (256, 1152, False),
+            (128, 128, True), (2048, 512, False), (8, 12, True), (64, 576, 'cl'), (128, 1152, 'cl'), (16, 100, 'cl5')]
+    items, refs, singles = [], [], []
+    for dB, dA, bias in dims:
+        Bi = torch.randn(dB, dB, device='cuda'); Bi = Bi @ Bi.T / dB
+        Ai = torch.randn(dA, dA, device='cuda'); Ai = Ai @ Ai.T / dA
+        G = torch.randn(dB, dA, device='cuda')
+        if isinstance(bias, str):          # a convolution gradient in the channels-last layout (3x3 or 5x5 window)
+            k = 5 if bias == 'cl5' else 3
+            G = G.view(dB, dA // (k * k), k, k).contiguous(memory_format=torch.channels_last)
+            assert not G.is_contiguous()
+            bias = False
+        b = torch.randn(dB, device='cuda') if bias else None
+        assert K.kron_precond_groupable(Bi, Ai, G, b)
+        refs.append((0.5 * Bi.double() @ G.double().reshape(dB, dA) @ Ai.double(),
+                     0.5 * Bi.double() @ b.double() if bias else None))
+        Gs, bs = G.contiguous().clone(), (b.clone() if bias else None)
+        K.kron_precond(Bi, Ai, Gs, bs, grad_scale=0.5)
+        singles.append((Gs, bs))
+        items.append((Bi, Ai, G, b))
+    print('grouped precondition', flush=True)
+    K.kron_precond_grouped(items, grad_scale=0.5)
+    torch.cuda.synchronize()
+    for (Bi, Ai, G, b), (rw, rb), (Gs, bs) in zip(items, refs, singles):
+        assert relerr(G.reshape(rw.shape), rw) < 5e-6, (tuple(G.shape), relerr(G.reshape(rw.shape), rw))
+        assert relerr(G.reshape(rw.shape), Gs.double().reshape(rw.shape)) < 5e-6
+        if b is not None:
+            assert relerr(b, rb) < 1e-5
+    assert not K.kron_precond_groupable(torch.eye(6, device='cuda'), torch.eye(8, device='cuda'),
+                                        torch.zeros(6, 8, device='cuda'))
+    assert not K.kron_precond_groupable(torch.eye(8, device='cuda'), torch.eye(8, device='cuda'),
+                                        torch.zeros(8, 8, device='cuda', dtype=torch.float64))
+
+
 @pytest.mark.parametrize('dB,dA,bias', [(4, 5, True), (10, 784, True), (512, 512, True), (64, 147, False),
                                         (300, 1152, False)])
 def test_kron_precond_matches_oracle(K, dB, dA, bias):

@@ -242,7 +242,7 @@ def test_small_cnn_bf16_autocast(channels_last):
 
 
 def test_config2_linear_4096_batch8192_bf16_ema():
-    """BASELINE config 2 at full size: Linear(4096, 4096), 8192 rows, bf16 activations, fp32 factors with EMA.
+    """The large single-layer configuration at full size: Linear(4096, 4096), 8192 rows, bf16 activations, fp32 factors with EMA.
     The factors are compared with fp64 products of the same rounded values, the inverses through the identity
     (A + lam I) A_inv = I, the preconditioned gradient with B_inv G A_inv in fp64."""
     torch.manual_seed(5)
@@ -280,7 +280,7 @@ def test_config2_linear_4096_batch8192_bf16_ema():
 
 
 def test_resnet50_batch64_channels_last_properties():
-    """BASELINE's benchmark configuration at full size, checked through properties that do not need a CPU run of
+    """The benchmark configuration (ResNet-50, batch 64) at full size, checked through properties that do not need a CPU run of
     the model: every conv A factor against an fp64 product of the unfolded input the GPU produced, every inverse
     through its defining identity, and the preconditioned gradients against B_inv G A_inv recomputed in fp64 from
     the stored inverses (sampled layers, to keep the host time down)."""
@@ -347,7 +347,7 @@ def test_resnet50_batch64_channels_last_properties():
 
 
 def test_resnet18_cifar_batch128_fp32_properties():
-    """BASELINE's third configuration at full size (fp32, NCHW, batch 128, Conv2d factors up to 4608 x 4608), checked
+    """The ResNet-18 configuration at full size (fp32, NCHW, batch 128, Conv2d factors up to 4608 x 4608), checked
     through the same size-independent properties as the ResNet-50 test."""
     torch.manual_seed(8)
     bs, damping, ema = 128, 1e-3, 0.5

@@ -251,7 +251,7 @@ def test_block_partitioner_and_dimension_merging():
 
 
 def test_shampoo_gpt2_small_weight_shapes_full_size():
-    """BASELINE's fifth configuration at the real weight shapes of one decoder block (768 x 2304 attention input,
+    """The transformer configuration at the real weight shapes of one decoder block (768 x 2304 attention input,
     768 x 768 attention output, 768 x 3072 and 3072 x 768 MLP): statistics against fp64 products of the very
     gradients, inverse fourth roots through the closed form of the ridged statistic, and the preconditioned
     gradient against P_L^T G P_R recomputed in fp64 from the stored roots."""
