@@ -50,6 +50,7 @@ class FisherMaker(GradientMaker):
     def __init__(self, model, config):
         super().__init__(model)
         self.config: FisherConfig = config
+        self.before_inverse_wait = None      # optional callable, run right before the host waits for the inverses
 
     def zero_fisher(self, fvp=False):
         attr = self.config.fvp_attr if fvp else self.config.fisher_attr
@@ -162,14 +163,17 @@ class FisherMaker(GradientMaker):
             self.replace_fisher_with_inv(damping)
         if loss_grad_after_fisher:
             loss.backward()
-        if deferred is not None:
-            deferred.finish(config.fisher_attr)
         if calc_loss_grad:
-            # the loss was summed over the batch: divide gradients and loss by the data size
+            # the loss was summed over the batch: divide gradients and loss by the data size (enqueued before the
+            # host waits for the inverse flags, so that nothing is left to launch between that wait and the caller)
             grads = [p.grad for p in model.parameters() if p.grad is not None]
             if grads:
                 torch._foreach_div_(grads, data_size)     # one launch for all parameters
             loss.div_(data_size)
+        if deferred is not None:
+            if self.before_inverse_wait is not None:
+                self.before_inverse_wait()      # host work of the caller that needs no flags: the device is still busy
+            deferred.finish(config.fisher_attr)
         return self._model_output, loss
 
     def _register_fisher(self, cxt: OperationContext, prescale=1.0):

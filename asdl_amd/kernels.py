@@ -680,9 +680,9 @@ def _grouped_operand_ok(ptr, ld, contiguous_extent):
     return ptr % 16 == 0 and ld % 4 == 0 and contiguous_extent % 4 == 0
 
 
-def gemm_grouped_raw(specs, device, pieces=3):
-    """One launch for many products C_i <- alpha_i * op(A_i) op(B_i).  specs: tuples (a_ptr, lda, b_ptr, ldb, c_ptr,
-    ldc, M, N, K, transA, transB, alpha) of device addresses of float32 matrices with contiguous rows."""
+def _gemm_grouped_table(specs, device):
+    """(device table, rows, tiles) for ak_gemm_f32_grouped.  specs: tuples (a_ptr, lda, b_ptr, ldb, c_ptr, ldc, M, N, K,
+    transA, transB, alpha) of device addresses of float32 matrices with contiguous rows."""
     rows, first = [], 0
     for a, lda, b, ldb, c, ldc, M, N, K, tA, tB, alpha in sorted(specs, key=lambda sp: -sp[8]):
         if M <= 0 or N <= 0 or K <= 0:
@@ -695,10 +695,19 @@ def gemm_grouped_raw(specs, device, pieces=3):
         rows.append((a, b, c, lda, ldb, ldc, M, N, K, int(bool(tA)) | (int(bool(tB)) << 1), _float_bits(alpha), first))
         first += ((M + 127) // 128) * ((N + 127) // 128)
     if not rows:
-        return
-    table = device_table(tuple(rows), device)
-    rc = _lib.load().ak_gemm_f32_grouped(int(pieces), ctypes.c_void_p(table.data_ptr()), len(rows), first, _stream())
-    _lib.check(rc, 'ak_gemm_f32_grouped')
+        return None, 0, 0
+    return device_table(tuple(rows), device), len(rows), first
+
+
+def _launch_gemm_grouped(table, count, tiles, pieces):
+    if count:
+        rc = _lib.load().ak_gemm_f32_grouped(int(pieces), ctypes.c_void_p(table.data_ptr()), count, tiles, _stream())
+        _lib.check(rc, 'ak_gemm_f32_grouped')
+
+
+def gemm_grouped_raw(specs, device, pieces=3):
+    """One launch for many products C_i <- alpha_i * op(A_i) op(B_i) (specs as for _gemm_grouped_table)."""
+    _launch_gemm_grouped(*_gemm_grouped_table(specs, device), pieces)
 
 
 def gemm_grouped(problems, pieces=3):
@@ -744,62 +753,83 @@ def kron_precond_groupable(B_inv, A_inv, grad_w, grad_b=None):
     return dB % 4 == 0 and dA % 4 == 0 and all(t.data_ptr() % 16 == 0 for t in (B_inv, A_inv, grad_w))
 
 
-def kron_precond_grouped(items, grad_scale=1.0):
+class KronPrecondPlan:
     """kron_precond for many modules in a handful of launches: all B_inv @ G, then all (.) @ A_inv, then all
     B_inv @ bias; channels-last convolution gradients are gathered into the contiguous layout before and
     scattered back after, one launch each.  items: (B_inv, A_inv, grad_w, grad_b or None), each accepted by
-    kron_precond_groupable; in place."""
-    if not items:
-        return
-    lib = _lib.load()
-    dev = items[0][0].device
-    n_w = sum(it[2].numel() for it in items)
-    n_cl = sum(it[2].numel() for it in items if not it[2].is_contiguous())
-    n_b = sum(it[0].shape[0] for it in items if it[3] is not None)
-    buf, _ = workspace(4 * (n_w + n_cl + n_b), dev)
-    base = buf.data_ptr()
-    first, second, layout, layout_rows, off = [], [], [], 0, 0
-    for B_inv, A_inv, g, _ in items:
-        dB, dA = B_inv.shape[0], A_inv.shape[0]
-        t = base + 4 * off
-        off += dB * dA
-        g_ptr = g.data_ptr()
-        if not g.is_contiguous():
-            g_ptr = base + 4 * off
+    kron_precond_groupable.  Construction does all host work (address tables, their upload); launch() only
+    enqueues the kernels, so a caller can prepare while the device is still busy producing the operands.  The
+    plan refers to the tensors by address: launch() is valid for as long as ``items`` are alive and unmoved."""
+
+    def __init__(self, items, grad_scale=1.0):
+        self.items = list(items)
+        self.grad_scale = float(grad_scale)
+        if not self.items:
+            return
+        dev = self.items[0][0].device
+        n_w = sum(it[2].numel() for it in self.items)
+        n_cl = sum(it[2].numel() for it in self.items if not it[2].is_contiguous())
+        n_b = sum(it[0].shape[0] for it in self.items if it[3] is not None)
+        self._buf, _ = workspace(4 * (n_w + n_cl + n_b), dev)       # kept alive with the plan
+        base = self._buf.data_ptr()
+        first, second, layout, layout_rows, off = [], [], [], 0, 0
+        for B_inv, A_inv, g, _ in self.items:
+            dB, dA = B_inv.shape[0], A_inv.shape[0]
+            t = base + 4 * off
             off += dB * dA
-            layout.append((g.data_ptr(), g_ptr, g.shape[1], g.shape[2] * g.shape[3], layout_rows))
-            layout_rows += dB
-        first.append((B_inv.data_ptr(), dB, g_ptr, dA, t, dA, dB, dA, dB, 0, 0, 1.0))
-        # the inverses are symmetric: reading A_inv as its transpose makes both operands contiguous along k
-        second.append((t, dA, A_inv.data_ptr(), dA, g_ptr, dA, dB, dA, dA, 0, 1, grad_scale))
-    layout_table = device_table(tuple(layout), dev) if layout else None
-    if layout:
-        rc = lib.ak_weight_layout_grouped(ctypes.c_void_p(layout_table.data_ptr()), len(layout), layout_rows, 1, _stream())
-        _lib.check(rc, 'ak_weight_layout_grouped')
-    # all 24 mantissa bits: the terms of these sums cancel (entries of the inverses reach 1/damping), and what a
-    # shorter split loses relative to the terms shows up magnified in the result
-    gemm_grouped_raw(first, dev, pieces=3)
-    gemm_grouped_raw(second, dev, pieces=3)
-    if layout:
-        rc = lib.ak_weight_layout_grouped(ctypes.c_void_p(layout_table.data_ptr()), len(layout), layout_rows, 0, _stream())
-        _lib.check(rc, 'ak_weight_layout_grouped')
-    rows, blocks, tmps, biases = [], 0, [], []
-    flat = buf[:4 * (n_w + n_cl + n_b)].view(torch.float32)
-    for B_inv, _, _, b in items:
-        if b is None:
-            continue
-        dB = B_inv.shape[0]
-        rows.append((B_inv.data_ptr(), b.data_ptr(), base + 4 * off, dB, blocks))
-        tmps.append(flat[off:off + dB])
-        biases.append(b.view(-1))
-        blocks += (dB + 3) // 4
-        off += dB
-    if rows:
-        table = device_table(tuple(rows), dev)
-        rc = lib.ak_gemv_f32_grouped(ctypes.c_void_p(table.data_ptr()), len(rows), blocks, float(grad_scale), _stream())
-        _lib.check(rc, 'ak_gemv_f32_grouped')
-        with _on_launch_stream():
-            torch._foreach_copy_(biases, tmps)
+            g_ptr = g.data_ptr()
+            if not g.is_contiguous():
+                g_ptr = base + 4 * off
+                off += dB * dA
+                layout.append((g.data_ptr(), g_ptr, g.shape[1], g.shape[2] * g.shape[3], layout_rows))
+                layout_rows += dB
+            first.append((B_inv.data_ptr(), dB, g_ptr, dA, t, dA, dB, dA, dB, 0, 0, 1.0))
+            # the inverses are symmetric: reading A_inv as its transpose makes both operands contiguous along k
+            second.append((t, dA, A_inv.data_ptr(), dA, g_ptr, dA, dB, dA, dA, 0, 1, self.grad_scale))
+        self._layout = (device_table(tuple(layout), dev), len(layout), layout_rows) if layout else None
+        self._first = _gemm_grouped_table(first, dev)
+        self._second = _gemm_grouped_table(second, dev)
+        rows, blocks, self._tmps, self._biases = [], 0, [], []
+        flat = self._buf[:4 * (n_w + n_cl + n_b)].view(torch.float32)
+        for B_inv, _, _, b in self.items:
+            if b is None:
+                continue
+            dB = B_inv.shape[0]
+            rows.append((B_inv.data_ptr(), b.data_ptr(), base + 4 * off, dB, blocks))
+            self._tmps.append(flat[off:off + dB])
+            self._biases.append(b.view(-1))
+            blocks += (dB + 3) // 4
+            off += dB
+        self._gemv = (device_table(tuple(rows), dev), len(rows), blocks) if rows else None
+
+    def _convert_layout(self, to_contiguous):
+        if self._layout is not None:
+            table, count, rows = self._layout
+            rc = _lib.load().ak_weight_layout_grouped(ctypes.c_void_p(table.data_ptr()), count, rows, to_contiguous,
+                                                      _stream())
+            _lib.check(rc, 'ak_weight_layout_grouped')
+
+    def launch(self):
+        if not self.items:
+            return
+        self._convert_layout(1)
+        # all 24 mantissa bits: the terms of these sums cancel (entries of the inverses reach 1/damping), and what
+        # a shorter split loses relative to the terms shows up magnified in the result
+        _launch_gemm_grouped(*self._first, 3)
+        _launch_gemm_grouped(*self._second, 3)
+        self._convert_layout(0)
+        if self._gemv is not None:
+            table, count, blocks = self._gemv
+            rc = _lib.load().ak_gemv_f32_grouped(ctypes.c_void_p(table.data_ptr()), count, blocks, self.grad_scale,
+                                                 _stream())
+            _lib.check(rc, 'ak_gemv_f32_grouped')
+            with _on_launch_stream():
+                torch._foreach_copy_(self._biases, self._tmps)
+
+
+def kron_precond_grouped(items, grad_scale=1.0):
+    """In place, for all items: grad_w <- grad_scale * B_inv @ grad_w @ A_inv, grad_b <- grad_scale * B_inv @ grad_b."""
+    KronPrecondPlan(items, grad_scale).launch()
 
 
 # ------------------------------------------------------------------------------ Shampoo inverse root

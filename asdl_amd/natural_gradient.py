@@ -25,6 +25,7 @@ _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KF
 _kernel_shapes = [SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_UNIT_WISE]
 _norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 PRECONDITION_STREAMS = 6      # side streams over which precondition() spreads the layers
+PREPARE_PRECONDITION_EARLY = True      # host side of precondition() while the device still works on the inverses
 GROUPED_PRECONDITION = True      # all Kronecker-factored modules in three launches instead of one stream-juggled chain per module
 
 __all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
@@ -130,10 +131,14 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         if ema_decay != _invalid_ema_decay:
             scale *= ema_decay
             prescale = 1 - ema_decay          # applied to the old factors inside the factor kernels
-        self.delegate_forward_and_backward(self.fisher_maker, data_size=config.data_size, scale=scale,
-                                           accumulate=self.do_accumulate, calc_loss_grad=True,
-                                           calc_inv=not self.do_accumulate, damping=config.damping,
-                                           accumulate_prescale=prescale)
+        self.fisher_maker.before_inverse_wait = self.prepare_precondition if PREPARE_PRECONDITION_EARLY else None
+        try:
+            self.delegate_forward_and_backward(self.fisher_maker, data_size=config.data_size, scale=scale,
+                                               accumulate=self.do_accumulate, calc_loss_grad=True,
+                                               calc_inv=not self.do_accumulate, damping=config.damping,
+                                               accumulate_prescale=prescale)
+        finally:
+            self.fisher_maker.before_inverse_wait = None
 
     def update_preconditioner(self, damping=None, module_name=None, kron=None, zero_curvature=False):
         if not self.do_accumulate:
@@ -170,8 +175,7 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             raise NotImplementedError('precondition(vectors=...) is not on this path')
         if grad_scale is None:
             grad_scale = self.grad_scale
-        work = [(module, shape) for shape in _kernel_shapes for module in self.modules_for(shape)
-                if module in self.modules_for_curvature]
+        work = self._precondition_work()
         if use_inv and GROUPED_PRECONDITION:
             work = self._precondition_grouped(work, grad_scale)
         grads = [m.weight.grad for m, _ in work if getattr(m, 'weight', None) is not None and m.weight.grad is not None]
@@ -198,11 +202,17 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             done.record(st)
             main.wait_event(done)
 
-    def _precondition_grouped(self, work, grad_scale):
-        """Preconditions every Kronecker-factored module whose operands the grouped kernels take, all in the same
-        three launches (B_inv G for every module, (.) A_inv for every module, B_inv bias), and returns the rest of
-        ``work`` for the per-module path.  Same arithmetic per module as Kron.mvp(use_inv=True, inplace=True)."""
-        items, rest = [], []
+    def _precondition_work(self):
+        return [(module, shape) for shape in _kernel_shapes for module in self.modules_for(shape)
+                if module in self.modules_for_curvature]
+
+    def _plan_grouped(self, work, grad_scale):
+        """Collects every Kronecker-factored module whose operands the grouped kernels take into one
+        kernels.KronPrecondPlan (B_inv G for every module, (.) A_inv for every module, B_inv bias: a handful of
+        launches, same arithmetic per module as Kron.mvp(use_inv=True, inplace=True)).  Returns
+        (plan, rest of ``work`` for the per-module path, signature) or None when fewer than two modules qualify;
+        the signature lists the objects the plan was built from."""
+        items, rest, signature = [], [], []
         for module, shape in work:
             kron = self._get_module_symmatrix(module, shape) if shape in (SHAPE_KRON, SHAPE_SWIFT_KRON) else None
             weight = getattr(module, 'weight', None)
@@ -216,13 +226,51 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                 if not has_bias or grad_b is not None:
                     if kernels.kron_precond_groupable(kron.B_inv, kron.A_inv, weight.grad, grad_b):
                         item = (kron.B_inv, kron.A_inv, weight.grad.data, None if grad_b is None else grad_b.data)
+                        signature.append((module, shape, kron, kron.A_inv, kron.B_inv, weight.grad, grad_b))
             if item is None:
                 rest.append((module, shape))
             else:
                 items.append(item)
         if len(items) < 2:
+            return None
+        return kernels.KronPrecondPlan(items, grad_scale), rest, signature
+
+    def prepare_precondition(self):
+        """Does the host side of the coming precondition() ahead of time.  update_curvature() has this called
+        after the loss backward pass is enqueued and before the host waits for the inverses' flags, i.e. while the
+        device is busy: when the wait returns, precondition() only has to launch.  precondition() checks that the
+        plan still describes the current inverses and gradients and builds a new one if not."""
+        self._precond_plan = None
+        if not GROUPED_PRECONDITION:
+            return
+        work = self._precondition_work()
+        planned = self._plan_grouped(work, self.grad_scale)
+        if planned is not None:
+            self._precond_plan = (planned, [m for m, _ in work])
+
+    def _take_plan(self, work, grad_scale):
+        """The plan of prepare_precondition() if it still holds (same modules, inverses and gradient tensors)."""
+        prepared, self._precond_plan = getattr(self, '_precond_plan', None), None
+        if prepared is None:
+            return None
+        (plan, rest, signature), modules = prepared
+        if plan.grad_scale != float(grad_scale) or len(modules) != len(work) or \
+                any(m is not w for m, (w, _) in zip(modules, work)):
+            return None
+        for module, shape, kron, A_inv, B_inv, grad_w, grad_b in signature:
+            if self._get_module_symmatrix(module, shape) is not kron or kron.A_inv is not A_inv or \
+                    kron.B_inv is not B_inv or module.weight.grad is not grad_w or \
+                    (grad_b is not None and module.bias.grad is not grad_b):
+                return None
+        return plan, rest, signature
+
+    def _precondition_grouped(self, work, grad_scale):
+        """Preconditions the modules the grouped kernels take and returns the rest of ``work``."""
+        planned = self._take_plan(work, grad_scale) or self._plan_grouped(work, grad_scale)
+        if planned is None:
             return work
-        kernels.kron_precond_grouped(items, grad_scale)
+        plan, rest, _ = planned
+        plan.launch()
         return rest
 
     def _precondition_module(self, module, shape=None, vectors=None, vec_weight=None, vec_bias=None,

@@ -443,6 +443,57 @@ def test_early_start_of_inverses_gives_the_same_result(network, monkeypatch):
             assert relerr(eager[key], lazy[key]) < 3e-2, key
 
 
+def test_grouped_precondition_and_its_early_preparation_give_the_per_module_result(monkeypatch):
+    """natural_gradient.GROUPED_PRECONDITION preconditions all modules in a handful of launches and
+    PREPARE_PRECONDITION_EARLY builds that plan before the inverses' flags are read.  A layer whose A factor is
+    all zero (no bias, zero input) gets no inverse: the plan prepared early must be dropped then, the gradient of
+    that layer stays raw, the others match the per-module path; a gradient replaced by the user between
+    update_curvature() and precondition() must be the one that is preconditioned."""
+    import asdl_amd.natural_gradient as ng_mod
+
+    def run(grouped, early, zero_input, replace_grad=False):
+        monkeypatch.setattr(ng_mod, 'GROUPED_PRECONDITION', grouped)
+        monkeypatch.setattr(ng_mod, 'PREPARE_PRECONDITION_EARLY', early)
+        torch.manual_seed(11)
+        class Gate(nn.Module):
+            def forward(self, x):
+                return x * 0 if zero_input else x
+
+        model = nn.Sequential(nn.Linear(8, 16), Gate(), nn.Linear(16, 12, bias=False), nn.Tanh(),
+                              nn.Linear(12, 8), nn.ReLU(), nn.Linear(8, 4)).cuda()
+        with torch.no_grad():
+            model[4].bias.fill_(0.5)
+        x = torch.randn(32, 8).cuda()
+        t = torch.randint(0, 4, (32,)).cuda()
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=32, damping=1e-2), fisher_type='fisher_emp')
+        grads = {}
+        for step in range(2):
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+            if replace_grad:
+                gm.update_curvature()
+                model[4].weight.grad = torch.ones_like(model[4].weight.grad)
+                gm.precondition()
+            else:
+                gm.forward_and_backward()
+            for name, p in model.named_parameters():
+                grads[(step, name)] = p.grad.detach().cpu().clone()
+        return grads, model
+
+    for zero_input in (False, True):
+        ref, model = run(False, False, zero_input)
+        if zero_input:
+            assert model[2].fisher.kron.A_inv is None          # all-zero factor: never inverted
+        for grouped, early in ((True, False), (True, True)):
+            got, _ = run(grouped, early, zero_input)
+            for key in ref:
+                assert grad_close(got[key], ref[key], 1e-5), (zero_input, grouped, early, key)
+    ref, _ = run(False, False, False, replace_grad=True)
+    got, _ = run(True, True, False, replace_grad=True)
+    for key in ref:
+        assert grad_close(got[key], ref[key], 1e-5), key
+
+
 @pytest.mark.parametrize('tag', ['cnn2_fisher_emp_ema0.5_int2', 'cnn_fisher_mc_ema-1', 'cnnbn_fisher_emp_ema-1'])
 def test_factor_side_stream_gives_the_golden_results(tag, monkeypatch):
     """fisher.FACTOR_SIDE_STREAM (off by default: ordering the side stream costs more host time per hook than the
