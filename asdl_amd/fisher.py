@@ -51,6 +51,8 @@ class FisherMaker(GradientMaker):
         super().__init__(model)
         self.config: FisherConfig = config
         self.before_inverse_wait = None      # optional callable, run right before the host waits for the inverses
+        self.after_factors = None            # optional callable, run when the factors are final and before the loss
+                                             # backward pass is enqueued; may return an object with finish()
 
     def zero_fisher(self, fvp=False):
         attr = self.config.fvp_attr if fvp else self.config.fisher_attr
@@ -161,7 +163,10 @@ class FisherMaker(GradientMaker):
 
         if inv_after_fisher:
             self.replace_fisher_with_inv(damping)
+        early = None
         if loss_grad_after_fisher:
+            if self.after_factors is not None:
+                early = self.after_factors()     # e.g. the caller's inverse update, enqueued beside the pass below
             loss.backward()
         if calc_loss_grad:
             # the loss was summed over the batch: divide gradients and loss by the data size (enqueued before the
@@ -170,10 +175,13 @@ class FisherMaker(GradientMaker):
             if grads:
                 torch._foreach_div_(grads, data_size)     # one launch for all parameters
             loss.div_(data_size)
-        if deferred is not None:
+        if deferred is not None or early is not None:
             if self.before_inverse_wait is not None:
                 self.before_inverse_wait()      # host work of the caller that needs no flags: the device is still busy
-            deferred.finish(config.fisher_attr)
+            if deferred is not None:
+                deferred.finish(config.fisher_attr)
+            if early is not None:
+                early.finish()
         return self._model_output, loss
 
     def _register_fisher(self, cxt: OperationContext, prescale=1.0):

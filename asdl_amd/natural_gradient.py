@@ -25,6 +25,7 @@ _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KF
 _kernel_shapes = [SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_UNIT_WISE]
 _norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 PRECONDITION_STREAMS = 6      # side streams over which precondition() spreads the layers
+OVERLAP_INVERSE_UPDATE = True           # EMA mode: update_preconditioner()'s inverses beside the loss backward pass
 PREPARE_PRECONDITION_EARLY = True      # host side of precondition() while the device still works on the inverses
 GROUPED_PRECONDITION = True      # all Kronecker-factored modules in three launches instead of one stream-juggled chain per module
 
@@ -132,6 +133,8 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             scale *= ema_decay
             prescale = 1 - ema_decay          # applied to the old factors inside the factor kernels
         self.fisher_maker.before_inverse_wait = self.prepare_precondition if PREPARE_PRECONDITION_EARLY else None
+        self.fisher_maker.after_factors = self._update_preconditioner_early \
+            if getattr(self, '_inverse_update_follows', False) else None
         try:
             self.delegate_forward_and_backward(self.fisher_maker, data_size=config.data_size, scale=scale,
                                                accumulate=self.do_accumulate, calc_loss_grad=True,
@@ -139,14 +142,24 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                                                accumulate_prescale=prescale)
         finally:
             self.fisher_maker.before_inverse_wait = None
+            self.fisher_maker.after_factors = None
 
-    def update_preconditioner(self, damping=None, module_name=None, kron=None, zero_curvature=False):
-        if not self.do_accumulate:
-            return
-        if kron is None:
-            kron = ['A', 'B']
-        if damping is None:
-            damping = self.config.damping
+    def forward_and_backward(self):
+        """The template of the base class.  With accumulated (EMA) factors the inverses are a step of their own,
+        update_preconditioner(); when that step follows update_curvature() in this very call, its Kronecker part is
+        enqueued as soon as the factors are final, beside the loss backward pass, instead of after it."""
+        step = self.state['step']
+        self._inverse_update_follows = bool(
+            OVERLAP_INVERSE_UPDATE and self.do_accumulate and self.do_update_curvature(step)
+            and self.do_update_preconditioner(step))
+        self._kron_inverses_current = False
+        try:
+            return super().forward_and_backward()
+        finally:
+            self._inverse_update_follows = False
+            self._kron_inverses_current = False
+
+    def _curvature_matrices(self, module_name=None):
         matrices, units = [], []
         for shape in _kernel_shapes:
             for name, module in self.named_modules_for(shape):
@@ -157,6 +170,30 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                 matrix = self._get_module_symmatrix(module, shape)
                 if matrix is not None:
                     (units if shape == SHAPE_UNIT_WISE else matrices).append(matrix)
+        return matrices, units
+
+    def _update_preconditioner_early(self):
+        """The Kronecker part of update_preconditioner() with its default arguments, enqueued only: returns the
+        pending inverses (finish() reads their flags).  GPU factors only."""
+        matrices, _ = self._curvature_matrices()
+        if not matrices or not all(k.has_A and k.has_B and k.A.is_cuda for k in matrices):
+            return None
+        pending = batched_update_inv(matrices, self.config.damping, defer=True)
+        self._kron_inverses_current = pending is not None
+        return pending
+
+    def update_preconditioner(self, damping=None, module_name=None, kron=None, zero_curvature=False):
+        if not self.do_accumulate:
+            return
+        if kron is None:
+            kron = ['A', 'B']
+        if damping is None:
+            damping = self.config.damping
+        matrices, units = self._curvature_matrices(module_name)
+        if getattr(self, '_kron_inverses_current', False) and module_name is None and not zero_curvature \
+                and set(kron) == {'A', 'B'} and damping == self.config.damping:
+            matrices = []        # already inverted beside the loss backward pass of this call
+            self._kron_inverses_current = False
         batched_update_inv(matrices, damping, calc_A_inv='A' in kron, calc_B_inv='B' in kron)
         for unit in units:
             unit.update_inv(damping)

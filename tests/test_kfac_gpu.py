@@ -494,6 +494,41 @@ def test_grouped_precondition_and_its_early_preparation_give_the_per_module_resu
         assert grad_close(got[key], ref[key], 1e-5), key
 
 
+@pytest.mark.parametrize('pi', [1, 2])
+def test_overlapped_inverse_update_in_ema_mode_gives_the_same_result(pi, monkeypatch):
+    """natural_gradient.OVERLAP_INVERSE_UPDATE: with accumulated factors and a sampled Fisher, the inverses of
+    update_preconditioner() are enqueued beside the loss backward pass when that step follows in the same call.
+    Same kernels on the same factors: bit for bit the result of the sequential order, also when the inverses are
+    only due every second step."""
+    import asdl_amd.natural_gradient as ng_mod
+
+    def run(overlap):
+        monkeypatch.setattr(ng_mod, 'OVERLAP_INVERSE_UPDATE', overlap)
+        torch.manual_seed(3)
+        model = bench_models.mlp().cuda()
+        x, t = torch.randn(32, 784).cuda(), torch.randint(0, 10, (32,)).cuda()
+        config = PreconditioningConfig(data_size=32, damping=1e-2, ema_decay=0.5, curvature_upd_interval=1,
+                                       preconditioner_upd_interval=pi)
+        gm = KfacGradientMaker(model, config, fisher_type='fisher_mc', seed=5)
+        out = {}
+        for step in range(4):
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+            gm.forward_and_backward()
+            for name, m in model.named_modules():
+                if isinstance(m, nn.Linear):
+                    out[(step, name, 'A')] = m.fisher.kron.A.clone()
+                    out[(step, name, 'A_inv')] = m.fisher.kron.A_inv.clone()
+                    out[(step, name, 'B_inv')] = m.fisher.kron.B_inv.clone()
+                    out[(step, name, 'grad')] = m.weight.grad.clone()
+        return out
+
+    seq, ovl = run(False), run(True)
+    assert seq.keys() == ovl.keys()
+    for key in seq:
+        assert torch.equal(seq[key], ovl[key]), key
+
+
 @pytest.mark.parametrize('tag', ['cnn2_fisher_emp_ema0.5_int2', 'cnn_fisher_mc_ema-1', 'cnnbn_fisher_emp_ema-1'])
 def test_factor_side_stream_gives_the_golden_results(tag, monkeypatch):
     """fisher.FACTOR_SIDE_STREAM (off by default: ordering the side stream costs more host time per hook than the
