@@ -229,6 +229,40 @@ static __global__ __launch_bounds__(256) void uw_nonzero_kernel(const float* __r
   if (__syncthreads_or(any) && threadIdx.x == 0) flag[0] = 1;
 }
 
+// uw_nonzero_kernel + uw_inv_kernel for many modules in one launch.  `table`: one row of 6 int64 per module: blocks,
+// inv, flags (addresses; flags = int[2] preset to {0, 0x7fffffff}), F, first block (blocks of 256 features, running
+// sum), damping (float bits).
+static __global__ __launch_bounds__(256) void uw_inv_grouped_kernel(const int64_t* __restrict__ table, int count) {
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[static_cast<int64_t>(mid) * 6 + 4] <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * 6;
+  const float* __restrict__ blocks = reinterpret_cast<const float*>(r[0]);
+  float* __restrict__ inv = reinterpret_cast<float*>(r[1]);
+  int* flags = reinterpret_cast<int*>(r[2]);
+  const int64_t F = r[3];
+  const float damping = __builtin_bit_cast(float, static_cast<uint32_t>(r[5]));
+  const int64_t f = static_cast<int64_t>(w - r[4]) * 256 + threadIdx.x;
+  int any = 0;
+  if (f < F) {
+    const float b0 = blocks[f * 4], b1 = blocks[f * 4 + 1], b2 = blocks[f * 4 + 2], b3 = blocks[f * 4 + 3];
+    any = (b0 != 0.f) | (b1 != 0.f) | (b2 != 0.f) | (b3 != 0.f);
+    const float a = b0 + damping, d = b3 + damping;
+    const float det = a * d - b1 * b2;
+    if (det == 0.f || det != det) atomicMin(flags + 1, static_cast<int>(f) + 1);
+    const float q = 1.f / det;
+    inv[f * 4] = d * q;
+    inv[f * 4 + 1] = -b1 * q;
+    inv[f * 4 + 2] = -b2 * q;
+    inv[f * 4 + 3] = a * q;
+  }
+  if (__syncthreads_or(any) && threadIdx.x == 0) flags[0] = 1;
+}
+
 static __global__ void uw_reset_kernel(int* flag, int* info) {
   flag[0] = 0;
   info[0] = 0x7fffffff;
@@ -241,6 +275,28 @@ static __global__ __launch_bounds__(256) void uw_mvp_kernel(const float* __restr
   const float w = vw[f] * scale, b = vb[f] * scale;
   vw[f] = mat[f * 4] * w + mat[f * 4 + 1] * b;
   vb[f] = mat[f * 4 + 2] * w + mat[f * 4 + 3] * b;
+}
+
+// The same for many modules in one launch.  `table`: one row of 5 int64 per module: blocks, vec_weight, vec_bias
+// (addresses), F, first block (blocks of 256 features, running sum).
+static __global__ __launch_bounds__(256) void uw_mvp_grouped_kernel(const int64_t* __restrict__ table, int count,
+                                                                    float scale) {
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[static_cast<int64_t>(mid) * 5 + 4] <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * 5;
+  const float* __restrict__ mat = reinterpret_cast<const float*>(r[0]);
+  float* __restrict__ vw = reinterpret_cast<float*>(r[1]);
+  float* __restrict__ vb = reinterpret_cast<float*>(r[2]);
+  const int64_t f = static_cast<int64_t>(w - r[4]) * 256 + threadIdx.x;
+  if (f >= r[3]) return;
+  const float wv = vw[f] * scale, bv = vb[f] * scale;
+  vw[f] = mat[f * 4] * wv + mat[f * 4 + 1] * bv;
+  vb[f] = mat[f * 4 + 2] * wv + mat[f * 4 + 3] * bv;
 }
 
 constexpr int64_t kUwChunkRows = 64;
@@ -337,5 +393,26 @@ extern "C" int ak_unit_wise_mvp(const float* mat, int64_t F, float* vec_weight, 
   if (mat == nullptr || vec_weight == nullptr || vec_bias == nullptr || F <= 0) return AK_ERR_ARG;
   hipLaunchKernelGGL(uw_mvp_kernel, dim3(static_cast<unsigned>((F + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), mat, F, vec_weight, vec_bias, scale);
+  return check_launch();
+}
+
+extern "C" int ak_unit_wise_mvp_grouped(const int64_t* table, int count, int64_t total_blocks, float scale,
+                                        ak_stream_t stream) {
+  using namespace ak;
+  if (count < 0 || total_blocks < 0 || total_blocks > (1ll << 30)) return AK_ERR_ARG;
+  if (count == 0 || total_blocks == 0) return AK_OK;
+  if (table == nullptr) return AK_ERR_ARG;
+  hipLaunchKernelGGL(uw_mvp_grouped_kernel, dim3(static_cast<unsigned>(total_blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), table, count, scale);
+  return check_launch();
+}
+
+extern "C" int ak_unit_wise_inv_grouped(const int64_t* table, int count, int64_t total_blocks, ak_stream_t stream) {
+  using namespace ak;
+  if (count < 0 || total_blocks < 0 || total_blocks > (1ll << 30)) return AK_ERR_ARG;
+  if (count == 0 || total_blocks == 0) return AK_OK;
+  if (table == nullptr) return AK_ERR_ARG;
+  hipLaunchKernelGGL(uw_inv_grouped_kernel, dim3(static_cast<unsigned>(total_blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), table, count);
   return check_launch();
 }

@@ -13,7 +13,7 @@ from .core import no_centered_cov
 from .grad_maker import GradientMaker, LOSS_CROSS_ENTROPY, LOSS_MSE
 from .matrices import *
 from .operations import OperationContext
-from .symmatrix import SymMatrix, batched_update_inv
+from .symmatrix import SymMatrix, batched_unit_update_inv, batched_update_inv
 from .utils import skip_param_grad
 
 __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
@@ -201,13 +201,14 @@ class FisherMaker(GradientMaker):
 
     def replace_fisher_with_inv(self, damping):
         attr = self.config.fisher_attr
-        krons = []
+        krons, units = [], []
         for module in self.model.modules():
             fisher: SymMatrix = getattr(module, attr, None)
             if fisher is not None and fisher.has_kron:
                 krons.append(fisher.kron)
             if fisher is not None and fisher.has_unit:
-                fisher.unit.update_inv(damping, replace=True)
+                units.append(fisher.unit)
+        batched_unit_update_inv(units, damping, replace=True)
         batched_update_inv(krons, damping=damping, replace=True)
 
     def _fisher_loop(self, closure):

@@ -446,6 +446,31 @@ def unit_wise_inv(blocks, damping, out=None):
     return out, flags
 
 
+def unit_wise_inv_grouped(blocks_list, dampings, outs=None):
+    """unit_wise_inv for many modules in two launches.  Returns (list of inverses, flags [count, 2] int32 on the
+    device, one (non-zero, first singular block) pair per module).  outs: optional list of output tensors or None."""
+    _require_gpu(*blocks_list)
+    count = len(blocks_list)
+    dev = blocks_list[0].device
+    invs = []
+    for i, blocks in enumerate(blocks_list):
+        if blocks.dtype != torch.float32 or blocks.ndim != 3 or blocks.shape[1:] != (2, 2) or not blocks.is_contiguous():
+            raise ValueError('blocks has to be a contiguous float32 [f, 2, 2] tensor')
+        out = outs[i] if outs is not None else None
+        invs.append(out if out is not None else torch.empty_like(blocks))
+    with _on_launch_stream():
+        flags = device_ints(((0, 0x7fffffff),) * count, dev, dtype=torch.int32).clone()
+    rows, first = [], 0
+    for i, (blocks, inv) in enumerate(zip(blocks_list, invs)):
+        F = blocks.shape[0]
+        rows.append((blocks.data_ptr(), inv.data_ptr(), flags.data_ptr() + 8 * i, F, first, _float_bits(dampings[i])))
+        first += (F + 255) // 256
+    table = device_table(tuple(rows), dev)
+    rc = _lib.load().ak_unit_wise_inv_grouped(ctypes.c_void_p(table.data_ptr()), count, first, _stream())
+    _lib.check(rc, 'ak_unit_wise_inv_grouped')
+    return invs, flags
+
+
 def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
     """[vec_weight, vec_bias][f] <- mat[f] @ (scale * [vec_weight, vec_bias][f]) in place."""
     _require_gpu(mat, vec_weight, vec_bias)
@@ -761,9 +786,23 @@ class KronPrecondPlan:
     enqueues the kernels, so a caller can prepare while the device is still busy producing the operands.  The
     plan refers to the tensors by address: launch() is valid for as long as ``items`` are alive and unmoved."""
 
-    def __init__(self, items, grad_scale=1.0):
+    def __init__(self, items, grad_scale=1.0, unit_items=()):
+        """unit_items: (inv [F, 2, 2], grad_w [F], grad_b [F]) of the unit-wise modules (contiguous float32):
+        one more launch applies all their 2 x 2 blocks."""
         self.items = list(items)
+        self.unit_items = list(unit_items)
         self.grad_scale = float(grad_scale)
+        self._units = None
+        if self.unit_items:
+            rows, blocks = [], 0
+            for inv, gw, gb in self.unit_items:
+                F = inv.shape[0]
+                if any(t.dtype != torch.float32 or not t.is_contiguous() for t in (inv, gw, gb)) or \
+                        gw.numel() != F or gb.numel() != F or tuple(inv.shape[1:]) != (2, 2):
+                    raise ValueError('unit-wise items are float32 [F, 2, 2] blocks with [F] weight and bias gradients')
+                rows.append((inv.data_ptr(), gw.data_ptr(), gb.data_ptr(), F, blocks))
+                blocks += (F + 255) // 256
+            self._units = (device_table(tuple(rows), self.unit_items[0][0].device), len(rows), blocks)
         if not self.items:
             return
         dev = self.items[0][0].device
@@ -810,6 +849,11 @@ class KronPrecondPlan:
             _lib.check(rc, 'ak_weight_layout_grouped')
 
     def launch(self):
+        if self._units is not None:
+            table, count, blocks = self._units
+            rc = _lib.load().ak_unit_wise_mvp_grouped(ctypes.c_void_p(table.data_ptr()), count, blocks, self.grad_scale,
+                                                      _stream())
+            _lib.check(rc, 'ak_unit_wise_mvp_grouped')
         if not self.items:
             return
         self._convert_layout(1)

@@ -18,7 +18,7 @@ from .fisher import FisherConfig, get_fisher_maker
 from .grad_maker import LOSS_CROSS_ENTROPY
 from .matrices import *
 from .prec_grad_maker import PreconditionedGradientMaker, PreconditioningConfig
-from .symmatrix import SymMatrix, batched_update_inv
+from .symmatrix import SymMatrix, batched_unit_update_inv, batched_update_inv
 
 _invalid_ema_decay = -1
 _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KFE, SHAPE_UNIT_WISE, SHAPE_DIAG]
@@ -195,9 +195,9 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             matrices = []        # already inverted beside the loss backward pass of this call
             self._kron_inverses_current = False
         batched_update_inv(matrices, damping, calc_A_inv='A' in kron, calc_B_inv='B' in kron)
-        for unit in units:
-            unit.update_inv(damping)
-            if zero_curvature:
+        batched_unit_update_inv(units, damping)
+        if zero_curvature:
+            for unit in units:
                 unit.mul_(0)
         if zero_curvature:
             with torch.no_grad():
@@ -249,11 +249,21 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         launches, same arithmetic per module as Kron.mvp(use_inv=True, inplace=True)).  Returns
         (plan, rest of ``work`` for the per-module path, signature) or None when fewer than two modules qualify;
         the signature lists the objects the plan was built from."""
-        items, rest, signature = [], [], []
+        items, unit_items, rest, signature = [], [], [], []
         for module, shape in work:
             kron = self._get_module_symmatrix(module, shape) if shape in (SHAPE_KRON, SHAPE_SWIFT_KRON) else None
             weight = getattr(module, 'weight', None)
             item = None
+            if shape == SHAPE_UNIT_WISE and weight is not None and weight.requires_grad and _bias_requires_grad(module):
+                unit = self._get_module_symmatrix(module, shape)
+                gw, gb = weight.grad, module.bias.grad
+                if unit is not None and unit.has_inv and gw is not None and gb is not None and \
+                        all(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() for t in (unit.inv, gw, gb)) \
+                        and unit.inv.ndim == 3 and tuple(unit.inv.shape[1:]) == (2, 2) \
+                        and gw.numel() == gb.numel() == unit.inv.shape[0]:
+                    unit_items.append((unit.inv, gw.data.view(-1), gb.data.view(-1)))
+                    signature.append((module, shape, unit, unit.inv, None, gw, gb))
+                    continue
             if kron is not None and kron.has_inv and weight is not None and weight.requires_grad \
                     and weight.grad is not None:
                 grad_b = None
@@ -268,9 +278,9 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                 rest.append((module, shape))
             else:
                 items.append(item)
-        if len(items) < 2:
+        if len(items) + len(unit_items) < 2:
             return None
-        return kernels.KronPrecondPlan(items, grad_scale), rest, signature
+        return kernels.KronPrecondPlan(items, grad_scale, unit_items), rest, signature
 
     def prepare_precondition(self):
         """Does the host side of the coming precondition() ahead of time.  update_curvature() has this called
@@ -294,10 +304,14 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         if plan.grad_scale != float(grad_scale) or len(modules) != len(work) or \
                 any(m is not w for m, (w, _) in zip(modules, work)):
             return None
-        for module, shape, kron, A_inv, B_inv, grad_w, grad_b in signature:
-            if self._get_module_symmatrix(module, shape) is not kron or kron.A_inv is not A_inv or \
-                    kron.B_inv is not B_inv or module.weight.grad is not grad_w or \
+        for module, shape, matrix, A_inv, B_inv, grad_w, grad_b in signature:
+            if self._get_module_symmatrix(module, shape) is not matrix or module.weight.grad is not grad_w or \
                     (grad_b is not None and module.bias.grad is not grad_b):
+                return None
+            if shape == SHAPE_UNIT_WISE:
+                if matrix.inv is not A_inv:
+                    return None
+            elif matrix.A_inv is not A_inv or matrix.B_inv is not B_inv:
                 return None
         return plan, rest, signature
 

@@ -462,6 +462,7 @@ class OperationContext:
         self._inverse_chunks = []
         self._pending_unit = []
         self._unit_flags = []
+        self._unit_flags_deferred = False
         self.factor_stream = None
         self.grad_edges = []       # autograd edges of the hooked module outputs of the latest forward pass
         self._eager_total = 0.0
@@ -555,10 +556,11 @@ class OperationContext:
             self._pending_unit.append(operation)
 
     def _invert_units(self):
-        """Damped inverses of the queued unit-wise blocks (one small launch each); their singularity flags are
-        read together in check_unit_flags()."""
+        """Damped inverses of the queued unit-wise blocks (one grouped launch); their singularity flags are read
+        together in check_unit_flags()."""
         ops = self._pending_unit
         self._pending_unit = []
+        todo = []
         for op in ops:
             blocks = op._op_results.pop('_unit_tmp', None)
             if blocks is None:
@@ -566,15 +568,21 @@ class OperationContext:
             store = op._op_results.setdefault(OP_COV_UNIT_WISE, {})
             prev = store.get('inv')
             reuse = prev is not None and prev.shape == blocks.shape
-            inv, flags = kernels.unit_wise_inv(blocks, op._damping, out=prev if reuse else None)
+            todo.append((op, store, blocks, prev if reuse else None))
+        if not todo:
+            return
+        invs, flags = kernels.unit_wise_inv_grouped([t[2] for t in todo], [t[0]._damping for t in todo],
+                                                    outs=[t[3] for t in todo])
+        for i, ((op, store, _, _), inv) in enumerate(zip(todo, invs)):
             store['inv'] = inv
-            self._unit_flags.append((op._module, flags))
+            self._unit_flags.append((op._module, flags[i]))
 
     def check_unit_flags(self):
         """torch.inverse raises for a singular block (asdl/operations/operation.py:317-320); here the flags of all
         modules are read with one copy."""
         pending = self._unit_flags
         self._unit_flags = []
+        self._unit_flags_deferred = False
         if not pending:
             return
         host = torch.stack([f for _, f in pending]).cpu().tolist()
@@ -619,10 +627,12 @@ class OperationContext:
         chunks = self._inverse_chunks
         self._inverse_chunks = []
         if not chunks:
-            self.check_unit_flags()
+            if not self._unit_flags_deferred:
+                self.check_unit_flags()
             return None
         deferred = DeferredInverses(chunks, self)
         if defer:
+            self._unit_flags_deferred = True      # read with the other flags in deferred.finish(), not by a later flush
             return deferred
         self.check_unit_flags()
         for pending, _ in chunks:

@@ -253,6 +253,27 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
     return None
 
 
+def batched_unit_update_inv(units, damping=_default_damping, replace=False):
+    """UnitWise.update_inv (asdl/symmatrix.py:687-699) for many modules: one grouped launch, then a single
+    device-to-host read for all zero / singular flags instead of one per module."""
+    units = [u for u in units if u is not None]
+    for u in units:
+        if not u.has_data:
+            raise ValueError('data do not exist.')
+    if not units:
+        return
+    invs, flags = kernels.unit_wise_inv_grouped([u.data for u in units], [float(damping)] * len(units))
+    host = flags.cpu().tolist()
+    for u, inv, (nonzero, bad) in zip(units, invs, host):
+        if not nonzero:
+            continue                       # an all-zero tensor keeps its old inverse (none)
+        if bad != 0x7fffffff:
+            raise torch.linalg.LinAlgError(f'unit-wise block {bad - 1} + damping is singular')
+        u.inv = inv
+        if replace:
+            u.data = None
+
+
 class Kron:
     def __init__(self, A, B, A_inv=None, B_inv=None):
         self.A: Tensor = A
@@ -438,17 +459,7 @@ class UnitWise:
 
     def update_inv(self, damping=_default_damping, replace=False):
         """asdl/symmatrix.py:687-699: an all-zero tensor keeps its old inverse (none)."""
-        if not self.has_data:
-            raise ValueError('data do not exist.')
-        inv, flags = kernels.unit_wise_inv(self.data, float(damping))
-        nonzero, bad = flags.cpu().tolist()
-        if not nonzero:
-            return
-        if bad != 0x7fffffff:
-            raise torch.linalg.LinAlgError(f'unit-wise block {bad - 1} + damping is singular')
-        self.inv = inv
-        if replace:
-            self.data = None
+        batched_unit_update_inv([self], damping, replace)
 
     def mvp(self, vec_weight, vec_bias, use_inv=False, inplace=False):
         """asdl/symmatrix.py:701-719 for modules with one (weight, bias) pair per block."""

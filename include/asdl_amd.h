@@ -171,11 +171,21 @@ int ak_unit_wise_stats(const void* y, int y_dtype, int64_t ysn, int64_t ysf, int
  * asdl/operations/operation.py:317-321. */
 int ak_unit_wise_inv(const float* blocks, int64_t F, float damping, float* inv, int* flags, ak_stream_t stream);
 
+/* ak_unit_wise_inv for many modules in one launch.  `table` is DEVICE memory, `count` rows of 6 int64: blocks,
+ * inv, flags (addresses; the caller presets each flags pair to {0, 0x7fffffff}), F, first_block (running sum of
+ * ceil(F/256)), damping (float bit pattern in the low 32 bits).  Same reference lines as ak_unit_wise_inv. */
+int ak_unit_wise_inv_grouped(const int64_t* table, int count, int64_t total_blocks, ak_stream_t stream);
+
 /* [vec_weight[f], vec_bias[f]] <- mat[f] @ (scale * [vec_weight[f], vec_bias[f]]) in place, mat = [F, 2, 2].
  * Replaces UnitWise.mvp for BatchNorm / LayerNorm (asdl/symmatrix.py:701-709, 716-719) and the grad_scale
  * pre-multiply of asdl/precondition/natural_gradient.py:535-538. */
 int ak_unit_wise_mvp(const float* mat, int64_t F, float* vec_weight, float* vec_bias, float scale,
                      ak_stream_t stream);
+
+/* ak_unit_wise_mvp for many modules in one launch.  `table` is DEVICE memory, `count` rows of 5 int64: mat,
+ * vec_weight, vec_bias (addresses), F, first_block (running sum of ceil(F/256)); total_blocks that sum over all
+ * rows.  The unit-wise modules of the loop at asdl/precondition/natural_gradient.py:481-486. */
+int ak_unit_wise_mvp_grouped(const int64_t* table, int count, int64_t total_blocks, float scale, ak_stream_t stream);
 
 /* ---- saved factors ----------------------------------------------------------------- */
 

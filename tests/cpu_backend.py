@@ -136,6 +136,15 @@ def unit_wise_inv(blocks, damping, out=None):
     return inv, flags
 
 
+def unit_wise_inv_grouped(blocks_list, dampings, outs=None):
+    invs, flags = [], []
+    for i, blocks in enumerate(blocks_list):
+        inv, fl = unit_wise_inv(blocks, dampings[i], out=outs[i] if outs is not None else None)
+        invs.append(inv)
+        flags.append(fl)
+    return invs, torch.stack(flags)
+
+
 def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
     w, b = R.unit_wise_mvp(mat, vec_weight * scale, vec_bias * scale)
     vec_weight.copy_(w)
@@ -146,5 +155,5 @@ def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
 def install(monkeypatch):
     from asdl_amd import kernels
     for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'cholesky_inv',
-                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_mvp', 'conv_patch_sum', 'smw_inv']:
+                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_inv_grouped', 'unit_wise_mvp', 'conv_patch_sum', 'smw_inv']:
         monkeypatch.setattr(kernels, name, globals()[name])

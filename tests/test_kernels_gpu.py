@@ -356,6 +356,41 @@ def test_gemm_split_matches_fp64(K, pieces, tol, tA, tB, M, N, K_):
     assert relerr(out2, 0.5 * ref - 2.0 * C0.double()) < tol
 
 
+def test_unit_wise_grouped_kernels_match_the_single_ones(K):
+    """Grouped inverse and grouped block-vector product of many modules against the per-module kernels (bit for
+    bit: same arithmetic per feature), including an all-zero module and a singular block."""
+    torch.manual_seed(9)
+    sizes = [64, 256, 300, 1, 2048, 512]
+    blocks = []
+    for F_ in sizes:
+        g = torch.randn(F_, 2, 2, device='cuda')
+        blocks.append((g @ g.transpose(1, 2)).contiguous())
+    blocks[3].zero_()                                   # all-zero module: flag 0
+    blocks[2][7] = torch.tensor([[-0.5, 0.0], [0.0, -0.5]], device='cuda')      # + damping 0.5 -> singular
+    dampings = [0.5] * len(sizes)
+    invs, flags = K.unit_wise_inv_grouped(blocks, dampings)
+    flags = flags.cpu().tolist()
+    for b, inv, fl in zip(blocks, invs, flags):
+        ref_inv, ref_fl = K.unit_wise_inv(b, 0.5)
+        assert fl == ref_fl.cpu().tolist()
+        assert torch.equal(torch.nan_to_num(inv, posinf=7.0, neginf=-7.0), torch.nan_to_num(ref_inv, posinf=7.0, neginf=-7.0))
+    assert flags[3][0] == 0 and flags[2][1] == 8 and flags[0] == [1, 0x7fffffff]
+    # grouped product through the plan
+    ws = [torch.randn(F_, device='cuda') for F_ in sizes]
+    bs = [torch.randn(F_, device='cuda') for F_ in sizes]
+    refs = []
+    for inv, w, b in zip(invs, ws, bs):
+        rw, rb = w.clone(), b.clone()
+        K.unit_wise_mvp(inv, rw, rb, 0.25)
+        refs.append((rw, rb))
+    K.KronPrecondPlan([], 0.25, unit_items=list(zip(invs, ws, bs))).launch()
+    torch.cuda.synchronize()
+    for i, ((rw, rb), w, b) in enumerate(zip(refs, ws, bs)):
+        if i == 2:
+            continue        # holds the singular block (inf / nan entries)
+        assert torch.equal(w, rw) and torch.equal(b, rb)
+
+
 def test_gemm_grouped_matches_fp64(K):
     """Products of very different sizes in one launch, each against its fp64 product; edge tiles, transposes,
     strided rows, a scale per product."""
