@@ -100,6 +100,9 @@ def _axis_statistic(grad, axis, out, alpha, beta):
         kernels.syrk_nt(grad.movedim(axis, 0).reshape(grad.shape[axis], -1).contiguous(), out=out, alpha=alpha, beta=beta)
 
 
+GROUPED_PRECONDITION = True      # matrix-shaped parameters: all their products in two launches
+
+
 def _precondition_block(grad, preconditioners):
     """tensordot(grad, P_j, [[0], [0]]) for every axis in turn (asdl/precondition/shampoo.py:358-364)."""
     cur = grad
@@ -242,5 +245,39 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
             self.last_root_stats[(n, exp)] = st
 
     def precondition(self):
-        for preconditioner in self.preconditioners:
+        """P_0^T G P_1 for every matrix-shaped parameter in two grouped launches (all G^T P_0, then all (.)^T P_1:
+        the per-axis tensordot chain of asdl/precondition/shampoo.py:351-367, on the split-bf16 kernel with all 24
+        mantissa bits); parameters with more axes, blocks or unaligned sizes go one at a time."""
+        specs_first, specs_second, rest, off = [], [], [], 0
+        grouped = []
+        for pc in self.preconditioners:
+            grad = pc.param.grad
+            shape = pc._transformed_shape
+            ok = GROUPED_PRECONDITION and grad is not None and len(shape) == 2 and tuple(grad.shape) == shape \
+                and len(pc.preconditioners) == 2 and grad.dtype == torch.float32 and grad.is_contiguous() \
+                and shape[0] % 4 == 0 and shape[1] % 4 == 0 and grad.data_ptr() % 16 == 0 \
+                and all(isinstance(q, torch.Tensor) and q.is_contiguous() and q.dtype == torch.float32
+                        and q.data_ptr() % 16 == 0 for q in pc.preconditioners) \
+                and tuple(pc.preconditioners[0].shape) == (shape[0], shape[0]) \
+                and tuple(pc.preconditioners[1].shape) == (shape[1], shape[1])
+            if ok:
+                grouped.append(pc)
+            else:
+                rest.append(pc)
+        if len(grouped) >= 2:
+            dev = grouped[0].param.device
+            buf, _ = kernels.workspace(4 * sum(pc.param.numel() for pc in grouped), dev)
+            base = buf.data_ptr()
+            for pc in grouped:
+                m, n = pc._transformed_shape
+                g, t = pc.param.grad.data_ptr(), base + 4 * off
+                off += m * n
+                # T[n, m] = G^T P_0, then G[m, n] <- T^T P_1
+                specs_first.append((g, n, pc.preconditioners[0].data_ptr(), m, t, m, n, m, m, 1, 0, 1.0))
+                specs_second.append((t, m, pc.preconditioners[1].data_ptr(), n, g, n, m, n, n, 1, 0, 1.0))
+            kernels.gemm_grouped_raw(specs_first, dev, pieces=3)
+            kernels.gemm_grouped_raw(specs_second, dev, pieces=3)
+        else:
+            rest = list(self.preconditioners)
+        for preconditioner in rest:
             preconditioner.precondition()

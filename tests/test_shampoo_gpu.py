@@ -216,6 +216,49 @@ def test_block_partitioned_preconditioner_matches_reference_golden(tag):
         assert relerr(param.grad, torch.from_numpy(z[f'step{step}/grad_out'])) < max(1e-3, 8 * worst_ref), (tag, step)
 
 
+def test_grouped_preconditioning_gives_the_per_parameter_result(monkeypatch):
+    """shampoo.GROUPED_PRECONDITION: the products of all matrix-shaped parameters in two launches, against the
+    per-parameter chain and against P_0^T G P_1 in fp64; a convolution weight and a matrix with an odd size in
+    the same model take the per-parameter way."""
+    import asdl_amd.shampoo as shampoo_mod
+
+    def run(grouped):
+        monkeypatch.setattr(shampoo_mod, 'GROUPED_PRECONDITION', grouped)
+        torch.manual_seed(21)
+        model = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.Flatten(), nn.Linear(8 * 6 * 6, 132), nn.ReLU(),
+                              nn.Linear(132, 260), nn.ReLU(), nn.Linear(260, 37), nn.ReLU(), nn.Linear(37, 8)).cuda()
+        x, t = torch.randn(16, 3, 6, 6).cuda(), torch.randint(0, 8, (16,)).cuda()
+        gm = ShampooGradientMaker(model, PreconditioningConfig(data_size=16, damping=1e-6))
+        gm.start_vector_fn = lambda count, n, dev: torch.linspace(-1, 1, count * n, device=dev).reshape(count, n)
+        out = {}
+        for step in range(2):
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+            raw = {}
+            orig = gm.precondition
+
+            def precondition_and_keep():
+                for name, p in model.named_parameters():
+                    raw[name] = p.grad.detach().double().clone()
+                orig()
+            gm.precondition = precondition_and_keep
+            gm.forward_and_backward()
+            gm.precondition = orig
+            for (name, p), pc in zip([(n_, p_) for n_, p_ in model.named_parameters() if p_.ndim > 1], gm.preconditioners):
+                out[(step, name)] = p.grad.detach().clone()
+                if p.ndim == 2:
+                    ref = pc.preconditioners[0].double().T @ raw[name] @ pc.preconditioners[1].double()
+                    # the roots of nearly singular statistics span many decades: the terms of these sums cancel
+                    assert relerr(p.grad, ref) < 1e-3, (grouped, step, name, relerr(p.grad, ref))
+                    print(f'grouped={grouped} step {step} {name}: {relerr(p.grad, ref):.2e}', flush=True)
+        return out
+
+    single, grouped = run(False), run(True)
+    assert single.keys() == grouped.keys()
+    for key in single:
+        assert relerr(grouped[key], single[key].double()) < 1e-3, key
+
+
 def test_block_partitioner_and_dimension_merging():
     from asdl_amd.shampoo import BlockPartitioner, Preconditioner, _merge_small_dims
     assert _merge_small_dims([1, 2, 512, 1, 2048, 1, 3, 4], 1024) == [1024, 2048, 12]
