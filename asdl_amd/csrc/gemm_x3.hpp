@@ -1,9 +1,11 @@
 // fp32 GEMM on the bf16 matrix cores: every fp32 operand element is split exactly into three bf16 pieces
-// (8 + 8 + 8 mantissa bits, by truncation, so hi + mid + lo == x), and the product is accumulated in fp32 from
-// the six piece products that matter:
+// (hi = x rounded to the nearest bf16, mid = x - hi rounded, lo = x - hi - mid, which needs no rounding any more:
+// hi + mid + lo == x), and the product is accumulated in fp32 from the six piece products that matter:
 //   x*y ~= hi*hi' + hi*mid' + mid*hi' + hi*lo' + lo*hi' + mid*mid'      (dropped terms are below 2^-24 |x y|),
 // i.e. the accuracy of an fp32 multiply at 6/16 of the cost of the fp32 MFMA.  With NSPLIT = 2 only hi and mid
-// are kept (16 mantissa bits, mid rounded to nearest; 3 products) for callers whose tolerance allows it.
+// are kept (16 mantissa bits, 3 products) for callers whose tolerance allows it.  Rounding to nearest (one packed
+// hardware conversion per two elements) leaves errors of either sign; cutting the pieces off instead would bias
+// every product towards zero, which a sum of squares (a Gram matrix) accumulates coherently.
 //
 // Same interface as gemm_f32_kernel (GemmParams: transposes, triangular contraction ranges, lower-triangle tile
 // modes, batches).  One work group = 4 waves (2x2) = one 128x128 tile, k-tiles of 32.  The fp32 panels are
@@ -20,6 +22,8 @@ namespace ak {
 
 #define AK_LDS3 __attribute__((address_space(3)))
 typedef uint32_t x3_u32x2 __attribute__((ext_vector_type(2)));
+typedef float x3_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 x3_bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int X3_BT = 128, X3_BK = 32;
 constexpr int X3_PLANE = X3_BT * X3_BK * 2;      // bytes of one bf16 plane of one operand panel
@@ -52,11 +56,6 @@ __device__ __forceinline__ void x3_fetch(X3Fetch& r, const float* __restrict__ P
   }
 }
 
-__device__ __forceinline__ uint32_t x3_pack_hi16(uint32_t lo_word, uint32_t hi_word) {
-  // bf16 (top halves) of two fp32 bit patterns into one dword: element 0 in the low half
-  return __builtin_amdgcn_perm(hi_word, lo_word, 0x07060302u);
-}
-
 // Splits the fetched panel into NSPLIT bf16 planes and writes them to the LDS.
 template <int NSPLIT>
 __device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char* panel, bool kcontig, int tid) {
@@ -71,26 +70,25 @@ __device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char
       const int krow = f >> 5, c4 = f & 31;
       off = (c4 >> 3) * 2048 + krow * 64 + (c4 & 7) * 8;
     }
-    uint32_t piece[NSPLIT][4];
+    // Every piece is the remainder rounded to the nearest bf16 (one packed conversion per pair of elements);
+    // x - hi and x - hi - mid are exact in fp32, and what is left after two pieces has at most 8 significant
+    // bits, so the third piece is exact: hi + mid + lo == x.
+    uint32_t pair[NSPLIT][2];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float rem = r.v[u][e];
+    for (int e = 0; e < 2; ++e) {
+      x3_f32x2 rem = {r.v[u][2 * e], r.v[u][2 * e + 1]};
 #pragma unroll
       for (int s = 0; s < NSPLIT; ++s) {
-        uint32_t bits = __builtin_bit_cast(uint32_t, rem);
-        // the last of two pieces is rounded to nearest even (halves the error and removes its bias); every
-        // other piece is cut off, which keeps the remainder exact (the third piece has no bits left to lose)
-        if (NSPLIT == 2 && s == 1) bits += 0x7fffu + ((bits >> 16) & 1u);
-        const uint32_t top = bits & 0xffff0000u;
-        piece[s][e] = top;
-        if (s + 1 < NSPLIT) rem -= __builtin_bit_cast(float, top);                // exact
+        const x3_bf16x2 h = __builtin_convertvector(rem, x3_bf16x2);
+        pair[s][e] = __builtin_bit_cast(uint32_t, h);
+        if (s + 1 < NSPLIT) rem -= __builtin_convertvector(h, x3_f32x2);
       }
     }
 #pragma unroll
     for (int s = 0; s < NSPLIT; ++s) {
       x3_u32x2 w;
-      w[0] = x3_pack_hi16(piece[s][0], piece[s][1]);
-      w[1] = x3_pack_hi16(piece[s][2], piece[s][3]);
+      w[0] = pair[s][0];
+      w[1] = pair[s][1];
       *reinterpret_cast<AK_LDS3 x3_u32x2*>(panel + s * X3_PLANE + off) = w;
     }
   }
@@ -231,10 +229,12 @@ static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
   gemm_x3_tile<NSPLIT>(p, blockIdx.y, blockIdx.x, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
 }
 
-// Grouped products: many independent C_i <- alpha_i * op(A_i) op(B_i) of different sizes in one launch, so that
-// products too small to fill the device share it and nothing waits on the host between them.  `table` holds one
-// row of GROUPED_ROW int64 per product: A, B, C, lda, ldb, ldc, M, N, K, transA | transB << 1, alpha (float bits in
-// the low word), first tile.  Tiles are numbered row-major inside a product, products in table order (longest
+// Grouped products: many independent C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i of different sizes in one
+// launch, so that products too small to fill the device share it and nothing waits on the host between them.
+// `table` holds one row of GROUPED_ROW int64 per product: A, B, C, lda, ldb, ldc, M, N, K,
+// transA | transB << 1 | symmetric << 2 (symmetric: M == N and the result is known to be symmetric, only the tiles
+// on and below the diagonal are computed and mirrored), alpha and beta (float bits in the low and high word),
+// first tile.  Tiles are numbered row-major inside a product, products in table order (longest
 // contraction first gives the best balance); work group w looks its product up by bisection on `first tile`.
 constexpr int GROUPED_ROW = 12;
 
@@ -259,8 +259,9 @@ static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64
   p.M = static_cast<int>(r[6]); p.N = static_cast<int>(r[7]); p.K = static_cast<int>(r[8]);
   p.transA = static_cast<int>(r[9] & 1); p.transB = static_cast<int>((r[9] >> 1) & 1);
   p.alpha = __builtin_bit_cast(float, static_cast<uint32_t>(r[10]));
-  p.beta = 0.f;
-  p.kmode = K_FULL; p.tile_mode = TILE_ALL;
+  p.beta = __builtin_bit_cast(float, static_cast<uint32_t>(static_cast<uint64_t>(r[10]) >> 32));
+  p.kmode = K_FULL;
+  p.tile_mode = (r[9] & 4) ? TILE_LOWER_MIRROR : TILE_ALL;     // symmetric result: lower tiles only, mirrored
   p.active = nullptr; p.active_stride = 0;
   p.split = NSPLIT;
   const int local = w - static_cast<int>(r[11]);

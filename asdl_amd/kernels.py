@@ -707,17 +707,24 @@ def _grouped_operand_ok(ptr, ld, contiguous_extent):
 
 def _gemm_grouped_table(specs, device):
     """(device table, rows, tiles) for ak_gemm_f32_grouped.  specs: tuples (a_ptr, lda, b_ptr, ldb, c_ptr, ldc, M, N, K,
-    transA, transB, alpha) of device addresses of float32 matrices with contiguous rows."""
+    transA, transB, alpha[, beta[, symmetric]]) of device addresses of float32 matrices with contiguous rows;
+    C <- alpha * op(A) op(B) + beta * C; symmetric: only the lower tiles are computed, and mirrored."""
     rows, first = [], 0
-    for a, lda, b, ldb, c, ldc, M, N, K, tA, tB, alpha in sorted(specs, key=lambda sp: -sp[8]):
+    for spec in sorted(specs, key=lambda sp: -sp[8]):
+        a, lda, b, ldb, c, ldc, M, N, K, tA, tB, alpha = spec[:12]
+        beta = spec[12] if len(spec) > 12 else 0.0
+        symmetric = bool(spec[13]) if len(spec) > 13 else False
         if M <= 0 or N <= 0 or K <= 0:
             continue
+        if symmetric and M != N:
+            raise ValueError('a symmetric product is square')
         if not (_grouped_operand_ok(a, lda, M if tA else K) and _grouped_operand_ok(b, ldb, K if tB else N)):
             raise ValueError('grouped products need 16-byte aligned operands whose leading dimension and '
                              'contiguous extent are multiples of 4')
         if lda < (M if tA else K) or ldb < (K if tB else N) or ldc < N:
             raise ValueError('leading dimension smaller than the row length')
-        rows.append((a, b, c, lda, ldb, ldc, M, N, K, int(bool(tA)) | (int(bool(tB)) << 1), _float_bits(alpha), first))
+        rows.append((a, b, c, lda, ldb, ldc, M, N, K, int(bool(tA)) | (int(bool(tB)) << 1) | (int(symmetric) << 2),
+                     _float_bits(alpha) | (_float_bits(beta) << 32), first))
         first += ((M + 127) // 128) * ((N + 127) // 128)
     if not rows:
         return None, 0, 0

@@ -218,16 +218,20 @@ int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, 
                 float* C, int64_t ldc, int batch, int64_t strideA, int64_t strideB, int64_t strideC,
                 ak_stream_t stream);
 
-/* Many products of different sizes in one launch: C_i <- alpha_i * op(A_i) op(B_i) on the bf16 matrix cores
- * (pieces = 2 or 3 as in ak_gemm_f32_split).  `table` is DEVICE memory, `count` rows of 12 int64:
- *   A, B, C (addresses), lda, ldb, ldc, M, N, K, transA | transB << 1, alpha (float bit pattern in the low
- *   32 bits), first_tile
+/* Many products of different sizes in one launch: C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i on the bf16
+ * matrix cores (pieces = 2 or 3 as in ak_gemm_f32_split).  `table` is DEVICE memory, `count` rows of 12 int64:
+ *   A, B, C (addresses), lda, ldb, ldc, M, N, K, transA | transB << 1 | symmetric << 2, alpha and beta (float
+ *   bit patterns in the low and the high 32 bits), first_tile
+ * (symmetric: M == N and op(A) op(B) is symmetric, e.g. G G^T: only the tiles on and below the diagonal are
+ * computed and mirrored, the result is exactly symmetric)
  * with first_tile the running sum of ceil(M/128) * ceil(N/128) over the rows before, and total_tiles that sum
  * over all rows.  Every operand has to satisfy what the split kernel needs (16-byte aligned addresses, leading
  * dimensions and the contiguous extents of both operands multiples of 4); the table cannot be checked from the
  * host.  Rows sorted by descending K balance best.  Replaces the per-module loop around Kron.mvp of
  * NaturalGradientMaker.precondition (asdl/precondition/natural_gradient.py:481-486, asdl/symmatrix.py:536-548):
- * one call computes Binv_i G_i for every module, a second one (.) Ainv_i. */
+ * one call computes Binv_i G_i for every module, a second one (.) Ainv_i; and the tensordot(G, G) statistics and
+ * the per-axis preconditioning of all matrix-shaped parameters of Shampoo (asdl/precondition/shampoo.py:331-339,
+ * 351-367). */
 int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t total_tiles, ak_stream_t stream);
 
 /* y_i <- alpha * M_i x_i for dense row-major [n_i, n_i] fp32 matrices, one launch.  `table` is DEVICE memory,

@@ -246,6 +246,9 @@ def test_grouped_preconditioning_gives_the_per_parameter_result(monkeypatch):
             gm.precondition = orig
             for (name, p), pc in zip([(n_, p_) for n_, p_ in model.named_parameters() if p_.ndim > 1], gm.preconditioners):
                 out[(step, name)] = p.grad.detach().clone()
+                for a, stat in enumerate(pc.statistics):
+                    out[(step, name, a)] = stat.detach().clone()
+                    assert torch.equal(stat, stat.T)
                 if p.ndim == 2:
                     ref = pc.preconditioners[0].double().T @ raw[name] @ pc.preconditioners[1].double()
                     # the roots of nearly singular statistics span many decades: the terms of these sums cancel
@@ -256,7 +259,12 @@ def test_grouped_preconditioning_gives_the_per_parameter_result(monkeypatch):
     single, grouped = run(False), run(True)
     assert single.keys() == grouped.keys()
     for key in single:
-        assert relerr(grouped[key], single[key].double()) < 1e-3, key
+        if len(key) == 3:
+            # statistics: same kernels either way; the convolution backward kernels of the library are not
+            # reproducible bit for bit from run to run, so the raw gradients may differ in the last bits
+            assert relerr(grouped[key], single[key].double()) < 1e-5, key
+        else:
+            assert relerr(grouped[key], single[key].double()) < 1e-3, key
 
 
 def test_block_partitioner_and_dimension_merging():
