@@ -241,6 +241,9 @@ def _contiguous(x):
         return x.contiguous()
 
 
+FACTOR_STREAM_BATCH = 16      # hook calls per ordering of the factor stream after the main stream
+
+
 class FactorStream:
     """A side stream (default priority) for the statistics kernels of the hooks.  ``run(fn, *tensors)`` orders the
     side stream after everything the calling thread's current stream holds, runs ``fn`` with this thread's kernel
@@ -260,6 +263,8 @@ class FactorStream:
             self._events.append(ev)
         self._next = 0
         self._keep = []
+        self._pending = []
+        self._flushing = False
 
     def _event(self):
         ev = self._events[self._next]
@@ -267,18 +272,41 @@ class FactorStream:
         return ev
 
     def run(self, fn, *tensors):
-        main = _stream_handle(self.device)
-        _lib.check(_lib.load().ak_stream_order(ctypes.c_void_p(main), ctypes.c_void_p(self.handle), self._event()),
-                   'ak_stream_order')
+        """Queues ``fn``; every ``batch`` queued calls are run together behind one ordering of the side stream
+        after the caller's stream (that ordering costs tens of microseconds of host time, more than a hook has to
+        spare).  ``fn`` must not depend on anything but its arguments; its results are only valid after join()."""
+        self._pending.append(fn)
         self._keep.append(tensors)
-        _override.handle, _override.stream = self.handle, self.stream
+        if len(self._pending) >= FACTOR_STREAM_BATCH:
+            self._flush()
+
+    def _flush(self):
+        if self._flushing or not self._pending:
+            return
+        self._flushing = True
+        saved = (getattr(_override, 'handle', None), getattr(_override, 'stream', None))
         try:
-            fn()
+            main = _stream_handle(self.device)
+            _lib.check(_lib.load().ak_stream_order(ctypes.c_void_p(main), ctypes.c_void_p(self.handle), self._event()),
+                       'ak_stream_order')
+            fns, self._pending = self._pending, []
+            _override.handle, _override.stream = self.handle, self.stream
+            for fn in fns:
+                fn()
         finally:
-            _override.handle = _override.stream = None
+            _override.handle, _override.stream = saved
+            self._flushing = False
 
     def join(self):
-        main = _stream_handle(self.device)
+        """Runs what is still queued and makes the caller's stream wait for the side stream.  Called from inside a
+        queued call (a hook that starts the early inverses), it covers the calls that have run so far."""
+        self._flush()
+        saved = (getattr(_override, 'handle', None), getattr(_override, 'stream', None))
+        _override.handle = _override.stream = None
+        try:
+            main = _stream_handle(self.device)
+        finally:
+            _override.handle, _override.stream = saved
         _lib.check(_lib.load().ak_stream_order(ctypes.c_void_p(self.handle), ctypes.c_void_p(main), self._event()),
                    'ak_stream_order')
         keep, self._keep = self._keep, []
