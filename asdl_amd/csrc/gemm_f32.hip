@@ -184,3 +184,5 @@ extern "C" void ak_debug_set_gemm_split_threshold(int min_groups, int min_k) {
   ak::g_x3_min_groups = min_groups;
   ak::g_x3_min_k = min_k;
 }
+
+extern "C" void ak_debug_set_gemm_double_buffer(int on) { ak::g_x3_double_buffer = on; }

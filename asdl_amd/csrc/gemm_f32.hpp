@@ -199,6 +199,7 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
 
 namespace ak {
 
+inline int g_x3_double_buffer = 1;                     // tuning hook (ak_debug_set_gemm_double_buffer)
 inline int g_x3_min_groups = 100, g_x3_min_k = 256;   // tuning hook (ak_debug_set_gemm_split_threshold)
 
 inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
@@ -210,8 +211,18 @@ inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   // fill most of the device; below that the 64 x 64 tiles of the fp32 kernel spread the work better.
   if (p.split >= 2 && work_groups >= g_x3_min_groups && p.K >= g_x3_min_k && gemm_x3_ok(p)) {
     dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
-    if (p.split == 2) hipLaunchKernelGGL(gemm_x3_kernel<2>, grid, dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(gemm_x3_kernel<3>, grid, dim3(256), 0, stream, p);
+    // three pieces: the double-buffered loop (one work group per CU, MFMAs and split arithmetic interleaved by
+    // hand), one instantiation per pair of operand layouts; two pieces: the single-buffered loop
+    if (p.split == 3 && g_x3_double_buffer) {
+      if (p.transA == 0 && p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 1>), grid, dim3(256), 0, stream, p);
+      else if (p.transA == 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 0>), grid, dim3(256), 0, stream, p);
+      else if (p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 1>), grid, dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 0>), grid, dim3(256), 0, stream, p);
+    } else if (p.split == 2) {
+      hipLaunchKernelGGL((gemm_x3_kernel<2, false>), grid, dim3(256), 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((gemm_x3_kernel<3, false>), grid, dim3(256), 0, stream, p);
+    }
     return check_launch();
   }
   // 128 x 128 tiles when they alone fill the 256 CUs twice over, else 64 x 64 tiles (four times the work groups)

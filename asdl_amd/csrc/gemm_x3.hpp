@@ -8,12 +8,19 @@
 // every product towards zero, which a sum of squares (a Gram matrix) accumulates coherently.
 //
 // Same interface as gemm_f32_kernel (GemmParams: transposes, triangular contraction ranges, lower-triangle tile
-// modes, batches).  One work group = 4 waves (2x2) = one 128x128 tile, k-tiles of 32.  The fp32 panels are
-// fetched into registers one k-tile ahead, split and written to the LDS as bf16 planes after the MFMAs of the
-// current k-tile.  An operand whose contraction index is contiguous in memory is kept as [row][32 k] with the
-// 16-byte chunks of a row XOR-swizzled by (row/4)%4, so that the ds_read_b128 of 16 consecutive rows hits 64
-// different banks; one whose row/column index is contiguous is kept as [32 columns][32 k-rows][64 B] blocks
-// and read with ds_read_b64_tr_b16 (no bank conflicts, no transposed copies).
+// modes, batches).  One work group = 4 waves (2x2) = one 128x128 tile, k-tiles of 32.  An operand whose contraction
+// index is contiguous in memory is kept in the LDS as [row][32 k] with the 16-byte chunks of a row XOR-swizzled by
+// (row/4)%4, so that the ds_read_b128 of 16 consecutive rows hits 64 different banks; one whose row/column index
+// is contiguous is kept as [32 columns][32 k-rows][64 B] blocks and read with ds_read_b64_tr_b16 (no bank
+// conflicts, no transposed copies).
+//
+// Two main loops.  Single-buffered (two work groups per CU, which overlap each other): the fp32 panels are fetched
+// into registers one k-tile ahead, split and written to the LDS after the MFMAs of the current k-tile, two
+// barriers per k-tile.  Double-buffered (DB, 96 KB of LDS, one work group per CU): one barrier per k-tile and a
+// fixed instruction order in which every MFMA is followed by a sixth of the split of one float4 of the next
+// k-tile, so that the vector ALU works in the shadow of the matrix pipe; the operand layouts are template
+// parameters there, which makes the loop body a single basic block.  Measured on 4096^3: 776 -> 697 us, on
+// 2048^3 (one tile per CU) 150 -> 96 us.
 #pragma once
 #include <type_traits>
 #include "common.hpp"
@@ -54,6 +61,33 @@ __device__ __forceinline__ void x3_fetch(X3Fetch& r, const float* __restrict__ P
       r.v[u] = ok ? w : z;
     }
   }
+}
+
+// One of this thread's four float4 of a panel (chunk u of x3_fetch).
+template <bool INTERIOR>
+__device__ __forceinline__ floatx4 x3_fetch_one(const float* __restrict__ P, int64_t ld, bool kcontig, int r0, int r_end,
+                                                int k0, int k_end, int tid, int u) {
+  const int f = tid + 256 * u;
+  int outer, inner, o_end, i_end;
+  if (kcontig) { outer = r0 + (f >> 3); inner = k0 + 4 * (f & 7); o_end = r_end; i_end = k_end; }
+  else { outer = k0 + (f >> 5); inner = r0 + 4 * (f & 31); o_end = k_end; i_end = r_end; }
+  if (INTERIOR) return *reinterpret_cast<const floatx4*>(P + static_cast<int64_t>(outer) * ld + inner);
+  const bool ok = outer < o_end && inner < i_end;
+  const float* src = ok ? P + static_cast<int64_t>(outer) * ld + inner : P;
+  const floatx4 w = *reinterpret_cast<const floatx4*>(src);
+  const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+  return ok ? w : z;
+}
+
+// Byte offset of chunk u inside a plane (the layouts of x3_stash).
+__device__ __forceinline__ uint32_t x3_chunk_offset(bool kcontig, int tid, int u) {
+  const int f = tid + 256 * u;
+  if (kcontig) {
+    const int row = f >> 3, c4 = f & 7;
+    return row * 64 + 16 * ((c4 >> 1) ^ ((row >> 2) & 3)) + 8 * (c4 & 1);
+  }
+  const int krow = f >> 5, c4 = f & 31;
+  return (c4 >> 3) * 2048 + krow * 64 + (c4 & 7) * 8;
 }
 
 // Splits the fetched panel into NSPLIT bf16 planes and writes them to the LDS.
@@ -109,9 +143,10 @@ __device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bo
 }
 
 // One 128 x 128 tile (ti, tj) of batch entry z of the product described by p.
-template <int NSPLIT>
+template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1>
 __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj, int z, AK_LDS3 unsigned char* lds) {
   constexpr int BT = X3_BT, BK = X3_BK;
+  constexpr int BUF = 2 * NSPLIT * X3_PLANE;        // both operands' planes of one k-tile
   AK_LDS3 unsigned char* panelA = lds;
   AK_LDS3 unsigned char* panelB = lds + NSPLIT * X3_PLANE;
   if (p.active != nullptr && p.active[static_cast<int64_t>(z) * p.active_stride] == 0) return;
@@ -130,7 +165,8 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
   const float* __restrict__ A = p.A + static_cast<int64_t>(z) * p.sA;
   const float* __restrict__ B = p.B + static_cast<int64_t>(z) * p.sB;
   float* __restrict__ C = p.C_list != nullptr ? p.C_list[z] : p.C + static_cast<int64_t>(z) * p.sC;
-  const bool a_kc = (p.transA == 0), b_kc = (p.transB != 0);
+  // operand layouts: fixed at compile time where the caller knows them (one basic block per loop body then)
+  const bool a_kc = AKC < 0 ? (p.transA == 0) : (AKC != 0), b_kc = BKC < 0 ? (p.transB != 0) : (BKC != 0);
   const int i0 = ti * BT, j0 = tj * BT;
 
   floatx16 acc[2][2];
@@ -144,60 +180,144 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
   const int nk = kbeg < kend ? (kend - kbeg + BK - 1) / BK : 0;
   const bool interior = i0 + BT <= p.M && j0 + BT <= p.N && (kend - kbeg) % BK == 0;
 
+  // The MFMAs of one k-tile, operands read from the planes at `buf`.
+  auto multiply = [&](AK_LDS3 unsigned char* buf) {
+    AK_LDS3 unsigned char* pa = buf;
+    AK_LDS3 unsigned char* pb = buf + NSPLIT * X3_PLANE;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      bf16x8 fa[2][NSPLIT], fb[2][NSPLIT];
+#pragma unroll
+      for (int s = 0; s < NSPLIT; ++s) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) fa[a][s] = x3_frag(pa + s * X3_PLANE, a_kc, 64 * wr + 32 * a + l32, h, lane);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) fb[b][s] = x3_frag(pb + s * X3_PLANE, b_kc, 64 * wc + 32 * b + l32, h, lane);
+      }
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          // smallest terms first
+          if constexpr (NSPLIT >= 3) {
+            acc[a][b] = mfma_bf16(fa[a][1], fb[b][1], acc[a][b]);
+            acc[a][b] = mfma_bf16(fa[a][0], fb[b][2], acc[a][b]);
+            acc[a][b] = mfma_bf16(fa[a][2], fb[b][0], acc[a][b]);
+          }
+          if constexpr (NSPLIT >= 2) {
+            acc[a][b] = mfma_bf16(fa[a][0], fb[b][1], acc[a][b]);
+            acc[a][b] = mfma_bf16(fa[a][1], fb[b][0], acc[a][b]);
+          }
+          acc[a][b] = mfma_bf16(fa[a][0], fb[b][0], acc[a][b]);
+        }
+    }
+  };
+
   auto mainloop = [&](auto interior_tag) {
     constexpr bool INTERIOR = decltype(interior_tag)::value;
     X3Fetch ra, rb;
+    auto fetch = [&](int kt) {
+      const int k0 = kbeg + kt * BK;
+      x3_fetch<INTERIOR>(ra, A, p.lda, a_kc, i0, p.M, k0, kend, tid);
+      x3_fetch<INTERIOR>(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, tid);
+    };
+    auto stash = [&](AK_LDS3 unsigned char* buf) {
+      x3_stash<NSPLIT>(ra, buf, a_kc, tid);
+      x3_stash<NSPLIT>(rb, buf + NSPLIT * X3_PLANE, b_kc, tid);
+    };
     if (nk > 0) {
-      x3_fetch<INTERIOR>(ra, A, p.lda, a_kc, i0, p.M, kbeg, kend, tid);
-      x3_fetch<INTERIOR>(rb, B, p.ldb, b_kc, j0, p.N, kbeg, kend, tid);
-      x3_stash<NSPLIT>(ra, panelA, a_kc, tid);
-      x3_stash<NSPLIT>(rb, panelB, b_kc, tid);
+      fetch(0);
+      stash(lds);
     }
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-      if (kt + 1 < nk) {                    // next k-tile's global loads fly during this one's MFMAs
-        const int k0 = kbeg + (kt + 1) * BK;
-        x3_fetch<INTERIOR>(ra, A, p.lda, a_kc, i0, p.M, k0, kend, tid);
-        x3_fetch<INTERIOR>(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, tid);
-      }
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        bf16x8 fa[2][NSPLIT], fb[2][NSPLIT];
-#pragma unroll
-        for (int s = 0; s < NSPLIT; ++s) {
-#pragma unroll
-          for (int a = 0; a < 2; ++a) fa[a][s] = x3_frag(panelA + s * X3_PLANE, a_kc, 64 * wr + 32 * a + l32, h, lane);
-#pragma unroll
-          for (int b = 0; b < 2; ++b) fb[b][s] = x3_frag(panelB + s * X3_PLANE, b_kc, 64 * wc + 32 * b + l32, h, lane);
-        }
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int b = 0; b < 2; ++b) {
-            // smallest terms first
-            if constexpr (NSPLIT >= 3) {
-              acc[a][b] = mfma_bf16(fa[a][1], fb[b][1], acc[a][b]);
-              acc[a][b] = mfma_bf16(fa[a][0], fb[b][2], acc[a][b]);
-              acc[a][b] = mfma_bf16(fa[a][2], fb[b][0], acc[a][b]);
-            }
-            if constexpr (NSPLIT >= 2) {
-              acc[a][b] = mfma_bf16(fa[a][0], fb[b][1], acc[a][b]);
-              acc[a][b] = mfma_bf16(fa[a][1], fb[b][0], acc[a][b]);
-            }
-            acc[a][b] = mfma_bf16(fa[a][0], fb[b][0], acc[a][b]);
-          }
-      }
-      __syncthreads();                      // everybody is done reading this k-tile
-      if (kt + 1 < nk) {
-        x3_stash<NSPLIT>(ra, panelA, a_kc, tid);
-        x3_stash<NSPLIT>(rb, panelB, b_kc, tid);
-      }
+    if constexpr (DB) {
+      // Two LDS buffers, one barrier per k-tile: the split and store of k-tile kt+1 (into the other buffer) and
+      // the global loads of k-tile kt+2 are issued ahead of the MFMAs of k-tile kt, in whose shadow they run.
+      if (nk > 1) fetch(1);
       __syncthreads();
+      int kt = 0;
+      if constexpr (NSPLIT == 3 && AKC >= 0 && BKC >= 0) {
+        // Fixed instruction order, one matrix instruction at a time: MFMA m of this k-tile, then one sixth of
+        // the split of one float4 of the next k-tile (a packed conversion, two unpacks, two subtractions: about
+        // as many cycles as the MFMA keeps the matrix pipe busy); after the sixth sixth the three LDS stores of
+        // that float4 and the global load that refills its registers from the k-tile after next.  48 MFMAs, 48
+        // sixths (8 float4 per thread x 3 pieces x 2 pairs).
+        uint32_t offA[4], offB[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { offA[u] = x3_chunk_offset(a_kc, tid, u); offB[u] = x3_chunk_offset(b_kc, tid, u); }
+        for (; kt + 2 < nk; ++kt) {
+          AK_LDS3 unsigned char* cur = lds + (kt & 1) * BUF;
+          AK_LDS3 unsigned char* nxt = lds + ((kt + 1) & 1) * BUF;
+          const int k2 = kbeg + (kt + 2) * BK;
+          // all LDS reads of this k-tile first: the stores into the other buffer cannot be proven not to alias
+          bf16x8 fa[2][2][NSPLIT], fb[2][2][NSPLIT];
+          auto read_frags = [&](int h) {
+#pragma unroll
+            for (int q = 0; q < NSPLIT; ++q) {
+#pragma unroll
+              for (int a = 0; a < 2; ++a) fa[h][a][q] = x3_frag(cur + q * X3_PLANE, a_kc, 64 * wr + 32 * a + l32, h, lane);
+#pragma unroll
+              for (int b = 0; b < 2; ++b)
+                fb[h][b][q] = x3_frag(cur + (NSPLIT + q) * X3_PLANE, b_kc, 64 * wc + 32 * b + l32, h, lane);
+            }
+          };
+          read_frags(0);
+          read_frags(1);
+          __builtin_amdgcn_sched_barrier(0);
+          uint32_t pair[NSPLIT][2];
+          x3_f32x2 rem;
+#pragma unroll
+          for (int m = 0; m < 48; ++m) {
+            {   // matrix instruction m: (h, a, b) and the term, smallest terms first
+              constexpr int PA[6] = {1, 0, 2, 0, 1, 0}, PB[6] = {1, 2, 0, 1, 0, 0};
+              const int h = m / 24, ab = (m % 24) / 6, t = m % 6;
+              acc[ab >> 1][ab & 1] = mfma_bf16(fa[h][ab >> 1][PA[t]], fb[h][ab & 1][PB[t]], acc[ab >> 1][ab & 1]);
+            }
+            {   // sixth m of the split: float4 u (0..3 of A, 4..7 of B), pair e, piece q
+              const int u = m / 6, q = (m % 6) / 2, e = m % 2;
+              const floatx4& v = u < 4 ? ra.v[u & 3] : rb.v[u & 3];
+              if (q == 0) rem = x3_f32x2{v[2 * e], v[2 * e + 1]};
+              else rem = x3_f32x2{v[2 * e], v[2 * e + 1]} - __builtin_convertvector(__builtin_bit_cast(x3_bf16x2, pair[0][e]), x3_f32x2)
+                         - (q == 2 ? __builtin_convertvector(__builtin_bit_cast(x3_bf16x2, pair[1][e]), x3_f32x2) : x3_f32x2{0.f, 0.f});
+              pair[q][e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rem, x3_bf16x2));
+              if (m % 6 == 5) {
+                AK_LDS3 unsigned char* dst = (u < 4 ? nxt + offA[u & 3] : nxt + NSPLIT * X3_PLANE + offB[u & 3]);
+#pragma unroll
+                for (int w = 0; w < NSPLIT; ++w) {
+                  x3_u32x2 word;
+                  word[0] = pair[w][0];
+                  word[1] = pair[w][1];
+                  *reinterpret_cast<AK_LDS3 x3_u32x2*>(dst + w * X3_PLANE) = word;
+                }
+                if (u < 4) ra.v[u & 3] = x3_fetch_one<INTERIOR>(A, p.lda, a_kc, i0, p.M, k2, kend, tid, u & 3);
+                else rb.v[u & 3] = x3_fetch_one<INTERIOR>(B, p.ldb, b_kc, j0, p.N, k2, kend, tid, u & 3);
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          __syncthreads();
+        }
+      }
+      for (; kt < nk; ++kt) {
+        AK_LDS3 unsigned char* cur = lds + (kt & 1) * BUF;
+        AK_LDS3 unsigned char* nxt = lds + ((kt + 1) & 1) * BUF;
+        if (kt + 1 < nk) stash(nxt);
+        multiply(cur);
+        __syncthreads();
+      }
+    } else {
+      __syncthreads();
+      for (int kt = 0; kt < nk; ++kt) {
+        if (kt + 1 < nk) fetch(kt + 1);       // next k-tile's global loads fly during this one's MFMAs
+        multiply(lds);
+        __syncthreads();                      // everybody is done reading this k-tile
+        if (kt + 1 < nk) stash(lds);
+        __syncthreads();
+      }
     }
   };
   if (interior) mainloop(std::true_type{});
   else mainloop(std::false_type{});
-  (void)g;
+  (void)g; (void)panelA; (void)panelB;
 
   // the partial products of (i, j) and (j, i) are summed in different orders, so a mirrored result takes both
   // triangles of a diagonal tile from the lower one
@@ -223,10 +343,10 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
     }
 }
 
-template <int NSPLIT>
+template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1>
 static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
-  gemm_x3_tile<NSPLIT>(p, blockIdx.y, blockIdx.x, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
+  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[(DB ? 2 : 1) * 2 * NSPLIT * X3_PLANE];
+  gemm_x3_tile<NSPLIT, DB, AKC, BKC>(p, blockIdx.y, blockIdx.x, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // Grouped products: many independent C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i of different sizes in one
@@ -268,7 +388,9 @@ static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64
   const int tn = (p.N + X3_BT - 1) / X3_BT;
   const int ti = local / tn, tj = local - ti * tn;
   if (ti * X3_BT >= p.M) return;            // a table whose tile count overstates this product
-  gemm_x3_tile<NSPLIT>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+  // two work groups per CU with the single-buffered loop serve the mix of long and short contractions of a
+  // grouped launch better than one work group with the double-buffered loop (measured: 0.99 against 1.25 ms)
+  gemm_x3_tile<NSPLIT, false>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // The split kernel takes operands whose 16-byte chunks never straddle the end of a row.
