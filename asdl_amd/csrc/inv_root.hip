@@ -9,6 +9,8 @@
 
 namespace ak {
 
+inline int g_root_split = 3;      // products of the Newton iteration: 3 = split-bf16 kernel (fp32-grade accuracy), 0 = fp32 MFMA
+
 constexpr int RCHUNKS = 64;   // partial-reduction chunks per matrix
 
 struct RootState {
@@ -316,6 +318,7 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
     GemmParams g = make_gemm(0, 0, N, N, N, 1.f, A, n, B, n, 0.f, C, n);
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.active = st.active; g.active_stride = 1;
+    g.split = g_root_split;
     return launch_gemm(g, batch, s);
   };
   for (int it = 0; it < max_iter; ++it) {
@@ -378,3 +381,7 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
   hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
   return check_launch();
 }
+
+// Tuning hook, not part of the interface: 0 = the fp32 MFMA kernel, 3 = the three-piece split kernel for the
+// products of the Newton iteration.
+extern "C" void ak_debug_set_root_split(int pieces) { ak::g_root_split = pieces; }
