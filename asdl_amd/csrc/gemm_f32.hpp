@@ -102,13 +102,12 @@ __device__ __forceinline__ void gemm_frag(float (&f)[8], const float* __restrict
   }
 }
 
+// One BT x BT tile (ti, tj) of batch entry z of the product described by p; lds: [2][2][PANEL] floats.
 template <int TI>
-static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
+__device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int tj, int z,
+                                              float (*lds)[2][GemmTile<64 * TI>::PANEL]) {
   constexpr int BT = 64 * TI;
-  __shared__ __attribute__((aligned(16))) float lds[2][2][GemmTile<BT>::PANEL];
-  const int z = blockIdx.z;
   if (p.active != nullptr && p.active[static_cast<int64_t>(z) * p.active_stride] == 0) return;
-  const int tj = blockIdx.x, ti = blockIdx.y;
   if (p.tile_mode != TILE_ALL && ti < tj) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave >> 1, wc = wave & 1, g = lane >> 5, l32 = lane & 31;
@@ -191,6 +190,12 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
         if (mirror) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
       }
     }
+}
+
+template <int TI>
+static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(16))) float lds[2][2][GemmTile<64 * TI>::PANEL];
+  gemm_f32_tile<TI>(p, blockIdx.y, blockIdx.x, blockIdx.z, lds);
 }
 
 }  // namespace ak

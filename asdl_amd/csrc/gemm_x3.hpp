@@ -358,10 +358,9 @@ static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
 // contraction first gives the best balance); work group w looks its product up by bisection on `first tile`.
 constexpr int GROUPED_ROW = 12;
 
-template <int NSPLIT>
-static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
-  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
-  const int w = blockIdx.x;
+// Product and tile of work group w of a grouped launch; false for a tile the table overstates.
+__device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table, int count, int w, GemmParams& p,
+                                               int& ti, int& tj) {
   int lo = 0, hi = count - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
@@ -369,7 +368,6 @@ static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64
     else hi = mid - 1;
   }
   const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * GROUPED_ROW;
-  GemmParams p;
   p.A = reinterpret_cast<const float*>(r[0]);
   p.B = reinterpret_cast<const float*>(r[1]);
   p.C = reinterpret_cast<float*>(r[2]);
@@ -383,14 +381,32 @@ static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64
   p.kmode = K_FULL;
   p.tile_mode = (r[9] & 4) ? TILE_LOWER_MIRROR : TILE_ALL;     // symmetric result: lower tiles only, mirrored
   p.active = nullptr; p.active_stride = 0;
-  p.split = NSPLIT;
+  p.split = 0;
   const int local = w - static_cast<int>(r[11]);
   const int tn = (p.N + X3_BT - 1) / X3_BT;
-  const int ti = local / tn, tj = local - ti * tn;
-  if (ti * X3_BT >= p.M) return;            // a table whose tile count overstates this product
+  ti = local / tn;
+  tj = local - ti * tn;
+  return ti * X3_BT < p.M;
+}
+
+template <int NSPLIT>
+static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
+  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
+  GemmParams p;
+  int ti, tj;
+  if (!grouped_lookup(table, count, blockIdx.x, p, ti, tj)) return;
   // two work groups per CU with the single-buffered loop serve the mix of long and short contractions of a
   // grouped launch better than one work group with the double-buffered loop (measured: 0.99 against 1.25 ms)
   gemm_x3_tile<NSPLIT, false>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+}
+
+// The same with true fp32 products (v_mfma_f32_32x32x2_f32, one accumulation per k): 128 x 128 tiles as above.
+static __global__ __launch_bounds__(256) void gemm_f32_grouped_kernel(const int64_t* __restrict__ table, int count) {
+  __shared__ __attribute__((aligned(16))) float lds[2][2][GemmTile<128>::PANEL];
+  GemmParams p;
+  int ti, tj;
+  if (!grouped_lookup(table, count, blockIdx.x, p, ti, tj)) return;
+  gemm_f32_tile<2>(p, ti, tj, 0, lds);
 }
 
 // The split kernel takes operands whose 16-byte chunks never straddle the end of a row.

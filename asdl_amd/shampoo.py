@@ -101,6 +101,7 @@ def _axis_statistic(grad, axis, out, alpha, beta):
 
 
 GROUPED_PRECONDITION = True      # matrix-shaped parameters: all their preconditioning products in two launches
+GROUPED_STATISTIC_MIN_DIM = 1024  # statistics of this size and up go into one grouped launch (with GROUPED_PRECONDITION)
 
 
 def _precondition_block(grad, preconditioners):
@@ -152,14 +153,16 @@ class Preconditioner:
             raise TypeError('Shampoo statistics are float32: keep parameters (and so their gradients) in float32')
         return self._partitioner.partition(grad.detach().reshape(self._transformed_shape))
 
-    def update_statistics(self):
+    def update_statistics(self, skip_axes=()):
+        """``skip_axes``: axes whose statistic the caller has updated itself (the gradient maker's grouped launch)."""
         ema_decay = self.config.ema_decay
         alpha, beta = (1.0, 1.0) if ema_decay == _invalid else (float(ema_decay), 1.0 - float(ema_decay))
         ndim = len(self._transformed_shape)
         for j, block in enumerate(self._blocks_of_grad()):
             block = block if block.is_contiguous() else block.contiguous()
             for i in range(ndim):
-                _axis_statistic(block, i, self.statistics[j * ndim + i], alpha, beta)
+                if i not in skip_axes:
+                    _axis_statistic(block, i, self.statistics[j * ndim + i], alpha, beta)
 
     def update_preconditioners(self):
         """L^(-1/exponent) of every statistic, one at a time (asdl/precondition/shampoo.py:341-349); the gradient
@@ -253,11 +256,33 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
         return grouped, [pc for pc in self.preconditioners if id(pc) not in taken]
 
     def update_curvature(self):
-        # The statistics stay on the fp32 MFMA SYRK kernels, one parameter at a time: the inverse roots of
-        # ill-conditioned statistics magnify what a different summation changes in the last bits, and the grouped
-        # split-bf16 product moved the roots of the golden runs further from the exact ones than the bar allows.
+        """Statistics of every axis (asdl/precondition/shampoo.py:331-339).  The large ones of matrix-shaped
+        parameters (GROUPED_STATISTIC_MIN_DIM and up), G G^T or G^T G, run in one grouped launch of the fp32 MFMA
+        tile kernel (true fp32 products, one accumulation per k like the SYRK kernels; lower tiles, mirrored: exactly
+        symmetric; the EMA folded into alpha / beta).  Small statistics stay on the SYRK kernels, one at a time: the
+        inverse roots of small, ill-conditioned statistics magnify what a different summation order changes in the
+        last bits, and the golden runs of the reference pin those."""
+        grouped, _ = self._split_groupable()
+        done = {}
+        if grouped:
+            ema_decay = self.config.ema_decay
+            alpha, beta = (1.0, 1.0) if ema_decay == _invalid else (float(ema_decay), 1.0 - float(ema_decay))
+            specs = []
+            for pc in grouped:
+                m, n = pc._transformed_shape
+                g = pc.param.grad.data_ptr()
+                axes = []
+                if m >= GROUPED_STATISTIC_MIN_DIM:
+                    specs.append((g, n, g, n, pc.statistics[0].data_ptr(), m, m, m, n, 0, 1, alpha, beta, True))
+                    axes.append(0)
+                if n >= GROUPED_STATISTIC_MIN_DIM:
+                    specs.append((g, n, g, n, pc.statistics[1].data_ptr(), n, n, n, m, 1, 0, alpha, beta, True))
+                    axes.append(1)
+                done[id(pc)] = tuple(axes)
+            if specs:
+                kernels.gemm_grouped_raw(specs, grouped[0].param.device, pieces=0)
         for preconditioner in self.preconditioners:
-            preconditioner.update_statistics()
+            preconditioner.update_statistics(skip_axes=done.get(id(preconditioner), ()))
 
     def update_preconditioner(self):
         """All inverse roots of one size in one batched call (per matrix:

@@ -219,7 +219,8 @@ int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, 
                 ak_stream_t stream);
 
 /* Many products of different sizes in one launch: C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i on the bf16
- * matrix cores (pieces = 2 or 3 as in ak_gemm_f32_split).  `table` is DEVICE memory, `count` rows of 12 int64:
+ * matrix cores (pieces = 2 or 3 as in ak_gemm_f32_split) or with true fp32 products (pieces = 0, the fp32 MFMA, one
+ * accumulation per k; needs no alignment).  `table` is DEVICE memory, `count` rows of 12 int64:
  *   A, B, C (addresses), lda, ldb, ldc, M, N, K, transA | transB << 1 | symmetric << 2, alpha and beta (float
  *   bit patterns in the low and the high 32 bits), first_tile
  * (symmetric: M == N and op(A) op(B) is symmetric, e.g. G G^T: only the tiles on and below the diagonal are

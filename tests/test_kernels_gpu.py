@@ -413,17 +413,19 @@ def test_gemm_grouped_matches_fp64(K):
         for (A, B, C, tA, tB, alpha), ref in zip(problems, refs):
             assert relerr(C, ref) < tol, (tuple(C.shape), A.shape, relerr(C, ref))
     # accumulate form and symmetric products (lower tiles, mirrored) through the raw table
-    G = torch.randn(260, 516, device='cuda')
-    S0 = torch.randn(260, 260, device='cuda'); S0 = S0 + S0.T
-    S1 = torch.randn(516, 516, device='cuda'); S1 = S1 + S1.T
-    r0 = 0.3 * G.double() @ G.double().T + 0.7 * S0.double()
-    r1 = 0.3 * G.double().T @ G.double() + 0.7 * S1.double()
-    g = G.data_ptr()
-    K.gemm_grouped_raw([(g, 516, g, 516, S0.data_ptr(), 260, 260, 260, 516, 0, 1, 0.3, 0.7, True),
-                        (g, 516, g, 516, S1.data_ptr(), 516, 516, 516, 260, 1, 0, 0.3, 0.7, True)], G.device, pieces=3)
-    torch.cuda.synchronize()
-    assert relerr(S0, r0) < 2e-6 and relerr(S1, r1) < 2e-6
-    assert torch.equal(S0, S0.T) and torch.equal(S1, S1.T)
+    for pieces in (3, 0):          # 0: the grouped kernel with true fp32 products
+        G = torch.randn(260, 516, device='cuda')
+        S0 = torch.randn(260, 260, device='cuda'); S0 = S0 + S0.T
+        S1 = torch.randn(516, 516, device='cuda'); S1 = S1 + S1.T
+        r0 = 0.3 * G.double() @ G.double().T + 0.7 * S0.double()
+        r1 = 0.3 * G.double().T @ G.double() + 0.7 * S1.double()
+        g = G.data_ptr()
+        K.gemm_grouped_raw([(g, 516, g, 516, S0.data_ptr(), 260, 260, 260, 516, 0, 1, 0.3, 0.7, True),
+                            (g, 516, g, 516, S1.data_ptr(), 516, 516, 516, 260, 1, 0, 0.3, 0.7, True)], G.device,
+                           pieces=pieces)
+        torch.cuda.synchronize()
+        assert relerr(S0, r0) < 2e-6 and relerr(S1, r1) < 2e-6, pieces
+        assert torch.equal(S0, S0.T) and torch.equal(S1, S1.T), pieces
     with pytest.raises(ValueError):
         K.gemm_grouped([(torch.randn(6, 6, device='cuda'), torch.randn(6, 6, device='cuda'),
                          torch.empty(6, 6, device='cuda'), False, False, 1.0)])       # extents not multiples of 4
