@@ -44,10 +44,12 @@ def parse():
     ap.add_argument('--with-batchnorm', action='store_true',
                     help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
                          '(the headline configuration ignores them, as the reference training script does)')
-    ap.add_argument('--workload', default='resnet50', choices=['resnet50', 'linear4096'],
+    ap.add_argument('--workload', default='resnet50', choices=['resnet50', 'linear4096', 'shampoo_gpt2'],
                     help="resnet50: the headline benchmark.  linear4096: the large single-layer configuration, a single "
                          'Linear 4096x4096 with bias on 8192 bf16 rows, EMA 0.95 (factor + inverse + precondition of one '
-                         'large layer; its own metric name, not the headline)')
+                         'large layer; its own metric name, not the headline).  shampoo_gpt2: ShampooGradientMaker '
+                         'on a 12-layer GPT-2-small-shaped decoder, 8 x 1024 random tokens, bf16 autocast, statistics and '
+                         'preconditioning every step, inverse 4th roots every 10 steps, epsilon 1e-6 (own metric name)')
     ap.add_argument('--swift', action='store_true',
                     help='KfacGradientMaker(swift=True): factors of layers with fewer samples than columns are kept as '
                          'row matrices (SKFAC); not the headline configuration')
@@ -128,7 +130,9 @@ def main():
     autotune = not args.no_conv_autotune and args.memory_format == 'channels_last'
     torch.backends.cudnn.benchmark = autotune
     torch.manual_seed(0)
-    if args.workload == 'linear4096':
+    if args.workload == 'shampoo_gpt2':
+        pass                                             # built below, with its own gradient maker
+    elif args.workload == 'linear4096':
         model = nn.Sequential(nn.Linear(4096, 4096, bias=True)).to(dev)
         bs = 8192
         x = torch.randn(bs, 4096).to(dev).to(torch.bfloat16)
@@ -144,17 +148,30 @@ def main():
         t = torch.randint(0, 1000, (bs,)).to(dev)
         ignore = [] if args.with_batchnorm else [nn.BatchNorm2d]
         config = PreconditioningConfig(data_size=bs, damping=args.damping, ignore_modules=ignore)
-    gm = KfacGradientMaker(model, config, fisher_type=args.fisher, swift=args.swift)
-    opt = torch.optim.SGD(model.parameters(), lr=1e-4)
+    if args.workload == 'shampoo_gpt2':
+        from asdl_amd import ShampooGradientMaker
+        model = bench_models.gpt2_small().to(dev)       # token embedding and output head frozen (50257-wide)
+        bs = 8
+        x = torch.randint(0, 50257, (bs, 1024)).to(dev)
+        t = torch.randint(0, 50257, (bs * 1024,)).to(dev)
+        config = PreconditioningConfig(damping=1e-6, preconditioner_upd_interval=10)
+        gm = ShampooGradientMaker(model, config)
+        args.no_factor_timing = True
+    else:
+        gm = KfacGradientMaker(model, config, fisher_type=args.fisher, swift=args.swift)
+    opt = torch.optim.SGD([p for p in model.parameters() if p.requires_grad], lr=1e-4)
 
     def fwd(inp):
         with torch.autocast('cuda', dtype=torch.bfloat16):
             return model(inp).float()
 
+    def loss_fn(y, target):
+        return F.cross_entropy(y.reshape(-1, y.shape[-1]), target)
+
     def step():
         opt.zero_grad(set_to_none=True)
         dummy_y = gm.setup_model_call(fwd, x)
-        gm.setup_loss_call(F.cross_entropy, dummy_y, t)
+        gm.setup_loss_call(loss_fn, dummy_y, t)
         gm.forward_and_backward()
         opt.step()
 
@@ -235,6 +252,13 @@ def main():
         if 'roofline' in out:
             out['roofline']['traffic'] = None
             out['roofline']['kernel'] = 'factor statistics (syrk_dtl_kernel, 8192 x 4096 bf16 operands), SYRK FLOP M*d*(d+1)'
+    elif args.workload == 'shampoo_gpt2':
+        out['metric'] = 'Shampoo steps/s GPT-2-small decoder, 8x1024 tokens'
+        out['config'] = {'workload': 'Shampoo step (L/R statistics and preconditioning of the 49 trainable weight matrices '
+                                     'every step, inverse 4th roots every 10 steps, epsilon 1e-6) on a 12-layer '
+                                     'GPT-2-small-shaped decoder (d 768, 12 heads, MLP 3072; token embedding and output '
+                                     'head frozen), 8 x 1024 uniform random tokens, bf16 autocast forward/backward, '
+                                     'fp32 statistics and roots', 'batch': bs}
     elif not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(args)
     print(json.dumps(out))
