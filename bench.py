@@ -165,8 +165,11 @@ def main():
         with torch.autocast('cuda', dtype=torch.bfloat16):
             return model(inp).float()
 
-    def loss_fn(y, target):
+    def token_loss(y, target):
         return F.cross_entropy(y.reshape(-1, y.shape[-1]), target)
+
+    # the K-FAC makers call the loss with reduction='sum' themselves (as the reference's do) and need its keyword
+    loss_fn = token_loss if args.workload == 'shampoo_gpt2' else F.cross_entropy
 
     def step():
         opt.zero_grad(set_to_none=True)
