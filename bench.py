@@ -154,7 +154,7 @@ def main():
         bs = 8
         x = torch.randint(0, 50257, (bs, 1024)).to(dev)
         t = torch.randint(0, 50257, (bs * 1024,)).to(dev)
-        config = PreconditioningConfig(damping=1e-6, preconditioner_upd_interval=10)
+        config = PreconditioningConfig(damping=1e-6, curvature_upd_interval=1, preconditioner_upd_interval=10)
         gm = ShampooGradientMaker(model, config)
         args.no_factor_timing = True
     else:
