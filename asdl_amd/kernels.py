@@ -349,6 +349,7 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
 
 
 AK_ERR_UNSUPPORTED = -3
+NCHW_VIA_CHANNELS_LAST = True     # bf16 NCHW activations: transpose once, then the channels-last kernels
 
 
 def _is_channels_last(x):
@@ -376,6 +377,12 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     lib = _lib.load()
     h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
     few_channels = d <= 160 and kh * kw > 1 and x.dtype in (torch.bfloat16, torch.float32)   # the LDS-window kernel
+    if NCHW_VIA_CHANNELS_LAST and x.dtype == torch.bfloat16 and C % 8 == 0 and not few_channels \
+            and x.is_contiguous() and C > 1 and N * C * H * W >= (1 << 16):
+        # one transposing copy (memory-bound, a few microseconds) buys the direct-to-LDS kernels, which read rows of
+        # 8 channels as 16-byte chunks; the NCHW kernel stages every operand through registers
+        with _on_launch_stream():
+            x = x.contiguous(memory_format=torch.channels_last)
     if _is_channels_last(x) and ((x.dtype == torch.bfloat16 and C % 8 == 0) or few_channels):
         if (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0):
             return syrk_tn(x.permute(0, 2, 3, 1).reshape(N * H * W, C), out=out, alpha=alpha, beta=beta)
