@@ -63,6 +63,8 @@ _SIGNATURES = {
     'ak_weight_layout_grouped': (c_int, [c_ptr, c_int, c_i64, c_int, c_ptr]),
     'ak_kron_precond_ws_bytes': (c_size, [c_i64, c_i64]),
     'ak_kron_precond': (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr, c_size, c_ptr]),
+    'ak_kron_precond_static_max_floats': (c_i64, []),
+    'ak_kron_precond_static': (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
     'ak_inv_root_ws_bytes': (c_size, [c_i64, c_int]),
     'ak_inv_root_newton': (c_int, [c_ptr, c_i64, c_int, c_i64, c_int, c_f32, c_ptr, c_int, c_f32, c_int, c_f32,
                                    c_ptr, c_i64, c_ptr, c_ptr, c_size, c_ptr]),

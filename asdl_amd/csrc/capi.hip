@@ -10,6 +10,7 @@ extern "C" const char* ak_error_string(int code) {
     case AK_ERR_WORKSPACE: return "workspace missing or smaller than the matching *_ws_bytes() query";
     case AK_ERR_UNSUPPORTED: return "configuration not supported by this kernel";
     case AK_ERR_LAUNCH: return "HIP reported a kernel launch failure";
+    case AK_ERR_TOO_LARGE: return "sizes beyond the fixed maximum of this entry point's built-in scratch memory";
     default: return "unknown error code";
   }
 }

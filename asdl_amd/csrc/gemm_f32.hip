@@ -1,5 +1,6 @@
 // Dense fp32 products exposed through the C ABI: the general GEMM and the Kronecker
 // preconditioning G <- grad_scale * Binv G Ainv (+ bias <- grad_scale * Binv bias).
+#include <mutex>
 #include "gemm_f32.hpp"
 
 namespace ak {
@@ -117,30 +118,77 @@ extern "C" size_t ak_kron_precond_ws_bytes(int64_t dB, int64_t dA) {
   return static_cast<size_t>(dB * dA + dB) * sizeof(float);
 }
 
+namespace ak {
+
+// G <- grad_scale * Binv G Ainv through the intermediate T = [dB, dA] (+ dB floats behind it for the bias).
+static int kron_precond_run(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA, float* bias,
+                            float grad_scale, float* T, hipStream_t s) {
+  const int b = static_cast<int>(dB), a = static_cast<int>(dA);
+  // the inverses are symmetric: reading A^-1 as its transpose makes both operands of the second product
+  // contiguous along the contraction index
+  GemmParams g1 = make_gemm(0, 0, b, a, b, 1.f, Binv, dB, G, dA, 0.f, T, dA);
+  GemmParams g2 = make_gemm(0, 1, b, a, a, grad_scale, T, dA, Ainv, dA, 0.f, G, dA);
+  g1.split = g2.split = 3;
+  int rc = launch_gemm(g1, 1, s);
+  if (rc != AK_OK) return rc;
+  rc = launch_gemm(g2, 1, s);
+  if (rc != AK_OK) return rc;
+  if (bias != nullptr) {
+    float* tb = T + dB * dA;
+    hipLaunchKernelGGL(gemv_kernel, dim3(static_cast<unsigned>((dB + 3) / 4)), dim3(256), 0, s, Binv, bias, tb, dB,
+                       grad_scale);
+    hipLaunchKernelGGL(copy_kernel, dim3(static_cast<unsigned>((dB + 255) / 256)), dim3(256), 0, s, tb, bias, dB);
+  }
+  return check_launch();
+}
+
+// Intermediate of ak_kron_precond_static: one array per GPU, held from the first call on that GPU until the process
+// ends.  In host code `scratch` is only a handle for hipGetSymbolAddress; kernels get the address looked up below.
+constexpr int64_t STATIC_SCRATCH_FLOATS = 4ll << 20;      // 16 MiB
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[MAX_DEVICES];                 // device address of `scratch` on each GPU, null until looked up
+
+// Address of the current device's copy of `scratch` (looked up once per device, with that device current).
+static int static_scratch(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return AK_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    float* ptr = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr)
+      return AK_ERR_LAUNCH;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return AK_OK;
+}
+
+}  // namespace ak
+
 extern "C" int ak_kron_precond(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA, float* bias,
                                float grad_scale, void* ws, size_t ws_bytes, ak_stream_t stream) {
   if (Binv == nullptr || Ainv == nullptr || G == nullptr || dB <= 0 || dA <= 0 || dB > (1 << 30) || dA > (1 << 30))
     return AK_ERR_ARG;
   if (ws == nullptr || ws_bytes < ak_kron_precond_ws_bytes(dB, dA)) return AK_ERR_WORKSPACE;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  float* T = static_cast<float*>(ws);
-  const int b = static_cast<int>(dB), a = static_cast<int>(dA);
-  // the inverses are symmetric: reading A^-1 as its transpose makes both operands of the second product
-  // contiguous along the contraction index
-  ak::GemmParams g1 = ak::make_gemm(0, 0, b, a, b, 1.f, Binv, dB, G, dA, 0.f, T, dA);
-  ak::GemmParams g2 = ak::make_gemm(0, 1, b, a, a, grad_scale, T, dA, Ainv, dA, 0.f, G, dA);
-  g1.split = g2.split = 3;
-  int rc = ak::launch_gemm(g1, 1, s);
+  return ak::kron_precond_run(Binv, Ainv, G, dB, dA, bias, grad_scale, static_cast<float*>(ws),
+                              static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t ak_kron_precond_static_max_floats(void) { return ak::STATIC_SCRATCH_FLOATS; }
+
+extern "C" int ak_kron_precond_static(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA,
+                                      float* bias, float grad_scale, ak_stream_t stream) {
+  if (Binv == nullptr || Ainv == nullptr || G == nullptr || dB <= 0 || dA <= 0 || dB > (1 << 30) || dA > (1 << 30))
+    return AK_ERR_ARG;
+  if (dB * dA + dB > ak::STATIC_SCRATCH_FLOATS) return AK_ERR_TOO_LARGE;
+  float* T = nullptr;
+  const int rc = ak::static_scratch(&T);
   if (rc != AK_OK) return rc;
-  rc = ak::launch_gemm(g2, 1, s);
-  if (rc != AK_OK) return rc;
-  if (bias != nullptr) {
-    float* tb = T + dB * dA;
-    hipLaunchKernelGGL(ak::gemv_kernel, dim3(static_cast<unsigned>((dB + 3) / 4)), dim3(256), 0, s, Binv, bias, tb, dB,
-                       grad_scale);
-    hipLaunchKernelGGL(ak::copy_kernel, dim3(static_cast<unsigned>((dB + 255) / 256)), dim3(256), 0, s, tb, bias, dB);
-  }
-  return ak::check_launch();
+  // both products overwrite their whole output without reading it, so what the last call left in T does not matter
+  return ak::kron_precond_run(Binv, Ainv, G, dB, dA, bias, grad_scale, T, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t total_tiles,

@@ -732,6 +732,24 @@ def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
     return grad_w, grad_b
 
 
+def kron_precond_static(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
+    """kron_precond through the entry point that brings its own scratch memory (a fixed array inside the library's
+    device image, no workspace, no allocation): for callers that must not allocate.  Raises KernelError when
+    dB * dA + dB exceeds the array; calls that overlap on one GPU race."""
+    _require_gpu(B_inv, A_inv, grad_w, grad_b)
+    dB, dA = B_inv.shape[0], A_inv.shape[0]
+    if grad_w.numel() != dB * dA or not grad_w.is_contiguous() or grad_w.dtype != torch.float32:
+        raise ValueError('grad_w has to be a contiguous float32 tensor with dB * dA elements')
+    if grad_b is not None and (grad_b.numel() != dB or not grad_b.is_contiguous() or grad_b.dtype != torch.float32):
+        raise ValueError('grad_b has to be a contiguous float32 vector with dB elements')
+    rc = _lib.load().ak_kron_precond_static(ctypes.c_void_p(B_inv.data_ptr()), ctypes.c_void_p(A_inv.data_ptr()),
+                                            ctypes.c_void_p(grad_w.data_ptr()), dB, dA,
+                                            ctypes.c_void_p(grad_b.data_ptr()) if grad_b is not None
+                                            else ctypes.c_void_p(0), grad_scale, _stream())
+    _lib.check(rc, 'ak_kron_precond_static')
+    return grad_w, grad_b
+
+
 def _float_bits(value):
     return struct.unpack('<I', struct.pack('<f', float(value)))[0]
 

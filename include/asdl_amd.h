@@ -37,6 +37,7 @@ extern "C" {
 #define AK_ERR_WORKSPACE -2  /* workspace missing or too small */
 #define AK_ERR_UNSUPPORTED -3
 #define AK_ERR_LAUNCH -4     /* hipGetLastError() reported a launch failure */
+#define AK_ERR_TOO_LARGE -5  /* sizes beyond the fixed maximum of an entry point that brings its own scratch memory */
 
 typedef void* ak_stream_t;
 
@@ -257,6 +258,18 @@ int ak_weight_layout_grouped(const int64_t* table, int count, int64_t total_rows
 size_t ak_kron_precond_ws_bytes(int64_t dB, int64_t dA);
 int ak_kron_precond(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA,
                     float* bias, float grad_scale, void* ws, size_t ws_bytes, ak_stream_t stream);
+
+/* ak_kron_precond without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, serving loops, harnesses that forbid hipMalloc): the [dB, dA] intermediate (and dB floats for the
+ * bias) lives in an array of ak_kron_precond_static_max_floats() floats (4 Mi floats = 16 MiB) that is part of the
+ * library's device image, one copy per GPU, held until the process ends.  dB*dA + dB beyond that maximum returns
+ * AK_ERR_TOO_LARGE and touches nothing.  Calls no hipMalloc / hipFree.  Nothing in the array has to start at zero
+ * (both products overwrite their whole output).  All calls on one GPU share the array: calls that may overlap on
+ * one GPU (different streams, different threads) race; order them on one stream.  Same results as ak_kron_precond.
+ * No counterpart in the reference. */
+int64_t ak_kron_precond_static_max_floats(void);
+int ak_kron_precond_static(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA,
+                           float* bias, float grad_scale, ak_stream_t stream);
 
 /* ---- Shampoo inverse p-th root ---------------------------------------------------- */
 
