@@ -33,6 +33,11 @@ _SIGNATURES = {
     'ak_kron_damping': (c_int, [c_ptr, c_ptr, c_ptr, c_int, c_f32, c_f32, c_ptr, c_ptr, c_ptr]),
     'ak_chol_inv_ws_bytes': (c_size, [c_i64, c_int]),
     'ak_chol_inv_batched': (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_size, c_ptr]),
+    'ak_chol_group_plan_bytes': (c_size, [c_ptr, c_int]),
+    'ak_chol_group_ws_bytes': (c_size, [c_ptr, c_int]),
+    'ak_chol_group_plan': (c_int, [c_ptr, c_int, c_ptr, c_size]),
+    'ak_chol_group_plan_launches': (c_int, [c_ptr]),
+    'ak_chol_inv_grouped': (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_size, c_ptr]),
     'ak_unit_wise_ws_bytes': (c_size, [c_i64, c_i64, c_i64]),
     'ak_unit_wise_stats': (c_int, [c_ptr, c_int, c_i64, c_i64, c_i64, c_ptr, c_int, c_i64, c_i64, c_i64, c_ptr, c_ptr,
                                    c_i64, c_i64, c_i64, c_f32, c_f32, c_ptr, c_ptr, c_size, c_ptr]),

@@ -1,0 +1,465 @@
+// out_m <- (A_m + lam_m I)^-1 for many symmetric positive definite fp32 matrices of DIFFERENT sizes in one call.
+//
+// Per matrix the arithmetic is the recursive blocked Cholesky of chol_inv.hip that carries the triangular inverse
+// along (work matrix W, lower triangle):
+//   F(lo, hi): n <= 128 -> one work group factors the diagonal block in the LDS and inverts the factor (chol_leaf.hpp)
+//              otherwise    F(lo, mid);  T1 = A21 M11^T;  { A22 -= T1 T1^T,  T2 = T1 M11 };  F(mid, hi);  M21 = -M22 T2
+//   out = M^T M.
+// T2 only needs T1 and M11, so it shares a launch with the trailing update: three product launches per node.
+//
+// What changes is the schedule.  The per-matrix sequences of steps (leaf | products) of ALL matrices are merged into
+// one sequence of "super-steps": super-step s holds, for every matrix whose next step has the type chosen for s,
+// that step.  One launch per super-step: a grouped leaf launch (one work group per diagonal block) or a grouped
+// product launch (one work group per 128 x 128 tile of any product of the step, split-bf16 MFMA tile of gemm_x3.hpp,
+// descriptor found by bisection on the running tile count).  The longest chain (the largest matrix) sets the number
+// of launches; the work of all smaller matrices runs in the shadow of its steps.  ResNet-50 (156 factors, 13 sizes):
+// about 150 launches instead of 620.
+//
+// The plan (descriptor tables, launch sequence) depends on the sizes only; every address in it is an offset into the
+// workspace.  The caller builds it once per size set on the host (ak_chol_group_plan), keeps a device copy, and
+// passes both to every call.
+//
+// Matrices are padded to a multiple of 4 columns with an identity block (the padded rows and columns drop out of the
+// result), which keeps every operand of the split kernel 16-byte aligned.  Only the lower triangle of the input is
+// read; the strictly upper 128-blocks of W are never touched.
+#include <algorithm>
+#include <cstring>
+#include <vector>
+#include "gemm_f32.hpp"
+#include "chol_leaf.hpp"
+
+namespace ak {
+
+constexpr int64_t CG_MAGIC = 0x3147524c4f4843ll;     // "CHOLGR1"
+constexpr int CG_COPY = 0, CG_LEAF = 1, CG_PROD = 2;
+constexpr int CG_FLAG_TRANSA = 1, CG_FLAG_TRANSB = 2, CG_FLAG_OUT_USER = 4;
+constexpr int CG_COPY_ROWS = 8;                       // rows of W one work group of the copy-in kernel writes
+
+struct CgHeader {
+  int64_t magic;
+  int64_t total_bytes;
+  int64_t ws_floats;
+  int64_t mats_off, steps_off, leaves_off, prods_off, map_off;     // byte offsets of the tables inside the plan
+  int32_t count, nsteps, nleaves, nprods;
+  int32_t copy_blocks, ntiles;
+};
+
+struct CgMat {
+  int64_t w_off;            // work matrix [dp, dp], offset in floats from the workspace base
+  int32_t d, dp;
+  int32_t first_copy_block, pad0;
+};
+
+struct CgStep {
+  int32_t type, first, count, grid;
+  int32_t first_tile, pad0;     // products: where the step's tile -> product map starts
+};
+
+struct CgLeafTask {
+  int64_t blk_off;          // the diagonal block, offset in floats from the workspace base
+  int32_t mat, lo, n, ld, d, pad0;
+};
+
+struct CgProd {
+  int64_t a_off, b_off, c_off;
+  int32_t lda, ldb, ldc;
+  int32_t M, N, K;
+  int32_t flags, kmode, tile_mode;
+  float alpha, beta;
+  int32_t mat;
+  int32_t first_tile, tiles_m, tiles_n;
+};
+
+struct CgArgs {
+  const unsigned char* plan;        // device copy of the plan
+  float* ws;
+  const float* const* A_list;
+  float* const* out_list;
+  const float* lam;
+  const int* skip;
+  int* info;
+  int lam_stride, skip_stride;
+};
+
+__device__ __forceinline__ bool cg_skipped(const CgArgs& a, int mat) {
+  return a.skip != nullptr && a.skip[static_cast<int64_t>(mat) * a.skip_stride] == 0;
+}
+
+// W_m <- lower(A_m) + lam_m I, padded rows carry the identity; info_m <- 0.  One work group per CG_COPY_ROWS rows of
+// one matrix (bisection on first_copy_block); a row is read and written up to its diagonal element only.
+static __global__ __launch_bounds__(256) void cg_copy_in_kernel(CgArgs a, int count) {
+  const CgHeader* __restrict__ h = reinterpret_cast<const CgHeader*>(a.plan);
+  const CgMat* __restrict__ mats = reinterpret_cast<const CgMat*>(a.plan + h->mats_off);
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (mats[mid].first_copy_block <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const CgMat m = mats[lo];
+  if (cg_skipped(a, lo)) return;
+  const int r0 = (w - m.first_copy_block) * CG_COPY_ROWS;
+  if (r0 == 0 && threadIdx.x == 0) a.info[lo] = 0;
+  const float* __restrict__ A = a.A_list[lo];
+  float* __restrict__ W = a.ws + m.w_off;
+  const float l = a.lam[static_cast<int64_t>(lo) * a.lam_stride];
+  const bool vec = (m.d % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
+#pragma unroll 1
+  for (int e = 0; e < CG_COPY_ROWS; ++e) {
+    const int r = r0 + e;
+    if (r >= m.dp) break;
+    float* __restrict__ dst = W + static_cast<int64_t>(r) * m.dp;
+    if (r >= m.d) {                                     // identity padding
+      for (int c = threadIdx.x; c <= r; c += 256) dst[c] = (c == r) ? 1.f : 0.f;
+      continue;
+    }
+    const float* __restrict__ src = A + static_cast<int64_t>(r) * m.d;
+    if (vec) {
+      for (int c = 4 * threadIdx.x; c <= r; c += 1024) {
+        floatx4 v = *reinterpret_cast<const floatx4*>(src + c);
+        if (r >= c && r < c + 4) v[r - c] += l;
+        *reinterpret_cast<floatx4*>(dst + c) = v;       // the elements right of the diagonal are never read
+      }
+    } else {
+      for (int c = threadIdx.x; c <= r; c += 256) dst[c] = src[c] + ((c == r) ? l : 0.f);
+    }
+  }
+}
+
+// One work group (16 waves) per leaf task of the step.  Every table is read with one load that depends on nothing
+// but the work group's index: a chain of dependent loads from cold device memory costs a microsecond per link.
+static __global__ __launch_bounds__(LEAF_THREADS) void cg_leaf_kernel(CgArgs a, const CgLeafTask* __restrict__ tasks) {
+  extern __shared__ __attribute__((aligned(16))) float leaf_smem[];
+  const CgLeafTask t = tasks[blockIdx.x];
+  const int live = a.skip != nullptr ? a.skip[static_cast<int64_t>(t.mat) * a.skip_stride] : 1;   // used at the end
+  const int tid = threadIdx.x;
+  leaf_block(a.ws + t.blk_off, t.ld, t.n, leaf_smem, tid);
+  const int bad = leaf_bad_pivot(leaf_smem);
+  // a bad pivot inside the identity padding cannot happen; one inside the matrix is reported like LAPACK's potrf.
+  // A skipped matrix's work area holds whatever the last call left there; its steps still run (they touch nothing
+  // but that work area) and report nothing.
+  if (tid == 0 && live != 0 && bad != 0 && t.lo + bad <= t.d && a.info[t.mat] == 0) a.info[t.mat] = t.lo + bad;
+}
+
+// Tile (ti, tj) number `local` of a product, longest contraction first where the range depends on the tile.
+__device__ __forceinline__ void cg_decode_tile(const CgProd& d, int local, int& ti, int& tj) {
+  if (d.tile_mode != TILE_ALL) {     // tiles on and below the diagonal, row by row (K_GE_MAXIJ: longest first)
+    ti = static_cast<int>((__builtin_sqrtf(8.f * static_cast<float>(local) + 1.f) - 1.f) * 0.5f);
+    while ((ti + 1) * (ti + 2) / 2 <= local) ++ti;
+    while (ti * (ti + 1) / 2 > local) --ti;
+    tj = local - ti * (ti + 1) / 2;
+    return;
+  }
+  switch (d.kmode) {
+    case K_LE_J:                     // k <= column tile: last column first
+      tj = d.tiles_n - 1 - local / d.tiles_m;
+      ti = local % d.tiles_m;
+      break;
+    case K_GE_J:                     // k >= column tile: first column first
+      tj = local / d.tiles_m;
+      ti = local % d.tiles_m;
+      break;
+    case K_LE_I:                     // k <= row tile: last row first
+      ti = d.tiles_m - 1 - local / d.tiles_n;
+      tj = local % d.tiles_n;
+      break;
+    default:
+      ti = local / d.tiles_n;
+      tj = local % d.tiles_n;
+      break;
+  }
+}
+
+// One work group per 128 x 128 tile of any product of the step; tile_map[w] = the product of work group w.
+static __global__ __launch_bounds__(256) void cg_prod_kernel(CgArgs a, const CgProd* __restrict__ prods,
+                                                             const int32_t* __restrict__ tile_map) {
+  __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * 3 * X3_PLANE];
+  const int w = blockIdx.x;
+  const CgProd d = prods[tile_map[w]];
+  // only the product that writes the caller's matrix has to respect the skip flag (see cg_leaf_kernel)
+  if ((d.flags & CG_FLAG_OUT_USER) && cg_skipped(a, d.mat)) return;
+  int ti, tj;
+  cg_decode_tile(d, w - d.first_tile, ti, tj);
+  GemmParams p;
+  p.A = a.ws + d.a_off;
+  p.B = a.ws + d.b_off;
+  p.C = (d.flags & CG_FLAG_OUT_USER) ? a.out_list[d.mat] : a.ws + d.c_off;
+  p.C_list = nullptr;
+  p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
+  p.sA = p.sB = p.sC = 0;
+  p.M = d.M; p.N = d.N; p.K = d.K;
+  p.transA = (d.flags & CG_FLAG_TRANSA) ? 1 : 0;
+  p.transB = (d.flags & CG_FLAG_TRANSB) ? 1 : 0;
+  p.alpha = d.alpha; p.beta = d.beta;
+  p.kmode = d.kmode; p.tile_mode = d.tile_mode;
+  p.active = nullptr; p.active_stride = 0;
+  p.split = 3;
+  gemm_x3_tile<3, false>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+}
+
+// ---- host: the plan ------------------------------------------------------------------------------------------
+
+struct CgOp {                 // one step of one matrix's own sequence
+  int type;
+  CgLeafTask leaf;
+  std::vector<CgProd> prods;
+};
+
+static int64_t cg_half(int64_t n) {
+  const int64_t nb = (n + LEAF - 1) / LEAF;
+  return LEAF * ((nb + 1) / 2);
+}
+
+// Floats of the T1 (and of the T2) pool of an n x n range: a node's panels live while its right half is factored.
+static int64_t cg_pool(int64_t n) {
+  if (n <= LEAF) return 0;
+  const int64_t s1 = cg_half(n), s2 = n - s1;
+  return std::max(cg_pool(s1), s1 * s2 + cg_pool(s2));
+}
+
+static int64_t cg_tiles(const CgProd& p) {
+  const int64_t tm = (p.M + 127) / 128, tn = (p.N + 127) / 128;
+  return p.tile_mode == TILE_ALL ? tm * tn : tm * (tm + 1) / 2;
+}
+
+static CgProd cg_prod(int mat, int flags, int M, int N, int K, float alpha, int64_t a, int lda, int64_t b, int ldb,
+                      float beta, int64_t c, int ldc, int kmode, int tile_mode) {
+  CgProd p;
+  std::memset(&p, 0, sizeof(p));
+  p.a_off = a; p.b_off = b; p.c_off = c;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.M = M; p.N = N; p.K = K;
+  p.flags = flags; p.kmode = kmode; p.tile_mode = tile_mode;
+  p.alpha = alpha; p.beta = beta;
+  p.mat = mat;
+  p.tiles_m = (M + 127) / 128;
+  p.tiles_n = (N + 127) / 128;
+  return p;
+}
+
+static void cg_range(std::vector<CgOp>& ops, int mat, int64_t w, int d, int dp, int64_t t1, int64_t t2, int lo, int hi,
+                     int64_t pool_off) {
+  const int n = hi - lo;
+  if (n <= LEAF) {
+    CgOp op;
+    op.type = CG_LEAF;
+    op.leaf = CgLeafTask{w + static_cast<int64_t>(lo) * dp + lo, mat, lo, n, dp, d, 0};
+    ops.push_back(op);
+    return;
+  }
+  const int mid = lo + static_cast<int>(cg_half(n));
+  cg_range(ops, mat, w, d, dp, t1, t2, lo, mid, pool_off);
+  const int s1 = mid - lo, s2 = hi - mid;
+  const int64_t W11 = w + static_cast<int64_t>(lo) * dp + lo, W21 = w + static_cast<int64_t>(mid) * dp + lo,
+                W22 = w + static_cast<int64_t>(mid) * dp + mid;
+  const int64_t T1 = t1 + pool_off, T2 = t2 + pool_off;
+  {
+    CgOp op;
+    op.type = CG_PROD;      // T1 = A21 M11^T
+    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, s2, s1, s1, 1.f, W21, dp, W11, dp, 0.f, T1, s1, K_LE_J, TILE_ALL));
+    ops.push_back(op);
+  }
+  {
+    CgOp op;
+    op.type = CG_PROD;      // A22 -= T1 T1^T (lower triangle);  T2 = T1 M11
+    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, s2, s2, s1, -1.f, T1, s1, T1, s1, 1.f, W22, dp, K_FULL, TILE_LOWER));
+    op.prods.push_back(cg_prod(mat, 0, s2, s1, s1, 1.f, T1, s1, W11, dp, 0.f, T2, s1, K_GE_J, TILE_ALL));
+    ops.push_back(op);
+  }
+  cg_range(ops, mat, w, d, dp, t1, t2, mid, hi, pool_off + static_cast<int64_t>(s1) * s2);
+  {
+    CgOp op;
+    op.type = CG_PROD;      // M21 = -M22 T2
+    op.prods.push_back(cg_prod(mat, 0, s2, s1, s2, -1.f, W22, dp, T2, s1, 0.f, W21, dp, K_LE_I, TILE_ALL));
+    ops.push_back(op);
+  }
+}
+
+struct CgPlan {
+  CgHeader h;
+  std::vector<CgMat> mats;
+  std::vector<CgStep> steps;
+  std::vector<CgLeafTask> leaves;
+  std::vector<CgProd> prods;
+  std::vector<int32_t> tile_map;
+};
+
+static inline int64_t cg_align(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+static bool cg_dims_ok(const int64_t* dims, int count) {
+  if (dims == nullptr || count <= 0 || count > (1 << 20)) return false;
+  for (int i = 0; i < count; ++i)
+    if (dims[i] <= 0 || dims[i] > 32768) return false;
+  return true;
+}
+
+static void cg_build(const int64_t* dims, int count, CgPlan& plan) {
+  std::vector<std::vector<CgOp>> seq(count);
+  int64_t off = 0;
+  int copy_blocks = 0;
+  plan.mats.resize(count);
+  for (int m = 0; m < count; ++m) {
+    const int d = static_cast<int>(dims[m]), dp = (d + 3) / 4 * 4;
+    const int64_t pool = cg_align(cg_pool(dp), 64);
+    CgMat& cm = plan.mats[m];
+    cm.w_off = off; cm.d = d; cm.dp = dp; cm.first_copy_block = copy_blocks; cm.pad0 = 0;
+    copy_blocks += (dp + CG_COPY_ROWS - 1) / CG_COPY_ROWS;
+    const int64_t t1 = off + cg_align(static_cast<int64_t>(dp) * dp, 64), t2 = t1 + pool;
+    off = t2 + pool;
+    cg_range(seq[m], m, cm.w_off, d, dp, t1, t2, 0, dp, 0);
+    CgOp fin;
+    fin.type = CG_PROD;     // out = M^T M, both triangles
+    fin.prods.push_back(cg_prod(m, CG_FLAG_TRANSA | CG_FLAG_OUT_USER, d, d, dp, 1.f, cm.w_off, dp, cm.w_off, dp, 0.f, 0, d,
+                                K_GE_MAXIJ, TILE_LOWER_MIRROR));
+    seq[m].push_back(fin);
+  }
+  plan.steps.push_back(CgStep{CG_COPY, 0, count, copy_blocks, 0, 0});
+  // Merge: the matrix with the most steps left decides the type of the next super-step; every matrix whose next
+  // step has that type takes part.
+  std::vector<size_t> cur(count, 0);
+  for (;;) {
+    int lead = -1;
+    size_t most = 0;
+    for (int m = 0; m < count; ++m) {
+      const size_t left = seq[m].size() - cur[m];
+      if (left > most) { most = left; lead = m; }
+    }
+    if (lead < 0) break;
+    const int type = seq[lead][cur[lead]].type;
+    CgStep st{type, 0, 0, 0, 0, 0};
+    if (type == CG_LEAF) {
+      st.first = static_cast<int>(plan.leaves.size());
+      for (int m = 0; m < count; ++m)
+        if (cur[m] < seq[m].size() && seq[m][cur[m]].type == CG_LEAF) plan.leaves.push_back(seq[m][cur[m]++].leaf);
+      st.count = static_cast<int>(plan.leaves.size()) - st.first;
+      st.grid = st.count;
+    } else {
+      std::vector<CgProd> ps;
+      for (int m = 0; m < count; ++m)
+        if (cur[m] < seq[m].size() && seq[m][cur[m]].type == CG_PROD) {
+          for (const CgProd& p : seq[m][cur[m]].prods) ps.push_back(p);
+          ++cur[m];
+        }
+      // longest contraction first: the long tiles start early, the short ones fill the tail
+      std::stable_sort(ps.begin(), ps.end(), [](const CgProd& x, const CgProd& y) { return x.K > y.K; });
+      int64_t tiles = 0;
+      st.first_tile = static_cast<int>(plan.tile_map.size());
+      for (size_t i = 0; i < ps.size(); ++i) {
+        ps[i].first_tile = static_cast<int>(tiles);
+        const int64_t n = cg_tiles(ps[i]);
+        tiles += n;
+        plan.tile_map.insert(plan.tile_map.end(), static_cast<size_t>(n), static_cast<int32_t>(i));
+      }
+      st.first = static_cast<int>(plan.prods.size());
+      st.count = static_cast<int>(ps.size());
+      st.grid = static_cast<int>(tiles);
+      plan.prods.insert(plan.prods.end(), ps.begin(), ps.end());
+    }
+    plan.steps.push_back(st);
+  }
+  CgHeader& h = plan.h;
+  std::memset(&h, 0, sizeof(h));
+  h.magic = CG_MAGIC;
+  h.ws_floats = off;
+  h.count = count;
+  h.nsteps = static_cast<int>(plan.steps.size());
+  h.nleaves = static_cast<int>(plan.leaves.size());
+  h.nprods = static_cast<int>(plan.prods.size());
+  h.copy_blocks = copy_blocks;
+  h.ntiles = static_cast<int>(plan.tile_map.size());
+  int64_t b = cg_align(sizeof(CgHeader), 64);
+  h.mats_off = b; b = cg_align(b + plan.mats.size() * sizeof(CgMat), 64);
+  h.steps_off = b; b = cg_align(b + plan.steps.size() * sizeof(CgStep), 64);
+  h.leaves_off = b; b = cg_align(b + plan.leaves.size() * sizeof(CgLeafTask), 64);
+  h.prods_off = b; b = cg_align(b + plan.prods.size() * sizeof(CgProd), 64);
+  h.map_off = b; b = cg_align(b + plan.tile_map.size() * sizeof(int32_t), 64);
+  h.total_bytes = b;
+}
+
+}  // namespace ak
+
+extern "C" size_t ak_chol_group_plan_bytes(const int64_t* dims, int count) {
+  if (!ak::cg_dims_ok(dims, count)) return 0;
+  ak::CgPlan plan;
+  ak::cg_build(dims, count, plan);
+  return static_cast<size_t>(plan.h.total_bytes);
+}
+
+extern "C" size_t ak_chol_group_ws_bytes(const int64_t* dims, int count) {
+  if (!ak::cg_dims_ok(dims, count)) return 0;
+  int64_t off = 0;
+  for (int m = 0; m < count; ++m) {
+    const int64_t dp = (dims[m] + 3) / 4 * 4;
+    off += ak::cg_align(dp * dp, 64) + 2 * ak::cg_align(ak::cg_pool(dp), 64);
+  }
+  return static_cast<size_t>(off) * sizeof(float);
+}
+
+extern "C" int ak_chol_group_plan(const int64_t* dims, int count, void* plan_host, size_t plan_bytes) {
+  using namespace ak;
+  if (!cg_dims_ok(dims, count) || plan_host == nullptr) return AK_ERR_ARG;
+  CgPlan plan;
+  cg_build(dims, count, plan);
+  if (plan_bytes < static_cast<size_t>(plan.h.total_bytes)) return AK_ERR_WORKSPACE;
+  unsigned char* out = static_cast<unsigned char*>(plan_host);
+  std::memset(out, 0, static_cast<size_t>(plan.h.total_bytes));
+  std::memcpy(out, &plan.h, sizeof(CgHeader));
+  std::memcpy(out + plan.h.mats_off, plan.mats.data(), plan.mats.size() * sizeof(CgMat));
+  std::memcpy(out + plan.h.steps_off, plan.steps.data(), plan.steps.size() * sizeof(CgStep));
+  if (!plan.leaves.empty()) std::memcpy(out + plan.h.leaves_off, plan.leaves.data(), plan.leaves.size() * sizeof(CgLeafTask));
+  if (!plan.prods.empty()) std::memcpy(out + plan.h.prods_off, plan.prods.data(), plan.prods.size() * sizeof(CgProd));
+  if (!plan.tile_map.empty())
+    std::memcpy(out + plan.h.map_off, plan.tile_map.data(), plan.tile_map.size() * sizeof(int32_t));
+  return AK_OK;
+}
+
+extern "C" int ak_chol_group_plan_launches(const void* plan_host) {
+  if (plan_host == nullptr) return AK_ERR_ARG;
+  const ak::CgHeader* h = static_cast<const ak::CgHeader*>(plan_host);
+  return h->magic == ak::CG_MAGIC ? h->nsteps : AK_ERR_ARG;
+}
+
+extern "C" int ak_chol_inv_grouped(const void* plan_host, const void* plan_dev, const float* const* A_list,
+                                   float* const* out_list, const float* lam, int lam_stride, const int* skip_flags,
+                                   int skip_stride, int* info, void* ws, size_t ws_bytes, ak_stream_t stream) {
+  using namespace ak;
+  if (plan_host == nullptr || plan_dev == nullptr || A_list == nullptr || out_list == nullptr || lam == nullptr ||
+      info == nullptr)
+    return AK_ERR_ARG;
+  const unsigned char* ph = static_cast<const unsigned char*>(plan_host);
+  const CgHeader* h = reinterpret_cast<const CgHeader*>(ph);
+  if (h->magic != CG_MAGIC || h->count <= 0 || h->nsteps <= 0) return AK_ERR_ARG;
+  if (ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 255) != 0 ||
+      ws_bytes < static_cast<size_t>(h->ws_floats) * sizeof(float))
+    return AK_ERR_WORKSPACE;
+  static bool leaf_attr_set = false;     // idempotent; a benign race sets it twice at worst
+  if (!leaf_attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(cg_leaf_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(LEAF_LDS_BYTES)) != hipSuccess)
+      return AK_ERR_LAUNCH;
+    leaf_attr_set = true;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CgArgs a;
+  a.plan = static_cast<const unsigned char*>(plan_dev);
+  a.ws = static_cast<float*>(ws);
+  a.A_list = A_list; a.out_list = out_list;
+  a.lam = lam; a.skip = skip_flags; a.info = info;
+  a.lam_stride = lam_stride; a.skip_stride = skip_stride;
+  const CgStep* steps = reinterpret_cast<const CgStep*>(ph + h->steps_off);
+  for (int i = 0; i < h->nsteps; ++i) {
+    const CgStep& st = steps[i];
+    if (st.grid <= 0) continue;
+    if (st.type == CG_COPY)
+      hipLaunchKernelGGL(cg_copy_in_kernel, dim3(st.grid), dim3(256), 0, s, a, h->count);
+    else if (st.type == CG_LEAF)
+      hipLaunchKernelGGL(cg_leaf_kernel, dim3(st.grid), dim3(LEAF_THREADS), LEAF_LDS_BYTES, s, a,
+                         reinterpret_cast<const CgLeafTask*>(a.plan + h->leaves_off) + st.first);
+    else
+      hipLaunchKernelGGL(cg_prod_kernel, dim3(st.grid), dim3(256), 0, s, a,
+                         reinterpret_cast<const CgProd*>(a.plan + h->prods_off) + st.first,
+                         reinterpret_cast<const int32_t*>(a.plan + h->map_off) + st.first_tile);
+  }
+  return check_launch();
+}

@@ -323,6 +323,30 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
   // triangles of a diagonal tile from the lower one
   const bool mirror = (p.tile_mode == TILE_LOWER_MIRROR);
   const bool lower_only = (p.tile_mode == TILE_LOWER) || (mirror && ti == tj);
+  if (p.beta != 0.f) {
+    // all loads of C first: interleaved with the stores they would wait for one another (the compiler cannot tell
+    // that the rows differ), one memory latency per element
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int gj = j0 + 64 * wc + 32 * b + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int gi = i0 + 64 * wr + 32 * a + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          float c = 0.f;
+          if (gj < p.N && gi < p.M && !(lower_only && gi < gj)) c = C[static_cast<int64_t>(gi) * p.ldc + gj];
+          acc[a][b][r] = p.alpha * acc[a][b][r] + p.beta * c;
+        }
+      }
+  } else {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] *= p.alpha;
+  }
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -334,10 +358,8 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
         const int gi = i0 + 64 * wr + 32 * a + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (gi >= p.M) continue;
         if (lower_only && gi < gj) continue;
-        float v = p.alpha * acc[a][b][r];
-        float* dst = C + static_cast<int64_t>(gi) * p.ldc + gj;
-        if (p.beta != 0.f) v += p.beta * *dst;
-        *dst = v;
+        const float v = acc[a][b][r];
+        C[static_cast<int64_t>(gi) * p.ldc + gj] = v;
         if (mirror && gi != gj) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
       }
     }

@@ -672,6 +672,68 @@ def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1
     return info
 
 
+_chol_plans = {}
+
+
+class CholGroupPlan:
+    """Launch plan of ak_chol_inv_grouped for one tuple of matrix sizes: built on the host by the library, kept in
+    pinned memory (the library reads the launch sequence from it on every call) with a copy on the device (the
+    kernels read their descriptors from it)."""
+
+    def __init__(self, dims, device):
+        lib = _lib.load()
+        self.dims = tuple(int(d) for d in dims)
+        arr = (ctypes.c_int64 * len(self.dims))(*self.dims)
+        nbytes = lib.ak_chol_group_plan_bytes(arr, len(self.dims))
+        if nbytes == 0:
+            raise ValueError(f'no grouped Cholesky plan for sizes {self.dims}')
+        self.ws_bytes = lib.ak_chol_group_ws_bytes(arr, len(self.dims))
+        self.host = torch.empty(nbytes, dtype=torch.uint8).pin_memory()
+        _lib.check(lib.ak_chol_group_plan(arr, len(self.dims), ctypes.c_void_p(self.host.data_ptr()), nbytes),
+                   'ak_chol_group_plan')
+        self.launches = lib.ak_chol_group_plan_launches(ctypes.c_void_p(self.host.data_ptr()))
+        with _on_launch_stream():
+            self.dev = self.host.to(device, non_blocking=True)
+
+
+def chol_group_plan(dims, device):
+    dev = torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), tuple(int(d) for d in dims))
+    plan = _chol_plans.get(key)
+    if plan is None:
+        if len(_chol_plans) > 64:
+            _chol_plans.clear()
+        plan = _chol_plans[key] = CholGroupPlan(dims, dev)
+    return plan
+
+
+def chol_inv_grouped(mats, outs, lam, lam_stride=1, active=None, active_stride=1, info=None):
+    """outs[m] <- (mats[m] + lam[m*lam_stride] I)^-1 for square matrices of any mix of sizes, all in one call:
+    the steps of all matrices are merged into one sequence of grouped launches (csrc/chol_group.hip).  Returns the
+    device ``info`` tensor (int32 [len(mats)], 0 = ok, k > 0 = leading minor k not positive definite)."""
+    _require_gpu(*mats, *outs, lam, active)
+    dev = mats[0].device
+    for a, o in zip(mats, outs):
+        if a.dtype != torch.float32 or a.ndim != 2 or a.shape[0] != a.shape[1] or not a.is_contiguous():
+            raise ValueError('matrices have to be contiguous square float32 tensors')
+        if o.dtype != torch.float32 or o.shape != a.shape or not o.is_contiguous():
+            raise ValueError('every output has to be a contiguous float32 tensor of its matrix\'s shape')
+    if len(outs) != len(mats):
+        raise ValueError('one output per matrix')
+    if info is None:
+        info = torch.empty(len(mats), dtype=torch.int32, device=dev)
+    plan = chol_group_plan([m.shape[0] for m in mats], dev)
+    ws, ws_bytes, keep = _ws_args(plan.ws_bytes, dev)
+    pa, po = device_ptr_array(mats), device_ptr_array(outs)
+    rc = _lib.load().ak_chol_inv_grouped(
+        ctypes.c_void_p(plan.host.data_ptr()), ctypes.c_void_p(plan.dev.data_ptr()), ctypes.c_void_p(pa.data_ptr()),
+        ctypes.c_void_p(po.data_ptr()), ctypes.c_void_p(lam.data_ptr()), lam_stride,
+        ctypes.c_void_p(active.data_ptr()) if active is not None else ctypes.c_void_p(0), active_stride,
+        ctypes.c_void_p(info.data_ptr()), ws, ws_bytes, _stream())
+    _lib.check(rc, 'ak_chol_inv_grouped')
+    return info
+
+
 def cholesky_inv(X, damping=1e-7):
     """(X + damping I)^-1; raises torch.linalg.LinAlgError when X + damping I is not positive
     definite (reads the device info word, i.e. synchronises)."""

@@ -65,7 +65,9 @@ def _load_from_numpy(path, device=None):
 
 
 _side_stream_cache = {}
-N_SIDE_STREAMS = 8     # size groups of a batched inverse that may run side by side
+N_SIDE_STREAMS = 8     # groups of a batched inverse that may run side by side
+GROUPED_INVERSE = True  # all square factors of a call in one merged launch sequence (kernels.chol_inv_grouped);
+                        # False: one batched inverse per distinct size, spread over the side streams
 
 
 def _side_streams(device, n):
@@ -77,6 +79,7 @@ def _side_streams(device, n):
 
 
 _enqueue_workers = {}
+_next_side_stream = 0
 
 
 def _worker(stream_index):
@@ -185,9 +188,14 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         if calc_B_inv:
             entry = (2 * i + 1, B_list[i], k, 'B')
             (groups[B_list[i].shape[0]] if B_list[i].shape[0] == B_list[i].shape[1] else low_rank).append(entry)
-    # Each size group is an independent chain of small launches: spread the groups over a few side streams
-    # (default priority) so that their launch latencies overlap; everything joins the caller's stream again.
-    order = sorted(groups, key=lambda d: d ** 3 * len(groups[d]), reverse=True)
+    # GROUPED_INVERSE: every square factor of the call goes into one grouped inverse, whose launches carry the steps
+    # of all matrices at once.  Otherwise each size group is an independent chain of small launches, and the groups
+    # are spread over a few side streams (default priority) so that their launch latencies overlap.  Either way
+    # everything joins the caller's stream again.
+    if GROUPED_INVERSE and groups:
+        merged = [e for d in sorted(groups, reverse=True) for e in groups[d]]
+        groups = {-1: merged}
+    order = sorted(groups, key=lambda d: sum(e[1].shape[0] ** 3 for e in groups[d]), reverse=True)
     prepared = []
     for d in order:
         entries = groups[d]
@@ -215,12 +223,22 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         entries, outs, lam_g, act_g, info = group
         if act_g is None:          # a low-rank factor
             kernels.smw_inv(entries[0][1], lam_g, out=outs[0], info=info)
+        elif GROUPED_INVERSE:
+            kernels.chol_inv_grouped([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
         else:
             kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
 
     if use_streams:
         main = torch.cuda.current_stream()
-        side = _side_streams(dev, min(N_SIDE_STREAMS, len(prepared)))
+        # successive calls start on different side streams (each with its own enqueue thread and workspace), so
+        # that an early batch and the remainder of one step run side by side
+        global _next_side_stream
+        pool = _side_streams(dev, N_SIDE_STREAMS)
+        first = _next_side_stream % len(pool)
+        n_used = min(len(pool), len(prepared))
+        _next_side_stream += n_used
+        chosen = [(first + i) % len(pool) for i in range(n_used)]
+        side = [pool[i] for i in chosen]
         start = torch.cuda.Event()
         start.record(main)
         per_stream = [prepared[i::len(side)] for i in range(len(side))]
@@ -234,7 +252,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
                 done.record(st)
             return done
 
-        for si, (st, groups_of_stream) in enumerate(zip(side, per_stream)):
+        for si, st, groups_of_stream in zip(chosen, side, per_stream):
             if defer:
                 futures.append(_worker(si).submit(run_stream, st, groups_of_stream))
             else:

@@ -149,6 +149,27 @@ int ak_chol_inv_batched(const float* const* A_list, float* const* out_list, int6
                         const float* lam, int lam_stride, const int* skip_flags, int skip_stride,
                         int* info, void* ws, size_t ws_bytes, ak_stream_t stream);
 
+/* ak_chol_inv_batched for `count` matrices of different sizes dims[m] in one call: the per-matrix sequences of
+ * steps (LDS-resident diagonal block | panel and trailing products) are merged into one sequence of grouped
+ * launches, so that the chains of the small matrices run in the shadow of the largest one's and nothing waits on
+ * the host (ResNet-50: 156 factors of 13 sizes, about 150 launches).  The launch plan depends on the sizes only:
+ *   ak_chol_group_plan_bytes / ak_chol_group_ws_bytes  bytes of the plan / of the device workspace (0: bad sizes);
+ *   ak_chol_group_plan        fills plan_host (HOST memory); the caller keeps it and a byte copy in device memory;
+ *   ak_chol_group_plan_launches  kernel launches one call enqueues;
+ *   ak_chol_inv_grouped       plan_host and plan_dev are those two copies; A_list / out_list: device arrays of
+ *                             `count` device pointers (dense, ld = dims[m]); lam, skip_flags, info as in
+ *                             ak_chol_inv_batched, indexed by m; ws 256-byte aligned.
+ * Only the lower triangle of A_m is read; out_m is written in full (both triangles).
+ * Same reference lines as ak_chol_inv_batched; the loop it replaces is the per-module Kron.update_inv of
+ * NaturalGradientMaker.update_preconditioner (asdl/precondition/natural_gradient.py:419-443). */
+size_t ak_chol_group_plan_bytes(const int64_t* dims, int count);
+size_t ak_chol_group_ws_bytes(const int64_t* dims, int count);
+int ak_chol_group_plan(const int64_t* dims, int count, void* plan_host, size_t plan_bytes);
+int ak_chol_group_plan_launches(const void* plan_host);
+int ak_chol_inv_grouped(const void* plan_host, const void* plan_dev, const float* const* A_list,
+                        float* const* out_list, const float* lam, int lam_stride, const int* skip_flags,
+                        int skip_stride, int* info, void* ws, size_t ws_bytes, ak_stream_t stream);
+
 /* ---- unit-wise blocks (BatchNorm / LayerNorm) ------------------------------------- */
 
 /* blocks[f] <- beta*blocks[f] + alpha * sum_n [[gw^2, gw*gb], [gw*gb, gb^2]] for f < F, blocks = [F, 2, 2] fp32,

@@ -317,6 +317,88 @@ def test_chol_inv_batched_skip_and_info(K):
     assert int(info[0]) == 71
 
 
+def _spd(d, seed, rows=None):
+    g = torch.Generator().manual_seed(seed)
+    rows = 2 * d + 3 if rows is None else rows
+    X = torch.randn(rows, d, generator=g)
+    return X.T @ X / rows
+
+
+def test_chol_inv_grouped_mixed_sizes_match_oracle(K):
+    # one call for matrices of many sizes (ragged, not multiples of 4, single-leaf and multi-level ones)
+    dims = [1, 2, 10, 63, 64, 65, 128, 147, 200, 256, 384, 512, 576, 640, 1000, 1152, 129, 64, 256, 512]
+    mats = [_spd(d, 100 + i) for i, d in enumerate(dims)]
+    lams = [0.05 + 0.01 * (i % 5) for i in range(len(dims))]
+    print(f'chol_inv_grouped dims={dims}', flush=True)
+    dev = [m.cuda() for m in mats]
+    outs = [torch.full_like(m, 7.0) for m in dev]
+    info = K.chol_inv_grouped(dev, outs, torch.tensor(lams, device='cuda'))
+    torch.cuda.synchronize()
+    assert torch.all(info == 0)
+    for A, Ag, out, lam, d in zip(mats, dev, outs, lams, dims):
+        assert torch.equal(Ag.cpu(), A), 'input must be left unchanged'
+        ref64 = torch.linalg.inv(A.double() + lam * torch.eye(d, dtype=torch.float64))
+        assert relerr(out, R.cholesky_inv(A, lam)) < TOL_INV, d
+        assert relerr(out, ref64) < TOL_INV, d
+        assert torch.equal(out, out.T), d
+
+
+def test_chol_inv_grouped_reads_the_lower_triangle_only(K):
+    d = 300
+    A = _spd(d, 7)
+    junk = A.clone()
+    junk[torch.triu(torch.ones(d, d, dtype=torch.bool), diagonal=1)] = float('nan')
+    out = torch.empty(d, d, device='cuda')
+    info = K.chol_inv_grouped([junk.cuda()], [out], torch.tensor([0.1], device='cuda'))
+    assert int(info.cpu()[0]) == 0
+    assert relerr(out, R.cholesky_inv(A, 0.1)) < TOL_INV
+
+
+def test_chol_inv_grouped_skip_and_info(K):
+    dims = [96, 300, 96, 140, 520]
+    mats = [_spd(d, 40 + i).cuda() for i, d in enumerate(dims)]
+    mats[2] = -torch.eye(96).cuda()                                  # not positive definite at the first pivot
+    bad = torch.eye(520)
+    bad[400, 400] = -5.0                                             # fails in a later diagonal block
+    mats[4] = bad.cuda()
+    lam = torch.tensor([0.1, 0.2, 0.3, 0.4, 0.0], device='cuda')
+    active = torch.tensor([1, 0, 1, 1, 1], dtype=torch.int32, device='cuda')
+    outs = [torch.full_like(m, 7.0) for m in mats]
+    info = K.chol_inv_grouped(mats, outs, lam, active=active).cpu()
+    assert info[0] == 0 and info[3] == 0
+    assert info[2] == 1 and info[4] == 401
+    assert torch.all(outs[1] == 7.0)                                 # skipped: untouched
+    for b in (0, 3):
+        assert relerr(outs[b], R.cholesky_inv(mats[b].cpu(), float(lam[b]))) < TOL_INV
+    # strided lam / flags, and the same call twice (the plan and the workspace are reused)
+    lam2 = torch.zeros(5, 2, device='cuda')
+    lam2[:, 1] = lam
+    info = K.chol_inv_grouped(mats[:2], outs[:2], lam2[:, 1], lam_stride=2).cpu()
+    assert info[0] == 0 and info[1] == 0
+    assert relerr(outs[1], R.cholesky_inv(mats[1].cpu(), 0.2)) < TOL_INV
+
+
+@pytest.mark.parametrize('d', [2048, 2304, 4608])
+def test_chol_inv_large_matches_fp32_oracle_and_fp64(K, d):
+    # the sizes of the largest ResNet factors: deepest recursion, every level on the split-bf16 tile kernel
+    A = _spd(d, d, rows=2 * d)
+    lam = 0.05
+    eye = torch.eye(d, dtype=torch.float64)
+    ref64 = torch.linalg.inv(A.double() + lam * eye)
+    ref32 = R.cholesky_inv(A, lam)
+    print(f'chol_inv large d={d}', flush=True)
+    out_g = torch.empty(d, d, device='cuda')
+    info = K.chol_inv_grouped([A.cuda()], [out_g], torch.tensor([lam], device='cuda'))
+    out_b = K.cholesky_inv(A.cuda(), lam)
+    torch.cuda.synchronize()
+    assert int(info.cpu()[0]) == 0
+    for name, out in (('grouped', out_g), ('batched', out_b)):
+        e32, e64 = relerr(out, ref32), relerr(out, ref64)
+        print(f'  {name}: vs fp32 oracle {e32:.2e}, vs fp64 {e64:.2e} (oracle vs fp64 {relerr(ref32, ref64):.2e})', flush=True)
+        assert e32 < TOL_INV and e64 < TOL_INV
+        assert torch.equal(out, out.T)
+
+
 # ------------------------------------------------------------------ products
 @pytest.mark.parametrize('tA', [False, True])
 @pytest.mark.parametrize('tB', [False, True])
