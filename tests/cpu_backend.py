@@ -63,6 +63,9 @@ def chol_inv_batched(mats, outs, lam, lam_stride=1, active=None, active_stride=1
     return info
 
 
+chol_inv_grouped = chol_inv_batched    # same contract; the stand-in never needed equal sizes
+
+
 def cholesky_inv(X, damping=1e-7):
     return R.cholesky_inv(X, damping)
 
@@ -154,6 +157,6 @@ def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
 
 def install(monkeypatch):
     from asdl_amd import kernels
-    for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'cholesky_inv',
+    for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'chol_inv_grouped', 'cholesky_inv',
                  'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_inv_grouped', 'unit_wise_mvp', 'conv_patch_sum', 'smw_inv']:
         monkeypatch.setattr(kernels, name, globals()[name])
