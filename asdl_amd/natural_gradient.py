@@ -18,7 +18,7 @@ from .fisher import FisherConfig, get_fisher_maker
 from .grad_maker import LOSS_CROSS_ENTROPY
 from .matrices import *
 from .prec_grad_maker import PreconditionedGradientMaker, PreconditioningConfig
-from .symmatrix import SymMatrix, batched_unit_update_inv, batched_update_inv
+from .symmatrix import Kron, SymMatrix, UnitWise, batched_unit_update_inv, batched_update_inv
 
 _invalid_ema_decay = -1
 _module_level_shapes = [SHAPE_LAYER_WISE, SHAPE_KRON, SHAPE_SWIFT_KRON, SHAPE_KFE, SHAPE_UNIT_WISE, SHAPE_DIAG]
@@ -123,6 +123,64 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
     @property
     def do_accumulate(self):
         return self.config.ema_decay != _invalid_ema_decay
+
+    _STATE_TENSORS = (('kron', 'A'), ('kron', 'B'), ('kron', 'A_inv'), ('kron', 'B_inv'), ('unit', 'data'), ('unit', 'inv'))
+
+    def state_dict(self) -> dict:
+        """``step`` as in the reference (asdl/precondition/prec_grad_maker.py:129-133) plus, under ``curvature``, the
+        curvature state itself so that a resumed run continues where it stopped: per module name a dict
+        ``'<kron|unit>.<attribute>' -> tensor`` holding the Kronecker factors A, B (kept in EMA mode only; without EMA
+        they live in scratch memory and only the inverses exist), their inverses A_inv, B_inv, and the unit-wise
+        blocks and their inverses.  Tensors are clones on the device they live on."""
+        state = dict(self.state)
+        curvature = {}
+        for shape in _kernel_shapes:
+            for name, module in self.named_modules_for(shape):
+                fisher = self._get_module_fisher(module)
+                if fisher is None:
+                    continue
+                entry = curvature.setdefault(name, {})
+                for part, attr in self._STATE_TENSORS:
+                    holder = getattr(fisher, part, None)
+                    tensor = getattr(holder, attr, None) if holder is not None else None
+                    if isinstance(tensor, torch.Tensor):
+                        entry[f'{part}.{attr}'] = tensor.detach().clone()
+        state['curvature'] = {name: entry for name, entry in curvature.items() if entry}
+        return state
+
+    def load_state_dict(self, state_dict: dict):
+        """Restores ``step`` and, when present, the curvature state written by state_dict() (a reference-style
+        ``{'step': n}`` loads as before).  Factors and inverses are moved to the model's device; modules missing from
+        the model raise KeyError."""
+        self.state['step'] = state_dict['step']
+        curvature = state_dict.get('curvature')
+        if curvature is None:
+            return
+        named = {}
+        for shape in _kernel_shapes:
+            for name, module in self.named_modules_for(shape):
+                named[name] = module
+        for name, entry in curvature.items():
+            if name not in named:
+                raise KeyError(f'the saved curvature names module {name!r}, which this model does not have')
+            module = named[name]
+            device = next(module.parameters()).device
+            fisher = self._get_module_fisher(module)
+            if fisher is None:
+                fisher = SymMatrix()
+                setattr(module, self._fisher_attr, fisher)
+            for key, tensor in entry.items():
+                part, attr = key.split('.')
+                if (part, attr) not in self._STATE_TENSORS:
+                    raise KeyError(f'unknown curvature entry {key!r} of module {name!r}')
+                holder = getattr(fisher, part, None)
+                if holder is None:
+                    holder = Kron(A=None, B=None) if part == 'kron' else UnitWise()
+                    setattr(fisher, part, holder)
+                setattr(holder, attr, tensor.detach().to(device=device, dtype=torch.float32).clone().contiguous())
+                if part == 'kron':
+                    holder._A_dim = holder._B_dim = None
+        self._precond_plan = None
 
     def update_curvature(self):
         config = self.config

@@ -225,6 +225,36 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
         self.start_vector_fn = None     # optional: (count, n, device) -> [count, n] start vectors
         self.last_root_stats = {}
 
+    def state_dict(self) -> dict:
+        """``step`` as in the reference (asdl/precondition/prec_grad_maker.py:129-133) plus, under ``shampoo``, the
+        statistics and inverse roots of every preconditioned parameter (in the order of model.parameters()): a list of
+        ``{'shape': parameter shape, 'statistics': [tensor per axis], 'preconditioners': [tensor per axis]}``."""
+        state = dict(self.state)
+        state['shampoo'] = [dict(shape=tuple(pc.param.shape),
+                                 statistics=[s.detach().clone() for s in pc.statistics],
+                                 preconditioners=[q.detach().clone() for q in pc.preconditioners])
+                            for pc in self.preconditioners]
+        return state
+
+    def load_state_dict(self, state_dict: dict):
+        """Restores ``step`` and, when present, the statistics and roots written by state_dict(), in place (the
+        per-size group tensors the batched root update works on keep their storage)."""
+        self.state['step'] = state_dict['step']
+        saved = state_dict.get('shampoo')
+        if saved is None:
+            return
+        if len(saved) != len(self.preconditioners):
+            raise ValueError(f'the saved state holds {len(saved)} parameters, this model has {len(self.preconditioners)}')
+        with torch.no_grad():
+            for pc, entry in zip(self.preconditioners, saved):
+                if tuple(entry['shape']) != tuple(pc.param.shape):
+                    raise ValueError(f'saved parameter shape {tuple(entry["shape"])} != {tuple(pc.param.shape)}')
+                for mine, theirs in ((pc.statistics, entry['statistics']), (pc.preconditioners, entry['preconditioners'])):
+                    if len(mine) != len(theirs):
+                        raise ValueError('saved state and model disagree on the number of Kronecker factors')
+                    for dst, src in zip(mine, theirs):
+                        dst.copy_(src)
+
     def do_forward_and_backward(self, step=None):
         return True
 

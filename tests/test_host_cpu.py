@@ -138,7 +138,7 @@ def test_update_schedule_and_intervals():
                                                             curvature_upd_interval=2, ema_decay=0.1))
     assert [gm.do_update_preconditioner(s) for s in range(6)] == [True, False, False, True, False, False]
     assert [gm.do_update_curvature(s) for s in range(4)] == [True, False, True, False]
-    assert gm.state_dict() == {'step': 0}
+    assert gm.state_dict() == {'step': 0, 'curvature': {}}
     gm.load_state_dict({'step': 5})
     assert gm.state['step'] == 5
     gm2 = KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1, num_total_steps=4,
@@ -212,7 +212,73 @@ def test_kfac_host_logic_matches_reference_golden(tag, monkeypatch):
             if isinstance(m, (nn.Linear, nn.Conv2d)) and ema == -1:
                 assert m.fisher.kron.A is None and m.fisher.kron.B is None    # only inverses are kept
         opt.step()
-    assert gm.state_dict() == {'step': n_steps}
+    assert gm.state_dict()['step'] == n_steps
+
+
+def _resume_run(monkeypatch, ema, ci, pi, fisher_type, n_steps=4, stop=2):
+    """Gradients of an uninterrupted run and of one that is saved after ``stop`` steps and continued by a fresh
+    maker on a fresh copy of the model."""
+    cpu_backend.install(monkeypatch)
+    torch.manual_seed(3)
+    data = [(torch.randn(8, 5), torch.randint(4, (8,))) for _ in range(n_steps)]
+    init = get_mlp().state_dict()
+
+    def make():
+        model = get_mlp()
+        model.load_state_dict(init)
+        config = PreconditioningConfig(data_size=8, damping=1e-2, ema_decay=ema, curvature_upd_interval=ci,
+                                       preconditioner_upd_interval=pi)
+        return model, KfacGradientMaker(model, config, fisher_type=fisher_type, seed=1), \
+            torch.optim.SGD(model.parameters(), lr=0.05)
+
+    def step(model, gm, opt, x, t):
+        opt.zero_grad(set_to_none=True)
+        gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+        gm.forward_and_backward()
+        grads = [p.grad.clone() for p in model.parameters()]
+        opt.step()
+        return grads
+
+    model, gm, opt = make()
+    straight = [step(model, gm, opt, x, t) for x, t in data]
+    model, gm, opt = make()
+    resumed = [step(model, gm, opt, x, t) for x, t in data[:stop]]
+    saved = gm.state_dict()
+    weights = {k: v.clone() for k, v in model.state_dict().items()}
+    for m in model.modules():                   # poison the live state: the clone in `saved` must not alias it
+        fisher = getattr(m, 'fisher', None)
+        if fisher is not None and fisher.has_kron:
+            for attr in ('A', 'B', 'A_inv', 'B_inv'):
+                if getattr(fisher.kron, attr) is not None:
+                    getattr(fisher.kron, attr).fill_(float('nan'))
+    model, gm, opt = make()
+    model.load_state_dict(weights)
+    gm.load_state_dict(saved)
+    assert gm.state['step'] == stop
+    resumed += [step(model, gm, opt, x, t) for x, t in data[stop:]]
+    return straight, resumed, saved
+
+
+@pytest.mark.parametrize('ema,ci,pi,fisher_type', [(-1, 3, 3, FISHER_EMP), (0.3, 1, 3, FISHER_EMP), (0.5, 2, 2, FISHER_MC)])
+def test_state_dict_carries_the_curvature_through_a_resume(ema, ci, pi, fisher_type, monkeypatch):
+    """Stop after step 2 of 4 with update intervals that make steps 2 and 3 depend on curvature computed earlier
+    (stale inverses without EMA; running-average factors with EMA): the continued run has to reproduce the
+    uninterrupted one bit for bit."""
+    straight, resumed, saved = _resume_run(monkeypatch, ema, ci, pi, fisher_type)
+    entry = saved['curvature']['0']
+    assert {'kron.A_inv', 'kron.B_inv'} <= set(entry)
+    assert ('kron.A' in entry) == (ema != -1)
+    for a, b in zip(straight, resumed):
+        for ga, gb in zip(a, b):
+            assert torch.equal(ga, gb)
+
+
+def test_load_state_dict_accepts_the_reference_form_and_rejects_unknown_modules():
+    gm = KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1))
+    gm.load_state_dict({'step': 7})
+    assert gm.state_dict() == {'step': 7, 'curvature': {}}
+    with pytest.raises(KeyError, match='nosuch'):
+        gm.load_state_dict({'step': 1, 'curvature': {'nosuch': {'kron.A': torch.eye(2)}}})
 
 
 # ------------------------------------------------------------------ FisherMaker invariants (test/grad_maker/test_fisher.py)

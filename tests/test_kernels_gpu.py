@@ -6,6 +6,8 @@ summation-order differences, so the bf16 cases are in fact held to 1e-5 as well)
 1e-4 against the fp32 oracle where the matrix is well conditioned, otherwise both are compared with
 an fp64 inverse; preconditioned gradients 1e-3.
 """
+import time
+
 import pytest
 import torch
 import torch.nn as nn
@@ -378,7 +380,7 @@ def test_chol_inv_grouped_skip_and_info(K):
     assert relerr(outs[1], R.cholesky_inv(mats[1].cpu(), 0.2)) < TOL_INV
 
 
-@pytest.mark.parametrize('d', [2048, 2304, 4608])
+@pytest.mark.parametrize('d', [2048, 2304, 4096, 4608])
 def test_chol_inv_large_matches_fp32_oracle_and_fp64(K, d):
     # the sizes of the largest ResNet factors: deepest recursion, every level on the split-bf16 tile kernel
     A = _spd(d, d, rows=2 * d)

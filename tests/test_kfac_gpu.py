@@ -1,7 +1,7 @@
 """End-to-end K-FAC parity on the GPU: KfacGradientMaker (HIP kernels) against the reference's
 golden runs and against the CPU oracle on identical seeded inputs.
 
-Tolerances: inverses 1e-4, preconditioned gradients 1e-3 (relative Frobenius norm); looser only
+Tolerances: factors 1e-5, inverses 1e-4, preconditioned gradients 1e-3 (relative Frobenius norm); looser only
 where the test says why.
 """
 import copy
@@ -20,7 +20,7 @@ from oracle import cpu_ref as R
 import bench_models
 
 pytestmark = pytest.mark.gpu
-TOL_INV, TOL_GRAD = 1e-4, 1e-3
+TOL_FACTOR, TOL_INV, TOL_GRAD = 1e-5, 1e-4, 1e-3
 
 
 def relerr(a, b):
@@ -61,6 +61,7 @@ def test_kfac_gpu_matches_reference_golden(tag):
     gm = KfacGradientMaker(model, config, fisher_type=fisher_type, seed=seed, swift=tag.startswith('swift_'))
     opt = torch.optim.SGD(model.parameters(), lr=0.05)
     n_steps = len({k.split('/')[0] for k in z.files if k.startswith('step')})
+    worst = {}
     for step in range(n_steps):
         x, t = torch.from_numpy(z[f'step{step}/x']), torch.from_numpy(z[f'step{step}/t'])
         if replay is not None:
@@ -80,15 +81,22 @@ def test_kfac_gpu_matches_reference_golden(tag):
                 _, _, mname, which = key.split('/')
                 got = getattr(model.get_submodule(mname).fisher.kron, which)
                 assert got is not None, key
-                assert relerr(got, torch.from_numpy(z[key])) < 5e-4, (key, relerr(got, torch.from_numpy(z[key])))
+                e = relerr(got, torch.from_numpy(z[key]))
+                tol = TOL_INV if which.endswith('_inv') else TOL_FACTOR
+                worst[which] = max(worst.get(which, 0.0), e)
+                assert e < tol, (key, e)
             if key.startswith(f'step{step}/unit/'):
                 _, _, mname, which = key.split('/')
                 got = getattr(model.get_submodule(mname).fisher.unit, which)
                 assert got is not None, key
-                assert relerr(got, torch.from_numpy(z[key])) < 5e-4, (key, relerr(got, torch.from_numpy(z[key])))
+                e = relerr(got, torch.from_numpy(z[key]))
+                tol = TOL_INV if which == 'inv' else TOL_FACTOR
+                worst['unit.' + which] = max(worst.get('unit.' + which, 0.0), e)
+                assert e < tol, (key, e)
         for name, p in model.named_parameters():
             assert grad_close(p.grad, torch.from_numpy(z[f'step{step}/grad/{name}']), TOL_GRAD), (tag, step, name)
         opt.step()
+    print(f'golden {tag}: worst relative errors ' + ', '.join(f'{k} {v:.1e}' for k, v in sorted(worst.items())), flush=True)
 
 
 def _run_pair(model_cpu, x, t, damping, ema=-1, steps=1, autocast=False, fisher_type=FISHER_EMP, tol_grad=TOL_GRAD,
@@ -203,80 +211,110 @@ def test_small_cnn_bf16_autocast(channels_last):
             return model(inp).float()
 
     layers = [(n, m) for n, m in model.named_modules() if isinstance(m, (nn.Linear, nn.Conv2d))]
-    ins, gouts, handles = {}, {}, []
+    ins, gouts, raw, handles = {}, {}, {}, []
     for name, m in layers:
         def fhook(mod, inp, out, name=name):
             ins[name] = inp[0].detach()
             out.register_hook(lambda g, name=name: gouts.__setitem__(name, g.detach()))
         handles.append(m.register_forward_hook(fhook))
-    # raw (mean-reduced) gradients and captured tensors from a plain step
-    model.zero_grad(set_to_none=True)
-    F.cross_entropy(fwd(x), t).backward()
-    raw = {n: p.grad.detach().clone() for n, p in model.named_parameters()}
-    saw_bf16 = any(v.dtype == torch.bfloat16 for v in ins.values())
-    for h in handles:
-        h.remove()
-    assert saw_bf16, 'autocast should hand bf16 activations to the hooks'
-    if channels_last:
-        assert any(v.ndim == 4 and not v.is_contiguous() and v.is_contiguous(memory_format=torch.channels_last)
-                   for v in ins.values()), 'the hooks should see channels-last activations'
+        for pn, p in m.named_parameters(recurse=False):
+            handles.append(p.register_hook(lambda g, key=f'{name}.{pn}': raw.__setitem__(key, g.detach().clone())))
 
+    # the capture hooks stay on during the maker's own pass: the oracle gets the very tensors the kernels read
     gm = KfacGradientMaker(model, PreconditioningConfig(data_size=bs, damping=damping), fisher_type=FISHER_EMP)
     model.zero_grad(set_to_none=True)
     gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
     gm.forward_and_backward()
+    for h in handles:
+        h.remove()
+    assert any(v.dtype == torch.bfloat16 for v in ins.values()), 'autocast should hand bf16 activations to the hooks'
+    if channels_last:
+        assert any(v.ndim == 4 and not v.is_contiguous() and v.is_contiguous(memory_format=torch.channels_last)
+                   for v in ins.values()), 'the hooks should see channels-last activations'
+    worst = {}
     for name, m in layers:
         a = ins[name].float().cpu()
-        g = gouts[name].float().cpu() * bs            # hooks saw the mean-reduced loss; K-FAC uses the summed one
+        g = gouts[name].float().cpu()                 # the maker back-propagates the summed loss
         if isinstance(m, nn.Conv2d):
             A = R.conv_cov_kron_A(a, m.kernel_size, m.stride, m.padding) / bs
             B = R.conv_cov_kron_B(g) / bs
         else:
             A, B = R.linear_cov_kron_A(a) / bs, R.linear_cov_kron_B(g) / bs
         A_inv, B_inv = R.kron_update_inv(A, B, damping)
-        assert relerr(m.fisher.kron.A_inv, A_inv) < TOL_INV, (name, relerr(m.fisher.kron.A_inv, A_inv))
-        assert relerr(m.fisher.kron.B_inv, B_inv) < 5e-3, (name, relerr(m.fisher.kron.B_inv, B_inv))
-        w, b = R.kron_mvp(A_inv, B_inv, raw[name + '.weight'].cpu(), raw[name + '.bias'].cpu())
-        assert relerr(m.weight.grad, w) < 1e-2, (name, relerr(m.weight.grad, w))
-        assert relerr(m.bias.grad, b) < 1e-2
+        w, b = R.kron_mvp(A_inv, B_inv, raw[name + '.weight'].float().cpu() / bs, raw[name + '.bias'].float().cpu() / bs)
+        errs = dict(A_inv=relerr(m.fisher.kron.A_inv, A_inv), B_inv=relerr(m.fisher.kron.B_inv, B_inv),
+                    weight=relerr(m.weight.grad, w), bias=relerr(m.bias.grad, b))
+        for k, v in errs.items():
+            worst[k] = max(worst.get(k, 0.0), v)
+        assert errs['A_inv'] < TOL_INV and errs['B_inv'] < TOL_INV, (name, errs)
+        assert errs['weight'] < TOL_GRAD and errs['bias'] < TOL_GRAD, (name, errs)
+    print('bf16 autocast cnn: worst relative errors ' + ', '.join(f'{k} {v:.1e}' for k, v in worst.items()), flush=True)
 
 
 def test_config2_linear_4096_batch8192_bf16_ema():
-    """The large single-layer configuration at full size: Linear(4096, 4096), 8192 rows, bf16 activations, fp32 factors with EMA.
-    The factors are compared with fp64 products of the same rounded values, the inverses through the identity
-    (A + lam I) A_inv = I, the preconditioned gradient with B_inv G A_inv in fp64."""
+    """The large single-layer configuration at full size: Linear(4096, 4096) with bias, 8192 rows of bf16 activations
+    and output gradients, fp32 factors, damping 1e-3, EMA decay 0.95, two steps (the second one runs the
+    beta != 0 accumulate path of the factor kernels at 4096 x 4096).  Everything is judged against fp64 arithmetic on
+    the tensors the kernels read (captured by extra hooks during the maker's own pass): A and B against the fp64
+    running averages of the fp64 products, the inverses against fp64 inverses of those references and through
+    (F + lam I) F_inv = I, the preconditioned gradient against B_inv G A_inv in fp64 on the raw gradient."""
     torch.manual_seed(5)
-    M, d, damping, ema = 8192, 4096, 1e-3, 0.05
-    a = torch.randn(M, d).to(torch.bfloat16)
+    M, d, damping, ema = 8192, 4096, 1e-3, 0.95
     lin = nn.Linear(d, d).cuda()
     model = nn.Sequential(lin)
-    t = torch.randn(M, d).cuda() * 0.01
     config = PreconditioningConfig(data_size=M, damping=damping, ema_decay=ema)
     gm = KfacGradientMaker(model, config, fisher_type=FISHER_EMP, loss_type='mse')
 
     def fwd(inp):
         with torch.autocast('cuda', dtype=torch.bfloat16):
-            return model(inp).float()
+            return model(inp)                      # bf16 output: the output gradient reaches the hook in bf16
 
-    model.zero_grad(set_to_none=True)
-    gm.setup_loss_call(F.mse_loss, gm.setup_model_call(fwd, a.cuda()), t)
-    gm.forward_and_backward()
-    kron = lin.fisher.kron
-    a64 = a.cuda().double()                        # fp64 products on the device: torch's GEMM as independent reference
-    A_ref = ema * (a64.T @ a64) / M                # first EMA update: (1 - ema) * 0 + ema * statistic
-    assert relerr(kron.A, A_ref) < 1e-5
-    assert torch.equal(kron.A, kron.A.T)
-    assert abs(float(kron.A.diagonal().sum().double()) - ema * float((a64 ** 2).sum() / M)) < 1e-4 * float(A_ref.trace())
-    for which in ('A', 'B'):
-        F_, inv = getattr(kron, which).double(), getattr(kron, which + '_inv').double()
-        trA, trB = float(kron.A.diagonal().sum()), float(kron.B.diagonal().sum())
-        pi = (trA / trB) ** 0.5                    # dA == dB
-        lam = damping ** 0.5 * pi if which == 'A' else damping ** 0.5 / pi
-        lam = max(lam, 1e-7)
-        eye = torch.eye(d, dtype=torch.float64, device='cuda')
-        resid = (F_ + lam * eye) @ inv - eye
-        assert float(resid.norm()) / d ** 0.5 < 1e-3, (which, float(resid.norm()) / d ** 0.5)
-        assert torch.equal(getattr(kron, which + '_inv'), getattr(kron, which + '_inv').T)
+    def mse_fp32(y, target, reduction='mean'):
+        return F.mse_loss(y.float(), target.float(), reduction=reduction)
+
+    cap, handles = {}, []
+
+    def fhook(mod, inp, out):
+        cap['a'] = inp[0].detach()
+        out.register_hook(lambda g: cap.__setitem__('g', g.detach()))
+    handles.append(lin.register_forward_hook(fhook))
+    handles.append(lin.weight.register_hook(lambda g: cap.__setitem__('gw', g.detach().clone())))
+    handles.append(lin.bias.register_hook(lambda g: cap.__setitem__('gb', g.detach().clone())))
+    eye = torch.eye(d, dtype=torch.float64, device='cuda')
+    A_ref = B_ref = None
+    for step in range(2):
+        a = torch.randn(M, d).to(torch.bfloat16).cuda()
+        t = (torch.randn(M, d) * 0.01).to(torch.bfloat16).cuda()
+        model.zero_grad(set_to_none=True)
+        gm.setup_loss_call(mse_fp32, gm.setup_model_call(fwd, a), t)
+        print(f'config 2 step {step}', flush=True)
+        gm.forward_and_backward()
+        assert cap['a'].dtype == torch.bfloat16 and cap['g'].dtype == torch.bfloat16
+        a64, g64 = cap['a'].double(), cap['g'].double()
+        SA, SB = a64.T @ a64 / M, g64.T @ g64 / M
+        A_ref = ema * SA if A_ref is None else (1 - ema) * A_ref + ema * SA
+        B_ref = ema * SB if B_ref is None else (1 - ema) * B_ref + ema * SB
+        kron = lin.fisher.kron
+        errs = dict(A=relerr(kron.A, A_ref), B=relerr(kron.B, B_ref))
+        assert errs['A'] < TOL_FACTOR and errs['B'] < TOL_FACTOR, (step, errs)
+        assert torch.equal(kron.A, kron.A.T) and torch.equal(kron.B, kron.B.T)
+        pi = (float(A_ref.trace()) / float(B_ref.trace())) ** 0.5           # dA == dB
+        for which, ref, lam in (('A', A_ref, damping ** 0.5 * pi), ('B', B_ref, damping ** 0.5 / pi)):
+            lam = max(lam, 1e-7)
+            inv = getattr(kron, which + '_inv')
+            assert torch.equal(inv, inv.T)
+            errs[which + '_inv'] = relerr(inv, torch.linalg.inv(ref + lam * eye))
+            resid = (getattr(kron, which).double() + lam * eye) @ inv.double() - eye
+            errs[which + '_resid'] = float(resid.norm()) / d ** 0.5
+            assert errs[which + '_inv'] < TOL_INV and errs[which + '_resid'] < TOL_INV, (step, which, errs)
+        G = cap['gw'].double() / M
+        w_ref = kron.B_inv.double() @ G @ kron.A_inv.double()
+        b_ref = kron.B_inv.double() @ (cap['gb'].double() / M)
+        errs['weight'], errs['bias'] = relerr(lin.weight.grad, w_ref), relerr(lin.bias.grad, b_ref)
+        assert errs['weight'] < TOL_GRAD and errs['bias'] < TOL_GRAD, (step, errs)
+        print(f'config 2 step {step}: ' + ', '.join(f'{k} {v:.1e}' for k, v in errs.items()), flush=True)
+    for h in handles:
+        h.remove()
 
 
 def test_resnet50_batch64_channels_last_properties():
@@ -344,6 +382,95 @@ def test_resnet50_batch64_channels_last_properties():
     ref = m.fisher.kron.B_inv.double() @ G @ m.fisher.kron.A_inv.double()
     got = m.weight.grad.detach().double().reshape(m.weight.shape[0], -1)
     assert relerr(got, ref) < 1e-3, relerr(got, ref)
+
+
+def test_benchmark_path_resnet50_batch64_against_a_sequential_replay():
+    """The very code path bench.py times, at its size: ResNet-50, batch 64, channels-last, bf16 autocast, sampled
+    (MC) Fisher without EMA, inverses started from inside the backward hooks (fisher.EAGER_INVERSE) on side
+    streams fed by worker threads, the grouped preconditioning plan prepared before the flags are read.  On the
+    third step (the eager path needs the cost of an earlier step) extra hooks capture, for every Conv2d / Linear,
+    the activation and the output gradient the factor kernels read, and the raw gradient of the loss.  Afterwards
+    the same tensors go through the same operations one module after the other on the current stream, with one
+    batched inverse at the end and nothing running beside it, and through the per-module Kron.mvp.  The kernels
+    are deterministic, so an inverse that differs from its replay by more than rounding was computed from a factor
+    that was not final (or was overwritten) when its inverse ran."""
+    import asdl_amd.fisher as fisher_mod
+    import asdl_amd.natural_gradient as ng_mod
+    from asdl_amd.core import no_centered_cov
+    from asdl_amd.matrices import SHAPE_KRON
+    assert fisher_mod.EAGER_INVERSE and ng_mod.GROUPED_PRECONDITION and ng_mod.PREPARE_PRECONDITION_EARLY
+    torch.manual_seed(12)
+    bs, damping = 64, 1e-3
+    model = bench_models.resnet50().cuda().to(memory_format=torch.channels_last)
+    x = torch.randn(bs, 3, 224, 224).cuda().contiguous(memory_format=torch.channels_last)
+    t = torch.randint(0, 1000, (bs,)).cuda()
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    config = PreconditioningConfig(data_size=bs, damping=damping, ignore_modules=[nn.BatchNorm2d])
+    gm = KfacGradientMaker(model, config, fisher_type=FISHER_MC)
+    layers = [(n, m) for n, m in model.named_modules() if isinstance(m, (nn.Linear, nn.Conv2d))]
+    ins, gouts, raw, handles = {}, {}, {}, []
+    benchmark_flag = torch.backends.cudnn.benchmark
+    torch.backends.cudnn.benchmark = True
+    try:
+        for step in range(3):
+            if step == 2:
+                for name, m in layers:
+                    def fhook(mod, inp, out, name=name):
+                        ins[name] = inp[0].detach()
+                        # the sampled pass comes first; the loss backward pass fires the hook a second time
+                        out.register_hook(lambda g, name=name: gouts.setdefault(name, g.detach()))
+                    handles.append(m.register_forward_hook(fhook))
+                    for pn, p in m.named_parameters(recurse=False):
+                        handles.append(p.register_hook(
+                            lambda g, key=(name, pn): raw.__setitem__(key, g.detach().clone())))
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
+            print(f'benchmark path step {step}', flush=True)
+            gm.forward_and_backward()
+    finally:
+        torch.backends.cudnn.benchmark = benchmark_flag
+        for h in handles:
+            h.remove()
+    torch.cuda.synchronize()
+    got = {name: (m.fisher.kron.A_inv.clone(), m.fisher.kron.B_inv.clone(),
+                  {pn: p.grad.detach().clone() for pn, p in m.named_parameters(recurse=False)}) for name, m in layers}
+    assert len(ins) == len(gouts) == len(layers) == 54
+
+    # sequential replay of the captured tensors
+    replay = {}
+    with no_centered_cov(model, [SHAPE_KRON], ignore_modules=[nn.BatchNorm2d], calc_inv=True) as cxt:
+        cxt.set_damping(damping)
+        cxt.set_cov_scale(1.0 / bs)
+        for name, m in layers:
+            cxt.call_operations_in_forward(m, ins[name], None)
+            cxt.call_operations_in_backward(m, gouts[name])
+        torch.cuda.synchronize()
+        cxt.flush_inverses()
+        for name, m in layers:
+            replay[name] = cxt.cov_symmatrix(m, pop=True).kron
+    torch.cuda.synchronize()
+    worst = dict(A_inv=0.0, B_inv=0.0, weight=0.0, bias=0.0)
+    for name, m in layers:
+        kron = replay[name]
+        eA, eB = relerr(got[name][0], kron.A_inv), relerr(got[name][1], kron.B_inv)
+        worst['A_inv'], worst['B_inv'] = max(worst['A_inv'], eA), max(worst['B_inv'], eB)
+        assert eA < 1e-5 and eB < 1e-5, (name, eA, eB)
+        g_w = raw[(name, 'weight')] / bs
+        g_b = raw[(name, 'bias')] / bs if m.bias is not None else None
+        kron.mvp(vec_weight=g_w, vec_bias=g_b, use_inv=True, inplace=True)
+        e = relerr(got[name][2]['weight'], g_w)
+        worst['weight'] = max(worst['weight'], e)
+        assert e < 1e-5, (name, 'weight', e)
+        if g_b is not None:
+            e = relerr(got[name][2]['bias'], g_b)
+            worst['bias'] = max(worst['bias'], e)
+            assert e < 1e-5, (name, 'bias', e)
+    print('benchmark path vs sequential replay: worst relative differences ' +
+          ', '.join(f'{k} {v:.1e}' for k, v in worst.items()), flush=True)
 
 
 def test_resnet18_cifar_batch128_fp32_properties():
@@ -555,3 +682,57 @@ def test_fisher_attributes_and_steps_without_curvature_update():
         invs.append(kron.A_inv.clone())
     assert torch.equal(invs[0], invs[1])            # step 1 reuses the stale inverse
     assert gm.state_dict() == {'step': 3}
+
+
+@pytest.mark.parametrize('ema,ci,pi', [(-1, 3, 3), (0.4, 1, 3)])
+def test_state_dict_resume_continues_the_run(ema, ci, pi):
+    """Save after two of four steps (state_dict: step + Kronecker factors / inverses + unit-wise blocks), load into a
+    fresh maker on a fresh copy of the model (through torch.save / torch.load, as a checkpoint would), continue:
+    with update intervals of 3 the third step preconditions with inverses from before the save, and with EMA the
+    running averages carry on.  The empirical Fisher on an MLP with BatchNorm1d / LayerNorm (unit-wise blocks) is
+    deterministic, so the continued run has to equal the uninterrupted one bit for bit."""
+    import io
+    torch.manual_seed(21)
+    data = [(torch.randn(16, 12).cuda(), torch.randint(5, (16,)).cuda()) for _ in range(4)]
+
+    def net():
+        torch.manual_seed(22)
+        return nn.Sequential(nn.Linear(12, 16), nn.BatchNorm1d(16), nn.ReLU(), nn.Linear(16, 10), nn.LayerNorm(10),
+                             nn.Linear(10, 5)).cuda()
+
+    def make(model):
+        config = PreconditioningConfig(data_size=16, damping=1e-2, ema_decay=ema, curvature_upd_interval=ci,
+                                       preconditioner_upd_interval=pi)
+        return KfacGradientMaker(model, config, fisher_type=FISHER_EMP), torch.optim.SGD(model.parameters(), lr=0.05)
+
+    def step(model, gm, opt, x, t):
+        opt.zero_grad(set_to_none=True)
+        gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+        gm.forward_and_backward()
+        grads = [p.grad.clone() for p in model.parameters()]
+        opt.step()
+        return grads
+
+    model = net()
+    gm, opt = make(model)
+    straight = [step(model, gm, opt, x, t) for x, t in data]
+    model = net()
+    gm, opt = make(model)
+    resumed = [step(model, gm, opt, x, t) for x, t in data[:2]]
+    buf = io.BytesIO()
+    torch.save({'model': model.state_dict(), 'kfac': gm.state_dict()}, buf)
+    entry = gm.state_dict()['curvature']
+    assert {'kron.A_inv', 'kron.B_inv'} <= set(entry['0']) and 'unit.inv' in entry['1'] and 'unit.inv' in entry['4']
+    assert ('kron.A' in entry['0']) == (ema != -1) and ('unit.data' in entry['1']) == (ema != -1)
+    del model, gm, opt
+    buf.seek(0)
+    ckpt = torch.load(buf, weights_only=True)
+    model = net()
+    model.load_state_dict(ckpt['model'])
+    gm, opt = make(model)
+    gm.load_state_dict(ckpt['kfac'])
+    assert gm.state['step'] == 2
+    resumed += [step(model, gm, opt, x, t) for x, t in data[2:]]
+    for k, (a, b) in enumerate(zip(straight, resumed)):
+        for ga, gb in zip(a, b):
+            assert torch.equal(ga, gb), f'step {k}'

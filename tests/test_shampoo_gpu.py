@@ -337,3 +337,53 @@ def test_shampoo_gpt2_small_weight_shapes_full_size():
     for prec, g, p in zip(gm.preconditioners, grads, params):
         ref = prec.preconditioners[0].double().T @ g.double() @ prec.preconditioners[1].double()
         assert relerr(p.grad, ref) < 1e-4
+
+
+def test_state_dict_resume_continues_the_run():
+    """Save after three of six steps (step + statistics + inverse roots of every parameter), load into a fresh
+    maker on a fresh copy of the model, continue: roots are taken every 4th step, so steps 3 precondition with
+    loaded roots and the root update of step 4 works on statistics that were accumulated across the save."""
+    import io
+    torch.manual_seed(31)
+    data = [(torch.randn(16, 12).cuda(), torch.randint(5, (16,)).cuda()) for _ in range(6)]
+
+    def net():
+        torch.manual_seed(32)
+        return nn.Sequential(nn.Linear(12, 16), nn.ReLU(), nn.Linear(16, 8), nn.ReLU(), nn.Linear(8, 5)).cuda()
+
+    def make(model):
+        config = PreconditioningConfig(damping=1e-6, curvature_upd_interval=1, preconditioner_upd_interval=4)
+        gm = ShampooGradientMaker(model, config)
+        gen = torch.Generator().manual_seed(33)
+        gm.start_vector_fn = lambda count, n, device: (torch.rand(count, n, generator=gen) * 2 - 1).to(device)
+        return gm, torch.optim.SGD(model.parameters(), lr=0.05), gen
+
+    def step(model, gm, opt, x, t):
+        opt.zero_grad(set_to_none=True)
+        gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+        gm.forward_and_backward()
+        grads = [p.grad.clone() for p in model.parameters()]
+        opt.step()
+        return grads
+
+    model = net()
+    gm, opt, gen = make(model)
+    straight = [step(model, gm, opt, x, t) for x, t in data]
+    model = net()
+    gm, opt, gen = make(model)
+    resumed = [step(model, gm, opt, x, t) for x, t in data[:3]]
+    buf = io.BytesIO()
+    torch.save({'model': model.state_dict(), 'shampoo': gm.state_dict(), 'rng': gen.get_state()}, buf)
+    del model, gm, opt
+    buf.seek(0)
+    ckpt = torch.load(buf, weights_only=True)
+    model = net()
+    model.load_state_dict(ckpt['model'])
+    gm, opt, gen = make(model)
+    gen.set_state(ckpt['rng'])
+    gm.load_state_dict(ckpt['shampoo'])
+    assert gm.state['step'] == 3 and len(ckpt['shampoo']['shampoo']) == 3
+    resumed += [step(model, gm, opt, x, t) for x, t in data[3:]]
+    for k, (a, b) in enumerate(zip(straight, resumed)):
+        for ga, gb in zip(a, b):
+            assert torch.equal(ga, gb), f'step {k}'
