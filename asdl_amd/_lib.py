@@ -56,6 +56,7 @@ _SIGNATURES = {
     'ak_event_record': (c_int, [c_ptr, c_ptr]),
     'ak_stream_order': (c_int, [c_ptr, c_ptr, c_ptr]),
     'ak_event_elapsed_ms': (c_int, [c_ptr, c_ptr, ctypes.POINTER(ctypes.c_float)]),
+    'ak_copy_bytes': (c_int, [c_ptr, c_ptr, c_i64, c_ptr]),
     'ak_tril_pack': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     'ak_tril_unpack': (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_ptr]),
     'ak_gemm_f32': (c_int, [c_int, c_int, c_i64, c_i64, c_i64, c_f32, c_ptr, c_i64, c_ptr, c_i64, c_f32,

@@ -20,6 +20,8 @@ def sources():
 
 
 def build(verbose=True, jobs=8):
+    """AK_TUNING_HOOKS=1 in the environment adds the ak_debug_set_* / ak_debug_force_* setters (tuning runs only)."""
+    flags = FLAGS + (['-DAK_TUNING_HOOKS'] if os.environ.get('AK_TUNING_HOOKS') == '1' else [])
     os.makedirs(LIB_DIR, exist_ok=True)
     obj_dir = os.path.join(LIB_DIR, 'obj')
     os.makedirs(obj_dir, exist_ok=True)
@@ -28,7 +30,7 @@ def build(verbose=True, jobs=8):
     for src in sources():
         obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + '.o')
         objs.append(obj)
-        cmd = [HIPCC] + FLAGS + ['-c', src, '-o', obj]
+        cmd = [HIPCC] + flags + ['-c', src, '-o', obj]
         if verbose:
             print(' '.join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -227,7 +227,8 @@ extern "C" int ak_weight_layout_grouped(const int64_t* table, int count, int64_t
   return ak::check_launch();
 }
 
-// Tuning hook, not part of the interface: the smallest grid (in 128 x 128 tiles) and contraction length from which
+#ifdef AK_TUNING_HOOKS
+// Tuning builds only (-DAK_TUNING_HOOKS): the smallest grid (in 128 x 128 tiles) and contraction length from which
 // products that ask for the split-bf16 kernel get it.
 extern "C" void ak_debug_set_gemm_split_threshold(int min_groups, int min_k) {
   ak::g_x3_min_groups = min_groups;
@@ -235,3 +236,4 @@ extern "C" void ak_debug_set_gemm_split_threshold(int min_groups, int min_k) {
 }
 
 extern "C" void ak_debug_set_gemm_double_buffer(int on) { ak::g_x3_double_buffer = on; }
+#endif

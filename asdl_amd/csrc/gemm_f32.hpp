@@ -204,8 +204,14 @@ static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
 
 namespace ak {
 
-inline int g_x3_double_buffer = 1;                     // tuning hook (ak_debug_set_gemm_double_buffer)
-inline int g_x3_min_groups = 100, g_x3_min_k = 256;   // tuning hook (ak_debug_set_gemm_split_threshold)
+// Constants of the product library; variables that a setter can change only in tuning builds (-DAK_TUNING_HOOKS).
+#ifdef AK_TUNING_HOOKS
+inline int g_x3_double_buffer = 1;
+inline int g_x3_min_groups = 100, g_x3_min_k = 256;
+#else
+constexpr int g_x3_double_buffer = 1;
+constexpr int g_x3_min_groups = 100, g_x3_min_k = 256;
+#endif
 
 inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return AK_OK;

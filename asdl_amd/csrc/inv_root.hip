@@ -9,7 +9,12 @@
 
 namespace ak {
 
-inline int g_root_split = 3;      // products of the Newton iteration: 3 = split-bf16 kernel (fp32-grade accuracy), 0 = fp32 MFMA
+// products of the Newton iteration: 3 = split-bf16 kernel (fp32-grade accuracy), 0 = fp32 MFMA
+#ifdef AK_TUNING_HOOKS
+inline int g_root_split = 3;
+#else
+constexpr int g_root_split = 3;
+#endif
 
 constexpr int RCHUNKS = 64;   // partial-reduction chunks per matrix
 
@@ -382,6 +387,8 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
   return check_launch();
 }
 
-// Tuning hook, not part of the interface: 0 = the fp32 MFMA kernel, 3 = the three-piece split kernel for the
-// products of the Newton iteration.
+#ifdef AK_TUNING_HOOKS
+// Tuning builds only: 0 = the fp32 MFMA kernel, 3 = the three-piece split kernel for the products of the Newton
+// iteration.
 extern "C" void ak_debug_set_root_split(int pieces) { ak::g_root_split = pieces; }
+#endif

@@ -406,8 +406,15 @@ struct DtlPlan {
   size_t ws_bytes;
 };
 
-static int g_force_group = 0;            // tuning hook (ak_debug_force_gather_group); 0: the built-in choice
-static int g_force_bt = 0, g_force_ns = 0;   // tuning hook (ak_debug_force_syrk_plan); 0: use the model
+// 0: the built-in choice of the gather group / the cost model's tile size and split factor.  Only a tuning build
+// (-DAK_TUNING_HOOKS) can pin them.
+#ifdef AK_TUNING_HOOKS
+static int g_force_group = 0;
+static int g_force_bt = 0, g_force_ns = 0;
+#else
+constexpr int g_force_group = 0;
+constexpr int g_force_bt = 0, g_force_ns = 0;
+#endif
 
 // Tile size and split-K factor from a small cost model (microseconds, constants measured on MI355X): the
 // k-tiles of one split times the k-tile time of the most loaded CU, a fixed charge per work group, the
@@ -582,15 +589,17 @@ static bool nhwc_ok(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, i
 
 }  // namespace ak
 
-// Not part of the public interface: pins the channel group size of the gathered column order (0: built-in choice).
+#ifdef AK_TUNING_HOOKS
+// Tuning builds only: pins the channel group size of the gathered column order (0: built-in choice).
 extern "C" void ak_debug_force_gather_group(int group) { ak::g_force_group = group; }
 
-// Not part of the public interface: pins the tile size (64/128/256) and split-K factor of the direct-to-LDS
-// SYRK for tuning runs; (0, 0) restores the cost model.
+// Tuning builds only: pins the tile size (64/128/256) and split-K factor of the direct-to-LDS SYRK; (0, 0) restores
+// the cost model.
 extern "C" void ak_debug_force_syrk_plan(int bt, int nsplit) {
   ak::g_force_bt = bt;
   ak::g_force_ns = nsplit;
 }
+#endif
 
 extern "C" size_t ak_conv_syrk_nhwc_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh,
                                              int sw, int ph, int pw) {

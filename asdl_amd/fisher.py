@@ -11,6 +11,7 @@ from torch import Tensor
 
 from .core import no_centered_cov
 from .grad_maker import GradientMaker, LOSS_CROSS_ENTROPY, LOSS_MSE
+from .profiling import nvtx_range, phase_mark
 from .matrices import *
 from .operations import OperationContext
 from .symmatrix import SymMatrix, batched_unit_update_inv, batched_update_inv
@@ -132,11 +133,13 @@ class FisherMaker(GradientMaker):
                 # the backward pass that is still producing the others
                 cxt.set_eager_inverse(getattr(self, '_inverse_cost_prev', 0))
 
-            self.call_model()
-            loss = None
-            if self.is_fisher_emp or calc_loss_grad:
-                self.call_loss()
-                loss = self._loss
+            with nvtx_range('fwd'):
+                self.call_model()
+                loss = None
+                if self.is_fisher_emp or calc_loss_grad:
+                    self.call_loss()
+                    loss = self._loss
+            phase_mark('fwd')             # forward pass with the cov_kron_A kernels of its hooks
 
             def closure(nll_expr, retain_graph=False):
                 keep = retain_graph or loss_grad_after_fisher
@@ -149,11 +152,13 @@ class FisherMaker(GradientMaker):
                         # engine leaves out the weight-gradient kernels, whose results would be dropped.
                         torch.autograd.grad(nll_expr(), list(cxt.grad_edges), retain_graph=keep, allow_unused=True)
 
-            if self.is_fisher_emp:
-                closure(lambda: loss)
-            else:
-                self._fisher_loop(closure)
+            with nvtx_range('bwd'):
+                if self.is_fisher_emp:
+                    closure(lambda: loss)
+                else:
+                    self._fisher_loop(closure)
             cxt.join_factor_stream()
+            phase_mark('bwd_fisher')      # backward pass that feeds the cov_kron_B kernels (early inverses run beside it)
             cxt.finish_registered()
             # The inverses only need the factors: enqueue them now (side streams) and, when a loss backward
             # pass follows, let that pass run on the main stream meanwhile; the flags are read afterwards.
@@ -167,7 +172,8 @@ class FisherMaker(GradientMaker):
         if loss_grad_after_fisher:
             if self.after_factors is not None:
                 early = self.after_factors()     # e.g. the caller's inverse update, enqueued beside the pass below
-            loss.backward()
+            with nvtx_range('bwd'):
+                loss.backward()
         if calc_loss_grad:
             # the loss was summed over the batch: divide gradients and loss by the data size (enqueued before the
             # host waits for the inverse flags, so that nothing is left to launch between that wait and the caller)
@@ -175,6 +181,7 @@ class FisherMaker(GradientMaker):
             if grads:
                 torch._foreach_div_(grads, data_size)     # one launch for all parameters
             loss.div_(data_size)
+        phase_mark('bwd_loss')            # loss backward pass (the inverses run beside it on side streams)
         if deferred is not None or early is not None:
             if self.before_inverse_wait is not None:
                 self.before_inverse_wait()      # host work of the caller that needs no flags: the device is still busy
@@ -182,6 +189,7 @@ class FisherMaker(GradientMaker):
                 deferred.finish(config.fisher_attr)
             if early is not None:
                 early.finish()
+        phase_mark('upd_inv')             # what is left of the inverses once the loss backward pass has ended
         return self._model_output, loss
 
     def _register_fisher(self, cxt: OperationContext, prescale=1.0):

@@ -19,6 +19,7 @@ import torch
 import torch.nn as nn
 
 from . import kernels
+from .profiling import nvtx_range
 from .symmatrix import Kron, SymMatrix, UnitWise, batched_update_inv
 from .utils import UnfoldedInput, im2col_2d, original_requires_grad
 
@@ -156,6 +157,10 @@ class Operation:
         self._op_results[tmp_key] = buf
 
     def forward_post_process(self, in_data: torch.Tensor, out_data: torch.Tensor):
+        with nvtx_range('cov_kron_A'):
+            self._forward_post_process(in_data, out_data)
+
+    def _forward_post_process(self, in_data: torch.Tensor, out_data: torch.Tensor):
         module = self._module
         op_names = self._op_names
         if OP_SAVE_INPUTS in op_names:
@@ -180,6 +185,10 @@ class Operation:
             self._n_forward += 1
 
     def backward_pre_process(self, out_grads, vector: torch.Tensor = None):
+        with nvtx_range('cov_kron_B'):
+            self._backward_pre_process(out_grads, vector)
+
+    def _backward_pre_process(self, out_grads, vector: torch.Tensor = None):
         module = self._module
         op_names = self._op_names
         if not any(name in BWD_OPS for name in op_names):
@@ -351,6 +360,10 @@ class _NormOperation(Operation):
         return tensor
 
     def backward_pre_process(self, out_grads, vector=None):
+        with nvtx_range('cov_unit_wise'):
+            self._backward_pre_process(out_grads, vector)
+
+    def _backward_pre_process(self, out_grads, vector=None):
         module = self._module
         op_names = self._op_names
         if OP_SAVE_OUTGRADS in op_names:

@@ -13,6 +13,7 @@ import torch
 from torch import Tensor
 
 from . import kernels
+from .profiling import nvtx_range
 
 __all__ = ['SymMatrix', 'Kron', 'UnitWise', 'batched_update_inv', 'PendingInverses', 'matrix_to_tril', 'tril_to_matrix',
            'get_n_cols_by_tril']
@@ -219,14 +220,19 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
     infos, records, events, futures = [], [], [], []
     use_streams = mats_on_gpu and (len(prepared) > 1 or defer)
 
+    range_name = 'inv_kron' + ('_A' if calc_A_inv else '') + ('_B' if calc_B_inv else '')
+
     def run_group(group):
         entries, outs, lam_g, act_g, info = group
-        if act_g is None:          # a low-rank factor
-            kernels.smw_inv(entries[0][1], lam_g, out=outs[0], info=info)
-        elif GROUPED_INVERSE:
-            kernels.chol_inv_grouped([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
-        else:
-            kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1, info=info)
+        with nvtx_range(range_name):
+            if act_g is None:          # a low-rank factor
+                kernels.smw_inv(entries[0][1], lam_g, out=outs[0], info=info)
+            elif GROUPED_INVERSE:
+                kernels.chol_inv_grouped([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1,
+                                         info=info)
+            else:
+                kernels.chol_inv_batched([e[1] for e in entries], outs, lam_g, 1, active=act_g, active_stride=1,
+                                         info=info)
 
     if use_streams:
         main = torch.cuda.current_stream()

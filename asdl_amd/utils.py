@@ -5,11 +5,12 @@ import torch
 from torch import nn
 
 from . import kernels
+from .profiling import nvtx_range
 
 _REQUIRES_GRAD_ATTR = '_original_requires_grad'
 
 __all__ = ['original_requires_grad', 'record_original_requires_grad', 'restore_original_requires_grad',
-           'skip_param_grad', 'cholesky_inv', 'has_reduction', 'UnfoldedInput', 'im2col_2d']
+           'skip_param_grad', 'cholesky_inv', 'has_reduction', 'nvtx_range', 'UnfoldedInput', 'im2col_2d']
 
 
 def original_requires_grad(module=None, param_name=None, param=None):

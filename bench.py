@@ -44,12 +44,13 @@ def parse():
     ap.add_argument('--with-batchnorm', action='store_true',
                     help='do not ignore BatchNorm2d: the 53 BN layers get the unit-wise 2x2 blocks of the default K-FAC '
                          '(the headline configuration ignores them, as the reference training script does)')
-    ap.add_argument('--workload', default='resnet50', choices=['resnet50', 'linear4096', 'shampoo_gpt2'],
+    ap.add_argument('--workload', default='resnet50', choices=['resnet50', 'linear4096', 'shampoo_gpt2', 'hbm_kernels'],
                     help="resnet50: the headline benchmark.  linear4096: the large single-layer configuration, a single "
                          'Linear 4096x4096 with bias on 8192 bf16 rows, EMA 0.95 (factor + inverse + precondition of one '
                          'large layer; its own metric name, not the headline).  shampoo_gpt2: ShampooGradientMaker '
                          'on a 12-layer GPT-2-small-shaped decoder, 8 x 1024 random tokens, bf16 autocast, statistics and '
-                         'preconditioning every step, inverse 4th roots every 10 steps, epsilon 1e-6 (own metric name)')
+                         'preconditioning every step, inverse 4th roots every 10 steps, epsilon 1e-6 (own metric name).  '
+                         'hbm_kernels: achieved HBM bandwidth of the memory-bound kernels (bench_hbm.py, own JSON line)')
     ap.add_argument('--swift', action='store_true',
                     help='KfacGradientMaker(swift=True): factors of layers with fewer samples than columns are kept as '
                          'row matrices (SKFAC); not the headline configuration')
@@ -58,11 +59,17 @@ def parse():
                          'script examples/arxiv_results/train.py:227: MIOpen then times its convolution kernels once '
                          'per layer shape during the warm-up and keeps the fastest)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--cpu-batch', type=int, default=16,
-                    help='batch of the CPU baseline sample (its time is scaled to the full batch)')
+    ap.add_argument('--cpu-batch', type=int, default=0,
+                    help='batch of the CPU baseline sample; 0 (default): the full batch of the workload, nothing scaled')
+    ap.add_argument('--phase-steps', type=int, default=5,
+                    help='steps run after the timed region with phase marks on (events at the phase boundaries of the '
+                         'main stream): the per-phase breakdown in the `phases` object; 0 switches it off')
+    ap.add_argument('--ranges', action='store_true',
+                    help='emit roctx ranges with the reference\'s range names (cov_kron_A, cov_kron_B, inv_kron_A_B, '
+                         'fwd, bwd, upd_curv, upd_inv, precond) for `rocprofv3 --marker-trace`')
     ap.add_argument('--no-factor-timing', action='store_true')
     ap.add_argument('--traffic-calibration-mib', type=int, default=0,
-                    help='before the warm-up, launch one plain copy kernel (ak::debug_copy_kernel) of this many MiB: '
+                    help='before the warm-up, launch one plain copy kernel (ak::copy_bytes_kernel) of this many MiB: '
                          'the known traffic against which a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this '
                          'command is scaled')
     return ap.parse_args()
@@ -75,12 +82,12 @@ def cpu_baseline(args):
     import torch.nn.functional as F
     import bench_models
     from oracle import cpu_ref
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    # a one-GPU box gives a job 16 host cores whatever os.cpu_count() shows
+    cores = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
     torch.manual_seed(0)
     model = bench_models.resnet50()
-    bs = args.cpu_batch
+    bs = args.cpu_batch or args.batch
     x = torch.randn(bs, 3, 224, 224)
     t = torch.randint(0, 1000, (bs,))
 
@@ -101,13 +108,13 @@ def cpu_baseline(args):
     t0 = time.time()
     orc.forward_and_backward(x, t)
     dt = time.time() - t0
-    # forward/backward and factor statistics scale with the batch, inverses and preconditioning do not;
-    # scaling the whole sample linearly therefore over-estimates the CPU time per full step only slightly
-    # less than proportionally -- reported as measured on the sample, and scaled, both.
+    # forward/backward and factor statistics scale with the batch, inverses and preconditioning do not: a sample at
+    # a smaller batch, scaled linearly, over-estimates the CPU time of a full step
     scaled = dt * args.batch / bs
-    return {'value': 1.0 / scaled, 'unit': 'steps/s', 'cores': cores, 'kind': 'port',
-            'sample': f'one K-FAC step of the CPU oracle on ResNet-50 at batch {bs} took {dt:.1f} s; '
-                      f'value = 1 / (that time x {args.batch}/{bs})'}
+    sample = f'one K-FAC step of the CPU oracle (PyTorch CPU ops, {cores} threads) on ResNet-50 at batch {bs} took {dt:.1f} s'
+    if bs != args.batch:
+        sample += f'; value = 1 / (that time x {args.batch}/{bs})'
+    return {'value': 1.0 / scaled, 'unit': 'steps/s', 'cores': cores, 'kind': 'port', 'sample': sample}
 
 
 def main():
@@ -116,6 +123,10 @@ def main():
         print(f'bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}).',
               file=sys.stderr)
         sys.exit(2)
+    if args.workload == 'hbm_kernels':
+        import bench_hbm          # achieved bandwidth of the memory-bound kernels: its own JSON line
+        bench_hbm.main([])
+        return
     import torch
     import torch.nn as nn
     import torch.nn.functional as F
@@ -185,12 +196,14 @@ def main():
         src = torch.ones(n // 4, device=dev)
         dst = torch.empty_like(src)
         lib = _lib.load()
-        lib.ak_debug_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         torch.cuda.synchronize()
-        _lib.check(lib.ak_debug_copy(src.data_ptr(), dst.data_ptr(), n, None), 'ak_debug_copy')
+        _lib.check(lib.ak_copy_bytes(src.data_ptr(), dst.data_ptr(), n, None), 'ak_copy_bytes')
         torch.cuda.synchronize()
         del src, dst
 
+    if args.ranges:
+        from asdl_amd import profiling
+        profiling.enable_ranges(True)
     for i in range(args.warmup):
         step()
         if i == 0:
@@ -211,6 +224,29 @@ def main():
     kernels.set_timing_sink(None)
 
     ms_per_step = elapsed / args.steps * 1e3
+
+    phases = None
+    if args.phase_steps > 0:
+        # Separate, untimed steps: an event at every phase boundary of the main stream.  The phases are those of the
+        # reference's profiling example (examples/prof/time_step.py: fwd_bwd_upd_curv, upd_inv, precond, upd_param),
+        # with the curvature update split into its three passes.  Work on side streams (the inverses) shows up in the
+        # phase it runs beside; `upd_inv` is what is left of it after the loss backward pass.
+        from asdl_amd import profiling
+        marks = []
+        profiling.set_phase_sink(marks)
+        for _ in range(args.phase_steps):
+            profiling.phase_mark('begin')
+            step()
+            profiling.phase_mark('upd_param')
+        torch.cuda.synchronize()
+        profiling.set_phase_sink(None)
+        sums = {}
+        for (_, e0), (name, e1) in zip(marks, marks[1:]):
+            if name != 'begin':
+                sums[name] = sums.get(name, 0.0) + e0.elapsed_time(e1)
+        phases = {'steps': args.phase_steps, 'unit': 'ms per step',
+                  'ms': {k: round(v / args.phase_steps, 4) for k, v in sums.items()},
+                  'sum_ms': round(sum(sums.values()) / args.phase_steps, 4)}
     out = {
         'metric': 'K-FAC steps/s ResNet-50 bs64',
         'value': args.steps / elapsed,
@@ -264,6 +300,8 @@ def main():
                                      'fp32 statistics and roots', 'batch': bs}
     elif not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(args)
+    if phases is not None:
+        out['phases'] = phases
     print(json.dumps(out))
 
 

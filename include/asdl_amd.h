@@ -16,8 +16,11 @@
  *   - Return value: 0 ok; <0 bad argument (see ak_error_string).  Numerical failures
  *     (non positive-definite input) are reported through a device `info` word, like
  *     LAPACK's info, because they are only known once the stream has run.
- *   - Thread safety: entry points keep no mutable global state and may be called from
- *     any host thread (autograd hooks run on the engine's device thread).
+ *   - Thread safety: entry points may be called from any host thread (autograd hooks run on the
+ *     engine's device thread).  The only state the library keeps is caches behind mutexes (memoised
+ *     launch plans keyed by problem shape) and the per-device address of the static scratch array of
+ *     ak_kron_precond_static; no setter changes its behaviour (tuning setters exist only in builds
+ *     with -DAK_TUNING_HOOKS, which is not how the shipped library is built).
  */
 #ifndef ASDL_AMD_H
 #define ASDL_AMD_H
@@ -317,6 +320,13 @@ int ak_event_destroy(void* event);
 int ak_event_record(void* event, ak_stream_t stream);
 int ak_stream_order(ak_stream_t before, ak_stream_t after, void* event);
 int ak_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---- measurement aid (no counterpart in the reference) ----------------------------------- */
+
+/* dst <- src, `bytes` bytes (a multiple of 16), by a plain grid-stride kernel: exactly `bytes` read from and `bytes`
+ * written to device memory.  The known traffic against which FETCH_SIZE / WRITE_SIZE counter readings of the other
+ * kernels are scaled, and the yardstick for the achieved bandwidth of the memory-bound ones. */
+int ak_copy_bytes(const void* src, void* dst, int64_t bytes, ak_stream_t stream);
 
 #ifdef __cplusplus
 }
