@@ -40,6 +40,15 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(short4v lo, short4v hi) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// Lower-triangular tile enumeration: linear id -> (ti, tj), tj <= ti, row by row (id = ti (ti + 1) / 2 + tj).
+__device__ __forceinline__ void decode_lower_tile(int id, int& ti, int& tj) {
+  int row = static_cast<int>((__builtin_sqrtf(8.f * static_cast<float>(id) + 1.f) - 1.f) * 0.5f);
+  while (row * (row + 1) / 2 > id) --row;
+  while ((row + 1) * (row + 2) / 2 <= id) ++row;
+  ti = row;
+  tj = id - row * (row + 1) / 2;
+}
+
 // Upper-triangular tile enumeration: linear id -> (ti, tj), ti <= tj < T, row-major.
 __device__ __forceinline__ void decode_upper_tile(int id, int T, int& ti, int& tj) {
   int row = 0, len = T;

@@ -21,7 +21,8 @@ enum KMode {
 enum TileMode {
   TILE_ALL = 0,
   TILE_LOWER = 1,         // only tiles with ti >= tj, only elements with i >= j are written
-  TILE_LOWER_MIRROR = 2   // tiles with ti >= tj, mirrored into the upper triangle
+  TILE_LOWER_MIRROR = 2,  // tiles with ti >= tj, mirrored into the upper triangle
+  TILE_LINEAR_GRID = 4    // flag set by the launcher: blockIdx.x enumerates the tiles with ti >= tj row by row
 };
 
 struct GemmParams {
@@ -222,17 +223,23 @@ inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   // fill most of the device; below that the 64 x 64 tiles of the fp32 kernel spread the work better.
   if (p.split >= 2 && work_groups >= g_x3_min_groups && p.K >= g_x3_min_k && gemm_x3_ok(p)) {
     dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
+    GemmParams q = p;
+    if (lower && p.M == p.N) {                  // square result, lower tiles only: enumerate just those
+      const unsigned T = grid.x;
+      grid = dim3(T * (T + 1) / 2, 1, batch);
+      q.tile_mode |= TILE_LINEAR_GRID;
+    }
     // three pieces: the double-buffered loop (one work group per CU, MFMAs and split arithmetic interleaved by
     // hand), one instantiation per pair of operand layouts; two pieces: the single-buffered loop
     if (p.split == 3 && g_x3_double_buffer) {
-      if (p.transA == 0 && p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 1>), grid, dim3(256), 0, stream, p);
-      else if (p.transA == 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 0>), grid, dim3(256), 0, stream, p);
-      else if (p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 1>), grid, dim3(256), 0, stream, p);
-      else hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 0>), grid, dim3(256), 0, stream, p);
+      if (p.transA == 0 && p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 1>), grid, dim3(256), 0, stream, q);
+      else if (p.transA == 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 0>), grid, dim3(256), 0, stream, q);
+      else if (p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 1>), grid, dim3(256), 0, stream, q);
+      else hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 0>), grid, dim3(256), 0, stream, q);
     } else if (p.split == 2) {
-      hipLaunchKernelGGL((gemm_x3_kernel<2, false>), grid, dim3(256), 0, stream, p);
+      hipLaunchKernelGGL((gemm_x3_kernel<2, false>), grid, dim3(256), 0, stream, q);
     } else {
-      hipLaunchKernelGGL((gemm_x3_kernel<3, false>), grid, dim3(256), 0, stream, p);
+      hipLaunchKernelGGL((gemm_x3_kernel<3, false>), grid, dim3(256), 0, stream, q);
     }
     return check_launch();
   }

@@ -368,7 +368,12 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
 template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1>
 static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char x3_smem[(DB ? 2 : 1) * 2 * NSPLIT * X3_PLANE];
-  gemm_x3_tile<NSPLIT, DB, AKC, BKC>(p, blockIdx.y, blockIdx.x, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
+  int ti = blockIdx.y, tj = blockIdx.x;
+  if (p.tile_mode & TILE_LINEAR_GRID) {       // a launch of the lower tiles only: no work groups that exit at once
+    p.tile_mode &= ~TILE_LINEAR_GRID;
+    decode_lower_tile(blockIdx.x, ti, tj);
+  }
+  gemm_x3_tile<NSPLIT, DB, AKC, BKC>(p, ti, tj, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // Grouped products: many independent C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i of different sizes in one

@@ -17,6 +17,7 @@ constexpr int g_root_split = 3;
 #endif
 
 constexpr int RCHUNKS = 64;   // partial-reduction chunks per matrix
+constexpr int kRootSymmetricMinDim = 512;   // products of matrices this large compute the lower tiles only
 
 struct RootState {
   // per matrix, all device memory
@@ -275,11 +276,18 @@ extern "C" size_t ak_inv_root_ws_bytes(int64_t n, int batch) {
   return (static_cast<size_t>(batch) * (7 * n * n + 2 * n) + ak::root_state_floats(batch)) * sizeof(float);
 }
 
-extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
-                                  const float* v0, int max_power_iter, float power_tol, int max_iter, float tol,
-                                  float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
-                                  ak_stream_t stream) {
-  using namespace ak;
+namespace ak {
+
+// Workspace layout: M, Mnew, newroot, four product buffers, two vectors, then the per-matrix state; `active`
+// (int32 per matrix, non-zero while its Newton iteration runs) sits at root_active_offset().
+static size_t root_active_offset(int64_t n, int batch) {
+  return (static_cast<size_t>(batch) * (7 * n * n + 2 * n) + static_cast<size_t>(batch) * (4 + RCHUNKS + 2)) * sizeof(float);
+}
+
+// phases: 1 = power iteration, ridge and start of the Newton iteration; 2 = `iters` Newton iterations; 4 = statistics
+static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
+                        const float* v0, int max_power_iter, float power_tol, int max_iter, float tol, float* out,
+                        int64_t strideOut, float* stats, void* ws, size_t ws_bytes, ak_stream_t stream) {
   if (S == nullptr || v0 == nullptr || out == nullptr || stats == nullptr || n < 2 || batch <= 0 || p < 1 ||
       n > (1 << 20) || strideS < n * n || strideOut < n * n)
     return AK_ERR_ARG;
@@ -306,17 +314,22 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
   st.commit = reinterpret_cast<int*>(w); w += batch;
   st.count = reinterpret_cast<int*>(w); w += batch;
 
+  if (reinterpret_cast<unsigned char*>(st.active) != static_cast<unsigned char*>(ws) + root_active_offset(n, batch))
+    return AK_ERR_ARG;     // the layout above and root_active_offset() have to agree
   const dim3 gb(batch), gc(RCHUNKS, batch), b256(256);
-  hipLaunchKernelGGL(root_init_kernel, gb, b256, 0, s, st, v0, v, n);
-  const dim3 gmv(static_cast<unsigned>((n + 3) / 4), batch);
-  for (int it = 0; it < max_power_iter; ++it) {
-    hipLaunchKernelGGL(power_matvec_kernel, gmv, b256, 0, s, st, S, strideS, v, mv, n);
-    hipLaunchKernelGGL(power_update_kernel, gb, b256, 0, s, st, v, mv, n, power_tol, max_power_iter);
+  if (phases & 1) {
+    hipLaunchKernelGGL(root_init_kernel, gb, b256, 0, s, st, v0, v, n);
+    const dim3 gmv(static_cast<unsigned>((n + 3) / 4), batch);
+    for (int it = 0; it < max_power_iter; ++it) {
+      hipLaunchKernelGGL(power_matvec_kernel, gmv, b256, 0, s, st, S, strideS, v, mv, n);
+      hipLaunchKernelGGL(power_update_kernel, gb, b256, 0, s, st, v, mv, n, power_tol, max_power_iter);
+    }
+    hipLaunchKernelGGL(root_ridge_kernel, gc, b256, 0, s, st, S, strideS, n, ridge_eps);
+    hipLaunchKernelGGL(root_zscale_kernel, gb, dim3(64), 0, s, st, p);
+    hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, M, out, strideOut, n, p);
+    hipLaunchKernelGGL(root_begin_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
   }
-  hipLaunchKernelGGL(root_ridge_kernel, gc, b256, 0, s, st, S, strideS, n, ridge_eps);
-  hipLaunchKernelGGL(root_zscale_kernel, gb, dim3(64), 0, s, st, p);
-  hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, M, out, strideOut, n, p);
-  hipLaunchKernelGGL(root_begin_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
+  if (!(phases & 2)) iters = 0;
 
   const int N = static_cast<int>(n);
   auto mm = [&](const float* A, int64_t sA, const float* B, int64_t sB, float* C, int64_t sC) {
@@ -324,9 +337,13 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.active = st.active; g.active_stride = 1;
     g.split = g_root_split;
+    // Every matrix of the iteration is a polynomial of the one symmetric statistic, so every product is symmetric up
+    // to rounding: large ones compute the tiles on and below the diagonal only and mirror them (half the work; the
+    // results are then exactly symmetric).  Small ones keep the full product.
+    if (N >= kRootSymmetricMinDim) g.tile_mode = TILE_LOWER_MIRROR;
     return launch_gemm(g, batch, s);
   };
-  for (int it = 0; it < max_iter; ++it) {
+  for (int it = 0; it < iters; ++it) {
     float* T = buf[0];
     hipLaunchKernelGGL(newton_tmp_kernel, gc, b256, 0, s, st, M, T, n, p);
     int rc = mm(out, strideOut, T, nn, newroot, nn);            // new_root = root T
@@ -383,8 +400,32 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
     hipLaunchKernelGGL(newton_decide_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
     hipLaunchKernelGGL(newton_commit_kernel, gc, b256, 0, s, st, out, strideOut, newroot, M, Mnew, n);
   }
-  hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
+  if (phases & 4) hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
   return check_launch();
+}
+
+}  // namespace ak
+
+extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
+                                  const float* v0, int max_power_iter, float power_tol, int max_iter, float tol,
+                                  float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
+                                  ak_stream_t stream) {
+  return ak::inv_root_run(7, max_iter, S, n, batch, strideS, p, ridge_eps, v0, max_power_iter, power_tol, max_iter, tol,
+                          out, strideOut, stats, ws, ws_bytes, stream);
+}
+
+extern "C" size_t ak_inv_root_active_offset(int64_t n, int batch) {
+  if (n <= 0 || batch <= 0) return 0;
+  return ak::root_active_offset(n, batch);
+}
+
+extern "C" int ak_inv_root_newton_part(int phases, int iters, float* S, int64_t n, int batch, int64_t strideS, int p,
+                                       float ridge_eps, const float* v0, int max_power_iter, float power_tol,
+                                       int max_iter, float tol, float* out, int64_t strideOut, float* stats, void* ws,
+                                       size_t ws_bytes, ak_stream_t stream) {
+  if (phases < 1 || phases > 7 || iters < 0) return AK_ERR_ARG;
+  return ak::inv_root_run(phases, iters, S, n, batch, strideS, p, ridge_eps, v0, max_power_iter, power_tol, max_iter,
+                          tol, out, strideOut, stats, ws, ws_bytes, stream);
 }
 
 #ifdef AK_TUNING_HOOKS

@@ -399,7 +399,7 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_kernel(DtlPara
 constexpr int kDtlDirectSplits = 24;   // up to this many partials the epilogue pass sums them itself
 
 struct DtlPlan {
-  int bt;          // work-group tile: 64, 128 or 256
+  int bt;          // work-group tile: 64, 128, 192 or 256
   int T, nsplit;
   int group, ngroups;   // two-stage reduction: partials per first-stage sum, number of sums (0: single stage)
   int64_t ntiles, rows_per_split;
@@ -422,9 +422,10 @@ constexpr int g_force_bt = 0, g_force_ns = 0;
 static DtlPlan dtl_plan_search(int64_t M, int64_t d, int64_t max_rows_per_split, bool gather) {
   struct Cand { int bt; int occ; double t_alone, t_shared, t_fix; };
   // t_alone: k-tile time of a work group that has its CU to itself, t_shared: with `occ` of them on the CU
-  const Cand cands[3] = {{64, 4, 0.20, 0.20, 3.0},
+  const Cand cands[4] = {{64, 4, 0.20, 0.20, 3.0},
                          {128, 2, gather ? 0.40 : 0.25, 0.59, 4.0},
-                         {256, 1, gather ? 0.95 : 0.70, gather ? 0.95 : 0.70, 8.0}};
+                         {192, 1, gather ? 0.55 : 0.42, gather ? 0.55 : 0.42, 6.0},
+                         {256, 1, gather ? 0.82 : 0.62, gather ? 0.82 : 0.62, 8.0}};
   const int64_t ktiles = (M + kDtlBK - 1) / kDtlBK;
   DtlPlan best{};
   double best_cost = 1e300;
@@ -432,6 +433,7 @@ static DtlPlan dtl_plan_search(int64_t M, int64_t d, int64_t max_rows_per_split,
     if (g_force_bt != 0 && c.bt != g_force_bt) continue;
     if (g_force_bt == 0 && c.bt == 64 && d > 192) continue;
     if (g_force_bt == 0 && c.bt == 256 && d < 1024) continue;
+    if (g_force_bt == 0 && c.bt == 192 && d < 384) continue;
     const int64_t T = (d + c.bt - 1) / c.bt, ntiles = T * (T + 1) / 2;
     const int64_t slots = 256 * c.occ;
     const int64_t ns_cap = ktiles / 4 < 1 ? 1 : (ktiles / 4 > 1024 ? 1024 : ktiles / 4);
@@ -549,7 +551,8 @@ static int dtl_launch(DtlParams& p, const DtlPlan& pl, void* ws, size_t ws_bytes
   p.rows_per_split = pl.rows_per_split;
   p.ws = static_cast<float*>(ws);
   if (pl.bt == 64) return dtl_launch_cfg<2, 2, 1, 1, GATHER>(p, pl, stream);
-  if (pl.bt == 256) return dtl_launch_cfg<2, 2, 4, 4, GATHER>(p, pl, stream);
+  if (pl.bt == 256) return dtl_launch_cfg<2, 4, 4, 2, GATHER>(p, pl, stream);
+  if (pl.bt == 192) return dtl_launch_cfg<2, 2, 3, 3, GATHER>(p, pl, stream);
   return dtl_launch_cfg<2, 2, 2, 2, GATHER>(p, pl, stream);
 }
 

@@ -999,10 +999,18 @@ def kron_precond_grouped(items, grad_scale=1.0):
 
 
 # ------------------------------------------------------------------------------ Shampoo inverse root
-def inv_root_newton(S, p, ridge_eps, v0, out=None, max_power_iter=100, power_tol=1e-6, max_iter=100, tol=1e-6):
+ROOT_POLL_EVERY = 8      # Newton iterations enqueued between two reads of the convergence flags (0: never read them)
+
+
+def inv_root_newton(S, p, ridge_eps, v0, out=None, max_power_iter=100, power_tol=1e-6, max_iter=100, tol=1e-6,
+                    poll_every=None):
     """out[b] <- (S[b] + ridge_eps * lambda_max I)^(-1/p) for S = [batch, n, n] (or [n, n]); S keeps the
     ridge.  v0 = [batch, n] start vectors of the power iteration.  Returns (out, stats) with
-    stats = [batch, 4] = (lambda_max, power iterations, newton iterations, final error) on the device."""
+    stats = [batch, 4] = (lambda_max, power iterations, newton iterations, final error) on the device.
+    ``poll_every`` (default ROOT_POLL_EVERY): the Newton iterations are enqueued that many at a time and the host reads
+    the convergence flags in between (one small device-to-host copy), so that nothing is launched for a batch that has
+    converged; 0 enqueues all ``max_iter`` iterations without ever waiting (the kernels of converged matrices exit at
+    once).  The results are the same either way."""
     _require_gpu(S, v0, out)
     single = S.ndim == 2
     S3 = S.unsqueeze(0) if single else S
@@ -1022,9 +1030,23 @@ def inv_root_newton(S, p, ridge_eps, v0, out=None, max_power_iter=100, power_tol
     ws, ws_bytes, keep = _ws_args(_ws_need('ak_inv_root_ws_bytes', n, batch), S.device)
     strideS = S3.stride(0) if batch > 1 else n * n
     strideO = out3.stride(0) if batch > 1 else n * n
-    rc = lib.ak_inv_root_newton(ctypes.c_void_p(S3.data_ptr()), n, batch, strideS, int(p), float(ridge_eps),
-                                ctypes.c_void_p(v0.data_ptr()), int(max_power_iter), float(power_tol), int(max_iter),
-                                float(tol), ctypes.c_void_p(out3.data_ptr()), strideO,
-                                ctypes.c_void_p(stats.data_ptr()), ws, ws_bytes, _stream())
-    _lib.check(rc, 'ak_inv_root_newton')
+    poll = ROOT_POLL_EVERY if poll_every is None else int(poll_every)
+    args = (ctypes.c_void_p(S3.data_ptr()), n, batch, strideS, int(p), float(ridge_eps), ctypes.c_void_p(v0.data_ptr()),
+            int(max_power_iter), float(power_tol), int(max_iter), float(tol), ctypes.c_void_p(out3.data_ptr()), strideO,
+            ctypes.c_void_p(stats.data_ptr()), ws, ws_bytes, _stream())
+    if poll <= 0 or poll >= max_iter:
+        _lib.check(lib.ak_inv_root_newton(*args), 'ak_inv_root_newton')
+    else:
+        off = lib.ak_inv_root_active_offset(n, batch)
+        active = keep[off:off + 4 * batch].view(torch.int32)
+        _lib.check(lib.ak_inv_root_newton_part(1, 0, *args), 'ak_inv_root_newton_part')
+        done = 0
+        while done < max_iter:
+            with _on_launch_stream():
+                if not bool(active.any().item()):      # waits for what has been enqueued so far
+                    break
+            chunk = min(poll, max_iter - done)
+            _lib.check(lib.ak_inv_root_newton_part(2, chunk, *args), 'ak_inv_root_newton_part')
+            done += chunk
+        _lib.check(lib.ak_inv_root_newton_part(4, 0, *args), 'ak_inv_root_newton_part')
     return (out3[0] if single and out.ndim == 3 else out), stats

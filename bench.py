@@ -117,6 +117,87 @@ def cpu_baseline(args):
     return {'value': 1.0 / scaled, 'unit': 'steps/s', 'cores': cores, 'kind': 'port', 'sample': sample}
 
 
+def cpu_baseline_linear4096(args):
+    """One K-FAC step of the CPU oracle on the single Linear 4096 x 4096 at its full size (8192 bf16 rows, EMA 0.95)."""
+    import torch
+    import torch.nn as nn
+    from oracle import cpu_ref
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(4096, 4096, bias=True))
+    x = torch.randn(8192, 4096).to(torch.bfloat16)
+    t = torch.randint(0, 4096, (8192,))
+
+    class Wrapped:
+        def __call__(self, inp):
+            with torch.autocast('cpu', dtype=torch.bfloat16):
+                return model(inp).float()
+
+        def parameters(self):
+            return model.parameters()
+
+    orc = cpu_ref.KfacOracle(model, data_size=8192, damping=args.damping, ema_decay=0.95, fisher_type=args.fisher,
+                             factor_dtype=torch.float32)
+    orc.model = Wrapped()
+    t0 = time.time()
+    orc.forward_and_backward(x, t)
+    dt = time.time() - t0
+    return {'value': 1.0 / dt, 'unit': 'steps/s', 'cores': cores, 'kind': 'port',
+            'sample': f'one K-FAC step of the CPU oracle (PyTorch CPU ops, {cores} threads) on the full workload took {dt:.1f} s'}
+
+
+def cpu_baseline_shampoo(args, root_interval=10):
+    """Shampoo step of the CPU oracle on a bounded sample: one step without a root update at 2 x 1024 tokens (a
+    quarter of the batch; forward, backward, statistics, preconditioning), and the inverse 4th root of one statistic
+    of each size (768, 1024, 2304, 3072) taken from that step, scaled by how many statistics of that size the model
+    has and spread over the root interval."""
+    import torch
+    import torch.nn.functional as F
+    import bench_models
+    from oracle import cpu_ref
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    model = bench_models.gpt2_small()
+    frac = 4
+    x = torch.randint(0, 50257, (8 // frac, 1024))
+    t = torch.randint(0, 50257, (8 // frac * 1024,))
+
+    class Wrapped:
+        def __call__(self, inp):
+            with torch.autocast('cpu', dtype=torch.bfloat16):
+                return model(inp).float()
+
+        def parameters(self):
+            return model.parameters()
+
+    orc = cpu_ref.ShampooOracle(model, damping=1e-6, curvature_upd_interval=1, preconditioner_upd_interval=10 ** 9)
+    orc.model = Wrapped()
+    orc.step = 1                                   # not a root step
+    t0 = time.time()
+    orc.forward_and_backward(x, t, loss_fn=lambda y, tt: F.cross_entropy(y.reshape(-1, y.shape[-1]), tt))
+    t_step = time.time() - t0
+    counts, sample_stat = {}, {}
+    for stats in orc.stats:
+        for st in stats:
+            n = st.shape[0]
+            counts[n] = counts.get(n, 0) + 1
+            sample_stat.setdefault(n, st)
+    t_roots, parts = 0.0, []
+    for n in sorted(counts):
+        t0 = time.time()
+        _, iters, _ = cpu_ref.compute_power(sample_stat[n].clone(), 4, torch.rand(n) * 2 - 1, ridge_epsilon=1e-6)
+        dt = time.time() - t0
+        t_roots += dt * counts[n]
+        parts.append(f'n={n}: {dt:.1f} s ({iters} iterations) x {counts[n]}')
+    per_step = t_step * frac + t_roots / root_interval
+    return {'value': 1.0 / per_step, 'unit': 'steps/s', 'cores': cores, 'kind': 'port',
+            'sample': f'CPU oracle (PyTorch CPU ops, {cores} threads): one step without roots at 2 x 1024 tokens took '
+                      f'{t_step:.1f} s (x {frac} for the full batch); one inverse 4th root per statistic size: '
+                      + '; '.join(parts) + f'; value = 1 / (step + all roots / {root_interval})'}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -168,6 +249,18 @@ def main():
         config = PreconditioningConfig(damping=1e-6, curvature_upd_interval=1, preconditioner_upd_interval=10)
         gm = ShampooGradientMaker(model, config)
         args.no_factor_timing = True
+        # the dominant kernels of this workload are the products of the coupled Newton iteration: events around every
+        # root update of the timed region, FLOP from the iteration counts the update reports (8 n^3 per iteration)
+        root_records = []
+        plain_update = gm.update_preconditioner
+
+        def timed_update():
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            plain_update()
+            stop.record()
+            root_records.append((start, stop, {key: st for key, st in gm.last_root_stats.items()}))
+        gm.update_preconditioner = timed_update
     else:
         gm = KfacGradientMaker(model, config, fisher_type=args.fisher, swift=args.swift)
     opt = torch.optim.SGD([p for p in model.parameters() if p.requires_grad], lr=1e-4)
@@ -209,6 +302,8 @@ def main():
         if i == 0:
             torch.cuda.synchronize()
             print('bench.py: first warm-up step done (kernel selection, workspaces)', file=sys.stderr, flush=True)
+    if args.workload == 'shampoo_gpt2':
+        del root_records[:]
     sink = None if args.no_factor_timing else []
     kernels.set_timing_sink(sink, n_events=2 * 110 * args.steps)     # two events per factor call, made up front
     torch.cuda.synchronize()
@@ -298,8 +393,38 @@ def main():
                                      'GPT-2-small-shaped decoder (d 768, 12 heads, MLP 3072; token embedding and output '
                                      'head frozen), 8 x 1024 uniform random tokens, bf16 autocast forward/backward, '
                                      'fp32 statistics and roots', 'batch': bs}
-    elif not args.no_cpu_baseline:
-        out['cpu_baseline'] = cpu_baseline(args)
+        if root_records:
+            secs = sum(a.elapsed_time(b) for a, b, _ in root_records) * 1e-3
+            flops, executed_flops, iters = 0.0, 0.0, []
+            for _, _, stats in root_records:
+                for (n, exp), st in stats.items():
+                    it = st[:, 2].double().cpu()
+                    products = 2 + (exp - 1).bit_length()      # root T, T^p by squaring (p a power of two), T^p M
+                    f = float(it.sum()) * products * 2.0 * n ** 3
+                    flops += f
+                    # every fp32 product runs as 6 bf16 piece products; matrices of 512 and up are known to be
+                    # symmetric and only their T (T + 1) / 2 tiles of 128 on and below the diagonal are computed
+                    tiles = -(-n // 128)
+                    executed_flops += 6.0 * f * ((tiles + 1) / (2.0 * tiles) if n >= 512 else 1.0)
+                    iters.append(int(it.max()))
+            executed = executed_flops / secs / 1e12
+            out['roofline'] = {'bound': 'mfma', 'achieved': executed, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
+                               'frac': executed / BF16_MFMA_PEAK_TFLOPS, 'traffic': None,
+                               'kernel': 'products of the coupled Newton iteration (gemm_x3_kernel); `achieved` counts the '
+                                         'bf16 MFMA work executed: 6 piece products per fp32 product, lower tiles only '
+                                         'for the symmetric results; algorithmic_fp32_tflops counts the 2 n^3 per '
+                                         'product of the reference',
+                               'algorithmic_fp32_tflops': flops / secs / 1e12,
+                               'root_updates_timed': len(root_records),
+                               'ms_per_root_update': secs / len(root_records) * 1e3,
+                               'newton_iterations_max': max(iters)}
+    if not args.no_cpu_baseline:
+        if args.workload == 'linear4096':
+            out['cpu_baseline'] = cpu_baseline_linear4096(args)
+        elif args.workload == 'shampoo_gpt2':
+            out['cpu_baseline'] = cpu_baseline_shampoo(args)
+        else:
+            out['cpu_baseline'] = cpu_baseline(args)
     if phases is not None:
         out['phases'] = phases
     print(json.dumps(out))

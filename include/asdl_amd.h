@@ -311,6 +311,19 @@ int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, f
                        float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
                        ak_stream_t stream);
 
+/* The same computation in parts, for a host that stops enqueuing once every matrix has converged (the reference's
+ * `while error > tol and count < iter_count` of asdl/precondition/shampoo.py:508-521 ends there; the one-call form
+ * enqueues max_iter iterations whose kernels exit at once for converged matrices).  `phases` is a bit mask:
+ * 1 = power iteration, ridge and start; 2 = `iters` further Newton iterations; 4 = stats.  All parts of one
+ * computation get the same arguments and the same workspace, untouched in between.  Between parts the host may read
+ * the `batch` int32 words at ws + ak_inv_root_active_offset(n, batch) (after synchronising with the stream): word b is
+ * non-zero while matrix b still iterates.  ak_inv_root_newton == phases 7 with iters = max_iter. */
+size_t ak_inv_root_active_offset(int64_t n, int batch);
+int ak_inv_root_newton_part(int phases, int iters, float* S, int64_t n, int batch, int64_t strideS, int p,
+                            float ridge_eps, const float* v0, int max_power_iter, float power_tol, int max_iter,
+                            float tol, float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,
+                            ak_stream_t stream);
+
 /* ---- stream helpers (no counterpart in the reference) ------------------------------------ */
 
 /* For hosts that run the statistics kernels on a side stream: events of the HIP runtime this library is linked

@@ -281,6 +281,45 @@ def test_load_state_dict_accepts_the_reference_form_and_rejects_unknown_modules(
         gm.load_state_dict({'step': 1, 'curvature': {'nosuch': {'kron.A': torch.eye(2)}}})
 
 
+def test_module_called_twice_in_one_forward_gets_one_inverse_of_the_summed_factors(monkeypatch):
+    """A module that is called twice per forward pass (shared weights), without EMA.  This build sums the two
+    A contributions and the two B contributions and inverts once: (A1 + A2 + lam I)^-1.  The reference inverts inside
+    every backward call and adds the inverses up (asdl/operations/operation.py:267-279: accumulate_result on A_inv /
+    B_inv, and the forward hook keeps only the last input): (A2 + lam I)^-1 + (A2 + lam' I)^-1 with the first call's
+    input lost.  That is a deliberate divergence: the sum of the factors is the curvature block K-FAC defines, and it
+    is what both implementations compute in EMA mode.  No golden run of the reference covers shared modules."""
+    import oracle.cpu_ref as R
+    cpu_backend.install(monkeypatch)
+    torch.manual_seed(5)
+
+    class Twice(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.Linear(6, 6)
+            self.head = nn.Linear(6, 3)
+
+        def forward(self, x):
+            return self.head(torch.tanh(self.lin(torch.tanh(self.lin(x)))))
+
+    model = Twice()
+    x, t = torch.randn(10, 6), torch.randint(3, (10,))
+    ins, gouts = [], []
+    def capture(m, i, o):
+        ins.append(i[0].detach())
+        o.register_hook(lambda g: gouts.append(g.detach()))
+    handle = model.lin.register_forward_hook(capture)
+    gm = KfacGradientMaker(model, PreconditioningConfig(data_size=10, damping=1e-2), fisher_type=FISHER_EMP)
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+    gm.forward_and_backward()
+    handle.remove()
+    assert len(ins) == 2 and len(gouts) == 2
+    A = sum(R.linear_cov_kron_A(a) for a in ins) / 10
+    B = sum(R.linear_cov_kron_B(g) for g in gouts) / 10
+    A_inv, B_inv = R.kron_update_inv(A, B, 1e-2)
+    assert relerr(model.lin.fisher.kron.A_inv, A_inv) < 1e-5
+    assert relerr(model.lin.fisher.kron.B_inv, B_inv) < 1e-5
+
+
 # ------------------------------------------------------------------ FisherMaker invariants (test/grad_maker/test_fisher.py)
 @pytest.mark.parametrize('network', ['mlp', 'cnn'])
 @pytest.mark.parametrize('fisher_type', [FISHER_EMP, FISHER_MC, FISHER_EXACT])

@@ -90,6 +90,23 @@ def test_inv_root_closed_form(n, p, batch):
         assert abs(int(stats[b, 2]) - iters) <= 1, (int(stats[b, 2]), iters)
 
 
+def test_inv_root_polled_and_unpolled_enqueue_give_the_same_result():
+    """The host may stop enqueuing Newton iterations once the convergence flags are all zero (read every few
+    iterations) or enqueue all of them blindly: bit-equal roots and the same iteration counts."""
+    g = torch.Generator().manual_seed(77)
+    S = torch.empty(3, 96, 96)
+    for b in range(3):
+        X = torch.randn(40 * (b + 1), 96, generator=g)        # one rank-deficient, two full-rank statistics
+        S[b] = X.T @ X / X.shape[0]
+    v0 = (torch.rand(3, 96, generator=g) * 2 - 1).cuda()
+    r0, st0 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=0)
+    r1, st1 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=3)
+    r2, st2 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0)
+    assert torch.equal(r0, r1) and torch.equal(r0, r2)
+    assert torch.equal(st0, st1) and torch.equal(st0, st2)
+    assert 1 <= float(st0[:, 2].max()) < 100
+
+
 def test_compute_power_api_and_1x1():
     S = torch.tensor([[4.0]]).cuda()
     assert torch.equal(compute_power(S, 4).cpu(), torch.eye(1))
@@ -337,6 +354,108 @@ def test_shampoo_gpt2_small_weight_shapes_full_size():
     for prec, g, p in zip(gm.preconditioners, grads, params):
         ref = prec.preconditioners[0].double().T @ g.double() @ prec.preconditioners[1].double()
         assert relerr(p.grad, ref) < 1e-4
+
+
+def test_shampoo_gpt2_small_full_decoder_bf16_real_gradients():
+    """The transformer configuration as bench.py runs it: the 12-layer GPT-2-small-shaped decoder, 8 x 1024 random
+    tokens, bf16 autocast, epsilon 1e-6, statistics and roots from the REAL gradients of two steps.  After one or two
+    steps every statistic is rank deficient (a 768 x 2304 gradient leaves at least 1536 zero eigenvalues on its
+    long side), so after the ridge cond = 1e6: the regime in which the coupled Newton iteration is slow and no fp32
+    root is accurate.  Checked: every statistic against the fp64 sums of products of the captured gradients (1e-5);
+    the roots of the 768-wide statistics of two blocks against the CPU oracle run on the same statistic with the same
+    start vector, both measured against the fp64 closed form; one root of each larger size (2304, 3072, 1024) against
+    the fp64 closed form; every preconditioned gradient against P_L^T G P_R in fp64 from the stored roots (1e-3)."""
+    torch.manual_seed(13)
+    model = bench_models.gpt2_small().cuda()
+    x = torch.randint(0, 50257, (8, 1024)).cuda()
+    t = torch.randint(0, 50257, (8 * 1024,)).cuda()
+    gm = ShampooGradientMaker(model, PreconditioningConfig(damping=1e-6, curvature_upd_interval=1,
+                                                           preconditioner_upd_interval=1))
+    gen = torch.Generator().manual_seed(14)
+    starts = {}
+
+    def start_vectors(count, n, dev):
+        v = torch.rand(count, n, generator=gen) * 2 - 1
+        starts[n] = v
+        return v.to(dev)
+    gm.start_vector_fn = start_vectors
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    def token_loss(y, target):
+        return F.cross_entropy(y.reshape(-1, y.shape[-1]), target)
+
+    precs = gm.preconditioners
+    assert len(precs) == 49
+    sums = [[torch.zeros(n, n, dtype=torch.float64, device='cuda') for n in pc.param.shape] for pc in precs]
+    opt = torch.optim.SGD([p for p in model.parameters() if p.requires_grad], lr=1e-3)
+    for step in range(2):
+        opt.zero_grad(set_to_none=True)
+        gm.setup_loss_call(token_loss, gm.setup_model_call(fwd, x), t)
+        print(f'shampoo gpt2 full step {step}', flush=True)
+        # the template of forward_and_backward(), one phase at a time
+        gm.forward()
+        gm.backward()
+        raw = [pc.param.grad.detach().clone() for pc in precs]
+        for g, acc in zip(raw, sums):
+            acc[0] += g.double() @ g.double().T
+            acc[1] += g.double().T @ g.double()
+        before = [[s_.clone() for s_ in pc.statistics] for pc in precs] if step == 1 else None
+        gm.update_curvature()
+        worst = 0.0
+        for k, (pc, acc) in enumerate(zip(precs, sums)):
+            for j, (stat, ref) in enumerate(zip(pc.statistics, acc)):
+                if step == 0:
+                    e = relerr(stat, ref + 1e-12 * torch.eye(ref.shape[0], dtype=torch.float64, device='cuda'))
+                else:       # the first root update left its ridge in the stored statistic: compare the increment
+                    g = raw[k].double()
+                    inc = g @ g.T if j == 0 else g.T @ g
+                    e = relerr(stat.double() - before[k][j].double(), inc)
+                worst = max(worst, e)
+                assert e < (1e-5 if step == 0 else 1e-4), (step, k, j, e)
+        print(f'  statistics: worst relative error {worst:.1e}', flush=True)
+        stats_in = [[s_.clone() for s_ in pc.statistics] for pc in precs]
+        gm.update_preconditioner()
+        iters = {key: st[:, 2].max().item() for key, st in gm.last_root_stats.items()}
+        print(f'  Newton iterations (max per size group): {iters}', flush=True)
+        # roots of 768-wide statistics against the CPU oracle on the same input (blocks 0 and 11: c_proj, both sides)
+        members = {}
+        for k, pc in enumerate(precs):
+            for j, n in enumerate(pc.param.shape):
+                members.setdefault(n, []).append((k, j))
+        names = [n_ for n_, p_ in model.named_parameters() if p_.requires_grad and p_.ndim > 1]
+        picks = [(k, j) for k, nm in enumerate(names) if nm in ('h.0.c_proj.weight', 'h.11.c_proj.weight') for j in (0, 1)]
+        worst_ratio = 0.0
+        for k, j in picks:
+            n = precs[k].param.shape[j]
+            slot = members[n].index((k, j))
+            S = stats_in[k][j].cpu()
+            root_ref, it_ref, err_ref = R.compute_power(S.clone(), 4, starts[n][slot].clone(), ridge_epsilon=1e-6)
+            exact = _closed_form_root(precs[k].statistics[j], 4)      # the stored statistic holds the ridge now
+            e_ref, e_mine = relerr(root_ref, exact), relerr(precs[k].preconditioners[j], exact)
+            print(f'  root {names[k]} axis {j}: oracle {e_ref:.2e} ({it_ref} iterations), here {e_mine:.2e}', flush=True)
+            worst_ratio = max(worst_ratio, e_mine / max(e_ref, 1e-30))
+            assert e_mine <= max(4 * e_ref, 1e-4), (names[k], j, e_mine, e_ref)
+        # one root of each larger size against the fp64 closed form
+        for n in (1024, 2304, 3072):
+            k, j = members[n][0]
+            w, V = torch.linalg.eigh(precs[k].statistics[j].double())
+            exact = (V * w.clamp_min(1e-300) ** -0.25) @ V.T
+            e = relerr(precs[k].preconditioners[j], exact)
+            print(f'  root n={n} ({names[k]} axis {j}): distance from the fp64 closed form {e:.2e}', flush=True)
+            assert e < 5e-2, (n, e)
+        gm.precondition()
+        worst = 0.0
+        for pc, g in zip(precs, raw):
+            ref = pc.preconditioners[0].double().T @ g.double() @ pc.preconditioners[1].double()
+            e = relerr(pc.param.grad, ref)
+            worst = max(worst, e)
+            assert e < 1e-3, e
+        print(f'  preconditioned gradients: worst relative error {worst:.1e}', flush=True)
+        gm.state['step'] += 1
+        opt.step()
 
 
 def test_state_dict_resume_continues_the_run():
