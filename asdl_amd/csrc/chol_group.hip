@@ -30,15 +30,22 @@
 
 namespace ak {
 
-constexpr int64_t CG_MAGIC = 0x3147524c4f4843ll;     // "CHOLGR1"
+constexpr int64_t CG_MAGIC = 0x3247524c4f4843ll;     // "CHOLGR2"
 constexpr int CG_COPY = 0, CG_LEAF = 1, CG_PROD = 2;
 constexpr int CG_FLAG_TRANSA = 1, CG_FLAG_TRANSB = 2, CG_FLAG_OUT_USER = 4;
+// What an operand of a product holds, for the fp16-piece products (bits 4-5 of CgProd::flags: A, bits 6-7: B).  With
+// a = the largest diagonal element of A + lam I, every element is bounded in magnitude: a block of the (updated)
+// matrix by a, of its Cholesky factor L by sqrt(a), of M = L^-1 by 1 / sqrt(lam), of L21 L11^-1 by sqrt(a / lam).
+constexpr int CG_KIND_W = 0, CG_KIND_L = 1, CG_KIND_M = 2, CG_KIND_T2 = 3;
+constexpr int CG_SCALE_FLOATS = 8;                    // per matrix: the four scales, the fp16 switch, padding
+constexpr float CG_HALF_MAX_COND = 1073741824.f;      // 2^30: beyond it a matrix keeps the bf16 three-piece products
 constexpr int CG_COPY_ROWS = 8;                       // rows of W one work group of the copy-in kernel writes
 
 struct CgHeader {
   int64_t magic;
   int64_t total_bytes;
   int64_t ws_floats;
+  int64_t scales_off;       // floats from the workspace base: CG_SCALE_FLOATS per matrix
   int64_t mats_off, steps_off, leaves_off, prods_off, map_off;     // byte offsets of the tables inside the plan
   int32_t count, nsteps, nleaves, nprods;
   int32_t copy_blocks, ntiles;
@@ -79,6 +86,7 @@ struct CgArgs {
   const int* skip;
   int* info;
   int lam_stride, skip_stride;
+  float* scales;                    // ws + scales_off
 };
 
 __device__ __forceinline__ bool cg_skipped(const CgArgs& a, int mat) {
@@ -110,8 +118,11 @@ static __global__ __launch_bounds__(256) void cg_copy_in_kernel(CgArgs a, int co
     const int r = r0 + e;
     if (r >= m.dp) break;
     float* __restrict__ dst = W + static_cast<int64_t>(r) * m.dp;
-    if (r >= m.d) {                                     // identity padding
-      for (int c = threadIdx.x; c <= r; c += 256) dst[c] = (c == r) ? 1.f : 0.f;
+    if (r >= m.d) {
+      // padding: a diagonal block that drops out of the result.  Its value lam (1 when lam <= 0) stays inside the
+      // magnitude bounds the fp16-piece products scale their operands by (lam <= a, 1 / sqrt(lam) for the inverse).
+      const float pad = l > 0.f ? l : 1.f;
+      for (int c = threadIdx.x; c <= r; c += 256) dst[c] = (c == r) ? pad : 0.f;
       continue;
     }
     const float* __restrict__ src = A + static_cast<int64_t>(r) * m.d;
@@ -125,6 +136,46 @@ static __global__ __launch_bounds__(256) void cg_copy_in_kernel(CgArgs a, int co
       for (int c = threadIdx.x; c <= r; c += 256) dst[c] = src[c] + ((c == r) ? l : 0.f);
     }
   }
+}
+
+// Per matrix: the powers of two that bring each kind of operand into the range of fp16 (largest possible magnitude
+// -> (2^13, 2^14]), from a = max_i (A_ii + lam) and lam; and whether the matrix takes the fp16-piece products at
+// all: a > 0, lam > 0 and a / lam <= 2^30 (elements that are much smaller than their kind's bound lose relative, not
+// absolute accuracy; within that ratio the elements that matter keep 22 bits).  One work group per matrix.
+static __global__ __launch_bounds__(256) void cg_scale_kernel(CgArgs a, int count) {
+  __shared__ float red[4];
+  const int m = blockIdx.x;
+  const CgHeader* __restrict__ h = reinterpret_cast<const CgHeader*>(a.plan);
+  const CgMat cm = reinterpret_cast<const CgMat*>(a.plan + h->mats_off)[m];
+  float* __restrict__ sc = a.scales + static_cast<int64_t>(m) * CG_SCALE_FLOATS;
+  float amax = -3.0e38f;
+  const bool live = !cg_skipped(a, m);
+  if (live) {
+    const float* __restrict__ A = a.A_list[m];
+    for (int i = threadIdx.x; i < cm.d; i += 256) amax = fmaxf(amax, A[static_cast<int64_t>(i) * cm.d + i]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float lam = live ? a.lam[static_cast<int64_t>(m) * a.lam_stride] : 0.f;
+  amax += lam;
+  const bool half = live && lam > 0.f && amax > 0.f && amax < 3.0e38f && amax <= CG_HALF_MAX_COND * lam;
+  float s[4] = {1.f, 1.f, 1.f, 1.f};
+  if (half) {
+    const float bound[4] = {amax, sqrtf(amax), 1.f / sqrtf(lam), sqrtf(amax / lam)};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      int e;
+      frexpf(bound[k], &e);              // bound <= 2^e
+      s[k] = ldexpf(1.f, 14 - e);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) sc[k] = s[k];
+  sc[4] = half ? 1.f : 0.f;
 }
 
 // One work group (16 waves) per leaf task of the step.  Every table is read with one load that depends on nothing
@@ -195,7 +246,17 @@ static __global__ __launch_bounds__(256) void cg_prod_kernel(CgArgs a, const CgP
   p.kmode = d.kmode; p.tile_mode = d.tile_mode;
   p.active = nullptr; p.active_stride = 0;
   p.split = 3;
-  gemm_x3_tile<3, false>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+  p.scaleA = p.scaleB = 1.f;
+  const float* __restrict__ sc = a.scales + static_cast<int64_t>(d.mat) * CG_SCALE_FLOATS;
+  if (sc[4] != 0.f) {
+    // fp16 pieces: two per operand element, three matrix instructions per product instead of six
+    p.scaleA = sc[(d.flags >> 4) & 3];
+    p.scaleB = sc[(d.flags >> 6) & 3];
+    p.alpha = d.alpha / (p.scaleA * p.scaleB);      // powers of two: exact
+    gemm_x3_tile<2, false, -1, -1, true>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+  } else {
+    gemm_x3_tile<3, false>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+  }
 }
 
 // ---- host: the plan ------------------------------------------------------------------------------------------
@@ -223,10 +284,11 @@ static int64_t cg_tiles(const CgProd& p) {
   return p.tile_mode == TILE_ALL ? tm * tn : tm * (tm + 1) / 2;
 }
 
-static CgProd cg_prod(int mat, int flags, int M, int N, int K, float alpha, int64_t a, int lda, int64_t b, int ldb,
-                      float beta, int64_t c, int ldc, int kmode, int tile_mode) {
+static CgProd cg_prod(int mat, int flags, int kind_a, int kind_b, int M, int N, int K, float alpha, int64_t a, int lda,
+                      int64_t b, int ldb, float beta, int64_t c, int ldc, int kmode, int tile_mode) {
   CgProd p;
   std::memset(&p, 0, sizeof(p));
+  flags |= (kind_a << 4) | (kind_b << 6);
   p.a_off = a; p.b_off = b; p.c_off = c;
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.M = M; p.N = N; p.K = K;
@@ -257,21 +319,25 @@ static void cg_range(std::vector<CgOp>& ops, int mat, int64_t w, int d, int dp, 
   {
     CgOp op;
     op.type = CG_PROD;      // T1 = A21 M11^T
-    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, s2, s1, s1, 1.f, W21, dp, W11, dp, 0.f, T1, s1, K_LE_J, TILE_ALL));
+    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_W, CG_KIND_M, s2, s1, s1, 1.f, W21, dp, W11, dp, 0.f, T1, s1,
+                               K_LE_J, TILE_ALL));
     ops.push_back(op);
   }
   {
     CgOp op;
     op.type = CG_PROD;      // A22 -= T1 T1^T (lower triangle);  T2 = T1 M11
-    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, s2, s2, s1, -1.f, T1, s1, T1, s1, 1.f, W22, dp, K_FULL, TILE_LOWER));
-    op.prods.push_back(cg_prod(mat, 0, s2, s1, s1, 1.f, T1, s1, W11, dp, 0.f, T2, s1, K_GE_J, TILE_ALL));
+    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_L, CG_KIND_L, s2, s2, s1, -1.f, T1, s1, T1, s1, 1.f, W22, dp,
+                               K_FULL, TILE_LOWER));
+    op.prods.push_back(cg_prod(mat, 0, CG_KIND_L, CG_KIND_M, s2, s1, s1, 1.f, T1, s1, W11, dp, 0.f, T2, s1, K_GE_J,
+                               TILE_ALL));
     ops.push_back(op);
   }
   cg_range(ops, mat, w, d, dp, t1, t2, mid, hi, pool_off + static_cast<int64_t>(s1) * s2);
   {
     CgOp op;
     op.type = CG_PROD;      // M21 = -M22 T2
-    op.prods.push_back(cg_prod(mat, 0, s2, s1, s2, -1.f, W22, dp, T2, s1, 0.f, W21, dp, K_LE_I, TILE_ALL));
+    op.prods.push_back(cg_prod(mat, 0, CG_KIND_M, CG_KIND_T2, s2, s1, s2, -1.f, W22, dp, T2, s1, 0.f, W21, dp, K_LE_I,
+                               TILE_ALL));
     ops.push_back(op);
   }
 }
@@ -310,8 +376,8 @@ static void cg_build(const int64_t* dims, int count, CgPlan& plan) {
     cg_range(seq[m], m, cm.w_off, d, dp, t1, t2, 0, dp, 0);
     CgOp fin;
     fin.type = CG_PROD;     // out = M^T M, both triangles
-    fin.prods.push_back(cg_prod(m, CG_FLAG_TRANSA | CG_FLAG_OUT_USER, d, d, dp, 1.f, cm.w_off, dp, cm.w_off, dp, 0.f, 0, d,
-                                K_GE_MAXIJ, TILE_LOWER_MIRROR));
+    fin.prods.push_back(cg_prod(m, CG_FLAG_TRANSA | CG_FLAG_OUT_USER, CG_KIND_M, CG_KIND_M, d, d, dp, 1.f, cm.w_off, dp,
+                                cm.w_off, dp, 0.f, 0, d, K_GE_MAXIJ, TILE_LOWER_MIRROR));
     seq[m].push_back(fin);
   }
   plan.steps.push_back(CgStep{CG_COPY, 0, count, copy_blocks, 0, 0});
@@ -361,6 +427,8 @@ static void cg_build(const int64_t* dims, int count, CgPlan& plan) {
   CgHeader& h = plan.h;
   std::memset(&h, 0, sizeof(h));
   h.magic = CG_MAGIC;
+  h.scales_off = off;
+  off += cg_align(static_cast<int64_t>(count) * CG_SCALE_FLOATS, 64);
   h.ws_floats = off;
   h.count = count;
   h.nsteps = static_cast<int>(plan.steps.size());
@@ -393,6 +461,7 @@ extern "C" size_t ak_chol_group_ws_bytes(const int64_t* dims, int count) {
     const int64_t dp = (dims[m] + 3) / 4 * 4;
     off += ak::cg_align(dp * dp, 64) + 2 * ak::cg_align(ak::cg_pool(dp), 64);
   }
+  off += ak::cg_align(static_cast<int64_t>(count) * ak::CG_SCALE_FLOATS, 64);
   return static_cast<size_t>(off) * sizeof(float);
 }
 
@@ -447,13 +516,15 @@ extern "C" int ak_chol_inv_grouped(const void* plan_host, const void* plan_dev, 
   a.A_list = A_list; a.out_list = out_list;
   a.lam = lam; a.skip = skip_flags; a.info = info;
   a.lam_stride = lam_stride; a.skip_stride = skip_stride;
+  a.scales = a.ws + h->scales_off;
   const CgStep* steps = reinterpret_cast<const CgStep*>(ph + h->steps_off);
   for (int i = 0; i < h->nsteps; ++i) {
     const CgStep& st = steps[i];
     if (st.grid <= 0) continue;
-    if (st.type == CG_COPY)
+    if (st.type == CG_COPY) {
       hipLaunchKernelGGL(cg_copy_in_kernel, dim3(st.grid), dim3(256), 0, s, a, h->count);
-    else if (st.type == CG_LEAF)
+      hipLaunchKernelGGL(cg_scale_kernel, dim3(h->count), dim3(256), 0, s, a, h->count);
+    } else if (st.type == CG_LEAF)
       hipLaunchKernelGGL(cg_leaf_kernel, dim3(st.grid), dim3(LEAF_THREADS), LEAF_LDS_BYTES, s, a,
                          reinterpret_cast<const CgLeafTask*>(a.plan + h->leaves_off) + st.first);
     else

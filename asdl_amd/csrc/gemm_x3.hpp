@@ -31,6 +31,17 @@ namespace ak {
 typedef uint32_t x3_u32x2 __attribute__((ext_vector_type(2)));
 typedef float x3_f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 x3_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 x3_f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 x3_f16x8 __attribute__((ext_vector_type(8)));
+
+// One matrix instruction on 16-byte fragments that hold bf16 pieces, or (HALF) fp16 pieces.
+template <bool HALF>
+__device__ __forceinline__ floatx16 x3_mfma(bf16x8 a, bf16x8 b, floatx16 c) {
+  if constexpr (HALF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(x3_f16x8, a), __builtin_bit_cast(x3_f16x8, b), c, 0, 0, 0);
+  else
+    return mfma_bf16(a, b, c);
+}
 
 constexpr int X3_BT = 128, X3_BK = 32;
 constexpr int X3_PLANE = X3_BT * X3_BK * 2;      // bytes of one bf16 plane of one operand panel
@@ -90,9 +101,12 @@ __device__ __forceinline__ uint32_t x3_chunk_offset(bool kcontig, int tid, int u
   return (c4 >> 3) * 2048 + krow * 64 + (c4 & 7) * 8;
 }
 
-// Splits the fetched panel into NSPLIT bf16 planes and writes them to the LDS.
-template <int NSPLIT>
-__device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char* panel, bool kcontig, int tid) {
+// Splits the fetched panel into NSPLIT bf16 planes and writes them to the LDS.  HALF: fp16 pieces of scale * x
+// instead (11 significant bits each: two pieces carry 22 bits; `scale`, a power of two, brings the operand into the
+// range of fp16: the caller guarantees |scale * x| <= 2^15 and divides the result by the scales of both operands).
+template <int NSPLIT, bool HALF = false>
+__device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char* panel, bool kcontig, int tid,
+                                         float scale = 1.f) {
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int f = tid + 256 * u;
@@ -111,11 +125,18 @@ __device__ __forceinline__ void x3_stash(const X3Fetch& r, AK_LDS3 unsigned char
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       x3_f32x2 rem = {r.v[u][2 * e], r.v[u][2 * e + 1]};
+      if constexpr (HALF) rem *= scale;
 #pragma unroll
       for (int s = 0; s < NSPLIT; ++s) {
-        const x3_bf16x2 h = __builtin_convertvector(rem, x3_bf16x2);
-        pair[s][e] = __builtin_bit_cast(uint32_t, h);
-        if (s + 1 < NSPLIT) rem -= __builtin_convertvector(h, x3_f32x2);
+        if constexpr (HALF) {
+          const x3_f16x2 h = __builtin_convertvector(rem, x3_f16x2);
+          pair[s][e] = __builtin_bit_cast(uint32_t, h);
+          if (s + 1 < NSPLIT) rem -= __builtin_convertvector(h, x3_f32x2);
+        } else {
+          const x3_bf16x2 h = __builtin_convertvector(rem, x3_bf16x2);
+          pair[s][e] = __builtin_bit_cast(uint32_t, h);
+          if (s + 1 < NSPLIT) rem -= __builtin_convertvector(h, x3_f32x2);
+        }
       }
     }
 #pragma unroll
@@ -143,8 +164,9 @@ __device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bo
 }
 
 // One 128 x 128 tile (ti, tj) of batch entry z of the product described by p.
-template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1>
+template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool HALF = false>
 __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj, int z, AK_LDS3 unsigned char* lds) {
+  static_assert(!HALF || (NSPLIT == 2 && !DB), "fp16 pieces: two of them, single-buffered loop");
   constexpr int BT = X3_BT, BK = X3_BK;
   constexpr int BUF = 2 * NSPLIT * X3_PLANE;        // both operands' planes of one k-tile
   AK_LDS3 unsigned char* panelA = lds;
@@ -200,15 +222,15 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
         for (int b = 0; b < 2; ++b) {
           // smallest terms first
           if constexpr (NSPLIT >= 3) {
-            acc[a][b] = mfma_bf16(fa[a][1], fb[b][1], acc[a][b]);
-            acc[a][b] = mfma_bf16(fa[a][0], fb[b][2], acc[a][b]);
-            acc[a][b] = mfma_bf16(fa[a][2], fb[b][0], acc[a][b]);
+            acc[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], acc[a][b]);
+            acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], acc[a][b]);
+            acc[a][b] = x3_mfma<HALF>(fa[a][2], fb[b][0], acc[a][b]);
           }
           if constexpr (NSPLIT >= 2) {
-            acc[a][b] = mfma_bf16(fa[a][0], fb[b][1], acc[a][b]);
-            acc[a][b] = mfma_bf16(fa[a][1], fb[b][0], acc[a][b]);
+            acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][1], acc[a][b]);
+            acc[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][0], acc[a][b]);
           }
-          acc[a][b] = mfma_bf16(fa[a][0], fb[b][0], acc[a][b]);
+          acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][0], acc[a][b]);
         }
     }
   };
@@ -222,8 +244,8 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
       x3_fetch<INTERIOR>(rb, B, p.ldb, b_kc, j0, p.N, k0, kend, tid);
     };
     auto stash = [&](AK_LDS3 unsigned char* buf) {
-      x3_stash<NSPLIT>(ra, buf, a_kc, tid);
-      x3_stash<NSPLIT>(rb, buf + NSPLIT * X3_PLANE, b_kc, tid);
+      x3_stash<NSPLIT, HALF>(ra, buf, a_kc, tid, p.scaleA);
+      x3_stash<NSPLIT, HALF>(rb, buf + NSPLIT * X3_PLANE, b_kc, tid, p.scaleB);
     };
     if (nk > 0) {
       fetch(0);
@@ -409,6 +431,7 @@ __device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table
   p.tile_mode = (r[9] & 4) ? TILE_LOWER_MIRROR : TILE_ALL;     // symmetric result: lower tiles only, mirrored
   p.active = nullptr; p.active_stride = 0;
   p.split = 0;
+  p.scaleA = p.scaleB = 1.f;
   const int local = w - static_cast<int>(r[11]);
   const int tn = (p.N + X3_BT - 1) / X3_BT;
   ti = local / tn;
