@@ -27,8 +27,9 @@ FACTOR_TIMING_EVERY = 4     # steps between two steps whose factor launches are 
 # Device-memory bytes per factor call (fetched + written, average over the 108 calls of a step) of the default
 # workload, from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) of this script scaled by a plain copy kernel of
 # known size (--traffic-calibration-mib); counters cannot be read from inside the timed run, so the figure is recorded
-# here and reported only for the configuration it was measured on.  Algorithmic bytes of the same calls: 31.7e6.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 74.7e6
+# here, reported only for the configuration it was measured on and marked as such (`traffic_source`).  Algorithmic
+# bytes of the same calls: 31.7e6.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 76.0e6
 
 
 def parse():
@@ -372,6 +373,10 @@ def main():
         traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None
         out['roofline'] = {'bound': 'mfma', 'achieved': achieved, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
                            'frac': achieved / BF16_MFMA_PEAK_TFLOPS, 'traffic': traffic,
+                           'traffic_source': None if traffic is None else
+                           'not measured by this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command '
+                           '(profiles/factor_kernels_resnet50_bs64_hbm_traffic.txt), bytes per factor call',
+                           'floor_ms_per_step': 0.908 if default_workload else None,
                            'kernel': 'factor statistics (syrk_dtl_kernel; conv_patch_syrk_kernel for the 3-channel '
                                      'stem), SYRK FLOP M*d*(d+1)',
                            'launches_per_step': len(sink) // timed_steps,
