@@ -38,7 +38,7 @@ constexpr int CG_FLAG_TRANSA = 1, CG_FLAG_TRANSB = 2, CG_FLAG_OUT_USER = 4;
 // matrix by a, of its Cholesky factor L by sqrt(a), of M = L^-1 by 1 / sqrt(lam), of L21 L11^-1 by sqrt(a / lam).
 constexpr int CG_KIND_W = 0, CG_KIND_L = 1, CG_KIND_M = 2, CG_KIND_T2 = 3;
 constexpr int CG_SCALE_FLOATS = 8;                    // per matrix: the four scales, the fp16 switch, padding
-constexpr float CG_HALF_MAX_COND = 1073741824.f;      // 2^30: beyond it a matrix keeps the bf16 three-piece products
+constexpr float CG_HALF_MAX_COND = 65536.f;           // a / lam beyond 2^16: the matrix keeps the bf16 three-piece products
 constexpr int CG_COPY_ROWS = 8;                       // rows of W one work group of the copy-in kernel writes
 
 struct CgHeader {
@@ -140,8 +140,10 @@ static __global__ __launch_bounds__(256) void cg_copy_in_kernel(CgArgs a, int co
 
 // Per matrix: the powers of two that bring each kind of operand into the range of fp16 (largest possible magnitude
 // -> (2^13, 2^14]), from a = max_i (A_ii + lam) and lam; and whether the matrix takes the fp16-piece products at
-// all: a > 0, lam > 0 and a / lam <= 2^30 (elements that are much smaller than their kind's bound lose relative, not
-// absolute accuracy; within that ratio the elements that matter keep 22 bits).  One work group per matrix.
+// all: a > 0, lam > 0 and a / lam <= 2^16 (elements that are much smaller than their kind's bound lose relative, not
+// absolute accuracy; within that ratio the elements that matter keep 22 bits, and the condition number, at most d a / lam,
+// leaves the two bits the fp16 pieces have less than fp32 to spare before the factorization breaks down).  One work group
+// per matrix.
 static __global__ __launch_bounds__(256) void cg_scale_kernel(CgArgs a, int count) {
   __shared__ float red[4];
   const int m = blockIdx.x;

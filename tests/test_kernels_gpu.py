@@ -8,6 +8,8 @@ an fp64 inverse; preconditioned gradients 1e-3.
 """
 import time
 
+import numpy as np
+
 import pytest
 import torch
 import torch.nn as nn
@@ -378,6 +380,45 @@ def test_chol_inv_grouped_skip_and_info(K):
     info = K.chol_inv_grouped(mats[:2], outs[:2], lam2[:, 1], lam_stride=2).cpu()
     assert info[0] == 0 and info[1] == 0
     assert relerr(outs[1], R.cholesky_inv(mats[1].cpu(), 0.2)) < TOL_INV
+
+
+@pytest.mark.parametrize('scale,lam_rel', [(1e-8, 1e-2), (1e6, 1e-2), (1.0, 1e-4), (1e-3, 3e-5), (1.0, 1e-6), (3e-5, 1e-8), (1.0, 1e-12), (1e4, 0.0)])
+def test_chol_inv_grouped_operand_scaling(K, scale, lam_rel):
+    """The products of the grouped inverse run on fp16 pieces of operands scaled by powers of two that come from the
+    diagonal maximum and the damping; matrices whose bound a / lam exceeds 2^16 (or lam = 0) keep the bf16 three-piece
+    products.  Factors of very different magnitudes (1e-8 ... 1e6) and dampings from 1e-2 down to 1e-12 of the diagonal,
+    full-rank and rank-deficient, against fp64: the error has to stay at the level conditioning allows in fp32
+    (a few eps * cond), and nothing may overflow."""
+    d = 640
+    mats, lams = [], []
+    for rows, seed in ((2 * d, 1), (d // 4, 2)):                 # full rank; rank 160 of 640
+        A = _spd(d, 400 + seed, rows=rows) * scale
+        mats.append(A.cuda())
+        lams.append(lam_rel * float(A.diagonal().max()))
+    lam = torch.tensor(lams, device='cuda')
+    outs = [torch.empty_like(m) for m in mats]
+    print(f'chol_inv_grouped scaling scale={scale} lam_rel={lam_rel}', flush=True)
+    info = K.chol_inv_grouped(mats, outs, lam).cpu()
+    eye = torch.eye(d, dtype=torch.float64, device='cuda')
+    for i, (A, o) in enumerate(zip(mats, outs)):
+        W = A.double() + lams[i] * eye
+        ref = torch.linalg.inv(W)
+        cond = float(torch.linalg.cond(W))
+        try:                                  # what the reference's fp32 Cholesky makes of the same matrix
+            e_ref = relerr(R.cholesky_inv(A.cpu(), lams[i]), ref)
+        except torch.linalg.LinAlgError:
+            e_ref = None
+        if e_ref is None or not np.isfinite(e_ref) or e_ref > 1e-2:
+            # eps * cond >= 1: beyond what fp32 can factor; LAPACK's unblocked potrf may get through with a result
+            # that is wrong in the first digit where the blocked recursion here reports the lost definiteness
+            print(f'  matrix {i}: cond {cond:.1e} is out of reach of fp32 (oracle: {e_ref}; info here {int(info[i])})',
+                  flush=True)
+            continue
+        assert int(info[i]) == 0, (i, cond, int(info[i]), e_ref)
+        assert torch.isfinite(o).all()
+        e = relerr(o, ref)
+        print(f'  matrix {i}: cond {cond:.1e}, relative error {e:.1e} (fp32 oracle {e_ref:.1e})', flush=True)
+        assert e < max(1e-4, 8 * e_ref), (i, cond, e, e_ref)
 
 
 @pytest.mark.parametrize('d', [2048, 2304, 4096, 4608])
