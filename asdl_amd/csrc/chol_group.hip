@@ -38,7 +38,11 @@ constexpr int CG_FLAG_TRANSA = 1, CG_FLAG_TRANSB = 2, CG_FLAG_OUT_USER = 4;
 // matrix by a, of its Cholesky factor L by sqrt(a), of M = L^-1 by 1 / sqrt(lam), of L21 L11^-1 by sqrt(a / lam).
 constexpr int CG_KIND_W = 0, CG_KIND_L = 1, CG_KIND_M = 2, CG_KIND_T2 = 3;
 constexpr int CG_SCALE_FLOATS = 8;                    // per matrix: the four scales, the fp16 switch, padding
+#ifdef AK_TUNING_HOOKS
+static float CG_HALF_MAX_COND = 65536.f;              // tuning builds: ak_debug_set_chol_half_max_cond
+#else
 constexpr float CG_HALF_MAX_COND = 65536.f;           // a / lam beyond 2^16: the matrix keeps the bf16 three-piece products
+#endif
 constexpr int CG_COPY_ROWS = 8;                       // rows of W one work group of the copy-in kernel writes
 
 struct CgHeader {
@@ -144,7 +148,7 @@ static __global__ __launch_bounds__(256) void cg_copy_in_kernel(CgArgs a, int co
 // absolute accuracy; within that ratio the elements that matter keep 22 bits, and the condition number, at most d a / lam,
 // leaves the two bits the fp16 pieces have less than fp32 to spare before the factorization breaks down).  One work group
 // per matrix.
-static __global__ __launch_bounds__(256) void cg_scale_kernel(CgArgs a, int count) {
+static __global__ __launch_bounds__(256) void cg_scale_kernel(CgArgs a, int count, float max_cond) {
   __shared__ float red[4];
   const int m = blockIdx.x;
   const CgHeader* __restrict__ h = reinterpret_cast<const CgHeader*>(a.plan);
@@ -164,7 +168,7 @@ static __global__ __launch_bounds__(256) void cg_scale_kernel(CgArgs a, int coun
   amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   const float lam = live ? a.lam[static_cast<int64_t>(m) * a.lam_stride] : 0.f;
   amax += lam;
-  const bool half = live && lam > 0.f && amax > 0.f && amax < 3.0e38f && amax <= CG_HALF_MAX_COND * lam;
+  const bool half = live && lam > 0.f && amax > 0.f && amax < 3.0e38f && amax <= max_cond * lam;
   float s[4] = {1.f, 1.f, 1.f, 1.f};
   if (half) {
     const float bound[4] = {amax, sqrtf(amax), 1.f / sqrtf(lam), sqrtf(amax / lam)};
@@ -525,7 +529,7 @@ extern "C" int ak_chol_inv_grouped(const void* plan_host, const void* plan_dev, 
     if (st.grid <= 0) continue;
     if (st.type == CG_COPY) {
       hipLaunchKernelGGL(cg_copy_in_kernel, dim3(st.grid), dim3(256), 0, s, a, h->count);
-      hipLaunchKernelGGL(cg_scale_kernel, dim3(h->count), dim3(256), 0, s, a, h->count);
+      hipLaunchKernelGGL(cg_scale_kernel, dim3(h->count), dim3(256), 0, s, a, h->count, CG_HALF_MAX_COND);
     } else if (st.type == CG_LEAF)
       hipLaunchKernelGGL(cg_leaf_kernel, dim3(st.grid), dim3(LEAF_THREADS), LEAF_LDS_BYTES, s, a,
                          reinterpret_cast<const CgLeafTask*>(a.plan + h->leaves_off) + st.first);
@@ -536,3 +540,8 @@ extern "C" int ak_chol_inv_grouped(const void* plan_host, const void* plan_dev, 
   }
   return check_launch();
 }
+
+#ifdef AK_TUNING_HOOKS
+// Tuning builds only: the bound a / lam up to which a matrix takes the fp16-piece products (0: never).
+extern "C" void ak_debug_set_chol_half_max_cond(float v) { ak::CG_HALF_MAX_COND = v; }
+#endif

@@ -6,9 +6,11 @@
 //           (oy*sh - ph + ky, ox*sw - pw + kx), zeros outside the image.  The kernel works in the
 //           column order (c/G, ky, kx, c%G) for a group size G (a multiple of 8 dividing C): 8 consecutive
 //           columns are 16 contiguous bytes of x.  The epilogue applies the permutation to the (c,ky,kx)
-//           order of the dense factor, which stays inside blocks of G*kh*kw columns.  G = C makes the
-//           gathered rows longest (best for the loads), G = 8 keeps a tile's writes within a few cache
-//           lines (best for large factors, whose epilogue would otherwise scatter 4-byte writes).
+//           order of the dense factor, which stays inside blocks of G*kh*kw columns.  A column block of a
+//           panel is 32 columns wide, so any G that is a multiple of 32 gives the loads the same 64 contiguous
+//           bytes per row; the smaller G, the fewer cache lines the permuted 4-byte writes of a tile row are
+//           spread over (G = 32: 18 lines, two thirds of each filled by one tile; measured 3-11 % faster than
+//           G = 128).  G = 8 for the largest factors, whose direct epilogue writes 85 MB.
 //
 // One work group owns one BT x BT tile of the upper triangle and, with split-K, a slice of the M rows.
 // A k-tile is 32 rows.  Per k-tile and panel the LDS holds BT/32 column blocks, each [32 rows][32 cols]
@@ -639,7 +641,7 @@ extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C,
   p.kw = kw; p.KK = kh * kw; p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw;
   p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
   p.mWo = ak::make_magic(p.Wo); p.mHo = ak::make_magic(p.Ho); p.mKw = ak::make_magic(kw);
-  p.G = ak::g_force_group > 0 && p.Cin % ak::g_force_group == 0 ? ak::g_force_group : (d >= 3456 ? 8 : (p.Cin % 128 == 0 ? 128 : p.Cin));
+  p.G = ak::g_force_group > 0 && p.Cin % ak::g_force_group == 0 ? ak::g_force_group : (d >= 3456 ? 8 : (p.Cin % 32 == 0 ? 32 : p.Cin));
   p.mBlk = ak::make_magic(p.G * p.KK); p.mG = ak::make_magic(p.G);
   const ak::DtlPlan pl = ak::dtl_plan(M, d, INT64_MAX, true);
   return ak::dtl_launch<true>(p, pl, ws, ws_bytes, static_cast<hipStream_t>(stream));
