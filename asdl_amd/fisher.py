@@ -24,6 +24,10 @@ _invalid_data_size = -1
 FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (ordering the two streams costs ~30 us of host time per hook: more than the overlap gains)
 PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
 EAGER_INVERSE = True        # start the bulk of the inverses during a single sampled / empirical backward pass: the longest chains get a head start
+EAGER_INVERSE_SAMPLED = False   # ... also when a loss backward pass follows the sampled one.  That pass hides the
+                                # inverses anyway, and one grouped inverse for all factors after the sampled pass is
+                                # faster than an early batch plus a remainder (ResNet-50 batch 64: 27.55 against
+                                # 27.96-28.50 ms per step in one process)
 
 
 @dataclass
@@ -128,7 +132,8 @@ class FisherMaker(GradientMaker):
             if damping is not None:
                 cxt.set_damping(damping)
             cxt.set_cov_scale(scale)
-            if inv_with_fisher and self.single_backward_pass and EAGER_INVERSE:
+            if inv_with_fisher and self.single_backward_pass and EAGER_INVERSE and \
+                    (EAGER_INVERSE_SAMPLED or not loss_grad_after_fisher):
                 # every B factor is final when its hook has run: the bulk of the inverses may start behind
                 # the backward pass that is still producing the others
                 cxt.set_eager_inverse(getattr(self, '_inverse_cost_prev', 0))

@@ -384,10 +384,12 @@ def test_resnet50_batch64_channels_last_properties():
     assert relerr(got, ref) < 1e-3, relerr(got, ref)
 
 
-def test_benchmark_path_resnet50_batch64_against_a_sequential_replay():
+@pytest.mark.parametrize('early_batch', [False, True])
+def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch, monkeypatch):
     """The very code path bench.py times, at its size: ResNet-50, batch 64, channels-last, bf16 autocast, sampled
-    (MC) Fisher without EMA, inverses started from inside the backward hooks (fisher.EAGER_INVERSE) on side
-    streams fed by worker threads, the grouped preconditioning plan prepared before the flags are read.  On the
+    (MC) Fisher without EMA, the grouped inverse on a side stream fed by a worker thread beside the loss backward pass
+    (and, with ``early_batch``, a first batch started from inside the hooks of the sampled pass:
+    fisher.EAGER_INVERSE_SAMPLED), the grouped preconditioning plan prepared before the flags are read.  On the
     third step (the eager path needs the cost of an earlier step) extra hooks capture, for every Conv2d / Linear,
     the activation and the output gradient the factor kernels read, and the raw gradient of the loss.  Afterwards
     the same tensors go through the same operations one module after the other on the current stream, with one
@@ -399,6 +401,7 @@ def test_benchmark_path_resnet50_batch64_against_a_sequential_replay():
     from asdl_amd.core import no_centered_cov
     from asdl_amd.matrices import SHAPE_KRON
     assert fisher_mod.EAGER_INVERSE and ng_mod.GROUPED_PRECONDITION and ng_mod.PREPARE_PRECONDITION_EARLY
+    monkeypatch.setattr(fisher_mod, 'EAGER_INVERSE_SAMPLED', early_batch)
     torch.manual_seed(12)
     bs, damping = 64, 1e-3
     model = bench_models.resnet50().cuda().to(memory_format=torch.channels_last)
