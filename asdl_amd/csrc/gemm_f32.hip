@@ -77,6 +77,46 @@ static __global__ __launch_bounds__(256) void weight_layout_grouped_kernel(const
   }
 }
 
+// Largest magnitudes of many strided vectors in one launch.  `table`: one row of 5 int64 per vector: address, number
+// of elements, element stride, address of the float word the maximum is folded into (integer atomic maximum on the
+// bit pattern; the caller zeroes the words first), first block (blocks of ABSMAX_BLOCK elements, numbered in table order).
+constexpr int ABSMAX_BLOCK = 8192;
+
+static __global__ __launch_bounds__(256) void absmax_grouped_kernel(const int64_t* __restrict__ table, int count) {
+  __shared__ float red[4];
+  const int w = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[static_cast<int64_t>(mid) * 5 + 4] <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * 5;
+  const float* __restrict__ x = reinterpret_cast<const float*>(r[0]);
+  const int64_t n = r[1], stride = r[2];
+  const int64_t i0 = static_cast<int64_t>(w - r[4]) * ABSMAX_BLOCK;
+  const int64_t i1 = i0 + ABSMAX_BLOCK < n ? i0 + ABSMAX_BLOCK : n;
+  float m = 0.f;
+  if (stride == 1 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const int64_t iv = i0 + ((i1 - i0) & ~static_cast<int64_t>(3));      // i0 is a multiple of 4
+    for (int64_t i = i0 + 4 * threadIdx.x; i < iv; i += 1024) {
+      const floatx4 v = *reinterpret_cast<const floatx4*>(x + i);
+      m = fmaxf(fmaxf(m, fmaxf(fabsf(v[0]), fabsf(v[1]))), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    }
+    for (int64_t i = iv + threadIdx.x; i < i1; i += 256) m = fmaxf(m, fabsf(x[i]));      // the ragged end of the vector
+  } else {
+    for (int64_t i = i0 + threadIdx.x; i < i1; i += 256) m = fmaxf(m, fabsf(x[i * stride]));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    atomicMax(reinterpret_cast<unsigned int*>(r[3]), __builtin_bit_cast(unsigned int, m));
+  }
+}
+
 static __global__ void copy_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t n) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = src[i];
@@ -217,7 +257,7 @@ extern "C" int ak_kron_precond_static(const float* Binv, const float* Ainv, floa
 
 extern "C" int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t total_tiles,
                                    ak_stream_t stream) {
-  if (pieces != 0 && pieces != 2 && pieces != 3) return AK_ERR_ARG;
+  if (pieces != 0 && pieces != 2 && pieces != 3 && pieces != 22) return AK_ERR_ARG;
   if (count < 0 || total_tiles < 0 || total_tiles > (1ll << 30)) return AK_ERR_ARG;
   if (count == 0 || total_tiles == 0) return AK_OK;
   if (table == nullptr) return AK_ERR_ARG;
@@ -225,6 +265,7 @@ extern "C" int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, 
   const dim3 grid(static_cast<unsigned>(total_tiles));
   if (pieces == 0) hipLaunchKernelGGL(ak::gemm_f32_grouped_kernel, grid, dim3(256), 0, s, table, count);
   else if (pieces == 2) hipLaunchKernelGGL(ak::gemm_x3_grouped_kernel<2>, grid, dim3(256), 0, s, table, count);
+  else if (pieces == 22) hipLaunchKernelGGL((ak::gemm_x3_grouped_kernel<2, true>), grid, dim3(256), 0, s, table, count);
   else hipLaunchKernelGGL(ak::gemm_x3_grouped_kernel<3>, grid, dim3(256), 0, s, table, count);
   return ak::check_launch();
 }
@@ -236,6 +277,17 @@ extern "C" int ak_gemv_f32_grouped(const int64_t* table, int count, int64_t tota
   if (table == nullptr) return AK_ERR_ARG;
   hipLaunchKernelGGL(ak::gemv_grouped_kernel, dim3(static_cast<unsigned>(total_blocks)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), table, count, alpha);
+  return ak::check_launch();
+}
+
+extern "C" int64_t ak_absmax_block(void) { return ak::ABSMAX_BLOCK; }
+
+extern "C" int ak_absmax_grouped(const int64_t* table, int count, int64_t total_blocks, ak_stream_t stream) {
+  if (count < 0 || total_blocks < 0 || total_blocks > (1ll << 30)) return AK_ERR_ARG;
+  if (count == 0 || total_blocks == 0) return AK_OK;
+  if (table == nullptr) return AK_ERR_ARG;
+  hipLaunchKernelGGL(ak::absmax_grouped_kernel, dim3(static_cast<unsigned>(total_blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), table, count);
   return ak::check_launch();
 }
 

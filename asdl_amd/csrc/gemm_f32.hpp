@@ -40,6 +40,8 @@ struct GemmParams {
   int active_stride;
   int split;                // 0: fp32 MFMA; 2 / 3: bf16 MFMA on operands split into that many bf16 pieces (gemm_x3.hpp)
   float scaleA, scaleB;     // fp16-piece variant only: powers of two the operands are multiplied by before the split
+  float* absmax_out;        // optional (split kernels): max |C| of the result is folded into this word with an integer
+                            // atomic maximum on its bit pattern (the caller zeroes it first)
 };
 
 constexpr int GBT = 128, GBK = 16;     // GBT: granularity of the triangular contraction ranges (both tile sizes)
@@ -266,6 +268,7 @@ inline GemmParams make_gemm(int transA, int transB, int M, int N, int K, float a
   p.alpha = alpha; p.beta = beta;
   p.kmode = K_FULL; p.tile_mode = TILE_ALL;
   p.scaleA = p.scaleB = 1.f;
+  p.absmax_out = nullptr;
   p.active = nullptr; p.active_stride = 0;
   p.split = 0;
   return p;

@@ -369,6 +369,7 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][b][r] *= p.alpha;
   }
+  float vmax = 0.f;
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -381,10 +382,17 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
         if (gi >= p.M) continue;
         if (lower_only && gi < gj) continue;
         const float v = acc[a][b][r];
+        vmax = fmaxf(vmax, fabsf(v));
         C[static_cast<int64_t>(gi) * p.ldc + gj] = v;
         if (mirror && gi != gj) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
       }
     }
+  if (p.absmax_out != nullptr) {
+    // non-negative floats order like their bit patterns; NaN (a larger pattern than any number) propagates
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, o));
+    if (lane == 0) atomicMax(reinterpret_cast<unsigned int*>(p.absmax_out), __builtin_bit_cast(unsigned int, vmax));
+  }
 }
 
 template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1>
@@ -403,19 +411,26 @@ static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
 // `table` holds one row of GROUPED_ROW int64 per product: A, B, C, lda, ldb, ldc, M, N, K,
 // transA | transB << 1 | symmetric << 2 (symmetric: M == N and the result is known to be symmetric, only the tiles
 // on and below the diagonal are computed and mirrored), alpha and beta (float bits in the low and high word),
-// first tile.  Tiles are numbered row-major inside a product, products in table order (longest
+// first tile, then three optional addresses of float words: the largest magnitude in A, in B (from which the fp16-piece
+// kernel takes its operand scales; required there) and where to fold the largest magnitude of the result (any split
+// kernel), one spare.  Tiles are numbered row-major inside a product, products in table order (longest
 // contraction first gives the best balance); work group w looks its product up by bisection on `first tile`.
-constexpr int GROUPED_ROW = 12;
+constexpr int GROUPED_ROW = 16;
 
 // Product and tile of work group w of a grouped launch; false for a tile the table overstates.
-__device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table, int count, int w, GemmParams& p,
-                                               int& ti, int& tj) {
+__device__ __forceinline__ int grouped_row_of(const int64_t* __restrict__ table, int count, int w) {
   int lo = 0, hi = count - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
     if (table[static_cast<int64_t>(mid) * GROUPED_ROW + 11] <= w) lo = mid;
     else hi = mid - 1;
   }
+  return lo;
+}
+
+__device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table, int count, int w, GemmParams& p,
+                                               int& ti, int& tj) {
+  const int lo = grouped_row_of(table, count, w);
   const int64_t* __restrict__ r = table + static_cast<int64_t>(lo) * GROUPED_ROW;
   p.A = reinterpret_cast<const float*>(r[0]);
   p.B = reinterpret_cast<const float*>(r[1]);
@@ -432,6 +447,7 @@ __device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table
   p.active = nullptr; p.active_stride = 0;
   p.split = 0;
   p.scaleA = p.scaleB = 1.f;
+  p.absmax_out = reinterpret_cast<float*>(r[14]);
   const int local = w - static_cast<int>(r[11]);
   const int tn = (p.N + X3_BT - 1) / X3_BT;
   ti = local / tn;
@@ -439,15 +455,30 @@ __device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table
   return ti * X3_BT < p.M;
 }
 
-template <int NSPLIT>
+// The power of two that brings magnitudes up to `absmax` into (2^13, 2^14] (1 for zero, infinite or NaN input).
+__device__ __forceinline__ float x3_half_scale(float absmax) {
+  if (!(absmax > 0.f) || !(absmax < 3.0e38f)) return 1.f;
+  int e;
+  frexpf(absmax, &e);                  // absmax <= 2^e
+  return ldexpf(1.f, 14 - e);
+}
+
+template <int NSPLIT, bool HALF = false>
 static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
   __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
   GemmParams p;
   int ti, tj;
   if (!grouped_lookup(table, count, blockIdx.x, p, ti, tj)) return;
+  if constexpr (HALF) {
+    // fp16 pieces: the operands' largest magnitudes (device words named by the table row) give the scales
+    const int64_t* __restrict__ r = table + static_cast<int64_t>(grouped_row_of(table, count, blockIdx.x)) * GROUPED_ROW;
+    p.scaleA = x3_half_scale(*reinterpret_cast<const float*>(r[12]));
+    p.scaleB = x3_half_scale(*reinterpret_cast<const float*>(r[13]));
+    p.alpha = p.alpha / (p.scaleA * p.scaleB);       // powers of two: exact
+  }
   // two work groups per CU with the single-buffered loop serve the mix of long and short contractions of a
   // grouped launch better than one work group with the double-buffered loop (measured: 0.99 against 1.25 ms)
-  gemm_x3_tile<NSPLIT, false>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+  gemm_x3_tile<NSPLIT, false, -1, -1, HALF>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // The same with true fp32 products (v_mfma_f32_32x32x2_f32, one accumulation per k): 128 x 128 tiles as above.

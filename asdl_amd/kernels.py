@@ -852,13 +852,16 @@ def _grouped_operand_ok(ptr, ld, contiguous_extent):
 
 def _gemm_grouped_table(specs, device):
     """(device table, rows, tiles) for ak_gemm_f32_grouped.  specs: tuples (a_ptr, lda, b_ptr, ldb, c_ptr, ldc, M, N, K,
-    transA, transB, alpha[, beta[, symmetric]]) of device addresses of float32 matrices with contiguous rows;
-    C <- alpha * op(A) op(B) + beta * C; symmetric: only the lower tiles are computed, and mirrored."""
+    transA, transB, alpha[, beta[, symmetric[, absmax_a, absmax_b, absmax_c]]]) of device addresses of float32 matrices
+    with contiguous rows; C <- alpha * op(A) op(B) + beta * C; symmetric: only the lower tiles are computed, and
+    mirrored; absmax_*: addresses of float words (0: none) holding the operands' largest magnitudes (pieces = 22) and
+    receiving the result's."""
     rows, first = [], 0
     for spec in sorted(specs, key=lambda sp: -sp[8]):
         a, lda, b, ldb, c, ldc, M, N, K, tA, tB, alpha = spec[:12]
         beta = spec[12] if len(spec) > 12 else 0.0
         symmetric = bool(spec[13]) if len(spec) > 13 else False
+        max_a, max_b, max_c = spec[14:17] if len(spec) > 16 else (0, 0, 0)
         if M <= 0 or N <= 0 or K <= 0:
             continue
         if symmetric and M != N:
@@ -869,7 +872,7 @@ def _gemm_grouped_table(specs, device):
         if lda < (M if tA else K) or ldb < (K if tB else N) or ldc < N:
             raise ValueError('leading dimension smaller than the row length')
         rows.append((a, b, c, lda, ldb, ldc, M, N, K, int(bool(tA)) | (int(bool(tB)) << 1) | (int(symmetric) << 2),
-                     _float_bits(alpha) | (_float_bits(beta) << 32), first))
+                     _float_bits(alpha) | (_float_bits(beta) << 32), first, max_a, max_b, max_c, 0))
         first += ((M + 127) // 128) * ((N + 127) // 128)
     if not rows:
         return None, 0, 0
@@ -930,6 +933,10 @@ def kron_precond_groupable(B_inv, A_inv, grad_w, grad_b=None):
     return dB % 4 == 0 and dA % 4 == 0 and all(t.data_ptr() % 16 == 0 for t in (B_inv, A_inv, grad_w))
 
 
+HALF_PIECE_PRECONDITION = True     # grouped preconditioning on two fp16 pieces per element (3 matrix instructions per
+                                   # product instead of the 6 of the bf16 three-piece split); False: three bf16 pieces
+
+
 class KronPrecondPlan:
     """kron_precond for many modules in a handful of launches: all B_inv @ G, then all (.) @ A_inv, then all
     B_inv @ bias; channels-last convolution gradients are gathered into the contiguous layout before and
@@ -978,6 +985,24 @@ class KronPrecondPlan:
             # the inverses are symmetric: reading A_inv as its transpose makes both operands contiguous along k
             second.append((t, dA, A_inv.data_ptr(), dA, g_ptr, dA, dB, dA, dA, 0, 1, self.grad_scale))
         self._layout = (device_table(tuple(layout), dev), len(layout), layout_rows) if layout else None
+        self._half = bool(HALF_PIECE_PRECONDITION)
+        if self._half:
+            # Operand ranges for the fp16 pieces, per module: the largest magnitude of B_inv and of A_inv is their largest
+            # diagonal element (symmetric positive definite), that of the gradient is measured by one pass over it, that
+            # of the intermediate B_inv G by the first product's own epilogue.
+            block = _lib.load().ak_absmax_block()
+            self._mx = torch.zeros(len(self.items), 4, dtype=torch.float32, device=dev)
+            mx = self._mx.data_ptr()
+            rows, blocks = [], 0
+            for i, ((B_inv, A_inv, g, _), f1, f2) in enumerate(zip(self.items, first, second)):
+                dB, dA = B_inv.shape[0], A_inv.shape[0]
+                for ptr, n, stride, slot in ((B_inv.data_ptr(), dB, dB + 1, 0), (f1[2], dB * dA, 1, 1),
+                                             (A_inv.data_ptr(), dA, dA + 1, 2)):
+                    rows.append((ptr, n, stride, mx + 16 * i + 4 * slot, blocks))
+                    blocks += (n + block - 1) // block
+                first[i] = f1 + (0.0, False, mx + 16 * i, mx + 16 * i + 4, mx + 16 * i + 12)
+                second[i] = f2 + (0.0, False, mx + 16 * i + 12, mx + 16 * i + 8, 0)
+            self._absmax = (device_table(tuple(rows), dev), len(rows), blocks)
         self._first = _gemm_grouped_table(first, dev)
         self._second = _gemm_grouped_table(second, dev)
         rows, blocks, self._tmps, self._biases = [], 0, [], []
@@ -1009,10 +1034,19 @@ class KronPrecondPlan:
         if not self.items:
             return
         self._convert_layout(1)
-        # all 24 mantissa bits: the terms of these sums cancel (entries of the inverses reach 1/damping), and what
+        # 22 to 24 mantissa bits: the terms of these sums cancel (entries of the inverses reach 1/damping), and what
         # a shorter split loses relative to the terms shows up magnified in the result
-        _launch_gemm_grouped(*self._first, 3)
-        _launch_gemm_grouped(*self._second, 3)
+        if self._half:
+            with _on_launch_stream():
+                self._mx.zero_()
+            table, count, blocks = self._absmax
+            rc = _lib.load().ak_absmax_grouped(ctypes.c_void_p(table.data_ptr()), count, blocks, _stream())
+            _lib.check(rc, 'ak_absmax_grouped')
+            _launch_gemm_grouped(*self._first, 22)
+            _launch_gemm_grouped(*self._second, 22)
+        else:
+            _launch_gemm_grouped(*self._first, 3)
+            _launch_gemm_grouped(*self._second, 3)
         self._convert_layout(0)
         if self._gemv is not None:
             table, count, blocks = self._gemv

@@ -305,7 +305,7 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         """Collects every Kronecker-factored module whose operands the grouped kernels take into one
         kernels.KronPrecondPlan (B_inv G for every module, (.) A_inv for every module, B_inv bias: a handful of
         launches, same arithmetic per module as Kron.mvp(use_inv=True, inplace=True)).  Returns
-        (plan, rest of ``work`` for the per-module path, signature) or None when fewer than two modules qualify;
+        (plan, rest of ``work`` for the per-module path, signature) or None when no module qualifies;
         the signature lists the objects the plan was built from."""
         items, unit_items, rest, signature = [], [], [], []
         for module, shape in work:
@@ -336,8 +336,8 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
                 rest.append((module, shape))
             else:
                 items.append(item)
-        if len(items) + len(unit_items) < 2:
-            return None
+        if len(items) + len(unit_items) < (1 if kernels.HALF_PIECE_PRECONDITION else 2):
+            return None      # (a single module still gains from the grouped form's fp16-piece products)
         return kernels.KronPrecondPlan(items, grad_scale, unit_items), rest, signature
 
     def prepare_precondition(self):

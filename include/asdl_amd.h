@@ -245,9 +245,14 @@ int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, 
 
 /* Many products of different sizes in one launch: C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i on the bf16
  * matrix cores (pieces = 2 or 3 as in ak_gemm_f32_split) or with true fp32 products (pieces = 0, the fp32 MFMA, one
- * accumulation per k; needs no alignment).  `table` is DEVICE memory, `count` rows of 12 int64:
+ * accumulation per k; needs no alignment), or on two fp16 pieces per element (pieces = 22: 22 significant bits, three
+ * partial products; each operand is multiplied by the power of two that brings its largest magnitude, read from the
+ * float word absmax_A / absmax_B names, into (2^13, 2^14]).  `table` is DEVICE memory, `count` rows of 16 int64:
  *   A, B, C (addresses), lda, ldb, ldc, M, N, K, transA | transB << 1 | symmetric << 2, alpha and beta (float
- *   bit patterns in the low and the high 32 bits), first_tile
+ *   bit patterns in the low and the high 32 bits), first_tile, absmax_A, absmax_B, absmax_C, 0
+ * (absmax_A, absmax_B: addresses of float words, required for pieces = 22, ignored otherwise; absmax_C: 0 or the
+ * address of a float word into which the split kernels fold max |C_i| by an integer atomic maximum on the bit pattern:
+ * zero it first)
  * (symmetric: M == N and op(A) op(B) is symmetric, e.g. G G^T: only the tiles on and below the diagonal are
  * computed and mirrored, the result is exactly symmetric)
  * with first_tile the running sum of ceil(M/128) * ceil(N/128) over the rows before, and total_tiles that sum
@@ -263,6 +268,15 @@ int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t tot
 /* y_i <- alpha * M_i x_i for dense row-major [n_i, n_i] fp32 matrices, one launch.  `table` is DEVICE memory,
  * `count` rows of 5 int64: M, x, y (addresses, y not aliasing x), n, first_block, with first_block the running
  * sum of ceil(n/4).  The bias half of Kron.mvp (asdl/symmatrix.py:543-546) for all modules at once. */
+/* Largest magnitudes of `count` strided fp32 vectors in one launch (the operand ranges the fp16-piece grouped products
+ * scale by).  table: device array of 5 int64 per vector: address, number of elements, element stride (d + 1 walks the
+ * diagonal of a [d, d] matrix: for a symmetric positive definite matrix that is its largest magnitude), address of the
+ * float word the maximum is folded into (integer atomic maximum on the bit pattern: zero the words first), first block;
+ * blocks of ak_absmax_block() elements are numbered in table order, total_blocks of them.  No counterpart in the
+ * reference. */
+int64_t ak_absmax_block(void);
+int ak_absmax_grouped(const int64_t* table, int count, int64_t total_blocks, ak_stream_t stream);
+
 int ak_gemv_f32_grouped(const int64_t* table, int count, int64_t total_blocks, float alpha, ak_stream_t stream);
 
 /* Convolution weight gradients of many modules between the channels-last layout [Cout][kh*kw][Cin] and the

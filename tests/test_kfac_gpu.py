@@ -464,10 +464,18 @@ def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch
         assert eA < 1e-5 and eB < 1e-5, (name, eA, eB)
         g_w = raw[(name, 'weight')] / bs
         g_b = raw[(name, 'bias')] / bs if m.bias is not None else None
+        exact = kron.B_inv.double() @ g_w.double().reshape(kron.B_inv.shape[0], -1) @ kron.A_inv.double()
         kron.mvp(vec_weight=g_w, vec_bias=g_b, use_inv=True, inplace=True)
         e = relerr(got[name][2]['weight'], g_w)
         worst['weight'] = max(worst['weight'], e)
-        assert e < 1e-5, (name, 'weight', e)
+        # The grouped path multiplies two fp16 pieces per element (22 bits), the per-module path three bf16 pieces
+        # (24 bits); the sums cancel (entries of the inverses reach 1 / damping), most in the classifier, whose A factor
+        # has rank 64 of 2048: both are compared with the fp64 product of the very same inverses as well.
+        e_grouped = relerr(got[name][2]['weight'].reshape(exact.shape), exact)
+        e_single = relerr(g_w.reshape(exact.shape), exact)
+        worst['weight vs fp64 (grouped)'] = max(worst.get('weight vs fp64 (grouped)', 0.0), e_grouped)
+        worst['weight vs fp64 (per module)'] = max(worst.get('weight vs fp64 (per module)', 0.0), e_single)
+        assert e < 1e-4 and e_grouped < 1e-4 and e_single < 1e-4, (name, 'weight', e, e_grouped, e_single)
         if g_b is not None:
             e = relerr(got[name][2]['bias'], g_b)
             worst['bias'] = max(worst['bias'], e)
