@@ -890,6 +890,20 @@ def gemm_grouped_raw(specs, device, pieces=3):
     _launch_gemm_grouped(*_gemm_grouped_table(specs, device), pieces)
 
 
+def absmax_grouped(vectors, device):
+    """vectors: (address, elements, element stride, address of the float word that receives max |x|); one launch.  The
+    words have to be zero before (the maxima are folded in with an atomic maximum)."""
+    block = _lib.load().ak_absmax_block()
+    rows, blocks = [], 0
+    for ptr, n, stride, out in vectors:
+        rows.append((ptr, n, stride, out, blocks))
+        blocks += (n + block - 1) // block
+    if rows:
+        table = device_table(tuple(rows), device)
+        _lib.check(_lib.load().ak_absmax_grouped(ctypes.c_void_p(table.data_ptr()), len(rows), blocks, _stream()),
+                   'ak_absmax_grouped')
+
+
 def gemm_grouped(problems, pieces=3):
     """problems: (A, B, C, transA, transB, alpha) with 2-D float32 tensors whose rows are contiguous;
     C <- alpha * op(A) @ op(B) for all of them in one launch."""

@@ -100,6 +100,7 @@ def _axis_statistic(grad, axis, out, alpha, beta):
         kernels.syrk_nt(grad.movedim(axis, 0).reshape(grad.shape[axis], -1).contiguous(), out=out, alpha=alpha, beta=beta)
 
 
+HALF_PIECE_PRECONDITION = True     # grouped preconditioning on two fp16 pieces per element (kernels.KronPrecondPlan does the same)
 GROUPED_PRECONDITION = True      # matrix-shaped parameters: all their preconditioning products in two launches
 GROUPED_STATISTIC_MIN_DIM = 1024  # statistics of this size and up go into one grouped launch (with GROUPED_PRECONDITION)
 
@@ -339,14 +340,29 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
             dev = grouped[0].param.device
             buf, _ = kernels.workspace(4 * sum(pc.param.numel() for pc in grouped), dev)
             base = buf.data_ptr()
-            for pc in grouped:
+            half = HALF_PIECE_PRECONDITION
+            if half:
+                # operand ranges for the fp16 pieces: the roots are symmetric positive definite (largest magnitude on
+                # the diagonal), the gradients are measured, the intermediate by the first product's epilogue
+                mx = torch.zeros(len(grouped), 4, dtype=torch.float32, device=dev)
+                vectors = []
+            for i, pc in enumerate(grouped):
                 m, n = pc._transformed_shape
                 g, t = pc.param.grad.data_ptr(), base + 4 * off
                 off += m * n
+                p0, p1 = pc.preconditioners[0].data_ptr(), pc.preconditioners[1].data_ptr()
                 # T[n, m] = G^T P_0, then G[m, n] <- T^T P_1
-                specs_first.append((g, n, pc.preconditioners[0].data_ptr(), m, t, m, n, m, m, 1, 0, 1.0))
-                specs_second.append((t, m, pc.preconditioners[1].data_ptr(), n, g, n, m, n, n, 1, 0, 1.0))
-            kernels.gemm_grouped_raw(specs_first, dev, pieces=3)
-            kernels.gemm_grouped_raw(specs_second, dev, pieces=3)
+                first, second = (g, n, p0, m, t, m, n, m, m, 1, 0, 1.0), (t, m, p1, n, g, n, m, n, n, 1, 0, 1.0)
+                if half:
+                    w = mx.data_ptr() + 16 * i
+                    vectors += [(g, m * n, 1, w), (p0, m, m + 1, w + 4), (p1, n, n + 1, w + 8)]
+                    first += (0.0, False, w, w + 4, w + 12)
+                    second += (0.0, False, w + 12, w + 8, 0)
+                specs_first.append(first)
+                specs_second.append(second)
+            if half:
+                kernels.absmax_grouped(vectors, dev)
+            kernels.gemm_grouped_raw(specs_first, dev, pieces=22 if half else 3)
+            kernels.gemm_grouped_raw(specs_second, dev, pieces=22 if half else 3)
         for preconditioner in rest:
             preconditioner.precondition()
