@@ -347,6 +347,8 @@ def test_shampoo_gpt2_small_weight_shapes_full_size():
         for stat, root, ref in zip(prec.statistics, prec.preconditioners, acc):
             lam_max = float(torch.linalg.eigvalsh(ref)[-1])
             ridge = float((stat.double() - ref).diagonal().mean())      # the root computation leaves its ridge behind
+            print(f'  n={stat.shape[0]}: ridge read back from the diagonal off by {abs(ridge - 1e-6 * lam_max) / (1e-6 * lam_max):.3f} of it',
+                  flush=True)
             assert abs(ridge - 1e-6 * lam_max) < 0.1 * 1e-6 * lam_max
             exact = _closed_form_root(stat, 4)
             assert exact is not None and relerr(root, exact) < 5e-3, relerr(root, exact)
