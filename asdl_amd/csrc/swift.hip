@@ -147,6 +147,9 @@ extern "C" int ak_conv_patch_sum(const void* x, int dtype, int64_t sn, int64_t s
     const int64_t chunks = vec8 ? C / 8 : C;
     int cch = 1;
     while (cch < 256 && cch < chunks) cch *= 2;          // power of two <= 256 covering the chunks
+    // few taps and samples (a 1 x 1 window at batch 64: 64 work groups): narrower channel ranges per work group, down
+    // to 4 chunks = 64 contiguous bytes per position, until the grid fills the device
+    while (cch > 4 && static_cast<int64_t>(kh) * kw * N * ((chunks + cch - 1) / cch) < 1024) cch /= 2;
     const int64_t zblocks = (chunks + cch - 1) / cch;
     if (zblocks > 65535 || N > 65535) return AK_ERR_UNSUPPORTED;
     dim3 grid(kh * kw, static_cast<unsigned>(N), static_cast<unsigned>(zblocks));
