@@ -103,11 +103,21 @@ def test_grad_maker_matches_vanilla_autograd_for_every_calling_style():
 
     for flip, idx in [(False, 1), (True, 0)]:
         model.zero_grad(set_to_none=True)
-        dummy_y = gm.setup_model_call(model, x, targets=t, flip=flip)
-        gm._loss_fn = None
-        gm.setup_loss_repr(dummy_y[idx])
-        y, loss = gm.forward_and_backward()
+        gm_repr = GradientMaker(model)
+        dummy_y = gm_repr.setup_model_call(model, x, targets=t, flip=flip)
+        gm_repr.setup_loss_repr(dummy_y[idx])
+        y, loss = gm_repr.forward_and_backward()
         check(loss)
+        # a registered loss function wins over a loss expression (asdl/grad_maker.py:272-281)
+        gm_repr.setup_loss_call(lambda out: out[idx] * 2, dummy_y)
+        assert torch.allclose(gm_repr.forward_and_backward()[1], ref_loss * 2)
+
+    # delegation: the other maker runs what was registered here, results land in both
+    model.zero_grad(set_to_none=True)
+    other = GradientMaker(model)
+    y, loss = gm.delegate_forward_and_backward(other)
+    check(loss)
+    assert other.loss is gm.loss and other.model_output is gm.model_output
 
     with pytest.raises(TypeError):
         gm.setup_loss_repr('not a dummy')
@@ -120,6 +130,32 @@ def test_dummy_object_replays_attribute_item_and_call():
     assert asdl_amd.DummyObject().weight[0].numel().eval(lin) == 5
     d = asdl_amd.DummyObject()
     assert d['a'][1].eval({'a': [1, 2]}) == 2
+    # placeholders among the arguments of a recorded call are evaluated on the same base value
+    base = {'f': lambda a, b=0: 10 * a + b, 'x': 3, 'y': 4}
+    assert d['f'](d['x'], b=d['y']).eval(base) == 34
+    assert d['a'].eval({'a': 1}) == 1 and d.eval(7) == 7        # d itself was not changed by the longer paths
+
+
+def test_loss_reduction_override_for_functions_and_modules():
+    """A maker that names a reduction passes it as a keyword to loss functions and sets (then restores) the
+    attribute of loss modules; a loss without the option is refused (asdl/grad_maker.py:283-300)."""
+    class Summed(GradientMaker):
+        _loss_reduction = 'sum'
+
+    torch.manual_seed(0)
+    model = _Net()
+    x, t = torch.randn(4, 5), torch.randint(4, (4,))
+    expected = F.cross_entropy(model(x), t, reduction='sum')
+    gm = Summed(model)
+    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t, reduction='mean')
+    torch.testing.assert_close(gm.forward_and_backward()[1], expected)
+    crit = nn.CrossEntropyLoss()
+    gm.setup_loss_call(crit, gm.setup_model_call(model, x), t)
+    torch.testing.assert_close(gm.forward_and_backward()[1], expected)
+    assert crit.reduction == 'mean'
+    gm.setup_loss_call(lambda y, t: F.cross_entropy(y, t), gm.setup_model_call(model, x), t)
+    with pytest.raises(AttributeError):
+        gm.forward_and_backward()
 
 
 # ------------------------------------------------------------------ schedules
@@ -130,6 +166,22 @@ def test_update_schedule_and_intervals():
     assert s[:2] == [True, True] and sum(s) == 5
     assert get_update_schedule(4, 1.0) == [True] * 4
     assert get_update_schedule(6, 0.5, interval_type='step') == [True] * 3 + [False] * 3
+    # vectors worked out by hand from asdl/precondition/prec_grad_maker.py:204-254
+    T_, F_ = True, False
+    assert get_update_schedule(10, 0.5) == [T_, F_] * 5
+    assert get_update_schedule(10, 0.3) == [T_, F_, F_, T_, F_, F_, T_, F_, F_, F_]      # the 4th multiple of 3 is over budget
+    assert get_update_schedule(10, 0.5, 0.2) == [T_, T_, T_, F_, T_, F_, T_, F_, F_, F_]
+    assert get_update_schedule(10, 0.5, 0.2, reverse=True) == [T_, T_, T_, F_, T_, F_, T_, F_, F_, F_][::-1]
+    linear = get_update_schedule(20, 0.25, interval_type='linear')         # gaps 0, 2, 4, 6
+    assert [i for i, f in enumerate(linear) if f] == [0, 1, 4, 9, 16] and len(linear) == 20
+    with pytest.raises(ValueError):
+        get_update_schedule(10, 0.5, interval_type='linear')               # gaps 0, 1, 2, 3 end at step 11 of 10
+    with pytest.raises(ZeroDivisionError):
+        get_update_schedule(10, 0.2, interval_type='linear')               # two updates: n (n - 1) = 0
+    with pytest.raises(ValueError):
+        get_update_schedule(10, 0.2, warmup_ratio=0.5)
+    with pytest.raises(ValueError):
+        get_update_schedule(10, 0.5, interval_type='quadratic')
     with pytest.raises(ValueError):
         get_update_schedule(0)
     with pytest.raises(ValueError):
@@ -145,6 +197,29 @@ def test_update_schedule_and_intervals():
                                                              preconditioner_upd_ratio=0.5))
     with pytest.warns(UserWarning):
         assert gm2.do_update_preconditioner(10) is False
+    assert gm2.preconditioner_upd_schedule == [True, False, True, False] and gm2.curvature_upd_schedule is None
+    assert [gm2.do_update_curvature(s) for s in range(4)] == [True, False, True, False]      # follows the preconditioner
+    with pytest.warns(UserWarning):                      # a known horizon overrides the interval
+        gm3 = KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1, num_total_steps=4, ema_decay=0.1,
+                                                                 preconditioner_upd_interval=2, curvature_upd_ratio=1.,
+                                                                 preconditioner_upd_ratio=0.5))
+    assert gm3.curvature_upd_schedule == [True] * 4 and gm3.do_update_curvature(1) and not gm3.do_update_preconditioner(1)
+    gm4 = KfacGradientMaker(get_mlp(), PreconditioningConfig(data_size=1, preconditioner_upd_interval=4,
+                                                             preconditioner_warmup_steps=3))
+    assert [gm4.do_update_preconditioner(s) for s in range(9)] == [True] * 4 + [False] * 3 + [True, False]
+
+
+def test_module_selection_by_ignore_list_and_trainability():
+    model = nn.Sequential(nn.Linear(3, 3), nn.ReLU(), nn.Linear(3, 3), nn.Sequential(nn.Linear(3, 2)), nn.Linear(2, 2))
+    for p in model[4].parameters():
+        p.requires_grad_(False)
+    keys = lambda **kw: list(KfacGradientMaker(model, PreconditioningConfig(data_size=1, **kw)).module_dict.keys())
+    assert keys() == ['0', '2', '3/0']                           # leaves with trainable parameters, '/' for '.'
+    assert keys(ignore_modules=[model[0]]) == ['2', '3/0']
+    assert keys(ignore_modules=['3.']) == ['0', '2']
+    model_c = nn.Sequential(nn.Linear(3, 3), nn.Conv1d(3, 3, 1))
+    with pytest.warns(UserWarning):
+        assert list(KfacGradientMaker(model_c, PreconditioningConfig(data_size=1)).module_dict.keys()) == ['0']
 
 
 def test_config_defaults_match_reference():
