@@ -90,6 +90,34 @@ __device__ __forceinline__ void dtl_epilogue(floatx16 (&acc)[FR][FC], const DtlP
     syrk_epilogue<FR, FC>(acc, p.C, p.ldc, p.d, gi0, gj0, diag_tile, p.alpha, p.beta, lane);
   } else {
     const int g = lane >> 5, l32 = lane & 31;
+    // First acc <- alpha * acc + beta * C, then the stores, so that no read of C waits behind a store to C.  The
+    // reads are unconditional (clamped positions) and issued a 32 x 32 block's 16 at a time: under a per-element
+    // condition each gets a wait of its own and pays one memory latency.
+#pragma unroll
+    for (int a = 0; a < FR; ++a)
+#pragma unroll
+      for (int b = 0; b < FC; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] *= p.alpha;
+    if (p.beta != 0.f) {
+#pragma unroll
+      for (int b = 0; b < FC; ++b) {
+        const int64_t gj = gj0 + 32 * b + l32;
+        const int64_t oj = out_index<true>(gj < p.d ? gj : p.d - 1, p);
+#pragma unroll
+        for (int a = 0; a < FR; ++a) {
+          float c[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int64_t gi = gi0 + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3);
+            c[r] = p.C[out_index<true>(gi < p.d ? gi : p.d - 1, p) * p.ldc + oj];
+          }
+          __builtin_amdgcn_sched_barrier(0);      // keeps the multiply-adds (and their waits) below all the loads
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[a][b][r] += p.beta * c[r];
+        }
+      }
+    }
 #pragma unroll
     for (int b = 0; b < FC; ++b) {
       const int64_t gj = gj0 + 32 * b + l32;
@@ -104,10 +132,8 @@ __device__ __forceinline__ void dtl_epilogue(floatx16 (&acc)[FR][FC], const DtlP
           for (int e = 0; e < 4; ++e) {
             if (gi + e >= p.d) continue;
             const int64_t oi = out_index<true>(gi + e, p);
-            float v = p.alpha * acc[a][b][4 * q + e];
-            float* dst = p.C + oi * p.ldc + oj;
-            if (p.beta != 0.f) v += p.beta * *dst;
-            *dst = v;
+            const float v = acc[a][b][4 * q + e];
+            p.C[oi * p.ldc + oj] = v;
             if (!diag_tile) p.C[oj * p.ldc + oi] = v;
           }
         }
@@ -384,15 +410,22 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_kernel(DtlPara
   const int64_t gi = static_cast<int64_t>(ti) * BT + 32 * FR * wr + 32 * a + 8 * q + 4 * g;
   if (gj >= p.d) return;
   const int64_t oj = out_index<GATHER>(gj, p);
+  int64_t oi[4];
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {                    // rows beyond d are clamped for the reads and skipped by the stores
+    oi[e] = out_index<GATHER>(gi + e < p.d ? gi + e : p.d - 1, p);
+    v[e] = p.alpha * acc[e];
+  }
+  if (p.beta != 0.f) {                             // all reads of C before any store to it, none under a condition
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] += p.beta * p.C[oi[e] * p.ldc + oj];
+  }
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     if (gi + e >= p.d) continue;
-    const int64_t oi = out_index<GATHER>(gi + e, p);
-    float v = p.alpha * acc[e];
-    float* dst = p.C + oi * p.ldc + oj;
-    if (p.beta != 0.f) v += p.beta * *dst;
-    *dst = v;
-    if (ti != tj) p.C[oj * p.ldc + oi] = v;
+    p.C[oi[e] * p.ldc + oj] = v[e];
+    if (ti != tj) p.C[oj * p.ldc + oi[e]] = v[e];
   }
 }
 
