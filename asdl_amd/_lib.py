@@ -30,6 +30,9 @@ _SIGNATURES = {
     'ak_conv_syrk_nhwc_ws_bytes': (c_size, [c_i64, c_i64, c_i64, c_i64, c_int, c_int, c_int, c_int, c_int, c_int]),
     'ak_conv_syrk_nhwc': (c_int, [c_ptr, c_int, c_i64, c_i64, c_i64, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_f32, c_f32, c_ptr, c_i64, c_ptr, c_size, c_ptr]),
+    'ak_syrk_group_eligible': (c_int, [c_ptr]),
+    'ak_syrk_group_sizes': (c_int, [c_ptr, c_int, c_ptr, c_ptr]),
+    'ak_syrk_group_launch': (c_int, [c_ptr, c_int, c_ptr, c_ptr, c_size, c_ptr, c_size, c_ptr]),
     'ak_kron_damping': (c_int, [c_ptr, c_ptr, c_ptr, c_int, c_f32, c_f32, c_ptr, c_ptr, c_ptr]),
     'ak_chol_inv_ws_bytes': (c_size, [c_i64, c_int]),
     'ak_chol_inv_batched': (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_size, c_ptr]),

@@ -32,13 +32,13 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
     def stream_cxt():
         return torch.cuda.stream(stream) if use_stream else nullcontext()
 
-    def run_hook(fn, *tensors):
+    def run_hook(fn, *tensors, backward=False):
         fs = cxt.factor_stream
         if fs is None or not tensors[0].is_cuda:
             with stream_cxt():
                 fn()
             return
-        fs.run(fn, *tensors)
+        fs.run(fn, *tensors, backward=backward)
 
     try:
         for module, names in module_wise_assignments(model, *op_names, ignore_modules=ignore_modules, map_rule=map_rule):
@@ -62,7 +62,7 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
                         if not cxt.is_operation_registered(_m):
                             return None          # context already closed
                         g = grad.detach()
-                        run_hook(lambda: cxt.call_operations_in_backward(_m, g), g)
+                        run_hook(lambda: cxt.call_operations_in_backward(_m, g), g, backward=True)
                         return None
                     handles.append(out_data.register_hook(grad_hook))
                     # the graph edge the hook sits on: a backward pass restricted to these edges still fires

@@ -22,10 +22,13 @@
 // hand-over between waves with one barrier per k-tile.  Rows and columns outside the matrix (or taps
 // outside the image) are given a byte offset beyond the buffer range, for which the hardware returns
 // zeros, so the main loop has no masks and no branches.
+#include <algorithm>
 #include <cmath>
+#include <cstring>
 #include <initializer_list>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 #include <type_traits>
 #include "common.hpp"
 
@@ -156,8 +159,20 @@ struct DtlCfg {
   static_assert(NCB * (kDtlBK / 16) % NW == 0 && IPW >= 1, "loads must split evenly over the waves");
 };
 
+// Work groups go to the 8 XCDs round-robin by their linear index, and each XCD has its own L2.  Renumbering them so
+// that one XCD gets a contiguous range of work items lets the tiles of one split share the rows they read through
+// one L2 instead of fetching them once per XCD.
+__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t wgid, uint32_t nwg) {
+  const uint32_t xcd = wgid & 7, local = wgid >> 3, q = nwg >> 3, rem = nwg & 7;
+  return xcd * q + (xcd < rem ? xcd : rem) + local;
+}
+
+// Rows [k_begin, k_begin + rows) of the operand into tile (ti, tj) of one factor.  partial == nullptr: the result is
+// the factor's tile (alpha, beta, mirror image); otherwise the accumulators go to `partial` in accumulator order,
+// [(a, b, q)][thread] float4, for a reduction pass.
 template <int WR, int WC, int FR, int FC, bool GATHER>
-__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
+__device__ __forceinline__ void dtl_tile(const DtlParams& p, int ti, int tj, int64_t k_begin, int rows,
+                                         floatx4* __restrict__ partial) {
   using Cfg = DtlCfg<WR, WC, FR, FC, GATHER>;
   constexpr int NW = Cfg::NW, BT = Cfg::BT, NCB = Cfg::NCB, IPW = Cfg::IPW, BK = kDtlBK, S = kDtlStages;
   extern __shared__ __attribute__((aligned(1024))) unsigned char dtl_smem[];
@@ -167,25 +182,8 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = wave / WC, wc = wave % WC;
-  int ti, tj;
-  // Work groups go to the 8 XCDs round-robin by their linear index, and each XCD has its own L2.  Renumber them so
-  // that one XCD gets a contiguous range of (split, tile) pairs: the tiles of one split then share the rows they
-  // read through one L2 instead of fetching them once per XCD.
-  uint32_t tile_id, split_id;
-  {
-    const uint32_t nwg = gridDim.x * gridDim.y, wgid = blockIdx.x + blockIdx.y * gridDim.x;
-    const uint32_t xcd = wgid & 7, local = wgid >> 3, q = nwg >> 3, rem = nwg & 7;
-    const uint32_t logical = xcd * q + (xcd < rem ? xcd : rem) + local;
-    split_id = logical / gridDim.x;
-    tile_id = logical - split_id * gridDim.x;
-  }
-  decode_upper_tile(tile_id, p.T, ti, tj);
   const bool diag = (ti == tj);
   const int64_t i0 = static_cast<int64_t>(ti) * BT, j0 = static_cast<int64_t>(tj) * BT;
-  const int64_t k_begin = static_cast<int64_t>(split_id) * p.rows_per_split;
-  int64_t k_end = k_begin + p.rows_per_split;
-  if (k_end > p.M) k_end = p.M;
-  const int rows = k_begin < k_end ? static_cast<int>(k_end - k_begin) : 0;
   const int nk = (rows + BK - 1) / BK;
 
   // buffer descriptor: plain mode is based at this split's first row, gather mode at the tensor
@@ -344,12 +342,9 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
   else mainloop(std::false_type{});
 
   const int64_t gi0 = i0 + 32 * FR * wr, gj0 = j0 + 32 * FC * wc;
-  if (p.nsplit == 1) {
+  if (partial == nullptr) {
     dtl_epilogue<FR, FC, GATHER>(acc, p, gi0, gj0, diag, lane);
   } else {
-    // partial tile in accumulator order: [(a,b,q)][thread] float4
-    floatx4* dst = reinterpret_cast<floatx4*>(p.ws) +
-                   (static_cast<size_t>(split_id) * gridDim.x + tile_id) * (BT * BT / 4);
 #pragma unroll
     for (int a = 0; a < FR; ++a)
 #pragma unroll
@@ -357,9 +352,50 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           floatx4 w = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]};
-          dst[((a * FC + b) * 4 + q) * (NW * 64) + tid] = w;
+          partial[((a * FC + b) * 4 + q) * (NW * 64) + tid] = w;
         }
   }
+}
+
+// One factor per launch: grid (upper tiles, splits).
+template <int WR, int WC, int FR, int FC, bool GATHER>
+__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_kernel(DtlParams p) {
+  constexpr int BT = DtlCfg<WR, WC, FR, FC, GATHER>::BT;
+  const uint32_t logical = xcd_contiguous_id(blockIdx.x + blockIdx.y * gridDim.x, gridDim.x * gridDim.y);
+  const uint32_t split_id = logical / gridDim.x, tile_id = logical - split_id * gridDim.x;
+  int ti, tj;
+  decode_upper_tile(tile_id, p.T, ti, tj);
+  const int64_t k_begin = static_cast<int64_t>(split_id) * p.rows_per_split;
+  int64_t k_end = k_begin + p.rows_per_split;
+  if (k_end > p.M) k_end = p.M;
+  const int rows = k_begin < k_end ? static_cast<int>(k_end - k_begin) : 0;
+  floatx4* partial = nullptr;
+  if (p.nsplit > 1)
+    partial = reinterpret_cast<floatx4*>(p.ws) + (static_cast<size_t>(split_id) * gridDim.x + tile_id) * (BT * BT / 4);
+  dtl_tile<WR, WC, FR, FC, GATHER>(p, ti, tj, k_begin, rows, partial);
+}
+
+// Many factors per launch.  Work item w (device table): a tile of a factor and a range of its rows.  The items of
+// one (factor, split) are adjacent, so the renumbering above still gives them one L2.
+struct DtlGroupItem {
+  int32_t factor, tile;
+  int32_t k_begin_tile, k_tiles;   // in k-tiles of kDtlBK rows
+  int64_t partial;                 // float4 index into the workspace, or -1: this item is the whole sum
+};
+
+template <int WR, int WC, int FR, int FC, bool GATHER>
+__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_grouped_kernel(const DtlParams* __restrict__ factors,
+                                                                        const DtlGroupItem* __restrict__ items,
+                                                                        floatx4* __restrict__ ws) {
+  const DtlGroupItem it = items[xcd_contiguous_id(blockIdx.x, gridDim.x)];
+  const DtlParams p = factors[it.factor];
+  int ti, tj;
+  decode_upper_tile(it.tile, p.T, ti, tj);
+  const int64_t k_begin = static_cast<int64_t>(it.k_begin_tile) * kDtlBK;
+  int64_t k_end = k_begin + static_cast<int64_t>(it.k_tiles) * kDtlBK;
+  if (k_end > p.M) k_end = p.M;
+  const int rows = k_begin < k_end ? static_cast<int>(k_end - k_begin) : 0;
+  dtl_tile<WR, WC, FR, FC, GATHER>(p, ti, tj, k_begin, rows, it.partial >= 0 ? ws + it.partial : nullptr);
 }
 
 // Split-K reduction, first stage (only for many splits): work group (tile, slot, g) sums partials
@@ -383,21 +419,16 @@ __global__ __launch_bounds__(NT) void syrk_dtl_reduce_kernel(const floatx4* __re
   dst[off + blockIdx.z * split_stride] = acc;
 }
 
-// Sums the (remaining) partials in a fixed order and applies the epilogue.  grid (tiles, 4*FR*FC): each work
-// group owns one float4 slot (a, b, q) of every thread's accumulators.
+// Sums n partial tiles (split_stride float4 apart) of tile (ti, tj) in a fixed order and applies the epilogue; one
+// work group per float4 slot (a, b, q) of every thread's accumulators.
 template <int WR, int WC, int FR, int FC, bool GATHER>
-__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_kernel(DtlParams p, const floatx4* __restrict__ part,
-                                                                         int n) {
+__device__ __forceinline__ void dtl_finalize_slot(const DtlParams& p, int ti, int tj, int slot,
+                                                  const floatx4* __restrict__ tile_part, size_t split_stride, int n) {
   constexpr int NW = WR * WC, BT = 32 * FR * WR;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave / WC, wc = wave % WC, g = lane >> 5, l32 = lane & 31;
-  int ti, tj;
-  decode_upper_tile(blockIdx.x, p.T, ti, tj);
-  const int slot = blockIdx.y;                     // (a * FC + b) * 4 + q
   const int q = slot & 3, b = (slot >> 2) % FC, a = (slot >> 2) / FC;
-  const size_t tile_f4 = BT * BT / 4;
-  const floatx4* src = part + blockIdx.x * tile_f4 + slot * (NW * 64) + tid;
-  const size_t split_stride = static_cast<size_t>(gridDim.x) * tile_f4;
+  const floatx4* src = tile_part + slot * (NW * 64) + tid;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   int s = 0;
   for (; s + 4 <= n; s += 4) {
@@ -427,6 +458,36 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_kernel(DtlPara
     p.C[oi[e] * p.ldc + oj] = v[e];
     if (ti != tj) p.C[oj * p.ldc + oi[e]] = v[e];
   }
+}
+
+// grid (tiles, 4*FR*FC)
+template <int WR, int WC, int FR, int FC, bool GATHER>
+__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_kernel(DtlParams p, const floatx4* __restrict__ part,
+                                                                         int n) {
+  constexpr int BT = 32 * FR * WR;
+  int ti, tj;
+  decode_upper_tile(blockIdx.x, p.T, ti, tj);
+  const size_t tile_f4 = BT * BT / 4;
+  dtl_finalize_slot<WR, WC, FR, FC, GATHER>(p, ti, tj, blockIdx.y, part + blockIdx.x * tile_f4,
+                                            static_cast<size_t>(gridDim.x) * tile_f4, n);
+}
+
+// The reduction pass of a grouped launch: grid (split tiles of all factors, 4*FR*FC).
+struct DtlGroupFin {
+  int32_t factor, tile, nparts, pad;
+  int64_t first, stride;           // float4 index of the first partial of the tile, distance to the next one
+};
+
+template <int WR, int WC, int FR, int FC, bool GATHER>
+__global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_grouped_kernel(const DtlParams* __restrict__ factors,
+                                                                                 const DtlGroupFin* __restrict__ fins,
+                                                                                 const floatx4* __restrict__ ws) {
+  const DtlGroupFin it = fins[blockIdx.x];
+  const DtlParams p = factors[it.factor];
+  int ti, tj;
+  decode_upper_tile(it.tile, p.T, ti, tj);
+  dtl_finalize_slot<WR, WC, FR, FC, GATHER>(p, ti, tj, blockIdx.y, ws + it.first, static_cast<size_t>(it.stride),
+                                            it.nparts);
 }
 
 // ---- host side ------------------------------------------------------------------------------------
@@ -625,7 +686,252 @@ static bool nhwc_ok(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, i
   return true;
 }
 
+// Gather geometry of a channels-last convolution input; false when the direct-to-LDS kernel cannot read it (16-byte
+// chunks must not straddle taps, offsets must fit the 32-bit buffer range, and the magic divisions by Wo, Ho, C and
+// kw must be exact over their operand ranges).
+static bool dtl_gather_params(DtlParams& p, const void* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw,
+                              int sh, int sw, int ph, int pw, int64_t Ho, int64_t Wo) {
+  const int64_t d = C * kh * kw, M = N * Ho * Wo;
+  if (C % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return false;
+  if (N * H * W * C * 2 > static_cast<int64_t>(kDtlRange)) return false;
+  if (M * (Wo > Ho ? Wo : Ho) >= (1ll << 32) || (d + 256) * d >= (1ll << 32)) return false;
+  p.X = x; p.M = M; p.d = d;
+  p.Cin = static_cast<int>(C); p.H = static_cast<int>(H); p.W = static_cast<int>(W);
+  p.kw = kw; p.KK = kh * kw; p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw;
+  p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
+  p.mWo = make_magic(p.Wo); p.mHo = make_magic(p.Ho); p.mKw = make_magic(kw);
+  p.G = g_force_group > 0 && p.Cin % g_force_group == 0 ? g_force_group : (d >= 3456 ? 8 : (p.Cin % 32 == 0 ? 32 : p.Cin));
+  p.mBlk = make_magic(p.G * p.KK); p.mG = make_magic(p.G);
+  return true;
+}
+
+// ---- many factors in one launch ---------------------------------------------------------------------------------
+// The factors of a whole forward or backward pass are small launches when taken one by one: a few tiles, split
+// along the rows to fill the device, each paying its ramp, its tail, its partial tiles and a reduction launch.
+// Taken together they fill the device with long work items: one launch per tile class, few splits, one reduction
+// launch per class.  A factor is described by kGroupSpecInts int64:
+//   [0] kind (0: X^T X of a bf16 [M, d] matrix, 1: unfolded channels-last bf16 [N, C, H, W] input)
+//   [1] operand address  [2] result address (fp32 [d, d])  [3] ldc  [4] alpha bits | beta bits << 32
+//   kind 0: [5] M  [6] d  [7] ldx          kind 1: [5] N  [6] C  [7] H  [8] W  [9] kh  [10] kw  [11..14] sh sw ph pw
+constexpr int kGroupSpecInts = 16;
+constexpr int kGroupClasses = 4;           // plain 128 / 192, gathered 128 / 192
+constexpr int kGroupMaxSplits = 32;
+
+struct GroupFactor {
+  DtlParams p;
+  int cls, bt;
+  int64_t ktiles, ntiles, kt_split, part_base;   // part_base: float4 index of this factor's partial tiles
+  int nsplit;
+};
+
+static int group_class(bool gather, int64_t d, int& bt) {
+  if (!gather) { bt = d >= 1536 ? 192 : 128; return bt == 128 ? 0 : 1; }
+  bt = d >= 576 ? 192 : 128;
+  return bt == 128 ? 2 : 3;
+}
+
+static bool group_decode(const int64_t* r, GroupFactor& f, int64_t& max_rows_per_split) {
+  DtlParams& p = f.p;
+  p = DtlParams{};
+  const void* x = reinterpret_cast<const void*>(r[1]);
+  p.C = reinterpret_cast<float*>(r[2]);
+  p.ldc = r[3];
+  const uint32_t abits = static_cast<uint32_t>(r[4] & 0xffffffffll), bbits = static_cast<uint32_t>(r[4] >> 32);
+  std::memcpy(&p.alpha, &abits, 4);
+  std::memcpy(&p.beta, &bbits, 4);
+  if (x == nullptr || p.C == nullptr) return false;
+  bool gather;
+  if (r[0] == 0) {
+    const int64_t M = r[5], d = r[6], ldx = r[7];
+    if (M <= 0 || d <= 0 || ldx < d || p.ldc < d || !syrk_dtl_plain_ok(x, M, d, ldx)) return false;
+    p.X = x; p.M = M; p.d = d;
+    p.row_bytes = static_cast<uint32_t>(ldx * 2);
+    p.Cin = 1; p.KK = 1;
+    max_rows_per_split = plain_max_rows(ldx);
+    gather = false;
+  } else if (r[0] == 1) {
+    const int64_t N = r[5], C = r[6], H = r[7], W = r[8];
+    const int kh = static_cast<int>(r[9]), kw = static_cast<int>(r[10]), sh = static_cast<int>(r[11]),
+              sw = static_cast<int>(r[12]), ph = static_cast<int>(r[13]), pw = static_cast<int>(r[14]);
+    int64_t Ho, Wo;
+    if (!nhwc_ok(x, N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return false;
+    if (conv_patch_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw) > 0) return false;     // the window kernel's case
+    if (p.ldc < C * kh * kw) return false;
+    if (!dtl_gather_params(p, x, N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return false;
+    // the widest factors fill the device on their own, with the 256-wide tile of 8 waves, whose register budget
+    // has no room for a descriptor read from memory
+    if (p.d >= 3456) return false;
+    max_rows_per_split = INT64_MAX;
+    gather = true;
+  } else {
+    return false;
+  }
+  f.cls = group_class(gather, p.d, f.bt);
+  p.T = static_cast<int>((p.d + f.bt - 1) / f.bt);
+  f.ntiles = static_cast<int64_t>(p.T) * (p.T + 1) / 2;
+  f.ktiles = (p.M + kDtlBK - 1) / kDtlBK;
+  return true;
+}
+
+struct GroupPlan {
+  std::vector<GroupFactor> factors;
+  std::vector<DtlGroupItem> items[kGroupClasses];
+  std::vector<DtlGroupFin> fins[kGroupClasses];
+  size_t ws_f4 = 0;                       // partial tiles, in float4
+  size_t off_factors = 0, off_items[kGroupClasses], off_fins[kGroupClasses], table_bytes = 0;
+};
+
+static int group_plan(const int64_t* specs, int n, GroupPlan& g) {
+  if (specs == nullptr || n <= 0) return AK_ERR_ARG;
+  g.factors.resize(n);
+  std::vector<int64_t> max_rows(n);
+  int64_t work[kGroupClasses] = {0, 0, 0, 0};
+  for (int i = 0; i < n; ++i) {
+    if (!group_decode(specs + static_cast<size_t>(i) * kGroupSpecInts, g.factors[i], max_rows[i])) return AK_ERR_UNSUPPORTED;
+    for (int j = 0; j < i; ++j)           // two items writing one result would race
+      if (g.factors[j].p.C == g.factors[i].p.C) return AK_ERR_ARG;
+    work[g.factors[i].cls] += g.factors[i].ntiles * g.factors[i].ktiles;
+  }
+  size_t ws_f4 = 0;
+  for (int c = 0; c < kGroupClasses; ++c) {
+    if (work[c] == 0) continue;
+    const int bt = (c == 0 || c == 2) ? 128 : 192;
+    const int64_t slots = 256 * (bt == 128 ? 2 : 1);
+    // about four items per slot of the device, none shorter than 32 k-tiles unless its factor is
+    int64_t chunk = (work[c] + slots * 4 - 1) / (slots * 4);
+    if (chunk < 32) chunk = 32;
+    std::vector<int> order;
+    for (int i = 0; i < n; ++i) {
+      GroupFactor& f = g.factors[i];
+      if (f.cls != c) continue;
+      int64_t ns = (f.ktiles + chunk - 1) / chunk;
+      if (ns > kGroupMaxSplits) ns = kGroupMaxSplits;
+      const int64_t max_kt = max_rows[i] / kDtlBK;
+      if (max_kt < 1) return AK_ERR_UNSUPPORTED;
+      if ((f.ktiles + ns - 1) / ns > max_kt) ns = (f.ktiles + max_kt - 1) / max_kt;
+      f.kt_split = (f.ktiles + ns - 1) / ns;
+      f.nsplit = static_cast<int>((f.ktiles + f.kt_split - 1) / f.kt_split);
+      f.p.nsplit = f.nsplit;
+      f.p.rows_per_split = f.kt_split * kDtlBK;
+      f.part_base = -1;
+      if (f.nsplit > 1) {
+        f.part_base = static_cast<int64_t>(ws_f4);
+        ws_f4 += static_cast<size_t>(f.nsplit) * f.ntiles * (static_cast<size_t>(bt) * bt / 4);
+      }
+      order.push_back(i);
+    }
+    // the longest items first: the short ones fill the tail
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int a, int b) { return g.factors[a].kt_split > g.factors[b].kt_split; });
+    const int64_t tile_f4 = static_cast<int64_t>(bt) * bt / 4;
+    for (int i : order) {
+      const GroupFactor& f = g.factors[i];
+      for (int s = 0; s < f.nsplit; ++s)
+        for (int64_t t = 0; t < f.ntiles; ++t) {
+          DtlGroupItem it;
+          it.factor = i;
+          it.tile = static_cast<int32_t>(t);
+          it.k_begin_tile = static_cast<int32_t>(s * f.kt_split);
+          it.k_tiles = static_cast<int32_t>(f.kt_split);
+          it.partial = f.nsplit > 1 ? f.part_base + (static_cast<int64_t>(s) * f.ntiles + t) * tile_f4 : -1;
+          g.items[c].push_back(it);
+        }
+      if (f.nsplit > 1)
+        for (int64_t t = 0; t < f.ntiles; ++t) {
+          DtlGroupFin fin;
+          fin.factor = i;
+          fin.tile = static_cast<int32_t>(t);
+          fin.nparts = f.nsplit;
+          fin.pad = 0;
+          fin.first = f.part_base + t * tile_f4;
+          fin.stride = f.ntiles * tile_f4;
+          g.fins[c].push_back(fin);
+        }
+    }
+  }
+  g.ws_f4 = ws_f4;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t at = off; off += (bytes + 255) & ~static_cast<size_t>(255); return at; };
+  g.off_factors = take(sizeof(DtlParams) * n);
+  for (int c = 0; c < kGroupClasses; ++c) {
+    g.off_items[c] = take(sizeof(DtlGroupItem) * g.items[c].size());
+    g.off_fins[c] = take(sizeof(DtlGroupFin) * g.fins[c].size());
+  }
+  g.table_bytes = off;
+  return AK_OK;
+}
+
+template <int WR, int WC, int FR, int FC, bool GATHER>
+static int group_launch_class(const GroupPlan& g, int c, const unsigned char* tables, floatx4* ws, hipStream_t stream) {
+  using Cfg = DtlCfg<WR, WC, FR, FC, GATHER>;
+  if (g.items[c].empty()) return AK_OK;
+  auto kern = syrk_dtl_grouped_kernel<WR, WC, FR, FC, GATHER>;
+  if (Cfg::LDS_BYTES > 64 * 1024) {
+    static bool attr_set = false;     // idempotent; a race sets it twice at worst
+    if (!attr_set) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              Cfg::LDS_BYTES) != hipSuccess)
+        return AK_ERR_LAUNCH;
+      attr_set = true;
+    }
+  }
+  const DtlParams* factors = reinterpret_cast<const DtlParams*>(tables + g.off_factors);
+  const DtlGroupItem* items = reinterpret_cast<const DtlGroupItem*>(tables + g.off_items[c]);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(g.items[c].size())), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, stream,
+                     factors, items, ws);
+  if (!g.fins[c].empty()) {
+    const DtlGroupFin* fins = reinterpret_cast<const DtlGroupFin*>(tables + g.off_fins[c]);
+    hipLaunchKernelGGL((syrk_dtl_finalize_grouped_kernel<WR, WC, FR, FC, GATHER>),
+                       dim3(static_cast<unsigned>(g.fins[c].size()), 4 * FR * FC), dim3(Cfg::NW * 64), 0, stream, factors,
+                       fins, static_cast<const floatx4*>(ws));
+  }
+  return check_launch();
+}
+
 }  // namespace ak
+
+extern "C" int ak_syrk_group_eligible(const int64_t* spec) {
+  if (spec == nullptr) return 0;
+  ak::GroupFactor f;
+  int64_t max_rows;
+  return ak::group_decode(spec, f, max_rows) && max_rows >= ak::kDtlBK ? 1 : 0;
+}
+
+extern "C" int ak_syrk_group_sizes(const int64_t* specs, int n, size_t* table_bytes, size_t* ws_bytes) {
+  if (table_bytes == nullptr || ws_bytes == nullptr) return AK_ERR_ARG;
+  ak::GroupPlan g;
+  const int rc = ak::group_plan(specs, n, g);
+  if (rc != AK_OK) return rc;
+  *table_bytes = g.table_bytes;
+  *ws_bytes = g.ws_f4 * sizeof(ak::floatx4);
+  return AK_OK;
+}
+
+extern "C" int ak_syrk_group_launch(const int64_t* specs, int n, void* host_stage, void* dev_tables, size_t table_bytes,
+                                    void* ws, size_t ws_bytes, ak_stream_t stream) {
+  ak::GroupPlan g;
+  int rc = ak::group_plan(specs, n, g);
+  if (rc != AK_OK) return rc;
+  if (host_stage == nullptr || dev_tables == nullptr || table_bytes < g.table_bytes) return AK_ERR_WORKSPACE;
+  if (g.ws_f4 > 0 && (ws == nullptr || ws_bytes < g.ws_f4 * sizeof(ak::floatx4))) return AK_ERR_WORKSPACE;
+  unsigned char* h = static_cast<unsigned char*>(host_stage);
+  ak::DtlParams* hf = reinterpret_cast<ak::DtlParams*>(h + g.off_factors);
+  for (int i = 0; i < n; ++i) hf[i] = g.factors[i].p;
+  for (int c = 0; c < ak::kGroupClasses; ++c) {
+    if (!g.items[c].empty())
+      std::memcpy(h + g.off_items[c], g.items[c].data(), sizeof(ak::DtlGroupItem) * g.items[c].size());
+    if (!g.fins[c].empty())
+      std::memcpy(h + g.off_fins[c], g.fins[c].data(), sizeof(ak::DtlGroupFin) * g.fins[c].size());
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (hipMemcpyAsync(dev_tables, host_stage, g.table_bytes, hipMemcpyHostToDevice, s) != hipSuccess) return AK_ERR_LAUNCH;
+  const unsigned char* t = static_cast<const unsigned char*>(dev_tables);
+  ak::floatx4* w = static_cast<ak::floatx4*>(ws);
+  if ((rc = ak::group_launch_class<2, 2, 2, 2, false>(g, 0, t, w, s)) != AK_OK) return rc;
+  if ((rc = ak::group_launch_class<2, 2, 3, 3, false>(g, 1, t, w, s)) != AK_OK) return rc;
+  if ((rc = ak::group_launch_class<2, 2, 2, 2, true>(g, 2, t, w, s)) != AK_OK) return rc;
+  return ak::group_launch_class<2, 2, 3, 3, true>(g, 3, t, w, s);
+}
 
 #ifdef AK_TUNING_HOOKS
 // Tuning builds only: pins the channel group size of the gathered column order (0: built-in choice).
@@ -662,20 +968,10 @@ extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C,
     if (rc != AK_ERR_UNSUPPORTED) return rc;
   }
   if (dtype != AK_BF16) return AK_ERR_UNSUPPORTED;
-  // 16-byte chunks must not straddle taps, offsets must fit the 32-bit buffer range, and the magic
-  // divisions by Wo, Ho, C and kw must be exact over their operand ranges
-  if (C % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return AK_ERR_UNSUPPORTED;
-  if (N * H * W * C * 2 > static_cast<int64_t>(ak::kDtlRange)) return AK_ERR_UNSUPPORTED;
-  if (M * (Wo > Ho ? Wo : Ho) >= (1ll << 32) || (d + 256) * d >= (1ll << 32)) return AK_ERR_UNSUPPORTED;
   ak::DtlParams p{};
-  p.X = x; p.C = A; p.M = M; p.d = d; p.ldc = lda;
+  if (!ak::dtl_gather_params(p, x, N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return AK_ERR_UNSUPPORTED;
+  p.C = A; p.ldc = lda;
   p.alpha = alpha; p.beta = beta;
-  p.Cin = static_cast<int>(C); p.H = static_cast<int>(H); p.W = static_cast<int>(W);
-  p.kw = kw; p.KK = kh * kw; p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw;
-  p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
-  p.mWo = ak::make_magic(p.Wo); p.mHo = ak::make_magic(p.Ho); p.mKw = ak::make_magic(kw);
-  p.G = ak::g_force_group > 0 && p.Cin % ak::g_force_group == 0 ? ak::g_force_group : (d >= 3456 ? 8 : (p.Cin % 32 == 0 ? 32 : p.Cin));
-  p.mBlk = ak::make_magic(p.G * p.KK); p.mG = ak::make_magic(p.G);
   const ak::DtlPlan pl = ak::dtl_plan(M, d, INT64_MAX, true);
   return ak::dtl_launch<true>(p, pl, ws, ws_bytes, static_cast<hipStream_t>(stream));
 }

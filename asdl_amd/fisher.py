@@ -21,6 +21,12 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
+GROUPED_FACTORS = True     # the Kronecker factors of a forward + backward pass in one grouped launch (kernels.FactorGroup) instead of one launch per factor
+GROUP_FLUSH_EVERY = (-1, 0)  # (forward, backward): launch the group after that many hooks of the pass (0: once, when the pass
+                             # has ended; -1: that pass launches its factors one by one).  The forward pass of the benchmark is
+                             # bound by the host's launch rate, so its factor kernels cost nothing where they are; the backward
+                             # pass is not (ResNet-50 batch 64 in one process: 27.1 ms per step with single launches, 27.5 with
+                             # (0, 0), 27.2 with (8, 0), 26.75 with (-1, 0))
 FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (ordering the two streams costs ~30 us of host time per hook: more than the overlap gains)
 PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
 EAGER_INVERSE = True        # start the bulk of the inverses during a single sampled / empirical backward pass: the longest chains get a head start
@@ -66,17 +72,22 @@ class FisherMaker(GradientMaker):
                 delattr(module, attr)
 
     def _factor_stream(self):
-        """Side stream (default priority) for the statistics kernels of the hooks, one per maker."""
-        if not FACTOR_SIDE_STREAM or not torch.cuda.is_available():
+        """Where the statistics kernels of the hooks go, one object per maker: a group that launches the factors of
+        the whole pass together (GROUPED_FACTORS), a side stream of default priority (FACTOR_SIDE_STREAM), or None
+        for one launch per factor on the caller's stream."""
+        if not (GROUPED_FACTORS or FACTOR_SIDE_STREAM) or not torch.cuda.is_available():
             return None
         p = next(self.model.parameters(), None)
         if p is None or not p.is_cuda:
             return None
+        from .kernels import DeferredFactors, FactorStream
+        kind = DeferredFactors if GROUPED_FACTORS else FactorStream
         fs = getattr(self, '_factor_stream_obj', None)
-        if fs is None or fs.device != p.device:
-            from .kernels import FactorStream
-            fs = FactorStream(p.device)
+        if type(fs) is not kind or fs.device != p.device:
+            fs = kind(p.device)
             self._factor_stream_obj = fs
+        if GROUPED_FACTORS:
+            fs.every = GROUP_FLUSH_EVERY
         return fs
 
     @property

@@ -73,8 +73,8 @@ def _timing_event():
 
 
 class _Timed:
-    def __init__(self, name, flops):
-        self.name, self.flops = name, flops
+    def __init__(self, name, flops, calls=1):
+        self.name, self.flops, self.calls = name, flops, calls      # calls: factors covered by the timed region
 
     def __enter__(self):
         self.timed = _timing_sink is not None and _timing_on
@@ -87,7 +87,7 @@ class _Timed:
         if self.timed:
             end = _timing_event()
             end.record()
-            _timing_sink.append((self.name, self.flops, self.start, end))
+            _timing_sink.append((self.name, self.flops, self.start, end, self.calls))
         return False
 
 
@@ -271,7 +271,7 @@ class FactorStream:
         self._next = (self._next + 1) % len(self._events)
         return ev
 
-    def run(self, fn, *tensors):
+    def run(self, fn, *tensors, backward=False):
         """Queues ``fn``; every ``batch`` queued calls are run together behind one ordering of the side stream
         after the caller's stream (that ordering costs tens of microseconds of host time, more than a hook has to
         spare).  ``fn`` must not depend on anything but its arguments; its results are only valid after join()."""
@@ -320,6 +320,139 @@ class FactorStream:
             pass
 
 
+# ------------------------------------------------------------------------------ factors of many layers in one launch
+_group = threading.local()         # .active: the FactorGroup that collects this thread's factor calls, or None
+GROUP_SPEC_INTS = 16
+_group_eligible = {}
+
+
+def _float_bits(v):
+    return struct.unpack('<I', struct.pack('<f', float(v)))[0]
+
+
+class FactorGroup:
+    """Collects the factor statistics that syrk_tn() / conv_syrk() are asked for while it is the calling thread's
+    active group and launches them together in flush(): the factors of a whole forward or backward pass are a few
+    tiles each, and one at a time each of them pays a launch ramp, a tail, its split-K partial tiles and a reduction
+    launch.  The operands and results are kept alive until flush().  A call whose result tensor is already in the
+    group flushes first (a second contribution to the same factor has to come after the first)."""
+    SLOTS = 4
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._rows, self._keep, self._outs, self._flops = [], [], set(), 0
+        self._sizes = {}
+        self._slots = [dict(host=None, dev=None, event=None) for _ in range(self.SLOTS)]
+        self._next = 0
+
+    def __len__(self):
+        return len(self._rows)
+
+    @staticmethod
+    def eligible(row, align_key):
+        """Can the single-factor call described by ``row`` join a group?  (A pure function of the shape, the
+        alignment of the operand and the kind of call: cached.)"""
+        key = (tuple(row[:1] + row[3:4] + row[5:]), align_key)
+        ok = _group_eligible.get(key)
+        if ok is None:
+            arr = (ctypes.c_int64 * GROUP_SPEC_INTS)(*row)
+            ok = bool(_lib.load().ak_syrk_group_eligible(ctypes.cast(arr, ctypes.c_void_p)))
+            if len(_group_eligible) > 4096:
+                _group_eligible.clear()
+            _group_eligible[key] = ok
+        return ok
+
+    def add(self, row, flops, *tensors):
+        if row[2] in self._outs:
+            self.flush()
+        self._rows.append(row)
+        self._outs.add(row[2])
+        self._keep.append(tensors)
+        self._flops += flops
+
+    def flush(self):
+        """Launches what has been collected on the calling thread's launch stream."""
+        if not self._rows:
+            return
+        rows, self._rows, keep, self._keep = self._rows, [], self._keep, []
+        flops, self._flops, self._outs = self._flops, 0, set()
+        lib = _lib.load()
+        import numpy as np
+        specs = np.ascontiguousarray(np.array(rows, dtype=np.int64))
+        specs_ptr = ctypes.c_void_p(specs.ctypes.data)
+        sig = tuple((r[0], r[3]) + tuple(r[5:]) + (r[1] & 15,) for r in rows)
+        sizes = self._sizes.get(sig)
+        if sizes is None:
+            tb, wb = ctypes.c_size_t(0), ctypes.c_size_t(0)
+            _lib.check(lib.ak_syrk_group_sizes(specs_ptr, len(rows), ctypes.byref(tb), ctypes.byref(wb)),
+                       'ak_syrk_group_sizes')
+            if len(self._sizes) > 64:
+                self._sizes.clear()
+            sizes = self._sizes[sig] = (tb.value, wb.value)
+        table_bytes, ws_bytes = sizes
+        slot = self._slots[self._next]
+        self._next = (self._next + 1) % self.SLOTS
+        if slot['event'] is not None:
+            slot['event'].synchronize()          # the copy that last read this slot's host memory has long run
+        if slot['host'] is None or slot['host'].numel() < table_bytes:
+            slot['host'] = torch.empty(max(table_bytes, 1 << 16), dtype=torch.uint8).pin_memory()
+            slot['dev'] = torch.empty(slot['host'].numel(), dtype=torch.uint8, device=self.device)
+            slot['event'] = torch.cuda.Event()
+        ws, ws_size, ws_keep = _ws_args(ws_bytes, self.device)
+        with _Timed('syrk_group', flops, calls=len(rows)):
+            rc = lib.ak_syrk_group_launch(specs_ptr, len(rows), ctypes.c_void_p(slot['host'].data_ptr()),
+                                          ctypes.c_void_p(slot['dev'].data_ptr()), slot['host'].numel(),
+                                          ws, ws_size, _stream(self.device))
+        _lib.check(rc, 'ak_syrk_group_launch')
+        st = getattr(_override, 'stream', None)
+        slot['event'].record(st if st is not None else torch.cuda.current_stream(self.device))
+        del keep
+
+
+class DeferredFactors:
+    """Stands where a FactorStream stands (OperationContext.factor_stream): the hook operations run at once, on the
+    caller's stream, but the factor statistics they ask for are collected in a FactorGroup; join() launches what is
+    left of them.  ``every`` = (forward, backward): the group is also launched after that many hook calls of the
+    pass (0: only at join(); -1: the hooks of that pass launch their factors one by one, as without a group)."""
+
+    def __init__(self, device, every=(0, 0)):
+        self.device = torch.device(device)
+        self.group = FactorGroup(self.device)
+        self.every = tuple(every)
+        self._count = 0
+
+    def run(self, fn, *tensors, backward=False):
+        every = self.every[1 if backward else 0]
+        if every < 0:
+            self.group.flush()
+            fn()
+            return
+        saved = getattr(_group, 'active', None)
+        _group.active = self.group
+        try:
+            fn()
+        finally:
+            _group.active = saved
+        self._count += 1
+        if every > 0 and self._count >= every:
+            self._count = 0
+            self.group.flush()
+
+    def join(self):
+        self._count = 0
+        self.group.flush()
+        return []
+
+
+def _group_take(row, flops, align_key, *tensors):
+    """True when the calling thread has an active group and it has taken the call."""
+    grp = getattr(_group, 'active', None)
+    if grp is None or not FactorGroup.eligible(row, align_key):
+        return False
+    grp.add(row, flops, *tensors)
+    return True
+
+
 # ------------------------------------------------------------------------------ factors
 def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     """out <- beta*out + alpha * x^T x for x = [M, d] (rows may be strided, columns contiguous)."""
@@ -338,6 +471,11 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
         beta = 0.0
     if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
         raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
+    if x.dtype == torch.bfloat16 and getattr(_group, 'active', None) is not None:
+        row = [0, x.data_ptr(), out.data_ptr(), out.stride(0), _float_bits(alpha) | (_float_bits(beta) << 32),
+               M, d, ldx] + [0] * 8
+        if _group_take(row, M * d * (d + 1), x.data_ptr() & 15, x, out):
+            return out
     lib = _lib.load()
     need = _ws_need('ak_syrk_tn_ws_bytes', M, d)
     ws, ws_bytes, keep = _ws_args(need, x.device)
@@ -386,6 +524,11 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     if _is_channels_last(x) and ((x.dtype == torch.bfloat16 and C % 8 == 0) or few_channels):
         if (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0):
             return syrk_tn(x.permute(0, 2, 3, 1).reshape(N * H * W, C), out=out, alpha=alpha, beta=beta)
+        if x.dtype == torch.bfloat16 and getattr(_group, 'active', None) is not None:
+            row = [1, x.data_ptr(), out.data_ptr(), out.stride(0), _float_bits(alpha) | (_float_bits(beta) << 32),
+                   N, C, H, W, kh, kw, sh, sw, ph, pw, 0]
+            if _group_take(row, N * h_out * w_out * d * (d + 1), x.data_ptr() & 15, x, out):
+                return out
         need = _ws_need('ak_conv_syrk_nhwc_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
         ws, ws_bytes, keep = _ws_args(need, x.device)
         with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):

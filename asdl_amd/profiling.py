@@ -12,6 +12,8 @@ timing event on the current stream and append ``(name, event)`` to the list, so 
 between consecutive marks once the device is idle."""
 from contextlib import contextmanager
 
+import time
+
 import torch
 
 _ranges_on = False
@@ -53,4 +55,4 @@ def phase_mark(name):
         return
     event = torch.cuda.Event(enable_timing=True)
     event.record()
-    _phase_sink.append((name, event))
+    _phase_sink.append((name, event, time.perf_counter()))      # the host's clock too: which side bounds the phase?

@@ -69,6 +69,9 @@ def parse():
                     help='emit roctx ranges with the reference\'s range names (cov_kron_A, cov_kron_B, inv_kron_A_B, '
                          'fwd, bwd, upd_curv, upd_inv, precond) for `rocprofv3 --marker-trace`')
     ap.add_argument('--no-factor-timing', action='store_true')
+    ap.add_argument('--factor-launches', choices=['default', 'single', 'grouped'], default='default',
+                    help='single: one launch per Kronecker factor; grouped: the factors of a pass in one grouped launch '
+                         '(asdl_amd.fisher.GROUPED_FACTORS); default: the library\'s own setting')
     ap.add_argument('--traffic-calibration-mib', type=int, default=0,
                     help='before the warm-up, launch one plain copy kernel (ak::copy_bytes_kernel) of this many MiB: '
                          'the known traffic against which a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this '
@@ -214,6 +217,9 @@ def main():
     import torch.nn.functional as F
     import bench_models
     from asdl_amd import PreconditioningConfig, KfacGradientMaker, kernels
+    if args.factor_launches != 'default':
+        from asdl_amd import fisher as fisher_mod
+        fisher_mod.GROUPED_FACTORS = args.factor_launches == 'grouped'
 
     if not torch.cuda.is_available():
         print('bench.py needs a ROCm GPU.', file=sys.stderr)
@@ -336,12 +342,16 @@ def main():
             profiling.phase_mark('upd_param')
         torch.cuda.synchronize()
         profiling.set_phase_sink(None)
-        sums = {}
-        for (_, e0), (name, e1) in zip(marks, marks[1:]):
+        sums, host = {}, {}
+        for (_, e0, h0), (name, e1, h1) in zip(marks, marks[1:]):
             if name != 'begin':
                 sums[name] = sums.get(name, 0.0) + e0.elapsed_time(e1)
+                host[name] = host.get(name, 0.0) + (h1 - h0) * 1e3
+        # `ms`: between the events on the device; `host_ms`: between the moments the host enqueued them (a phase
+        # whose host time is close to its device time is bound by the host's launch rate)
         phases = {'steps': args.phase_steps, 'unit': 'ms per step',
                   'ms': {k: round(v / args.phase_steps, 4) for k, v in sums.items()},
+                  'host_ms': {k: round(v / args.phase_steps, 4) for k, v in host.items()},
                   'sum_ms': round(sum(sums.values()) / args.phase_steps, 4)}
     out = {
         'metric': 'K-FAC steps/s ResNet-50 bs64',
@@ -379,7 +389,8 @@ def main():
                            'floor_ms_per_step': 0.908 if default_workload else None,
                            'kernel': 'factor statistics (syrk_dtl_kernel; conv_patch_syrk_kernel for the 3-channel '
                                      'stem), SYRK FLOP M*d*(d+1)',
-                           'launches_per_step': len(sink) // timed_steps,
+                           'launches_per_step': sum(s[4] for s in sink) // timed_steps,
+                           'timed_regions_per_step': len(sink) // timed_steps,
                            'factor_ms_per_step': secs / timed_steps * 1e3,
                            'timed_steps': timed_steps,
                            'gemm_equiv_tflops': 2 * achieved}

@@ -88,6 +88,28 @@ int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C, int64_t H,
                       float alpha, float beta, float* A, int64_t lda,
                       void* ws, size_t ws_bytes, ak_stream_t stream);
 
+/* The statistics of many layers in one launch sequence: what ak_syrk_tn (bf16 operand, 16-byte aligned rows) and
+ * ak_conv_syrk_nhwc compute one factor at a time, i.e. Linear / Conv2d cov_kron_A and cov_kron_B
+ * (asdl/operations/linear.py:75-89, asdl/operations/conv.py:80-103) of a whole forward or backward pass, whose
+ * hooks the reference runs one by one (asdl/core.py:41-62).  Taken one at a time these factors are launches of a
+ * few tiles, split along the rows to fill the device; together they fill it with long work items and few splits.
+ * specs: HOST array of n rows of 16 int64:
+ *   [0] kind: 0 = X^T X of a bf16 [M, d] matrix, 1 = unfolded channels-last bf16 [N, C, H, W] input
+ *   [1] operand address (device)  [2] result address (device, fp32 [d, d])  [3] ldc
+ *   [4] alpha (float bits, low word) and beta (float bits, high word): result <- beta*result + alpha*statistic
+ *   kind 0: [5] M  [6] d  [7] ldx      kind 1: [5] N  [6] C  [7] H  [8] W  [9] kh  [10] kw  [11] sh  [12] sw  [13] ph  [14] pw
+ * ak_syrk_group_eligible: 1 when the row can be part of a group (else use the single-factor entry points: fp32
+ * operands, unaligned rows, few input channels, factors of 3456 columns and more).
+ * ak_syrk_group_sizes: bytes of the descriptor tables and of the workspace (partial tiles) of a group.
+ * ak_syrk_group_launch: host_stage is HOST memory of table_bytes (pinned, so that the copy is asynchronous) that
+ * the caller leaves alone until the stream has passed the copy; dev_tables and ws are device memory.  Two rows with
+ * the same result address are refused (AK_ERR_ARG): they would race.  Fixed summation order: results are
+ * reproducible bit for bit for a given list of shapes. */
+int ak_syrk_group_eligible(const int64_t* spec);
+int ak_syrk_group_sizes(const int64_t* specs, int n, size_t* table_bytes, size_t* ws_bytes);
+int ak_syrk_group_launch(const int64_t* specs, int n, void* host_stage, void* dev_tables, size_t table_bytes,
+                         void* ws, size_t ws_bytes, ak_stream_t stream);
+
 /* ---- damping ---------------------------------------------------------------------- */
 
 /* For each pair b < batch: tr(A_b), tr(B_b), the pi split

@@ -214,6 +214,86 @@ def test_syrk_tn_bf16_split_k_and_strided(K, M, d, ld):
     assert torch.equal(out, out.T)
 
 
+def _group_cases():
+    """(kind, args): plain [M, d] operands (with a row stride, ragged sizes, a result with a wide row stride) and
+    channels-last convolution inputs (3x3, strided 1x1, 5x5 with padding), small and at the benchmark's sizes."""
+    plain = [(64, 128, 128), (777, 264, 264), (333, 1000, 1000), (3000, 64, 64), (4096, 512, 520), (12544, 1024, 1024),
+             (3136, 2048, 2048), (50176, 256, 256), (100, 136, 136), (1500, 1600, 1608)]
+    conv = [(2, 32, 9, 9, 3, 1, 1), (4, 64, 14, 14, 3, 2, 1), (3, 24, 11, 11, 3, 1, 0), (8, 128, 28, 28, 3, 1, 1),
+            (2, 16, 13, 13, 5, 2, 2), (16, 64, 56, 56, 3, 1, 1), (4, 256, 14, 14, 1, 2, 0), (8, 256, 14, 14, 3, 1, 1)]
+    return plain, conv
+
+
+def test_factor_group_matches_the_single_launches_and_fp64(K):
+    """kernels.FactorGroup: the factors of many layers in one grouped launch per tile class.  Every result has to
+    agree with the fp64 product of the rounded operand to 1e-5 and to be exactly symmetric; alpha / beta (the EMA
+    form) and a second contribution to the same result (which forces a flush in between) are covered."""
+    import torch.nn.functional as F
+    plain, conv = _group_cases()
+    torch.manual_seed(3)
+    xs, outs, refs = [], [], []
+    grp = K.FactorGroup(torch.device('cuda'))
+    K._group.active = grp
+    try:
+        for i, (M, d, ld) in enumerate(plain):
+            x = torch.randn(M, ld, device='cuda').to(torch.bfloat16)[:, :d]
+            alpha, beta = (0.5, 0.0) if i % 3 else (0.25, 0.75)
+            out = torch.full((d, d + 8), 2.0, device='cuda')[:, :d] if i % 4 == 0 else torch.full((d, d), 2.0, device='cuda')
+            ref = alpha * (x.double().T @ x.double()) + beta * out.double()
+            r = K.syrk_tn(x, out=out, alpha=alpha, beta=beta)
+            assert r is out
+            xs.append(x); outs.append(out); refs.append(ref)
+        for (N, C, H, W, k, s, p) in conv:
+            x = torch.randn(N, C, H, W, device='cuda').to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+            d = C * k * k
+            u = F.unfold(x.double(), k, padding=p, stride=s).transpose(1, 2).reshape(-1, d)
+            out = torch.zeros(d, d, device='cuda')
+            K.conv_syrk(x, (k, k), (s, s), (p, p), out=out, alpha=2.0)
+            xs.append(x); outs.append(out); refs.append(2.0 * (u.T @ u))
+        assert len(grp) == len(plain) + len(conv), 'every case should have been taken by the group'
+        assert float(outs[1].abs().max()) == 2.0, 'nothing may be written before the flush'
+        # a second contribution to the first result: the group has to flush before it takes it
+        M, d, _ = plain[0]
+        x2 = torch.randn(M, d, device='cuda').to(torch.bfloat16)
+        refs[0] = refs[0] + (x2.double().T @ x2.double())
+        K.syrk_tn(x2, out=outs[0], alpha=1.0, beta=1.0)
+        assert len(grp) == 1
+        grp.flush()
+        assert len(grp) == 0
+    finally:
+        K._group.active = None
+    torch.cuda.synchronize()
+    for i, (out, ref) in enumerate(zip(outs, refs)):
+        assert relerr(out, ref) < 1e-5, (i, relerr(out, ref))
+        assert torch.equal(out, out.T), i
+    # the same calls one by one give the same factors up to the summation order
+    for i, (M, d, ld) in enumerate(plain[:4]):
+        single = K.syrk_tn(xs[i], alpha=1.0)
+        assert single.shape == (d, d)
+
+
+def test_factor_group_leaves_ineligible_calls_alone(K):
+    """fp32 operands, rows that are not 16-byte aligned, the few-channel stem and factors of 3456 columns and more are
+    launched at once even while a group is active."""
+    grp = K.FactorGroup(torch.device('cuda'))
+    K._group.active = grp
+    try:
+        x = torch.randn(300, 40, device='cuda')
+        out = K.syrk_tn(x)
+        assert len(grp) == 0 and relerr(out, x.double().T @ x.double()) < 1e-5
+        xb = torch.randn(300, 44, device='cuda').to(torch.bfloat16)        # 88-byte rows
+        out = K.syrk_tn(xb)
+        assert len(grp) == 0 and relerr(out, xb.double().T @ xb.double()) < 1e-5
+        stem = torch.randn(2, 3, 32, 32, device='cuda').to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+        K.conv_syrk(stem, (7, 7), (2, 2), (3, 3))
+        assert len(grp) == 0
+        wide = torch.randn(1, 512, 7, 7, device='cuda').to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+        K.conv_syrk(wide, (3, 3), (1, 1), (1, 1))
+        assert len(grp) == 0
+    finally:
+        K._group.active = None
+
+
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('N,C,hw', [(2, 4, (3, 3)), (8, 64, (7, 7)), (4, 130, (14, 14)), (2, 1000, (1, 1)),
                                     (3, 17, (28, 28)), (1, 257, (5, 9))])

@@ -461,7 +461,9 @@ def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch
         kron = replay[name]
         eA, eB = relerr(got[name][0], kron.A_inv), relerr(got[name][1], kron.B_inv)
         worst['A_inv'], worst['B_inv'] = max(worst['A_inv'], eA), max(worst['B_inv'], eB)
-        assert eA < 1e-5 and eB < 1e-5, (name, eA, eB)
+        # the run sums the rows of a factor in the grouped launch's order, the replay in the single launch's: the
+        # factors differ by ~1e-7 and the inverses by that times the condition number; 1e-4 is the bar for inverses
+        assert eA < 1e-4 and eB < 1e-4, (name, eA, eB)
         g_w = raw[(name, 'weight')] / bs
         g_b = raw[(name, 'bias')] / bs if m.bias is not None else None
         exact = kron.B_inv.double() @ g_w.double().reshape(kron.B_inv.shape[0], -1) @ kron.A_inv.double()
@@ -674,6 +676,66 @@ def test_factor_side_stream_gives_the_golden_results(tag, monkeypatch):
     import asdl_amd.fisher as fisher_mod
     monkeypatch.setattr(fisher_mod, 'FACTOR_SIDE_STREAM', True)
     test_kfac_gpu_matches_reference_golden(tag)
+
+
+@pytest.mark.parametrize('ema', [-1, 0.3])
+def test_grouped_factor_launches_give_the_single_launch_factors(ema, monkeypatch):
+    """fisher.GROUPED_FACTORS collects the bf16 Kronecker-factor statistics of a pass and launches them together
+    (kernels.FactorGroup), at the end of the pass or every few hooks (fisher.GROUP_FLUSH_EVERY).  On a channels-last
+    CNN under bf16 autocast (3x3, strided 1x1 and plain 1x1 convolutions, a Linear head; two steps, so that with EMA
+    the second one accumulates) every setting has to give the factors of the one-launch-per-factor path up to the
+    summation order (2e-6), inverses within 1e-4 and the same preconditioned gradients (1e-4)."""
+    import asdl_amd.fisher as fisher_mod
+    torch.manual_seed(31)
+    xs = [torch.randn(8, 16, 12, 12).cuda().contiguous(memory_format=torch.channels_last) for _ in range(2)]
+    ts = [torch.randint(10, (8,)).cuda() for _ in range(2)]
+
+    def run(grouped, every):
+        monkeypatch.setattr(fisher_mod, 'GROUPED_FACTORS', grouped)
+        monkeypatch.setattr(fisher_mod, 'GROUP_FLUSH_EVERY', every)
+        torch.manual_seed(32)
+        model = nn.Sequential(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU(), nn.Conv2d(32, 64, 1, stride=2), nn.ReLU(),
+                              nn.Conv2d(64, 64, 1), nn.ReLU(), nn.Conv2d(64, 32, 3, padding=1), nn.ReLU(),
+                              nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
+        model = model.to(memory_format=torch.channels_last)
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=8, damping=1e-2, ema_decay=ema),
+                               fisher_type=FISHER_EMP)
+
+        def fwd(inp):
+            with torch.autocast('cuda', dtype=torch.bfloat16):
+                return model(inp).float()
+        for x, t in zip(xs, ts):
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
+            gm.forward_and_backward()
+        torch.cuda.synchronize()
+        out = {}
+        for name, m in model.named_modules():
+            if hasattr(m, 'fisher'):
+                kron = m.fisher.kron
+                for key in ('A', 'B', 'A_inv', 'B_inv'):
+                    if getattr(kron, key) is not None:
+                        out[f'{name}.{key}'] = getattr(kron, key).clone()
+                out[f'{name}.grad'] = m.weight.grad.clone()
+        return out
+
+    from asdl_amd import kernels
+    taken = []
+    plain_add = kernels.FactorGroup.add
+    monkeypatch.setattr(kernels.FactorGroup, 'add', lambda self, row, *a: (taken.append(row[0]), plain_add(self, row, *a))[1])
+    ref = run(False, (0, 0))
+    assert not taken
+    assert any(k.endswith('A_inv') for k in ref) and (ema == -1 or any(k.endswith('.A') for k in ref))
+    for every in [(0, 0), (-1, 0), (2, 3), (1, 1)]:
+        del taken[:]
+        got = run(True, every)
+        # per step: B of the four convolutions (the Linear layer's 10 columns are not a multiple of 8), and with
+        # forward grouping A of the four layers that are not the few-channel stem
+        assert len(taken) == 2 * (4 if every[0] < 0 else 8) and (every[0] < 0 or 1 in taken), (every, taken)
+        assert got.keys() == ref.keys()
+        for key in ref:
+            tol = 2e-6 if key.endswith(('.A', '.B')) else 1e-4
+            assert relerr(got[key], ref[key]) < tol, (every, key, relerr(got[key], ref[key]))
 
 
 def test_fisher_attributes_and_steps_without_curvature_update():
