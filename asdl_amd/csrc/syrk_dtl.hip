@@ -26,7 +26,9 @@
 #include <cmath>
 #include <cstring>
 #include <initializer_list>
+#include <functional>
 #include <mutex>
+#include <queue>
 #include <unordered_map>
 #include <vector>
 #include <type_traits>
@@ -715,7 +717,7 @@ static bool dtl_gather_params(DtlParams& p, const void* x, int64_t N, int64_t C,
 //   kind 0: [5] M  [6] d  [7] ldx          kind 1: [5] N  [6] C  [7] H  [8] W  [9] kh  [10] kw  [11..14] sh sw ph pw
 constexpr int kGroupSpecInts = 16;
 constexpr int kGroupClasses = 4;           // plain 128 / 192, gathered 128 / 192
-constexpr int kGroupMaxSplits = 32;
+constexpr int kGroupMaxSplits = 96;         // partial tiles per tile that the reduction pass sums, one after the other
 
 struct GroupFactor {
   DtlParams p;
@@ -797,18 +799,66 @@ static int group_plan(const int64_t* specs, int n, GroupPlan& g) {
     if (work[c] == 0) continue;
     const int bt = (c == 0 || c == 2) ? 128 : 192;
     const int64_t slots = 256 * (bt == 128 ? 2 : 1);
-    // about four items per slot of the device, none shorter than 32 k-tiles unless its factor is
-    int64_t chunk = (work[c] + slots * 4 - 1) / (slots * 4);
-    if (chunk < 32) chunk = 32;
+    // The longest item a factor may have, in k-tiles ("chunk"): longer row ranges are split.  Candidates: no split at
+    // all, and 1/4 or 1/8 of the work per slot (coarser items balance well on paper only: work groups do not all
+    // run at one speed); each is judged by the finishing time of a greedy assignment of its items, longest first,
+    // to the slots (what the dispatcher does with the work groups in launch order) plus the traffic of the partial
+    // tiles it causes.  A group of a few wide factors thus stays unsplit, a pass of many narrow ones gets a few
+    // splits each.
+    auto splits_of = [&](int i, int64_t chunk) {
+      const GroupFactor& f = g.factors[i];
+      int64_t ns = (f.ktiles + chunk - 1) / chunk;
+      if (ns > kGroupMaxSplits) ns = kGroupMaxSplits;
+      const int64_t max_kt = max_rows[i] / kDtlBK;
+      if ((f.ktiles + ns - 1) / ns > max_kt) ns = (f.ktiles + max_kt - 1) / max_kt;
+      return ns < 1 ? int64_t{1} : ns;
+    };
+    int64_t longest = 0;
+    for (int i = 0; i < n; ++i) {
+      if (g.factors[i].cls != c) continue;
+      if (max_rows[i] / kDtlBK < 1) return AK_ERR_UNSUPPORTED;
+      longest = std::max(longest, g.factors[i].ktiles);
+    }
+    // microseconds per k-tile of a work group: two 128-wide ones share a CU (dtl_plan_search's t_shared), a 192-wide
+    // one has it to itself
+    const double t_kt = bt == 128 ? 0.55 : 0.45;
+    int64_t chunk = longest;
+    double best_cost = 1e300;
+    for (int k = 0; k <= 4; k += (k == 0 ? 3 : 1)) {
+      int64_t cand = k == 0 ? longest : (work[c] + slots * (1 << (k - 1)) - 1) / (slots * (1 << (k - 1)));
+      if (cand < 32) cand = 32;
+      if (cand > longest) cand = longest;
+      std::vector<int64_t> lens;                            // item lengths, longest first
+      double part_mb = 0.0;
+      int64_t most_splits = 1;
+      for (int i = 0; i < n; ++i) {
+        const GroupFactor& f = g.factors[i];
+        if (f.cls != c) continue;
+        const int64_t ns = splits_of(i, cand), len = (f.ktiles + ns - 1) / ns;
+        lens.insert(lens.end(), static_cast<size_t>(ns * f.ntiles), len);
+        if (ns > 1) part_mb += static_cast<double>(ns * f.ntiles) * bt * bt * 4.0 * 1e-6;
+        most_splits = std::max(most_splits, ns);
+      }
+      std::sort(lens.begin(), lens.end(), std::greater<int64_t>());
+      std::priority_queue<int64_t, std::vector<int64_t>, std::greater<int64_t>> busy;   // finishing times of the slots
+      int64_t makespan = 0;
+      for (int64_t len : lens) {
+        int64_t start = 0;
+        if (static_cast<int64_t>(busy.size()) >= slots) { start = busy.top(); busy.pop(); }
+        busy.push(start + len);
+        makespan = std::max(makespan, start + len);
+      }
+      // partial tiles: written once, read once, ~5 TB/s out of L2 / MALL; the reduction pass: a launch and a chain
+      // of dependent reads as long as the largest split count
+      const double cost = static_cast<double>(makespan) * t_kt + 2.0 * part_mb / 5.0 +
+                          (part_mb > 0 ? 4.0 + 0.15 * static_cast<double>(most_splits) : 0.0);
+      if (cost < best_cost) { best_cost = cost; chunk = cand; }
+    }
     std::vector<int> order;
     for (int i = 0; i < n; ++i) {
       GroupFactor& f = g.factors[i];
       if (f.cls != c) continue;
-      int64_t ns = (f.ktiles + chunk - 1) / chunk;
-      if (ns > kGroupMaxSplits) ns = kGroupMaxSplits;
-      const int64_t max_kt = max_rows[i] / kDtlBK;
-      if (max_kt < 1) return AK_ERR_UNSUPPORTED;
-      if ((f.ktiles + ns - 1) / ns > max_kt) ns = (f.ktiles + max_kt - 1) / max_kt;
+      const int64_t ns = splits_of(i, chunk);
       f.kt_split = (f.ktiles + ns - 1) / ns;
       f.nsplit = static_cast<int>((f.ktiles + f.kt_split - 1) / f.kt_split);
       f.p.nsplit = f.nsplit;

@@ -376,6 +376,23 @@ class FactorGroup:
             return
         rows, self._rows, keep, self._keep = self._rows, [], self._keep, []
         flops, self._flops, self._outs = self._flops, 0, set()
+        if len(rows) == 1:
+            # nothing to share a launch with: the single-factor entry points, whose plan search knows more tile
+            # sizes and a two-stage reduction
+            saved = getattr(_group, 'active', None)
+            _group.active = None
+            try:
+                x, out = keep[0][0], keep[0][1]
+                alpha = struct.unpack('<f', struct.pack('<I', rows[0][4] & 0xffffffff))[0]
+                beta = struct.unpack('<f', struct.pack('<I', rows[0][4] >> 32))[0]
+                if rows[0][0] == 0:
+                    syrk_tn(x, out=out, alpha=alpha, beta=beta)
+                else:
+                    r = rows[0]
+                    conv_syrk(x, (r[9], r[10]), (r[11], r[12]), (r[13], r[14]), out=out, alpha=alpha, beta=beta)
+            finally:
+                _group.active = saved
+            return
         lib = _lib.load()
         import numpy as np
         specs = np.ascontiguousarray(np.array(rows, dtype=np.int64))
