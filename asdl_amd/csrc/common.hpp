@@ -57,6 +57,12 @@ __device__ __forceinline__ void decode_upper_tile(int id, int T, int& ti, int& t
   tj = row + id;
 }
 
+// The SYRK epilogues read the old result (beta != 0) through a 32-bit buffer descriptor: results of 4 GiB and more
+// cannot be accumulated into.
+inline bool syrk_beta_ok(float beta, int64_t d, int64_t ldc) {
+  return beta == 0.f || ((d - 1) * ldc + d) * 4 < 0xFFFFFF00ll;
+}
+
 // Symmetric epilogue for one wave's accumulators of a BT x BT output tile at (ti, tj), ti <= tj.
 // acc[a][b] is the 32x32 MFMA tile at rows row0 + 32a, cols col0 + 32b of the WG tile.
 // Writes C[i][j] = beta*C[i][j] + alpha*acc and, off the diagonal tile, the mirror C[j][i].
@@ -68,7 +74,11 @@ __device__ __forceinline__ void syrk_epilogue(floatx16 (&acc)[TI][TJ], float* __
   const bool vec_mirror = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
   // Phase 1: acc <- alpha * acc (+ beta * C).  All reads of C come before the first store: the compiler cannot
   // prove that a store to C leaves a later read alone, so reads that follow stores are issued one memory latency
-  // after another (measured: +60 us on a 4096 x 4096 factor).
+  // after another.  The reads go through a buffer descriptor of C: one 32-bit offset register per 32 x 32 block and
+  // lane, the row within the block as a scalar offset, and rows beyond the matrix read as zero without a bounds
+  // test (a load under a per-element condition gets a wait of its own: 16 * TI * TJ memory latencies in a row;
+  // 64-bit addresses and clamped indices for as many loads in flight cost more registers than the widest tile has).
+  // Columns beyond d read whatever lies there inside the buffer; those accumulators are never stored.
 #pragma unroll
   for (int a = 0; a < TI; ++a)
 #pragma unroll
@@ -76,26 +86,23 @@ __device__ __forceinline__ void syrk_epilogue(floatx16 (&acc)[TI][TJ], float* __
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] *= alpha;
   if (beta != 0.f) {
+    // (the entry points refuse beta != 0 for a result of 4 GiB and more: syrk_beta_ok)
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(((d - 1) * ldc + d) * 4), 0x00020000);
+    const uint32_t ldc4 = static_cast<uint32_t>(ldc) * 4u;
 #pragma unroll
     for (int a = 0; a < TI; ++a) {
-      // Unconditional loads from clamped positions, a row of 32 x 32 blocks (16 * TJ loads) at a time: a load
-      // under a per-element condition gets a wait of its own, and the 16 * TI * TJ of them then pay one memory
-      // latency each.
-      float c[TJ][16];
 #pragma unroll
       for (int b = 0; b < TJ; ++b) {
-        const int64_t gj = gj0 + 32 * b + l32, rj = gj < d ? gj : d - 1;
+        const uint32_t voff = static_cast<uint32_t>(gi0 + 32 * a + 4 * g) * ldc4 +
+                              static_cast<uint32_t>(gj0 + 32 * b + l32) * 4u;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t gi = gi0 + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3);
-          c[b][r] = C[(gi < d ? gi : d - 1) * ldc + rj];
+          const float c = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, (8 * (r >> 2) + (r & 3)) * ldc4, 0));
+          acc[a][b][r] += beta * c;
         }
       }
-      __builtin_amdgcn_sched_barrier(0);          // keeps the multiply-adds (and their waits) below all the loads
-#pragma unroll
-      for (int b = 0; b < TJ; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += beta * c[b][r];
     }
   }
   // Phase 2: the tile and, off the diagonal, its mirror image.

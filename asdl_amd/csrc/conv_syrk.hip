@@ -598,6 +598,7 @@ extern "C" int ak_conv_syrk(const void* x, int dtype, int64_t N, int64_t C, int6
       sw <= 0 || ph < 0 || pw < 0)
     return AK_ERR_ARG;
   if (dtype != AK_BF16 && dtype != AK_F32) return AK_ERR_ARG;
+  if (!ak::syrk_beta_ok(beta, C * kh * kw, lda)) return AK_ERR_UNSUPPORTED;
   {  // few input channels: the window kernel
     const int rc = ak::conv_patch_syrk(x, dtype, C * H * W, H * W, W, 1, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,
                                        A, lda, ws, ws_bytes, static_cast<hipStream_t>(stream));

@@ -55,7 +55,7 @@ struct DtlParams {
   // gather geometry
   int Cin, H, W, kw, KK, sh, sw, ph, pw, Ho, Wo;
   int G;                          // channels per column group
-  uint32_t mWo, mHo, mKw, mBlk, mG;   // magic multipliers: Wo, Ho, kw, G*KK, G
+  uint32_t mWo, mHo, mKw, mBlk, mG, mKK;   // magic multipliers: Wo, Ho, kw, G*KK, G, KK
 };
 
 // 16 bytes per lane, global -> LDS at m0 + 16*lane.  The compiler does not see the LDS write: callers
@@ -96,8 +96,9 @@ __device__ __forceinline__ void dtl_epilogue(floatx16 (&acc)[FR][FC], const DtlP
   } else {
     const int g = lane >> 5, l32 = lane & 31;
     // First acc <- alpha * acc + beta * C, then the stores, so that no read of C waits behind a store to C.  The
-    // reads are unconditional (clamped positions) and issued a 32 x 32 block's 16 at a time: under a per-element
-    // condition each gets a wait of its own and pays one memory latency.
+    // reads go through a buffer descriptor of C (see syrk_epilogue): the four rows of an accumulator float4 are
+    // consecutive channels of one tap, KK result rows apart, so their row offsets are scalars; rows and columns
+    // beyond d get an out-of-range offset and read as zero.
 #pragma unroll
     for (int a = 0; a < FR; ++a)
 #pragma unroll
@@ -105,22 +106,34 @@ __device__ __forceinline__ void dtl_epilogue(floatx16 (&acc)[FR][FC], const DtlP
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][b][r] *= p.alpha;
     if (p.beta != 0.f) {
+      // (results of 4 GiB and more are refused on the host: (d + 256) * d < 2^32 / 4 is required of gathered factors)
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          p.C, 0, static_cast<int>(((p.d - 1) * p.ldc + p.d) * 4), 0x00020000);
+      const uint32_t ldc4 = static_cast<uint32_t>(p.ldc) * 4u, row_step = static_cast<uint32_t>(p.KK) * ldc4;
+      uint32_t row_off[FR][4];
+#pragma unroll
+      for (int a = 0; a < FR; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t gi = gi0 + 32 * a + 8 * q + 4 * g;
+          row_off[a][q] = gi < p.d ? static_cast<uint32_t>(out_index<true>(gi, p)) * ldc4 : kDtlOob;
+        }
 #pragma unroll
       for (int b = 0; b < FC; ++b) {
         const int64_t gj = gj0 + 32 * b + l32;
-        const int64_t oj = out_index<true>(gj < p.d ? gj : p.d - 1, p);
+        const uint32_t col_off = gj < p.d ? static_cast<uint32_t>(out_index<true>(gj, p)) * 4u : kDtlOob;
 #pragma unroll
-        for (int a = 0; a < FR; ++a) {
-          float c[16];
+        for (int a = 0; a < FR; ++a)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int64_t gi = gi0 + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3);
-            c[r] = p.C[out_index<true>(gi < p.d ? gi : p.d - 1, p) * p.ldc + oj];
+          for (int q = 0; q < 4; ++q) {
+            const bool ok = row_off[a][q] != kDtlOob && col_off != kDtlOob;
+            const uint32_t voff = ok ? row_off[a][q] + col_off : kDtlOob;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float c = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, e * row_step, 0));
+              acc[a][b][4 * q + e] += p.beta * c;
+            }
           }
-          __builtin_amdgcn_sched_barrier(0);      // keeps the multiply-adds (and their waits) below all the loads
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[a][b][r] += p.beta * c[r];
-        }
       }
     }
 #pragma unroll
@@ -492,6 +505,101 @@ __global__ __launch_bounds__(WR * WC * 64) void syrk_dtl_finalize_grouped_kernel
                                             it.nparts);
 }
 
+// Reduction pass of a GATHERED factor by output position.  The pass above takes the partial tiles in accumulator
+// order, whose neighbouring columns are KK floats apart in the result (working order (c/G, tap, c%G), result order
+// (c, tap)): every lane stores 4 bytes here and 4 bytes there, and the memory system writes 7 bytes for each one
+// stored.  Here a wave owns four result rows, (c .. c+3, tap) for a channel quad c, and 64 consecutive result
+// columns: its stores are whole 256-byte runs.  The four rows are consecutive working rows, i.e. ONE float4 of a
+// partial tile, if the element lies in a computed (upper) tile; below the diagonal the mirror image is read, four
+// floats from four float4.  grid (ceil(d / 64), ceil(d / 16)), 256 threads.
+template <int WR, int WC, int FR, int FC>
+__device__ __forceinline__ void dtl_finalize_out(const DtlParams& p, const floatx4* __restrict__ part, int64_t ntiles,
+                                                 int n, uint32_t col_block, uint32_t row_block) {
+  constexpr int NW = WR * WC, BT = 32 * FR * WR;
+  constexpr size_t tile_f4 = static_cast<size_t>(BT) * BT / 4;
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t d = static_cast<uint32_t>(p.d), KK = p.KK, G = p.G;
+  const uint32_t oj = col_block * 64 + lane;
+  const uint32_t rg = row_block * 4 + wave;                 // row group: (channel quad, tap)
+  if (rg * 4 >= d || oj >= d) return;
+  const uint32_t c4 = fastdiv(rg, p.mKK, KK), tap_i = rg - c4 * KK, ci = 4 * c4;
+  const uint32_t blk_i = fastdiv(ci, p.mG, G);
+  const uint32_t vi = blk_i * G * KK + tap_i * G + (ci - blk_i * G);      // first of four consecutive working rows
+  const uint32_t cj = fastdiv(oj, p.mKK, KK), tap_j = oj - cj * KK, blk_j = fastdiv(cj, p.mG, G);
+  const uint32_t vj = blk_j * G * KK + tap_j * G + (cj - blk_j * G);
+  const uint32_t ti = vi / BT, tj = vj / BT;
+  // float4 index and component of element (r, c) of a tile, in accumulator order
+  auto slot_of = [](uint32_t r, uint32_t c, uint32_t& e) {
+    const uint32_t wr = r / (32 * FR), a = (r % (32 * FR)) / 32, r32 = r % 32, q = r32 / 8, g = (r32 % 8) / 4;
+    const uint32_t wc = c / (32 * FC), b = (c % (32 * FC)) / 32, l32 = c % 32;
+    e = r32 % 4;
+    return ((a * FC + b) * 4 + q) * (NW * 64) + (wr * WC + wc) * 64 + g * 32 + l32;
+  };
+  const size_t split_stride = static_cast<size_t>(ntiles) * tile_f4;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (ti <= tj) {
+    const size_t tile = static_cast<size_t>(ti) * p.T - static_cast<size_t>(ti) * (ti - 1) / 2 + (tj - ti);
+    uint32_t e;
+    const floatx4* src = part + tile * tile_f4 + slot_of(vi % BT, vj % BT, e);     // e == 0: vi is a multiple of 4
+    int s = 0;
+    for (; s + 4 <= n; s += 4) {
+      const floatx4 w0 = src[(s + 0) * split_stride], w1 = src[(s + 1) * split_stride];
+      const floatx4 w2 = src[(s + 2) * split_stride], w3 = src[(s + 3) * split_stride];
+      acc += w0; acc += w1; acc += w2; acc += w3;
+    }
+    for (; s < n; ++s) acc += src[s * split_stride];
+  } else {
+    const size_t tile = static_cast<size_t>(tj) * p.T - static_cast<size_t>(tj) * (tj - 1) / 2 + (ti - tj);
+    const float* base = reinterpret_cast<const float*>(part + tile * tile_f4);
+    size_t off[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      uint32_t e;
+      const uint32_t f4 = slot_of(vj % BT, (vi + k) % BT, e);
+      off[k] = static_cast<size_t>(f4) * 4 + e;
+    }
+    for (int s = 0; s < n; ++s) {
+      const float* q = base + static_cast<size_t>(s) * split_stride * 4;
+      const float x0 = q[off[0]], x1 = q[off[1]], x2 = q[off[2]], x3 = q[off[3]];
+      acc[0] += x0; acc[1] += x1; acc[2] += x2; acc[3] += x3;
+    }
+  }
+  float* dst = p.C + (static_cast<int64_t>(ci) * KK + tap_i) * p.ldc + oj;       // rows are KK apart
+  const int64_t row_step = static_cast<int64_t>(KK) * p.ldc;
+  float v[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) v[k] = p.alpha * acc[k];
+  if (p.beta != 0.f) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] += p.beta * dst[k * row_step];
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) dst[k * row_step] = v[k];
+}
+
+template <int WR, int WC, int FR, int FC>
+__global__ __launch_bounds__(256) void syrk_dtl_finalize_out_kernel(DtlParams p, const floatx4* __restrict__ part,
+                                                                    int64_t ntiles, int n) {
+  dtl_finalize_out<WR, WC, FR, FC>(p, part, ntiles, n, blockIdx.x, blockIdx.y);
+}
+
+// The same for the gathered factors of a grouped launch: grid (column blocks x row blocks of the widest factor,
+// factors with partial tiles); work groups beyond a narrower factor's blocks leave at once.
+struct DtlGroupFinOut {
+  int32_t factor, nparts, col_blocks, pad;
+  int64_t first, ntiles;
+};
+
+template <int WR, int WC, int FR, int FC>
+__global__ __launch_bounds__(256) void syrk_dtl_finalize_out_grouped_kernel(const DtlParams* __restrict__ factors,
+                                                                            const DtlGroupFinOut* __restrict__ fins,
+                                                                            const floatx4* __restrict__ ws) {
+  const DtlGroupFinOut it = fins[blockIdx.y];
+  const DtlParams p = factors[it.factor];
+  const uint32_t row_block = blockIdx.x / it.col_blocks, col_block = blockIdx.x - row_block * it.col_blocks;
+  dtl_finalize_out<WR, WC, FR, FC>(p, ws + it.first, it.ntiles, it.nparts, col_block, row_block);
+}
+
 // ---- host side ------------------------------------------------------------------------------------
 
 constexpr int kDtlDirectSplits = 24;   // up to this many partials the epilogue pass sums them itself
@@ -635,8 +743,14 @@ static int dtl_launch_cfg(const DtlParams& p, const DtlPlan& pl, hipStream_t str
       part = sums;
       n = pl.ngroups;
     }
-    hipLaunchKernelGGL((syrk_dtl_finalize_kernel<WR, WC, FR, FC, GATHER>), dim3(ntiles, 4 * FR * FC),
-                       dim3(Cfg::NW * 64), 0, stream, p, part, n);
+    if constexpr (GATHER) {
+      const unsigned d = static_cast<unsigned>(p.d);
+      hipLaunchKernelGGL((syrk_dtl_finalize_out_kernel<WR, WC, FR, FC>), dim3((d + 63) / 64, (d + 15) / 16), dim3(256),
+                         0, stream, p, part, pl.ntiles, n);
+    } else {
+      hipLaunchKernelGGL((syrk_dtl_finalize_kernel<WR, WC, FR, FC, GATHER>), dim3(ntiles, 4 * FR * FC),
+                         dim3(Cfg::NW * 64), 0, stream, p, part, n);
+    }
   }
   return check_launch();
 }
@@ -703,7 +817,7 @@ static bool dtl_gather_params(DtlParams& p, const void* x, int64_t N, int64_t C,
   p.Ho = static_cast<int>(Ho); p.Wo = static_cast<int>(Wo);
   p.mWo = make_magic(p.Wo); p.mHo = make_magic(p.Ho); p.mKw = make_magic(kw);
   p.G = g_force_group > 0 && p.Cin % g_force_group == 0 ? g_force_group : (d >= 3456 ? 8 : (p.Cin % 32 == 0 ? 32 : p.Cin));
-  p.mBlk = make_magic(p.G * p.KK); p.mG = make_magic(p.G);
+  p.mBlk = make_magic(p.G * p.KK); p.mG = make_magic(p.G); p.mKK = make_magic(p.KK);
   return true;
 }
 
@@ -768,6 +882,7 @@ static bool group_decode(const int64_t* r, GroupFactor& f, int64_t& max_rows_per
   } else {
     return false;
   }
+  if (!syrk_beta_ok(p.beta, p.d, p.ldc)) return false;
   f.cls = group_class(gather, p.d, f.bt);
   p.T = static_cast<int>((p.d + f.bt - 1) / f.bt);
   f.ntiles = static_cast<int64_t>(p.T) * (p.T + 1) / 2;
@@ -778,9 +893,11 @@ static bool group_decode(const int64_t* r, GroupFactor& f, int64_t& max_rows_per
 struct GroupPlan {
   std::vector<GroupFactor> factors;
   std::vector<DtlGroupItem> items[kGroupClasses];
-  std::vector<DtlGroupFin> fins[kGroupClasses];
+  std::vector<DtlGroupFin> fins[kGroupClasses];           // plain classes: reduction by accumulator slot
+  std::vector<DtlGroupFinOut> fins_out[kGroupClasses];    // gathered classes: reduction by output position
+  unsigned fin_out_blocks[kGroupClasses] = {};
   size_t ws_f4 = 0;                       // partial tiles, in float4
-  size_t off_factors = 0, off_items[kGroupClasses], off_fins[kGroupClasses], table_bytes = 0;
+  size_t off_factors = 0, off_items[kGroupClasses], off_fins[kGroupClasses], off_fins_out[kGroupClasses], table_bytes = 0;
 };
 
 static int group_plan(const int64_t* specs, int n, GroupPlan& g) {
@@ -886,7 +1003,19 @@ static int group_plan(const int64_t* specs, int n, GroupPlan& g) {
           it.partial = f.nsplit > 1 ? f.part_base + (static_cast<int64_t>(s) * f.ntiles + t) * tile_f4 : -1;
           g.items[c].push_back(it);
         }
-      if (f.nsplit > 1)
+      if (f.nsplit > 1 && c >= 2) {
+        DtlGroupFinOut fin;
+        const unsigned d = static_cast<unsigned>(f.p.d);
+        fin.factor = i;
+        fin.nparts = f.nsplit;
+        fin.col_blocks = static_cast<int32_t>((d + 63) / 64);
+        fin.pad = 0;
+        fin.first = f.part_base;
+        fin.ntiles = f.ntiles;
+        g.fins_out[c].push_back(fin);
+        g.fin_out_blocks[c] = std::max(g.fin_out_blocks[c], ((d + 63) / 64) * ((d + 15) / 16));
+      }
+      if (f.nsplit > 1 && c < 2)
         for (int64_t t = 0; t < f.ntiles; ++t) {
           DtlGroupFin fin;
           fin.factor = i;
@@ -906,6 +1035,7 @@ static int group_plan(const int64_t* specs, int n, GroupPlan& g) {
   for (int c = 0; c < kGroupClasses; ++c) {
     g.off_items[c] = take(sizeof(DtlGroupItem) * g.items[c].size());
     g.off_fins[c] = take(sizeof(DtlGroupFin) * g.fins[c].size());
+    g.off_fins_out[c] = take(sizeof(DtlGroupFinOut) * g.fins_out[c].size());
   }
   g.table_bytes = off;
   return AK_OK;
@@ -934,6 +1064,14 @@ static int group_launch_class(const GroupPlan& g, int c, const unsigned char* ta
     hipLaunchKernelGGL((syrk_dtl_finalize_grouped_kernel<WR, WC, FR, FC, GATHER>),
                        dim3(static_cast<unsigned>(g.fins[c].size()), 4 * FR * FC), dim3(Cfg::NW * 64), 0, stream, factors,
                        fins, static_cast<const floatx4*>(ws));
+  }
+  if constexpr (GATHER) {
+    if (!g.fins_out[c].empty()) {
+      const DtlGroupFinOut* fins = reinterpret_cast<const DtlGroupFinOut*>(tables + g.off_fins_out[c]);
+      hipLaunchKernelGGL((syrk_dtl_finalize_out_grouped_kernel<WR, WC, FR, FC>),
+                         dim3(g.fin_out_blocks[c], static_cast<unsigned>(g.fins_out[c].size())), dim3(256), 0, stream,
+                         factors, fins, static_cast<const floatx4*>(ws));
+    }
   }
   return check_launch();
 }
@@ -972,6 +1110,8 @@ extern "C" int ak_syrk_group_launch(const int64_t* specs, int n, void* host_stag
       std::memcpy(h + g.off_items[c], g.items[c].data(), sizeof(ak::DtlGroupItem) * g.items[c].size());
     if (!g.fins[c].empty())
       std::memcpy(h + g.off_fins[c], g.fins[c].data(), sizeof(ak::DtlGroupFin) * g.fins[c].size());
+    if (!g.fins_out[c].empty())
+      std::memcpy(h + g.off_fins_out[c], g.fins_out[c].data(), sizeof(ak::DtlGroupFinOut) * g.fins_out[c].size());
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (hipMemcpyAsync(dev_tables, host_stage, g.table_bytes, hipMemcpyHostToDevice, s) != hipSuccess) return AK_ERR_LAUNCH;
@@ -1012,6 +1152,7 @@ extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C,
   const int64_t d = C * kh * kw, M = N * Ho * Wo;
   if (lda < d) return AK_ERR_ARG;
   if (dtype != AK_BF16 && dtype != AK_F32) return AK_ERR_ARG;
+  if (!ak::syrk_beta_ok(beta, d, lda)) return AK_ERR_UNSUPPORTED;
   {  // few input channels: the window kernel, any dtype and channel count
     const int rc = ak::conv_patch_syrk(x, dtype, H * W * C, 1, W * C, C, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,
                                        A, lda, ws, ws_bytes, static_cast<hipStream_t>(stream));

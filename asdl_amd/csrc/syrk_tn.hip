@@ -241,6 +241,7 @@ extern "C" size_t ak_syrk_tn_ws_bytes(int64_t M, int64_t d) {
 extern "C" int ak_syrk_tn(const void* X, int dtype, int64_t M, int64_t d, int64_t ldx, float alpha, float beta,
                           float* C, int64_t ldc, void* ws, size_t ws_bytes, ak_stream_t stream) {
   if (X == nullptr || C == nullptr || M < 0 || d <= 0 || ldx < d || ldc < d) return AK_ERR_ARG;
+  if (!ak::syrk_beta_ok(beta, d, ldc)) return AK_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == AK_BF16 && ak::syrk_dtl_plain_ok(X, M, d, ldx)) {
     const int rc = ak::syrk_dtl_plain(X, M, d, ldx, alpha, beta, C, ldc, ws, ws_bytes, s);

@@ -50,7 +50,8 @@ const char* ak_error_string(int code);
 /* ---- Kronecker-factor statistics -------------------------------------------------- */
 
 /* C <- beta*C + alpha * X^T X, X = [M, d] row-major (leading dimension ldx), C = [d, d] fp32,
- * full symmetric on exit (upper triangle computed, mirrored).  beta == 0 never reads C.
+ * full symmetric on exit (upper triangle computed, mirrored).  beta == 0 never reads C; beta != 0 needs C below
+ * 4 GiB (d < 32768 for ldc == d), else AK_ERR_UNSUPPORTED: this holds for all three statistics entry points.
  * Replaces Linear.cov_kron_A / cov_kron_B  (asdl/operations/linear.py:75-77, 87-89), the
  * `.mul_(cov_scale)` and `results[key] += value` passes (asdl/operations/operation.py:133-137,
  * 199-201, 264-266) and the EMA pre-scale Kron.mul_ (asdl/symmatrix.py:448-453), and the 2-D
