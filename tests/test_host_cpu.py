@@ -45,6 +45,25 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert b'workspace' in lib.ak_error_string(-2)
 
 
+def test_no_hot_kernel_spills_registers():
+    """asdl_amd.build writes the compiler's resource figures of every kernel next to the library.  The matrix-core
+    kernels keep their accumulators in registers for the whole k-loop: scratch memory (a spill) in one of them costs
+    a factor of two and more (it happened to the 256-wide gathered SYRK tile after an epilogue change), so none is
+    allowed outside the short list of kernels that have always had a few bytes."""
+    report = os.path.join(os.path.dirname(asdl_amd.__file__), 'lib', 'kernel_resources.txt')
+    if not os.path.exists(report):
+        pytest.skip('no kernel_resources.txt: the library was not built by asdl_amd.build in this tree')
+    allowed = {'conv_patch_syrk_kernel': 16, 'conv_syrk_kernel': 96}        # bytes per lane
+    rows = [l.split() for l in open(report) if l.strip() and not l.startswith('#')]
+    assert len(rows) > 100
+    spilled = []
+    for src, name, vgprs, agprs, scratch, occupancy, lds in rows:
+        limit = max([v for k, v in allowed.items() if k in name] or [0])
+        if int(scratch) > limit:
+            spilled.append((src, name, int(scratch)))
+    assert not spilled, spilled
+
+
 def test_product_refuses_cpu_tensors():
     from asdl_amd import kernels
     with pytest.raises(RuntimeError, match='ROCm device'):
