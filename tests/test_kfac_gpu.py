@@ -13,7 +13,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from asdl_amd import PreconditioningConfig, KfacGradientMaker, FISHER_EMP, FISHER_MC
+from asdl_amd import PreconditioningConfig, KfacGradientMaker, FISHER_EMP, FISHER_MC, FISHER_EXACT
 from conftest import GOLDEN
 from models_small import GOLDEN_KFAC
 from oracle import cpu_ref as R
@@ -678,13 +678,15 @@ def test_factor_side_stream_gives_the_golden_results(tag, monkeypatch):
     test_kfac_gpu_matches_reference_golden(tag)
 
 
-@pytest.mark.parametrize('ema', [-1, 0.3])
-def test_grouped_factor_launches_give_the_single_launch_factors(ema, monkeypatch):
+@pytest.mark.parametrize('ema,fisher_type,n_mc', [(-1, FISHER_EMP, 1), (0.3, FISHER_EMP, 1), (0.3, FISHER_MC, 2), (-1, FISHER_EXACT, 1)])
+def test_grouped_factor_launches_give_the_single_launch_factors(ema, fisher_type, n_mc, monkeypatch):
     """fisher.GROUPED_FACTORS collects the bf16 Kronecker-factor statistics of a pass and launches them together
     (kernels.FactorGroup), at the end of the pass or every few hooks (fisher.GROUP_FLUSH_EVERY).  On a channels-last
     CNN under bf16 autocast (3x3, strided 1x1 and plain 1x1 convolutions, a Linear head; two steps, so that with EMA
     the second one accumulates) every setting has to give the factors of the one-launch-per-factor path up to the
-    summation order (2e-6), inverses within 1e-4 and the same preconditioned gradients (1e-4)."""
+    summation order (2e-6), inverses within 1e-4 and the same preconditioned gradients (1e-4).  With two Monte-Carlo
+    samples or the exact Fisher (one backward pass per class) a factor receives several contributions per step: the
+    group has to launch before it takes the second one."""
     import asdl_amd.fisher as fisher_mod
     torch.manual_seed(31)
     xs = [torch.randn(8, 16, 12, 12).cuda().contiguous(memory_format=torch.channels_last) for _ in range(2)]
@@ -699,7 +701,7 @@ def test_grouped_factor_launches_give_the_single_launch_factors(ema, monkeypatch
                               nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
         model = model.to(memory_format=torch.channels_last)
         gm = KfacGradientMaker(model, PreconditioningConfig(data_size=8, damping=1e-2, ema_decay=ema),
-                               fisher_type=FISHER_EMP)
+                               fisher_type=fisher_type, n_mc_samples=n_mc, seed=7)
 
         def fwd(inp):
             with torch.autocast('cuda', dtype=torch.bfloat16):
@@ -729,9 +731,10 @@ def test_grouped_factor_launches_give_the_single_launch_factors(ema, monkeypatch
     for every in [(0, 0), (-1, 0), (2, 3), (1, 1)]:
         del taken[:]
         got = run(True, every)
-        # per step: B of the four convolutions (the Linear layer's 10 columns are not a multiple of 8), and with
-        # forward grouping A of the four layers that are not the few-channel stem
-        assert len(taken) == 2 * (4 if every[0] < 0 else 8) and (every[0] < 0 or 1 in taken), (every, taken)
+        # per step: B of the four convolutions once per backward pass (the Linear layer's 10 columns are not a
+        # multiple of 8), and with forward grouping A of the four layers that are not the few-channel stem
+        passes = {FISHER_EMP: 1, FISHER_MC: n_mc, FISHER_EXACT: 10}[fisher_type]
+        assert len(taken) == 2 * (4 * passes + (0 if every[0] < 0 else 4)) and (every[0] < 0 or 1 in taken), (every, taken)
         assert got.keys() == ref.keys()
         for key in ref:
             tol = 2e-6 if key.endswith(('.A', '.B')) else 1e-4
