@@ -1,6 +1,7 @@
 """Hook engine: the ``extend`` context attaches one Operation per supported leaf module and calls
 it from a forward hook and from a hook on the gradient of the module's output
 (role of asdl/core.py:20-97, 130-244)."""
+import sys
 from contextlib import contextmanager, nullcontext
 
 import torch
@@ -77,6 +78,13 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
         for handle in handles:
             handle.remove()
         cxt.clear_operations()
+        if hasattr(cxt.factor_stream, 'discard'):
+            # factor calls that were recorded but not launched yet: dropped if the pass ended in an exception,
+            # launched otherwise (the consumers above all call join_factor_stream() themselves)
+            if sys.exc_info()[0] is not None:
+                cxt.factor_stream.discard()
+            else:
+                cxt.factor_stream.join()
 
 
 def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, vectors=None, stream=None,

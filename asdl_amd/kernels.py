@@ -370,6 +370,10 @@ class FactorGroup:
         self._keep.append(tensors)
         self._flops += flops
 
+    def discard(self):
+        """Forgets what has been collected without launching it (a pass that ended in an exception)."""
+        self._rows, self._keep, self._outs, self._flops = [], [], set(), 0
+
     def flush(self):
         """Launches what has been collected on the calling thread's launch stream."""
         if not self._rows:
@@ -459,6 +463,10 @@ class DeferredFactors:
         self._count = 0
         self.group.flush()
         return []
+
+    def discard(self):
+        self._count = 0
+        self.group.discard()
 
 
 def _group_take(row, flops, align_key, *tensors):

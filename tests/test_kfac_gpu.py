@@ -741,6 +741,44 @@ def test_grouped_factor_launches_give_the_single_launch_factors(ema, fisher_type
             assert relerr(got[key], ref[key]) < tol, (every, key, relerr(got[key], ref[key]))
 
 
+def test_grouped_factors_are_dropped_when_the_pass_raises():
+    """Factor calls recorded by the hooks of a pass that ends in an exception are not launched later on (their
+    tensors belong to a step that never finished); the maker works as before on the next call."""
+    torch.manual_seed(41)
+    model = nn.Sequential(nn.Conv2d(16, 32, 1), nn.ReLU(), nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 16)).cuda()
+    model = model.to(memory_format=torch.channels_last)
+    gm = KfacGradientMaker(model, PreconditioningConfig(data_size=4, damping=1e-2), fisher_type=FISHER_EMP)
+    x = torch.randn(4, 16, 6, 6).cuda().contiguous(memory_format=torch.channels_last)
+    t = torch.randint(16, (4,)).cuda()
+    state = {'fail': True}
+
+    def fwd(inp):
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            return model(inp).float()
+
+    def loss_fn(y, target, reduction='mean'):
+        if state['fail']:
+            raise RuntimeError('boom')
+        return F.cross_entropy(y, target, reduction=reduction)
+
+    gm.setup_loss_call(loss_fn, gm.setup_model_call(fwd, x), t)
+    import asdl_amd.fisher as fisher_mod
+    saved = fisher_mod.GROUP_FLUSH_EVERY
+    fisher_mod.GROUP_FLUSH_EVERY = (0, 0)          # the forward hooks record too
+    try:
+        with pytest.raises(RuntimeError, match='boom'):
+            gm.forward_and_backward()
+        group = gm.fisher_maker._factor_stream_obj.group
+        assert len(group) == 0
+        state['fail'] = False
+        gm.forward_and_backward()
+        assert len(group) == 0
+    finally:
+        fisher_mod.GROUP_FLUSH_EVERY = saved
+    torch.cuda.synchronize()
+    assert model[0].fisher.kron.A_inv is not None and torch.isfinite(model[0].weight.grad).all()
+
+
 def test_fisher_attributes_and_steps_without_curvature_update():
     torch.manual_seed(4)
     model = bench_models.mlp(20, 16, 5).cuda()
