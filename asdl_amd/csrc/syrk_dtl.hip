@@ -583,6 +583,107 @@ __global__ __launch_bounds__(256) void syrk_dtl_finalize_out_kernel(DtlParams p,
   dtl_finalize_out<WR, WC, FR, FC>(p, part, ntiles, n, blockIdx.x, blockIdx.y);
 }
 
+// The same reduction, staged through the LDS: every partial tile is read with whole-line float4 loads and every
+// result line is stored whole, the mirror image included.  The permutation between the working order and the result
+// order stays inside a channel group of G * KK columns, so a work group takes four channels of rows (4 * KK result
+// rows: KK float4 rows of the partial tiles) and cpb channels of columns (cpb * KK result columns, cpb a divisor of
+// G), sums its float4 over the splits, scatters them into an LDS block in result order and stores the block row by
+// row.  Column blocks in a channel group right of the rows' group also store the transposed block (runs of 4 * KK
+// floats); blocks in the rows' own group are each computed by their own work group (elements whose tile lies below
+// the diagonal read the mirror image, four floats), blocks left of it are those transposed stores.
+// grid (Cin / cpb, Cin / 4), 256 threads, 4 * KK * (cpb * KK + 1) floats of LDS.
+template <int WR, int WC, int FR, int FC>
+__global__ __launch_bounds__(256) void syrk_dtl_finalize_blk_kernel(DtlParams p, const floatx4* __restrict__ part,
+                                                                    int64_t ntiles, int n, int cpb) {
+  constexpr int NW = WR * WC, BT = 32 * FR * WR;
+  constexpr size_t tile_f4 = static_cast<size_t>(BT) * BT / 4;
+  extern __shared__ float blk_lds[];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t KK = p.KK, G = p.G, GKK = G * KK;
+  const uint32_t ci0 = blockIdx.y * 4, cj0 = blockIdx.x * cpb;          // first channel of the rows / of the columns
+  const uint32_t grp_i = fastdiv(ci0, p.mG, G), grp_j = fastdiv(cj0, p.mG, G);
+  if (grp_j < grp_i) return;
+  const uint32_t cols = cpb * KK, rows = 4 * KK, lw = cols + 1;
+  auto slot_of = [](uint32_t r, uint32_t c, uint32_t& e) {
+    const uint32_t wr = r / (32 * FR), a = (r % (32 * FR)) / 32, r32 = r % 32, q = r32 / 8, g = (r32 % 8) / 4;
+    const uint32_t wc = c / (32 * FC), b = (c % (32 * FC)) / 32, l32 = c % 32;
+    e = r32 % 4;
+    return ((a * FC + b) * 4 + q) * (NW * 64) + (wr * WC + wc) * 64 + g * 32 + l32;
+  };
+  const size_t split_stride = static_cast<size_t>(ntiles) * tile_f4;
+  const uint32_t vi_base = grp_i * GKK + (ci0 - grp_i * G), vj_base = grp_j * GKK + (cj0 - grp_j * G);
+  for (uint32_t item = tid; item < KK * cols; item += 256) {
+    const uint32_t tap_i = item / cols, idx = item - tap_i * cols;
+    const uint32_t vi = vi_base + tap_i * G;                              // four consecutive working rows
+    const uint32_t ti = vi / BT;
+    {
+      const uint32_t tap_j = idx / cpb, cgl = idx - tap_j * cpb;
+      const uint32_t vj = vj_base + tap_j * G + cgl;
+      const uint32_t tj = vj / BT;
+      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+      if (ti <= tj) {
+        const size_t tile = static_cast<size_t>(ti) * p.T - static_cast<size_t>(ti) * (ti - 1) / 2 + (tj - ti);
+        uint32_t e;
+        const floatx4* src = part + tile * tile_f4 + slot_of(vi % BT, vj % BT, e);
+        int s = 0;
+        for (; s + 8 <= n; s += 8) {                                      // eight loads in flight, summed in order
+          floatx4 w[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) w[k] = src[(s + k) * split_stride];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc += w[k];
+        }
+        for (; s < n; ++s) acc += src[s * split_stride];
+      } else {
+        const size_t tile = static_cast<size_t>(tj) * p.T - static_cast<size_t>(tj) * (tj - 1) / 2 + (ti - tj);
+        const float* base = reinterpret_cast<const float*>(part + tile * tile_f4);
+        size_t off[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          uint32_t e;
+          const uint32_t f4 = slot_of(vj % BT, (vi + k) % BT, e);
+          off[k] = static_cast<size_t>(f4) * 4 + e;
+        }
+        int s = 0;
+        for (; s + 2 <= n; s += 2) {
+          const float* q0 = base + static_cast<size_t>(s) * split_stride * 4;
+          const float* q1 = q0 + split_stride * 4;
+          const float x0 = q0[off[0]], x1 = q0[off[1]], x2 = q0[off[2]], x3 = q0[off[3]];
+          const float y0 = q1[off[0]], y1 = q1[off[1]], y2 = q1[off[2]], y3 = q1[off[3]];
+          acc[0] += x0; acc[1] += x1; acc[2] += x2; acc[3] += x3;
+          acc[0] += y0; acc[1] += y1; acc[2] += y2; acc[3] += y3;
+        }
+        for (; s < n; ++s) {
+          const float* q = base + static_cast<size_t>(s) * split_stride * 4;
+          acc[0] += q[off[0]]; acc[1] += q[off[1]]; acc[2] += q[off[2]]; acc[3] += q[off[3]];
+        }
+      }
+      const uint32_t col = cgl * KK + tap_j;                              // result column inside the block
+#pragma unroll
+      for (int e = 0; e < 4; ++e) blk_lds[(e * KK + tap_i) * lw + col] = acc[e];
+    }
+  }
+  __syncthreads();
+  // the block, row by row: C[ci0 * KK + r][cj0 * KK + c]
+  float* dst = p.C + static_cast<int64_t>(ci0) * KK * p.ldc + static_cast<int64_t>(cj0) * KK;
+  for (uint32_t idx = tid; idx < rows * cols; idx += 256) {
+    const uint32_t r = idx / cols, c = idx - r * cols;
+    float v = p.alpha * blk_lds[r * lw + c];
+    float* q = dst + static_cast<int64_t>(r) * p.ldc + c;
+    if (p.beta != 0.f) v += p.beta * *q;
+    *q = v;
+    blk_lds[r * lw + c] = v;                                              // the mirror image stores the same value
+  }
+  if (grp_j == grp_i) return;
+  __syncthreads();
+  // the transposed block: C[cj0 * KK + c][ci0 * KK + r]
+  float* dst_t = p.C + static_cast<int64_t>(cj0) * KK * p.ldc + static_cast<int64_t>(ci0) * KK;
+  for (uint32_t idx = tid; idx < rows * cols; idx += 256) {
+    const uint32_t c = idx / rows, r = idx - c * rows;
+    dst_t[static_cast<int64_t>(c) * p.ldc + r] = blk_lds[r * lw + c];
+  }
+}
+
 // The same for the gathered factors of a grouped launch: grid (column blocks x row blocks of the widest factor,
 // factors with partial tiles); work groups beyond a narrower factor's blocks leave at once.
 struct DtlGroupFinOut {
@@ -717,6 +818,22 @@ static DtlPlan dtl_plan(int64_t M, int64_t d, int64_t max_rows_per_split, bool g
   return plan;
 }
 
+// Channels per column block of the LDS-staged reduction pass of a gathered factor (0: use the pass by output
+// position): a divisor of G small enough for 64 KB of LDS and for at least ~2 work groups per CU.
+static int dtl_blk_channels(const DtlParams& p) {
+  if (p.KK < 2 || p.Cin % 4 != 0 || p.G % 4 != 0 || p.Cin % p.G != 0) return 0;
+  int cpb = 0;
+  for (int c = p.G; c >= 4; c /= 2) {
+    if (p.G % c != 0) break;
+    const size_t lds = static_cast<size_t>(4 * p.KK) * (c * p.KK + 1) * sizeof(float);
+    if (lds > 64 * 1024) continue;
+    cpb = c;
+    const int64_t wgs = static_cast<int64_t>(p.Cin / c) * (p.Cin / 4) / 2;     // about half are above the diagonal
+    if (wgs >= 512) break;
+  }
+  return cpb;
+}
+
 template <int WR, int WC, int FR, int FC, bool GATHER>
 static int dtl_launch_cfg(const DtlParams& p, const DtlPlan& pl, hipStream_t stream) {
   using Cfg = DtlCfg<WR, WC, FR, FC, GATHER>;
@@ -745,8 +862,15 @@ static int dtl_launch_cfg(const DtlParams& p, const DtlPlan& pl, hipStream_t str
     }
     if constexpr (GATHER) {
       const unsigned d = static_cast<unsigned>(p.d);
-      hipLaunchKernelGGL((syrk_dtl_finalize_out_kernel<WR, WC, FR, FC>), dim3((d + 63) / 64, (d + 15) / 16), dim3(256),
-                         0, stream, p, part, pl.ntiles, n);
+      const int cpb = dtl_blk_channels(p);
+      if (cpb > 0) {
+        const size_t lds = static_cast<size_t>(4 * p.KK) * (cpb * p.KK + 1) * sizeof(float);
+        hipLaunchKernelGGL((syrk_dtl_finalize_blk_kernel<WR, WC, FR, FC>), dim3(p.Cin / cpb, p.Cin / 4), dim3(256), lds,
+                           stream, p, part, pl.ntiles, n, cpb);
+      } else {
+        hipLaunchKernelGGL((syrk_dtl_finalize_out_kernel<WR, WC, FR, FC>), dim3((d + 63) / 64, (d + 15) / 16),
+                           dim3(256), 0, stream, p, part, pl.ntiles, n);
+      }
     } else {
       hipLaunchKernelGGL((syrk_dtl_finalize_kernel<WR, WC, FR, FC, GATHER>), dim3(ntiles, 4 * FR * FC),
                          dim3(Cfg::NW * 64), 0, stream, p, part, n);

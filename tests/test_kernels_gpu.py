@@ -214,6 +214,35 @@ def test_syrk_tn_bf16_split_k_and_strided(K, M, d, ld):
     assert torch.equal(out, out.T)
 
 
+@pytest.mark.parametrize('N,C,H,k,s,p', [(8, 64, 28, 3, 1, 1),      # G = 32, 9 taps
+                                         (8, 24, 28, 3, 1, 1),      # G = C = 24 (not a multiple of 32)
+                                         (8, 32, 20, 5, 1, 2),      # 25 taps: four channels per column block
+                                         (8, 40, 24, 2, 2, 0),      # 4 taps, G = 40
+                                         (16, 8, 40, 5, 1, 2),      # G = 8 (few channels, but more than 160 columns)
+                                         (64, 256, 14, 3, 1, 1)])   # 8 channel groups: blocks right of the diagonal
+def test_gathered_factor_reduction_pass_variants(K, N, C, H, k, s, p):
+    """Split gathered factors end in a reduction pass that permutes the working column order (c/G, tap, c%G) into
+    the result order (c, tap), staged through the LDS in blocks of a few channels.  Shapes with different group
+    sizes G, tap counts and block counts, all of them split along the rows (their workspace query is non-zero),
+    against the fp64 product of the unfolded input; alpha and beta (the EMA form) included."""
+    import torch.nn.functional as F
+    from asdl_amd import _lib
+    assert _lib.load().ak_conv_syrk_nhwc_ws_bytes(N, C, H, H, k, k, s, s, p, p) > 0, 'this case should be split'
+    torch.manual_seed(C + k)
+    x = torch.randn(N, C, H, H, device='cuda').to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+    d = C * k * k
+    u = F.unfold(x.double(), k, padding=p, stride=s).transpose(1, 2).reshape(-1, d)
+    old = torch.randn(d, d, device='cuda')
+    old = old + old.T
+    ref = 0.25 * (u.T @ u) + 0.5 * old.double()
+    out = old.clone()
+    print(f'gathered reduction N={N} C={C} H={H} k={k} s={s} p={p}', flush=True)
+    K.conv_syrk(x, (k, k), (s, s), (p, p), out=out, alpha=0.25, beta=0.5)
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5
+    assert torch.equal(out, out.T)
+
+
 def _group_cases():
     """(kind, args): plain [M, d] operands (with a row stride, ragged sizes, a result with a wide row stride) and
     channels-last convolution inputs (3x3, strided 1x1, 5x5 with padding), small and at the benchmark's sizes."""
