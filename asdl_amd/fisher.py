@@ -22,11 +22,14 @@ __all__ = ['FisherConfig', 'get_fisher_maker', 'FisherMaker']
 _supported_types = [FISHER_EXACT, FISHER_MC, FISHER_EMP]
 _invalid_data_size = -1
 GROUPED_FACTORS = True     # the Kronecker factors of a forward + backward pass in one grouped launch (kernels.FactorGroup) instead of one launch per factor
-GROUP_FLUSH_EVERY = (-1, 0)  # (forward, backward): launch the group after that many hooks of the pass (0: once, when the pass
-                             # has ended; -1: that pass launches its factors one by one).  The forward pass of the benchmark is
-                             # bound by the host's launch rate, so its factor kernels cost nothing where they are; the backward
-                             # pass is not (ResNet-50 batch 64 in one process: 27.1 ms per step with single launches, 27.5 with
-                             # (0, 0), 27.2 with (8, 0), 26.75 with (-1, 0))
+GROUP_FLUSH_EVERY = (-2, 0)  # (forward, backward): launch the group after that many hooks of the pass (0: once, when the pass
+                             # has ended; -1: that pass launches its factors one by one; -2: it launches its unfolded
+                             # factors one by one and leaves its plain X^T X factors to the group).  The forward pass of
+                             # the benchmark sits at the balance of the host's launch rate and the device, so most of its
+                             # factor kernels cost nothing where they are, and the grouped plain factors take half the
+                             # time of their single launches; the backward pass is bound by the device (ResNet-50 batch
+                             # 64 in one process: 26.9 ms per step with single launches, 27.4 with (0, 0), 26.3 with
+                             # (-1, 0), 26.0 with (-2, 0))
 FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (ordering the two streams costs ~30 us of host time per hook: more than the overlap gains)
 PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
 EAGER_INVERSE = True        # start the bulk of the inverses during a single sampled / empirical backward pass: the longest chains get a head start

@@ -342,6 +342,7 @@ class FactorGroup:
         self.device = torch.device(device)
         self._rows, self._keep, self._outs, self._flops = [], [], set(), 0
         self._sizes = {}
+        self.plain_only = False      # take X^T X calls only: unfolded inputs are launched at once
         self._slots = [dict(host=None, dev=None, event=None) for _ in range(self.SLOTS)]
         self._next = 0
 
@@ -434,7 +435,8 @@ class DeferredFactors:
     """Stands where a FactorStream stands (OperationContext.factor_stream): the hook operations run at once, on the
     caller's stream, but the factor statistics they ask for are collected in a FactorGroup; join() launches what is
     left of them.  ``every`` = (forward, backward): the group is also launched after that many hook calls of the
-    pass (0: only at join(); -1: the hooks of that pass launch their factors one by one, as without a group)."""
+    pass (0: only at join(); -1: the hooks of that pass launch their factors one by one, as without a group; -2: only
+    the plain X^T X factors of that pass are collected, until join(), the unfolded ones are launched at once)."""
 
     def __init__(self, device, every=(0, 0)):
         self.device = torch.device(device)
@@ -444,16 +446,17 @@ class DeferredFactors:
 
     def run(self, fn, *tensors, backward=False):
         every = self.every[1 if backward else 0]
-        if every < 0:
+        if every == -1:
             self.group.flush()
             fn()
             return
-        saved = getattr(_group, 'active', None)
+        saved = getattr(_group, 'active', None), self.group.plain_only
         _group.active = self.group
+        self.group.plain_only = every == -2
         try:
             fn()
         finally:
-            _group.active = saved
+            _group.active, self.group.plain_only = saved
         self._count += 1
         if every > 0 and self._count >= every:
             self._count = 0
@@ -472,7 +475,7 @@ class DeferredFactors:
 def _group_take(row, flops, align_key, *tensors):
     """True when the calling thread has an active group and it has taken the call."""
     grp = getattr(_group, 'active', None)
-    if grp is None or not FactorGroup.eligible(row, align_key):
+    if grp is None or (grp.plain_only and row[0] != 0) or not FactorGroup.eligible(row, align_key):
         return False
     grp.add(row, flops, *tensors)
     return True

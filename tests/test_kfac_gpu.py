@@ -681,7 +681,8 @@ def test_factor_side_stream_gives_the_golden_results(tag, monkeypatch):
 @pytest.mark.parametrize('ema,fisher_type,n_mc', [(-1, FISHER_EMP, 1), (0.3, FISHER_EMP, 1), (0.3, FISHER_MC, 2), (-1, FISHER_EXACT, 1)])
 def test_grouped_factor_launches_give_the_single_launch_factors(ema, fisher_type, n_mc, monkeypatch):
     """fisher.GROUPED_FACTORS collects the bf16 Kronecker-factor statistics of a pass and launches them together
-    (kernels.FactorGroup), at the end of the pass or every few hooks (fisher.GROUP_FLUSH_EVERY).  On a channels-last
+    (kernels.FactorGroup), at the end of the pass or every few hooks, all or only the plain ones of the forward pass
+    (fisher.GROUP_FLUSH_EVERY).  On a channels-last
     CNN under bf16 autocast (3x3, strided 1x1 and plain 1x1 convolutions, a Linear head; two steps, so that with EMA
     the second one accumulates) every setting has to give the factors of the one-launch-per-factor path up to the
     summation order (2e-6), inverses within 1e-4 and the same preconditioned gradients (1e-4).  With two Monte-Carlo
@@ -728,13 +729,20 @@ def test_grouped_factor_launches_give_the_single_launch_factors(ema, fisher_type
     ref = run(False, (0, 0))
     assert not taken
     assert any(k.endswith('A_inv') for k in ref) and (ema == -1 or any(k.endswith('.A') for k in ref))
-    for every in [(0, 0), (-1, 0), (2, 3), (1, 1)]:
+    plain_forward = None
+    for every in [(0, 0), (-1, 0), (-2, 0), (2, 3), (-2, 2), (1, 1)]:
         del taken[:]
         got = run(True, every)
         # per step: B of the four convolutions once per backward pass (the Linear layer's 10 columns are not a
-        # multiple of 8), and with forward grouping A of the four layers that are not the few-channel stem
+        # multiple of 8), and with forward grouping A of the four layers that are not the few-channel stem; with
+        # -2 only those of them that are plain X^T X products (kind 0, like every B)
         passes = {FISHER_EMP: 1, FISHER_MC: n_mc, FISHER_EXACT: 10}[fisher_type]
-        assert len(taken) == 2 * (4 * passes + (0 if every[0] < 0 else 4)) and (every[0] < 0 or 1 in taken), (every, taken)
+        if plain_forward is None:
+            plain_forward = taken.count(0) - 2 * 4 * passes
+            assert 0 < plain_forward < 2 * 4
+        forward = {-1: 0, -2: plain_forward}.get(every[0], 2 * 4)
+        assert len(taken) == 2 * 4 * passes + forward and (every[0] < 0 or 1 in taken), (every, taken)
+        assert every[0] != -2 or 1 not in taken
         assert got.keys() == ref.keys()
         for key in ref:
             tol = 2e-6 if key.endswith(('.A', '.B')) else 1e-4
