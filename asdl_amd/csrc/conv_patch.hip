@@ -7,7 +7,16 @@
 // window: lane l of v_mfma_f32_32x32x2_f32 supplies patch element (32*block + l%32) of position (2*step + l/32).
 // The lower 32 x 32 tiles of the (padded) d x d result are spread over the 8 waves; a work group walks over
 // several strips and writes one partial per wave and tile slot, summed by a second kernel that also applies
-// alpha / beta and mirrors the result.  Input: fp32 or bf16 with arbitrary element strides (NCHW and NHWC alike).
+// alpha / beta and mirrors the result.  Input: fp32 with arbitrary element strides (NCHW and NHWC alike).
+//
+// bf16 input, and fp32 input that is to be rounded to bf16 (AK_F32_AS_BF16), goes to the bf16 matrix instruction
+// instead (conv_patch_bf16_kernel): the window is kept as bf16, a lane gathers the same patch element of 8
+// consecutive output positions of a row (v_mfma_f32_32x32x16_bf16 wants lane l to hold k = 8*(l/32) .. +7 of row
+// l%32, the same layout for both operands of X^T X, so one fragment per 32-block of patch elements serves as
+// row operand and as column operand), and every wave keeps ALL lower tiles (15 for d = 147) in its accumulators:
+// 5 fragments of 8 two-byte LDS reads feed 15 matrix instructions, which leaves the kernel bound by the matrix
+// cores and not by the LDS.  One work group of 4 waves per CU; the four waves' tiles are summed through the LDS
+// before they go to the workspace.
 #include "common.hpp"
 
 namespace ak {
@@ -28,7 +37,15 @@ struct PatchParams {
   int chan_inner;                // 1: channels are the fastest-moving input axis (NHWC)
   int d, nb, ntiles, tpw, KS;    // 32-blocks, lower tiles, tiles per wave, position slices per tile
   uint32_t mKK, mKw, mPC, mC, mPRPC;
-  float* ws;                     // [grid][wave][slot][16][64]
+  // bf16 kernel: its window is Q rows of L elements in the order of the input's memory, [window row][column][channel]
+  // for a channels-last input (Q = PR, L = PC*C) and [channel][window row][column] otherwise (Q = C*PR, L = PC);
+  // LDS row stride RSb.  Patch element (c, ky, kx) of output position (r, ox) of the strip is LDS element
+  // c*tap_c + ky*RSb + kx*tap_x + r*strh*RSb + ox*strw*tap_x.
+  int G;                         // groups of 8 output positions per output row
+  uint32_t mG;
+  int Q, L, RSb, tap_c, tap_x, lead, Lvalid;   // lead: window columns left of the input (padding), Lvalid: W*C or W
+  uint32_t mL;
+  float* ws;                     // [grid][wave][slot][16][64]; bf16 kernel: [grid][tile][16][64]
   int nwg;
   float alpha, beta;
   float* A;
@@ -236,11 +253,250 @@ static __global__ __launch_bounds__(256) void conv_patch_reduce_kernel(PatchPara
   if (i != j) p.A[static_cast<int64_t>(j) * p.lda + i] = v;
 }
 
+// ---- bf16 matrix-instruction variant ------------------------------------------------------------------------
+constexpr int kPbWaves = 4;
+constexpr int kPbThreads = kPbWaves * 64;
+constexpr int kPbStage = 64;                              // window elements per thread
+constexpr int kPbMaxWindow = kPbStage * kPbThreads;       // 16384 bf16 elements = 32 KB
+
+__device__ __forceinline__ uint32_t lds_u16(uint32_t byte_addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) uint16_t*>(byte_addr);
+}
+
+template <typename T>
+__device__ __forceinline__ uint16_t patch_bf16_bits(T v);
+template <>
+__device__ __forceinline__ uint16_t patch_bf16_bits<uint16_t>(uint16_t v) { return v; }
+template <>
+__device__ __forceinline__ uint16_t patch_bf16_bits<float>(float v) {      // round to nearest even
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
+}
+
+// NB: 32-blocks of patch elements (d <= 32 * NB); the wave holds the NB (NB + 1) / 2 lower tiles.  INNER: channels-last
+// input (x[n][iy][ix][c] contiguous).
+template <typename T, int NB, bool INNER>
+static __global__ __launch_bounds__(kPbThreads) void conv_patch_bf16_kernel(PatchParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char pb_smem[];
+  constexpr int NT = NB * (NB + 1) / 2;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, kg = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t smem_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(pb_smem));
+
+  // LDS byte address of this lane's patch element (at output position 0 of the strip) in each 32-block; padding
+  // elements (>= d) read element 0: their rows / columns are computed from any data and never stored
+  uint32_t tap[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const uint32_t i = static_cast<uint32_t>(32 * b + l32);
+    uint32_t o = 0;
+    if (i < static_cast<uint32_t>(p.d)) {
+      const uint32_t c = fastdiv(i, p.mKK, p.kh * p.kw);
+      const uint32_t rem = i - c * p.kh * p.kw;
+      const uint32_t ky = fastdiv(rem, p.mKw, p.kw);
+      const uint32_t kx = rem - ky * p.kw;
+      o = (c * p.tap_c + ky * p.RSb + kx * p.tap_x) * 2;
+    }
+    tap[b] = smem_base + o;
+  }
+  const uint32_t sw2 = static_cast<uint32_t>(p.strw * p.tap_x) * 2;       // bytes between neighbouring output positions
+  floatx16 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx16{};
+  const T* __restrict__ x = static_cast<const T*>(p.x);
+  const int window = p.Q * p.L;
+  const int sh = static_cast<int>(p.sh), sw = static_cast<int>(p.sw), sc = static_cast<int>(p.sc);
+
+  // Window elements of one strip, fetched into registers one strip ahead: element idx is column idx % L of window
+  // row idx / L.  The index is made opaque to the optimiser, so that row and column are recomputed for every strip
+  // instead of being kept in registers for all 64 elements, which the accumulators leave no room for.
+  T stage[kPbStage];
+  auto fetch = [&](int strip) {
+    const int n = strip / p.strips_per_image;
+    const int iy0 = (strip - n * p.strips_per_image) * p.R * p.strh - p.ph;
+    const T* __restrict__ xn = x + static_cast<int64_t>(n) * p.sn;
+#pragma unroll
+    for (int e = 0; e < kPbStage; ++e) {
+      int idx = tid + e * kPbThreads;
+      asm volatile("" : "+v"(idx));
+      const uint32_t q = fastdiv(idx, p.mL, p.L);
+      const int m = idx - static_cast<int>(q) * p.L - p.lead;      // column of the input row (times C + channel)
+      int iy, off;
+      if (INNER) {
+        iy = iy0 + static_cast<int>(q);
+        off = iy * sh + m;
+      } else {
+        const uint32_t c = fastdiv(q, p.mPRPC, p.PR);
+        iy = iy0 + static_cast<int>(q - c * p.PR);
+        off = static_cast<int>(c) * sc + iy * sh + m * sw;
+      }
+      T v = 0;
+      if (idx < window && static_cast<uint32_t>(iy) < static_cast<uint32_t>(p.H) &&
+          static_cast<uint32_t>(m) < static_cast<uint32_t>(p.Lvalid))
+        v = xn[off];
+      stage[e] = v;
+    }
+  };
+  auto stash = [&]() {
+    uint16_t* const win = reinterpret_cast<uint16_t*>(pb_smem);
+#pragma unroll
+    for (int e = 0; e < kPbStage; ++e) {
+      int idx = tid + e * kPbThreads;
+      asm volatile("" : "+v"(idx));
+      if (idx >= window) break;
+      const uint32_t q = fastdiv(idx, p.mL, p.L);
+      win[idx + q * (p.RSb - p.L)] = patch_bf16_bits<T>(stage[e]);
+    }
+  };
+  // the fragments of one step: 8 consecutive output positions (from byte offset off, `valid` of them exist) of this
+  // lane's patch element in every 32-block
+  auto load_frags = [&](bf16x8 (&f)[NB], uint32_t off, int valid) {
+    if (__all(valid == 8)) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const uint32_t a = tap[b] + off;
+        uint32_t w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) w[q] = lds_u16(a + (2 * q) * sw2) | (lds_u16(a + (2 * q + 1) * sw2) << 16);
+        f[b] = __builtin_bit_cast(bf16x8, w);
+      }
+    } else {                                   // end of a row / of the strip: missing positions are zero
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const uint32_t a = tap[b] + off;
+        uint32_t w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint32_t lo = lds_u16(2 * q < valid ? a + (2 * q) * sw2 : smem_base);
+          uint32_t hi = lds_u16(2 * q + 1 < valid ? a + (2 * q + 1) * sw2 : smem_base);
+          if (2 * q >= valid) lo = 0;
+          if (2 * q + 1 >= valid) hi = 0;
+          w[q] = lo | (hi << 16);
+        }
+        f[b] = __builtin_bit_cast(bf16x8, w);
+      }
+    }
+  };
+
+  if (static_cast<int>(blockIdx.x) < p.total_strips) fetch(blockIdx.x);
+  for (int strip = blockIdx.x; strip < p.total_strips; strip += gridDim.x) {
+    const int n = strip / p.strips_per_image;
+    const int oy0 = (strip - n * p.strips_per_image) * p.R;
+    const int rows = min(p.R, p.Ho - oy0);
+    __syncthreads();                              // the previous strip's reads are done
+    stash();
+    __syncthreads();
+    if (strip + static_cast<int>(gridDim.x) < p.total_strips) fetch(strip + gridDim.x);
+    const int ngroups = rows * p.G;               // groups of 8 positions; a step multiplies two of them
+    const int nsteps = (ngroups + 1) >> 1;
+    auto locate = [&](int st, uint32_t& off, int& valid) {
+      const int g = 2 * st + kg;
+      const uint32_t r = fastdiv(g, p.mG, p.G);
+      const int ox0 = (g - static_cast<int>(r) * p.G) * 8;
+      valid = g < ngroups ? min(8, p.Wo - ox0) : 0;
+      off = valid > 0 ? r * p.strh * p.RSb * 2 + ox0 * sw2 : 0;
+    };
+    if (wave < nsteps) {
+      bf16x8 cur[NB], nxt[NB];
+      uint32_t off;
+      int valid;
+      locate(wave, off, valid);
+      load_frags(cur, off, valid);
+      for (int st = wave; st < nsteps; st += kPbWaves) {
+        const bool more = st + kPbWaves < nsteps;
+        if (more) {                                // the next step's operands are read before this step's products
+          locate(st + kPbWaves, off, valid);
+          load_frags(nxt, off, valid);
+        }
+        int t = 0;
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+          for (int bj = 0; bj <= bi; ++bj, ++t) acc[t] = mfma_bf16(cur[bi], cur[bj], acc[t]);
+        if (more) {
+#pragma unroll
+          for (int b = 0; b < NB; ++b) cur[b] = nxt[b];
+        }
+      }
+    }
+  }
+  // The four waves' tiles are summed through the LDS in a fixed order, ((w3 + w2) + w1) + w0: a wave writes its tiles,
+  // the next one adds them to its own (write-only and read-only passes, so the LDS accesses of a pass are in flight
+  // together), and wave 0 stores the work group's partial.
+  float* const red = reinterpret_cast<float*>(pb_smem);
+  __syncthreads();
+  for (int w = kPbWaves - 1; w > 0; --w) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[(t * 16 + e) * 64 + lane] = acc[t][e];
+    }
+    __syncthreads();
+    if (wave == w - 1) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] += red[(t * 16 + e) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);          // a tile at a time: the reads of all tiles at once would not fit the registers
+      }
+    }
+    __syncthreads();
+  }
+  if (wave == 0) {
+    float* __restrict__ out = p.ws + static_cast<int64_t>(blockIdx.x) * NT * 1024;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) out[(t * 16 + e) * 64 + lane] = acc[t][e];
+  }
+}
+
+// Sums the work groups' partials: a block takes 32 groups of four neighbouring tile elements, its 8 thread rows a
+// slice of the partials each; the slices are added in a fixed order, then alpha / beta and the mirror image.
+static __global__ __launch_bounds__(256) void conv_patch_bf16_reduce_kernel(PatchParams p) {
+  __shared__ floatx4 part[8][32];
+  const int q = blockIdx.x * 32 + (threadIdx.x & 31), slice = threadIdx.x >> 5;
+  const floatx4* __restrict__ w = reinterpret_cast<const floatx4*>(p.ws) + q;
+  const int64_t step = static_cast<int64_t>(p.ntiles) * 256;
+  floatx4 s[4] = {floatx4{}, floatx4{}, floatx4{}, floatx4{}};
+  int g = slice;
+  for (; g + 24 < p.nwg; g += 32) {
+    s[0] += w[(g + 0) * step];
+    s[1] += w[(g + 8) * step];
+    s[2] += w[(g + 16) * step];
+    s[3] += w[(g + 24) * step];
+  }
+  for (; g < p.nwg; g += 8) s[0] += w[g * step];
+  part[slice][threadIdx.x & 31] = (s[0] + s[1]) + (s[2] + s[3]);
+  __syncthreads();
+  if (slice != 0) return;
+  floatx4 sum = part[0][threadIdx.x];
+#pragma unroll
+  for (int k = 1; k < 8; ++k) sum += part[k][threadIdx.x];
+  const int t = q >> 8, el = (q & 255) * 4;            // tile; reg * 64 + lane of the first of the four elements
+  int bi, bj;
+  patch_tile_blocks(t, bi, bj);
+  const int reg = el >> 6, lane = el & 63;
+  const int i = 32 * bi + 8 * (reg >> 2) + 4 * (lane >> 5) + (reg & 3);
+  if (i >= p.d) return;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int j = 32 * bj + (lane & 31) + k;
+    if (j >= p.d || (bi == bj && j > i)) continue;
+    float v = p.alpha * sum[k];
+    float* dst = p.A + static_cast<int64_t>(i) * p.lda + j;
+    if (p.beta != 0.f) v += p.beta * *dst;
+    *dst = v;
+    if (i != j) p.A[static_cast<int64_t>(j) * p.lda + i] = v;
+  }
+}
+
 // Fills the plan; false when the layer is not one for this kernel.
 static bool conv_patch_plan(PatchParams& p, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
                      int pw) {
   const int64_t d = C * kh * kw;
   if (d > kPatchMaxD || kh * kw == 1 || N > (1 << 20) || H > (1 << 15) || W > (1 << 15)) return false;
+  if (C * H * W >= (1ll << 31)) return false;           // offsets inside an image are 32-bit
   const int64_t Ho = (H + 2 * ph - kh) / sh + 1, Wo = (W + 2 * pw - kw) / sw + 1;
   if (Ho <= 0 || Wo <= 0) return false;
   const int64_t PC = (Wo - 1) * sw + kw;
@@ -273,10 +529,71 @@ static bool conv_patch_plan(PatchParams& p, int64_t N, int64_t C, int64_t H, int
   return true;
 }
 
+// The plan of the bf16 kernel for a layer conv_patch_plan() accepts (its window limit, in elements, is the wider
+// one): the strip height that minimises rounds of work groups x (matrix steps + window staging) per strip.
+static void conv_patch_bf16_plan(PatchParams& p) {
+  constexpr int kCUs = 256;
+  const int64_t PC = p.PC;
+  p.G = (p.Wo + 7) / 8;
+  p.mG = make_magic(p.G);
+  p.L = p.chan_inner ? p.PC * p.C : p.PC;
+  p.mL = make_magic(p.L);
+  p.RSb = p.L | 1;
+  p.tap_x = p.chan_inner ? p.C : 1;
+  p.lead = p.pw * p.tap_x;
+  p.Lvalid = p.W * p.tap_x;
+  const int64_t RS = p.RSb, rows_per = p.chan_inner ? 1 : p.C;
+  int best_r = p.R;                         // the fp32 kernel's strip height fits in any case
+  double best = 1e300;
+  for (int r = 1; r <= p.Ho && r <= 64; ++r) {
+    const int64_t PR = static_cast<int64_t>(r - 1) * p.strh + p.kh;
+    if (rows_per * PR * RS > kPbMaxWindow) break;
+    const int64_t strips = static_cast<int64_t>(p.N) * ((p.Ho + r - 1) / r);
+    if (strips > (1 << 30)) continue;
+    const int64_t rounds = (strips + kCUs - 1) / kCUs;
+    const int64_t steps = ((static_cast<int64_t>(r) * p.G + 1) / 2 + kPbWaves - 1) / kPbWaves;
+    const double cost = static_cast<double>(rounds) * (500.0 * steps + 24.0 * ((p.C * PR * PC + kPbThreads - 1) / kPbThreads) + 1500.0);
+    if (cost < best) { best = cost; best_r = r; }
+  }
+  p.R = best_r;
+  p.strips_per_image = (p.Ho + p.R - 1) / p.R;
+  p.total_strips = p.N * p.strips_per_image;
+  p.PR = (p.R - 1) * p.strh + p.kh;
+  p.mPRPC = make_magic(p.PR);
+  p.Q = p.chan_inner ? p.PR : p.C * p.PR;
+  p.tap_c = p.chan_inner ? 1 : p.PR * p.RSb;
+  p.nwg = p.total_strips < kCUs ? p.total_strips : kCUs;
+}
+
 size_t conv_patch_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw) {
   PatchParams p;
   if (!conv_patch_plan(p, N, C, H, W, kh, kw, sh, sw, ph, pw)) return 0;
-  return static_cast<size_t>(p.nwg) * kPatchWaves * 2 * 1024 * sizeof(float);
+  const size_t f32 = static_cast<size_t>(p.nwg) * kPatchWaves * 2 * 1024 * sizeof(float);
+  const size_t b16 = static_cast<size_t>(256) * p.ntiles * 1024 * sizeof(float);     // at most one partial per CU
+  return f32 > b16 ? f32 : b16;            // whichever kernel the dtype of the call selects
+}
+
+template <typename T, int NB>
+static void conv_patch_bf16_launch_nb(const PatchParams& p, hipStream_t stream) {
+  size_t lds = static_cast<size_t>(p.Q) * p.RSb * 2 + 2;
+  const size_t red = static_cast<size_t>(p.ntiles) * 1024 * sizeof(float);
+  if (red > lds) lds = red;
+  if (p.chan_inner) hipLaunchKernelGGL((conv_patch_bf16_kernel<T, NB, true>), dim3(p.nwg), dim3(kPbThreads), lds, stream, p);
+  else hipLaunchKernelGGL((conv_patch_bf16_kernel<T, NB, false>), dim3(p.nwg), dim3(kPbThreads), lds, stream, p);
+}
+
+template <typename T>
+static int conv_patch_bf16_launch(PatchParams& p, hipStream_t stream) {
+  conv_patch_bf16_plan(p);
+  switch (p.nb) {
+    case 1: conv_patch_bf16_launch_nb<T, 1>(p, stream); break;
+    case 2: conv_patch_bf16_launch_nb<T, 2>(p, stream); break;
+    case 3: conv_patch_bf16_launch_nb<T, 3>(p, stream); break;
+    case 4: conv_patch_bf16_launch_nb<T, 4>(p, stream); break;
+    default: conv_patch_bf16_launch_nb<T, 5>(p, stream); break;
+  }
+  hipLaunchKernelGGL(conv_patch_bf16_reduce_kernel, dim3(p.ntiles * 8), dim3(256), 0, stream, p);
+  return check_launch();
 }
 
 template <typename T>
@@ -294,13 +611,14 @@ int conv_patch_syrk(const void* x, int dtype, int64_t sn, int64_t sc, int64_t sh
   PatchParams p;
   if (!conv_patch_plan(p, N, C, H, W, kh, kw, sh, sw, ph, pw)) return AK_ERR_UNSUPPORTED;
   if (lda < p.d) return AK_ERR_ARG;
-  if (ws == nullptr || ws_bytes < static_cast<size_t>(p.nwg) * kPatchWaves * 2 * 1024 * sizeof(float))
-    return AK_ERR_WORKSPACE;
+  if (ws == nullptr || ws_bytes < conv_patch_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw)) return AK_ERR_WORKSPACE;
   p.x = x; p.sn = sn; p.sc = sc; p.sh = sh_el; p.sw = sw_el;
-  p.chan_inner = (sc == 1 && C > 1) ? 1 : 0;
+  p.chan_inner = (sc == 1 && sw_el == C && C > 1) ? 1 : 0;
   p.ws = static_cast<float*>(ws);
   p.alpha = alpha; p.beta = beta; p.A = A; p.lda = lda;
-  return dtype == AK_BF16 ? conv_patch_launch<uint16_t>(p, stream) : conv_patch_launch<float>(p, stream);
+  if (dtype == AK_BF16) return conv_patch_bf16_launch<uint16_t>(p, stream);
+  if (dtype == AK_F32_AS_BF16) return conv_patch_bf16_launch<float>(p, stream);
+  return conv_patch_launch<float>(p, stream);
 }
 
 }  // namespace ak

@@ -597,13 +597,14 @@ extern "C" int ak_conv_syrk(const void* x, int dtype, int64_t N, int64_t C, int6
   if (x == nullptr || A == nullptr || N <= 0 || C <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || sh <= 0 ||
       sw <= 0 || ph < 0 || pw < 0)
     return AK_ERR_ARG;
-  if (dtype != AK_BF16 && dtype != AK_F32) return AK_ERR_ARG;
+  if (dtype != AK_BF16 && dtype != AK_F32 && dtype != AK_F32_AS_BF16) return AK_ERR_ARG;
   if (!ak::syrk_beta_ok(beta, C * kh * kw, lda)) return AK_ERR_UNSUPPORTED;
   {  // few input channels: the window kernel
     const int rc = ak::conv_patch_syrk(x, dtype, C * H * W, H * W, W, 1, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,
                                        A, lda, ws, ws_bytes, static_cast<hipStream_t>(stream));
     if (rc != AK_ERR_UNSUPPORTED) return rc;
   }
+  if (dtype == AK_F32_AS_BF16) return AK_ERR_UNSUPPORTED;      // rounding on the fly is the window kernel's
   ak::ConvPlan plan;
   if (!ak::make_plan(plan, dtype == AK_BF16 ? 2 : 4, N, C, H, W, kh, kw, sh, sw, ph, pw)) return AK_ERR_UNSUPPORTED;
   if (lda < plan.p.d) return AK_ERR_ARG;

@@ -1275,7 +1275,7 @@ extern "C" int ak_conv_syrk_nhwc(const void* x, int dtype, int64_t N, int64_t C,
   if (A == nullptr || !ak::nhwc_ok(x, N, C, H, W, kh, kw, sh, sw, ph, pw, Ho, Wo)) return AK_ERR_ARG;
   const int64_t d = C * kh * kw, M = N * Ho * Wo;
   if (lda < d) return AK_ERR_ARG;
-  if (dtype != AK_BF16 && dtype != AK_F32) return AK_ERR_ARG;
+  if (dtype != AK_BF16 && dtype != AK_F32 && dtype != AK_F32_AS_BF16) return AK_ERR_ARG;
   if (!ak::syrk_beta_ok(beta, d, lda)) return AK_ERR_UNSUPPORTED;
   {  // few input channels: the window kernel, any dtype and channel count
     const int rc = ak::conv_patch_syrk(x, dtype, H * W * C, 1, W * C, C, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,

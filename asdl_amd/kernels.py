@@ -13,7 +13,7 @@ import torch
 
 from . import _lib
 
-AK_F32, AK_BF16 = 0, 1
+AK_F32, AK_BF16, AK_F32_AS_BF16 = 0, 1, 2
 
 _ws_lock = threading.Lock()
 _workspaces = {}
@@ -482,11 +482,19 @@ def _group_take(row, flops, align_key, *tensors):
 
 
 # ------------------------------------------------------------------------------ factors
-def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
-    """out <- beta*out + alpha * x^T x for x = [M, d] (rows may be strided, columns contiguous)."""
+def _as_bf16(x):
+    with _on_launch_stream():
+        return x.to(torch.bfloat16)
+
+
+def syrk_tn(x, out=None, alpha=1.0, beta=0.0, round_bf16=False):
+    """out <- beta*out + alpha * x^T x for x = [M, d] (rows may be strided, columns contiguous).  round_bf16: an
+    fp32 x is rounded to bf16 first (what a matmul does to it inside a bf16 autocast region)."""
     _require_gpu(x, out)
     if x.ndim != 2:
         raise ValueError(f'x.ndim has to be 2. Got {x.ndim}.')
+    if round_bf16 and x.dtype == torch.float32:
+        x = _as_bf16(x)
     if x.stride(1) != 1 and x.shape[1] > 1:
         x = _contiguous(x)
     M, d = x.shape
@@ -523,10 +531,12 @@ def _is_channels_last(x):
             and not x.is_contiguous())
 
 
-def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
+def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0, round_bf16=False):
     """out <- beta*out + alpha * sum_{n,pos} patch patch^T for x = [N, C, H, W], patches ordered (c, ky, kx);
     no division by the output size (fold it into alpha).  A channels-last bf16 x is read in place
-    (rows gathered from the NHWC memory); anything else goes through the NCHW kernel."""
+    (rows gathered from the NHWC memory); anything else goes through the NCHW kernel.  round_bf16: an fp32 x is
+    rounded to bf16 (what a matmul does to it inside a bf16 autocast region): while it is read, by the window
+    kernel of the few-channel layers, else by a cast beforehand."""
     _require_gpu(x, out)
     if x.ndim != 4:
         raise ValueError(f'x.ndim has to be 4. Got {x.ndim}.')
@@ -543,6 +553,14 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     lib = _lib.load()
     h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
     few_channels = d <= 160 and kh * kw > 1 and x.dtype in (torch.bfloat16, torch.float32)   # the LDS-window kernel
+    code = None
+    if round_bf16 and x.dtype == torch.float32:
+        if few_channels:
+            code = AK_F32_AS_BF16
+        else:
+            x = _as_bf16(x)
+    if code is None:
+        code = _dtype_code(x)
     if NCHW_VIA_CHANNELS_LAST and x.dtype == torch.bfloat16 and C % 8 == 0 and not few_channels \
             and x.is_contiguous() and C > 1 and N * C * H * W >= (1 << 16):
         # one transposing copy (memory-bound, a few microseconds) buys the direct-to-LDS kernels, which read rows of
@@ -560,7 +578,7 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
         need = _ws_need('ak_conv_syrk_nhwc_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
         ws, ws_bytes, keep = _ws_args(need, x.device)
         with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
-            rc = lib.ak_conv_syrk_nhwc(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw,
+            rc = lib.ak_conv_syrk_nhwc(ctypes.c_void_p(x.data_ptr()), code, N, C, H, W, kh, kw, sh, sw,
                                        ph, pw, alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0),
                                        ws, ws_bytes, _stream())
         if rc != AK_ERR_UNSUPPORTED:
@@ -570,8 +588,10 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
     need = _ws_need('ak_conv_syrk_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
     ws, ws_bytes, keep = _ws_args(need, x.device)
     with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
-        rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), N, C, H, W, kh, kw, sh, sw, ph, pw,
+        rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), code, N, C, H, W, kh, kw, sh, sw, ph, pw,
                               alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
+    if rc == AK_ERR_UNSUPPORTED and code == AK_F32_AS_BF16:     # a window too large for the LDS: cast, then the bf16 kernels
+        return conv_syrk(_as_bf16(x), kernel_size, stride, padding, out=out, alpha=alpha, beta=beta)
     _lib.check(rc, 'ak_conv_syrk')
     return out
 

@@ -46,6 +46,19 @@ __all__ = ['Operation', 'Linear', 'Conv2d', 'BatchNorm', 'LayerNorm', 'Operation
            'OP_COV_UNIT_WISE', 'OP_COV_UNIT_WISE_INV',
            'OP_SAVE_INPUTS', 'OP_SAVE_OUTPUTS', 'OP_SAVE_OUTGRADS']
 
+AUTOCAST_ROUNDS_FP32_OPERANDS = True
+
+
+def _autocast_rounds(x):
+    """True for an fp32 operand of an input factor that is computed inside a bf16 autocast region.  The reference
+    forms that factor with torch.matmul in its forward hook (asdl/operations/linear.py:75-77, conv.py:80-88), i.e.
+    inside the region, where matmul casts both operands to bf16 (and returns bf16).  Rounding the operand the same
+    way gives the statistic of the activation the layer itself consumed, on the bf16 matrix cores; the sums stay in
+    fp32.  Output gradients are not concerned: backward hooks run outside the region."""
+    return (AUTOCAST_ROUNDS_FP32_OPERANDS and x.dtype == torch.float32 and x.is_cuda
+            and torch.is_autocast_enabled('cuda') and torch.get_autocast_dtype('cuda') == torch.bfloat16)
+
+
 _FACTOR_CACHE_ATTR = '_asdl_amd_factor_cache'
 
 
@@ -270,7 +283,7 @@ class Linear(Operation):
 
     @staticmethod
     def cov_kron_A(module, in_data, out=None, alpha=1.0, beta=0.0):
-        return kernels.syrk_tn(in_data, out=out, alpha=alpha, beta=beta)      # f_in x f_in
+        return kernels.syrk_tn(in_data, out=out, alpha=alpha, beta=beta, round_bf16=_autocast_rounds(in_data))   # f_in x f_in
 
     @staticmethod
     def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):
@@ -312,7 +325,7 @@ class Conv2d(Operation):
             # already materialised [n, d, out_size] patches
             return kernels.syrk_nt(in_data, out=out, alpha=alpha / in_data.shape[-1], beta=beta)
         return kernels.conv_syrk(in_data.x, in_data.kernel_size, in_data.stride, in_data.padding, out=out,
-                                 alpha=alpha / in_data.out_size, beta=beta)
+                                 alpha=alpha / in_data.out_size, beta=beta, round_bf16=_autocast_rounds(in_data.x))
 
     @staticmethod
     def cov_kron_B(module, out_grads, out=None, alpha=1.0, beta=0.0):

@@ -34,6 +34,10 @@ extern "C" {
 
 #define AK_F32 0
 #define AK_BF16 1
+#define AK_F32_AS_BF16 2     /* fp32 in memory, every element rounded to the nearest bf16 (ties to even) as it is read:
+                                what torch.matmul does to an fp32 operand inside a bf16 autocast region, where the
+                                reference's hooks run.  ak_conv_syrk / ak_conv_syrk_nhwc only, and only for layers of
+                                the window kernel (C*kh*kw <= 160, kh*kw > 1); AK_ERR_UNSUPPORTED elsewhere */
 
 #define AK_OK 0
 #define AK_ERR_ARG -1        /* null pointer, negative size, unknown dtype */

@@ -6,7 +6,8 @@ import torch
 from oracle import cpu_ref as R
 
 
-def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
+def syrk_tn(x, out=None, alpha=1.0, beta=0.0, round_bf16=False):
+    x = x.bfloat16() if round_bf16 else x
     val = alpha * R.linear_cov_kron_A(x.float())
     if out is None:
         return val
@@ -14,7 +15,8 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0):
     return out
 
 
-def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0):
+def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0, round_bf16=False):
+    x = x.bfloat16() if round_bf16 else x
     col = R.im2col_2d(x.float(), kernel_size, stride, padding)
     m = col.transpose(0, 1).flatten(start_dim=1)
     val = alpha * (m @ m.T)

@@ -130,27 +130,36 @@ WINDOW_CASES = [
     (700, 3, 6, 6, (3, 3), (1, 1), (1, 1)),        # more strips than work groups
     (2, 3, 8, 40, (3, 5), (1, 8), (1, 2)),         # stride wider than the kernel, few output columns
     (1, 2, 5, 3, (5, 3), (1, 1), (0, 0)),          # a single output position
+    (2, 3, 224, 224, (7, 7), (2, 2), (3, 3)),      # the ImageNet stem at its size: 112 positions per output row
+    (2, 4, 20, 45, (3, 3), (3, 3), (0, 0)),        # stride 3, 15 positions per row: a full and a ragged group of 8
 ]
 
 
 @pytest.mark.parametrize('layout', ['nchw', 'channels_last'])
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, 'f32_as_bf16'])
 @pytest.mark.parametrize('case', WINDOW_CASES, ids=[str(c) for c in WINDOW_CASES])
 def test_conv_syrk_window_kernel_matches_oracle(K, dtype, layout, case):
+    """fp32 input: fp32 matrix instructions; bf16 input, and fp32 input that the kernel rounds to bf16 as it reads
+    it (round_bf16: what the reference's matmul does to it inside a bf16 autocast region), the bf16 ones.  The
+    oracle gets the rounded values: the sums are fp32 in every case."""
     N, C, H, W, k, s, p = case
-    x = _inputs((N, C, H, W), dtype, seed=N + 10 * C + H)
+    rounded = dtype == 'f32_as_bf16'
+    x = _inputs((N, C, H, W), torch.float32 if rounded else dtype, seed=N + 10 * C + H)
     out_size = ((H + 2 * p[0] - k[0]) // s[0] + 1) * ((W + 2 * p[1] - k[1]) // s[1] + 1)
-    ref = R.conv_cov_kron_A(x.float().double(), k, s, p) * out_size      # the plain sum over positions
+    seen = x.bfloat16() if rounded else x
+    ref = R.conv_cov_kron_A(seen.float().double(), k, s, p) * out_size      # the plain sum over positions
     print(f'conv_syrk window dtype={dtype} layout={layout} case={case}', flush=True)
     xg = x.cuda()
     if layout == 'channels_last':
         xg = xg.contiguous(memory_format=torch.channels_last)
-    out = K.conv_syrk(xg, k, s, p, alpha=0.5)
+    out = K.conv_syrk(xg, k, s, p, alpha=0.5, round_bf16=rounded)
     torch.cuda.synchronize()
     assert relerr(out, 0.5 * ref) < 1e-5
     assert torch.equal(out, out.T)
+    if rounded and N * out_size <= 4096:     # not the statistic of the unrounded input: the rounding is really applied
+        assert relerr(out, 0.5 * R.conv_cov_kron_A(x.double(), k, s, p) * out_size) > 1e-5
     # accumulation: out <- beta * out + alpha * stat
-    K.conv_syrk(xg, k, s, p, out=out, alpha=0.25, beta=2.0)
+    K.conv_syrk(xg, k, s, p, out=out, alpha=0.25, beta=2.0, round_bf16=rounded)
     torch.cuda.synchronize()
     assert relerr(out, 1.25 * ref) < 1e-5
     assert torch.equal(out, out.T)

@@ -233,7 +233,9 @@ def test_small_cnn_bf16_autocast(channels_last):
                    for v in ins.values()), 'the hooks should see channels-last activations'
     worst = {}
     for name, m in layers:
-        a = ins[name].float().cpu()
+        # forward hooks run inside the autocast region: an fp32 input (the first layer's) enters its factor rounded
+        # to bf16, as it enters the reference's torch.matmul there and the layer's own convolution
+        a = ins[name].bfloat16().float().cpu()
         g = gouts[name].float().cpu()                 # the maker back-propagates the summed loss
         if isinstance(m, nn.Conv2d):
             A = R.conv_cov_kron_A(a, m.kernel_size, m.stride, m.padding) / bs
@@ -317,6 +319,47 @@ def test_config2_linear_4096_batch8192_bf16_ema():
         h.remove()
 
 
+@pytest.mark.parametrize('rounds', [True, False])
+def test_fp32_inputs_of_a_bf16_autocast_region_enter_the_A_factor_rounded(rounds, monkeypatch):
+    """The reference forms the A factor with torch.matmul inside its forward hook (asdl/operations/linear.py:75-77,
+    conv.py:80-88), i.e. inside the caller's autocast region, where an fp32 operand is cast to bf16.
+    operations.AUTOCAST_ROUNDS_FP32_OPERANDS does the same to an fp32 module input (first layers): the factor is the
+    fp32 sum over the bf16-rounded input, 1e-5 from the oracle on the rounded values and clearly away from the one on
+    the unrounded values; switched off, or outside an autocast region, the fp32 values are used as they are."""
+    import asdl_amd.operations as ops_mod
+    monkeypatch.setattr(ops_mod, 'AUTOCAST_ROUNDS_FP32_OPERANDS', rounds)
+    torch.manual_seed(17)
+    bs = 4
+    conv = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.ReLU(), nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(8, 8)).cuda()
+    mlp = nn.Sequential(nn.Linear(24, 16), nn.ReLU(), nn.Linear(16, 8)).cuda()
+    for model, x in ((conv, torch.randn(bs, 3, 6, 6).cuda()), (mlp, torch.randn(bs, 24).cuda())):
+        t = torch.randint(8, (bs,)).cuda()
+        for autocast in (True, False):
+            def fwd(inp):
+                with torch.autocast('cuda', dtype=torch.bfloat16, enabled=autocast):
+                    return model(inp).float()
+            ema = 0.5                         # with a moving average the factors are kept beside their inverses
+            for m in model.modules():         # a fresh average for every run
+                if hasattr(m, 'fisher'):
+                    delattr(m, 'fisher')
+            gm = KfacGradientMaker(model, PreconditioningConfig(data_size=bs, damping=1e-2, ema_decay=ema),
+                                   fisher_type=FISHER_EMP)
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
+            gm.forward_and_backward()
+            first = model[0]
+            stat = {}
+            for key, seen in (('rounded', x.bfloat16().double().cpu()), ('plain', x.double().cpu())):
+                if isinstance(first, nn.Conv2d):
+                    stat[key] = ema * R.conv_cov_kron_A(seen, first.kernel_size, first.stride, first.padding) / bs
+                else:
+                    stat[key] = ema * R.linear_cov_kron_A(seen) / bs
+            want, other = ('rounded', 'plain') if rounds and autocast else ('plain', 'rounded')
+            A = first.fisher.kron.A
+            assert relerr(A, stat[want]) < 1e-5, (type(first).__name__, autocast, relerr(A, stat[want]))
+            assert relerr(A, stat[other]) > 1e-4, (type(first).__name__, autocast, relerr(A, stat[other]))
+
+
 def test_resnet50_batch64_channels_last_properties():
     """The benchmark configuration (ResNet-50, batch 64) at full size, checked through properties that do not need a CPU run of
     the model: every conv A factor against an fp64 product of the unfolded input the GPU produced, every inverse
@@ -352,7 +395,7 @@ def test_resnet50_batch64_channels_last_properties():
     for name in picks:
         m = mods[name]
         kron = m.fisher.kron
-        a = ins[name].float()
+        a = ins[name].bfloat16().float()     # conv1's fp32 images enter its factor rounded to bf16 (autocast region)
         g = gouts[name].float()              # summed loss inside the maker: these are the K-FAC out-grads
         if isinstance(m, nn.Conv2d):
             u = F.unfold(a.contiguous().double(), m.kernel_size, padding=m.padding, stride=m.stride)   # [n, d, hw]
@@ -449,7 +492,8 @@ def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch
         cxt.set_damping(damping)
         cxt.set_cov_scale(1.0 / bs)
         for name, m in layers:
-            cxt.call_operations_in_forward(m, ins[name], None)
+            with torch.autocast('cuda', dtype=torch.bfloat16):      # as the forward hooks of the run
+                cxt.call_operations_in_forward(m, ins[name], None)
             cxt.call_operations_in_backward(m, gouts[name])
         torch.cuda.synchronize()
         cxt.flush_inverses()
