@@ -29,7 +29,7 @@ FACTOR_TIMING_EVERY = 4     # steps between two steps whose factor launches are 
 # known size (--traffic-calibration-mib); counters cannot be read from inside the timed run, so the figure is recorded
 # here, reported only for the configuration it was measured on and marked as such (`traffic_source`).  Algorithmic
 # bytes of the same calls: 31.7e6.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 66.5e6    # FETCH_SIZE + WRITE_SIZE of the factor kernels per step / 108 factors (see profiles/)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 70.8e6    # FETCH_SIZE + WRITE_SIZE of the factor kernels per step / 108 factors (see profiles/)
 
 
 def parse():
@@ -387,7 +387,7 @@ def main():
                            'not measured by this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command '
                            '(profiles/factor_kernels_resnet50_bs64_hbm_traffic.txt), bytes per factor call',
                            'floor_ms_per_step': 0.908 if default_workload else None,
-                           'kernel': 'factor statistics (syrk_dtl_kernel; conv_patch_syrk_kernel for the 3-channel '
+                           'kernel': 'factor statistics (syrk_dtl_kernel, single and grouped; conv_patch_bf16_kernel for the 3-channel '
                                      'stem), SYRK FLOP M*d*(d+1)',
                            'launches_per_step': sum(s[4] for s in sink) // timed_steps,
                            'timed_regions_per_step': len(sink) // timed_steps,
