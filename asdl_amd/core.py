@@ -10,7 +10,7 @@ from torch.autograd.graph import GradientEdge
 
 from .matrices import *
 from .operations import *
-from .operations import FWD_OPS, BWD_OPS
+from .operations import FWD_OPS, BWD_OPS, BWD_OPS_WITH_INPUTS
 from .utils import record_original_requires_grad
 
 _supported_module_classes = (nn.Linear, nn.Conv2d, nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
@@ -55,9 +55,13 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
             if not (has_fwd or has_bwd):
                 continue
 
-            def forward_hook(_module, in_data, out_data, _has_bwd=has_bwd):
-                x, y = in_data[0].detach(), out_data.detach()
-                run_hook(lambda: cxt.call_operations_in_forward(_module, x, y), x, y)
+            # only the stored outputs and the unit-wise statistics look at the module's output
+            needs_out = OP_SAVE_OUTPUTS in names or any(n in BWD_OPS_WITH_INPUTS for n in names)
+
+            def forward_hook(_module, in_data, out_data, _has_bwd=has_bwd, _needs_out=needs_out):
+                x = in_data[0].detach()
+                y = out_data.detach() if _needs_out else None
+                run_hook(lambda: cxt.call_operations_in_forward(_module, x, y), x)
                 if _has_bwd and out_data.requires_grad:
                     def grad_hook(grad, _m=_module):
                         if not cxt.is_operation_registered(_m):
@@ -139,12 +143,14 @@ def module_wise_assignments(model, *assign_rules, ignore_modules=None, map_rule=
             raise ValueError(f'({key}, _) is already assigned.')
         specified[key] = list(values)
 
+    ignored_ids = {id(m) for m in ignore_modules if isinstance(m, nn.Module)}
+    ignored_classes = tuple(cls for cls in ignore_modules if isinstance(cls, type))
+    ignored_keywords = [keyword for keyword in ignore_modules if isinstance(keyword, str)]
+    name_rules = [key for key in specified if isinstance(key, str)]
     for name, module in named_supported_modules(model):
-        if any(module is m for m in ignore_modules if isinstance(m, nn.Module)):
+        if id(module) in ignored_ids or isinstance(module, ignored_classes):
             continue
-        if any(isinstance(module, cls) for cls in ignore_modules if isinstance(cls, type)):
-            continue
-        if any(keyword in name for keyword in ignore_modules if isinstance(keyword, str)):
+        if ignored_keywords and any(keyword in name for keyword in ignored_keywords):
             continue
         requires_grad = False
         for attr in ['weight', 'bias']:
@@ -157,8 +163,8 @@ def module_wise_assignments(model, *assign_rules, ignore_modules=None, map_rule=
         info = (name, module) if named else (module,)
         if module in specified:
             values = specified[module]
-        elif any(isinstance(key, str) and key in name for key in specified):
-            values = specified[next(key for key in specified if isinstance(key, str) and key in name)]
+        elif name_rules and any(key in name for key in name_rules):
+            values = specified[next(key for key in name_rules if key in name)]
         elif module.__class__ in specified:
             values = specified[module.__class__]
         else:

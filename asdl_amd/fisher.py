@@ -71,8 +71,7 @@ class FisherMaker(GradientMaker):
     def zero_fisher(self, fvp=False):
         attr = self.config.fvp_attr if fvp else self.config.fisher_attr
         for module in self.model.modules():
-            if hasattr(module, attr):
-                delattr(module, attr)
+            module.__dict__.pop(attr, None)      # a plain attribute: set by setattr(module, attr, SymMatrix)
 
     def _factor_stream(self):
         """Where the statistics kernels of the hooks go, one object per maker: a group that launches the factors of
@@ -162,14 +161,15 @@ class FisherMaker(GradientMaker):
 
             def closure(nll_expr, retain_graph=False):
                 keep = retain_graph or loss_grad_after_fisher
-                with skip_param_grad(model, disable=loss_grad_with_fisher):
-                    if loss_grad_with_fisher or not PRUNED_FISHER_BACKWARD or not cxt.grad_edges:
+                if loss_grad_with_fisher or not PRUNED_FISHER_BACKWARD or not cxt.grad_edges:
+                    with skip_param_grad(model, disable=loss_grad_with_fisher):
                         nll_expr().backward(retain_graph=keep)
-                    else:
-                        # No parameter takes a gradient from this pass: differentiate with respect to the
-                        # hooked module outputs only.  Every hook fires as in a full pass; the autograd
-                        # engine leaves out the weight-gradient kernels, whose results would be dropped.
-                        torch.autograd.grad(nll_expr(), list(cxt.grad_edges), retain_graph=keep, allow_unused=True)
+                else:
+                    # No parameter takes a gradient from this pass: differentiate with respect to the
+                    # hooked module outputs only.  Every hook fires as in a full pass; the autograd
+                    # engine leaves out the weight-gradient kernels, whose results would be dropped, and
+                    # accumulates into no .grad, so the parameters' requires_grad flags stay as they are.
+                    torch.autograd.grad(nll_expr(), list(cxt.grad_edges), retain_graph=keep, allow_unused=True)
 
             with nvtx_range('bwd'):
                 if self.is_fisher_emp:
