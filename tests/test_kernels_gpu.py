@@ -199,6 +199,34 @@ def test_conv_syrk_channels_last_matches_oracle(K, case):
     assert relerr(out, out2.double()) < 1e-5
 
 
+@pytest.mark.parametrize('layout', ['nchw', 'channels_last'])
+def test_round_bf16_outside_the_window_kernel_is_a_cast(K, layout):
+    """round_bf16 for operands the window kernel does not take (many channels, 1x1 windows, plain rows): the wrappers
+    cast to bf16 and use the bf16 kernels; the C entry points answer AK_ERR_UNSUPPORTED to AK_F32_AS_BF16 there."""
+    import ctypes
+    from asdl_amd import _lib
+    x = _inputs((2, 32, 10, 10), torch.float32, seed=5)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last) if layout == 'channels_last' else x.cuda()
+    for k, s, p in (((3, 3), (1, 1), (1, 1)), ((1, 1), (1, 1), (0, 0))):
+        ref = R.conv_cov_kron_A(x.bfloat16().double(), k, s, p)
+        out_size = ((10 + 2 * p[0] - k[0]) // s[0] + 1) ** 2
+        out = K.conv_syrk(xg, k, s, p, alpha=1.0 / out_size, round_bf16=True)
+        assert relerr(out, ref) < 1e-5
+        assert relerr(out, R.conv_cov_kron_A(x.double(), k, s, p)) > 1e-5
+    rows = _inputs((300, 48), torch.float32, seed=6)
+    out = K.syrk_tn(rows.cuda(), round_bf16=True)
+    assert relerr(out, R.linear_cov_kron_A(rows.bfloat16().double())) < 1e-5
+    assert relerr(out, R.linear_cov_kron_A(rows.double())) > 1e-5
+    # the C ABI itself: the third dtype code is the window kernel's only
+    A = torch.empty(288, 288, device='cuda')
+    lib = _lib.load()
+    args = (ctypes.c_void_p(xg.data_ptr()), K.AK_F32_AS_BF16, 2, 32, 10, 10, 3, 3, 1, 1, 1, 1, 1.0, 0.0,
+            ctypes.c_void_p(A.data_ptr()), 288, ctypes.c_void_p(0), 0, ctypes.c_void_p(0))
+    fn = lib.ak_conv_syrk_nhwc if layout == 'channels_last' else lib.ak_conv_syrk
+    assert fn(*args) == K.AK_ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+
+
 def test_conv_syrk_channels_last_ema_accumulate(K):
     x = _inputs((4, 16, 10, 10), torch.bfloat16, 1)
     x2 = _inputs((4, 16, 10, 10), torch.bfloat16, 2)
