@@ -48,6 +48,7 @@ _SIGNATURES = {
     'ak_unit_wise_mvp': (c_int, [c_ptr, c_i64, c_ptr, c_ptr, c_f32, c_ptr]),
     'ak_unit_wise_mvp_grouped': (c_int, [c_ptr, c_int, c_i64, c_f32, c_ptr]),
     'ak_unit_wise_inv_grouped': (c_int, [c_ptr, c_int, c_i64, c_ptr]),
+    'ak_identity_where_zero': (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_ptr]),
     'ak_conv_patch_sum': (c_int, [c_ptr, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_f32, c_f32, c_ptr, c_i64, c_ptr]),
     'ak_kron_damping_swift': (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_f32, c_f32, c_ptr, c_ptr, c_ptr]),

@@ -131,7 +131,29 @@ static __global__ __launch_bounds__(256) void damping_scan_swift_kernel(const fl
   if (__syncthreads_or(any) && threadIdx.x == 0) atomicOr(&nonzero_out[2 * b + f], 1);
 }
 
+// Identity into the matrices whose factor was all zero (flag 0); the others are left alone.
+__global__ __launch_bounds__(256) void identity_where_zero_kernel(float* const* __restrict__ out_list,
+                                                                   const int64_t* __restrict__ dims,
+                                                                   const int* __restrict__ nonzero,
+                                                                   const int64_t* __restrict__ flag_index) {
+  const int m = blockIdx.y;
+  if (nonzero[flag_index[m]] != 0) return;
+  const int64_t d = dims[m], total = d * d;
+  float* __restrict__ out = out_list[m];
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * 256)
+    out[i] = (i / d == i % d) ? 1.f : 0.f;
+}
+
 }  // namespace ak
+
+extern "C" int ak_identity_where_zero(float* const* out_list, const int64_t* dims, const int* nonzero,
+                                      const int64_t* flag_index, int count, ak_stream_t stream) {
+  if (out_list == nullptr || dims == nullptr || nonzero == nullptr || flag_index == nullptr || count <= 0)
+    return AK_ERR_ARG;
+  hipLaunchKernelGGL(ak::identity_where_zero_kernel, dim3(32, count), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     out_list, dims, nonzero, flag_index);
+  return ak::check_launch();
+}
 
 extern "C" int ak_kron_damping_swift(const float* const* A_list, const float* const* B_list, const int64_t* dims,
                                      const float* eig_scale, int batch, float damping, float eps, float* lam_out,

@@ -32,6 +32,14 @@ GROUP_FLUSH_EVERY = (-2, 0)  # (forward, backward): launch the group after that 
                              # (-1, 0), 26.0 with (-2, 0))
 FACTOR_SIDE_STREAM = False  # statistics kernels of the hooks on a side stream (ordering the two streams costs ~30 us of host time per hook: more than the overlap gains)
 PRUNED_FISHER_BACKWARD = True   # sampled / exact Fisher passes skip the weight-gradient kernels (their results are never used)
+LATE_INVERSE_FLAGS = False  # Read the zero / not-positive-definite flags of an update with calc_loss_grad only when the next
+                            # update reaches the same point (FisherMaker.late_inverse_flags; check_late_flags() after
+                            # the last one) instead of waiting for them before the preconditioning is enqueued: the
+                            # host then never waits for the device inside a step and prepares the next step while the
+                            # device finishes this one.  The price is the reference's error behaviour: a factor
+                            # that is not positive definite raises torch.linalg.LinAlgError one update late, and an
+                            # all-zero factor, whose inverse the reference skips, preconditions with the identity
+                            # until then.  Off by default; bench.py switches it on and says so.
 EAGER_INVERSE = True        # start the bulk of the inverses during a single sampled / empirical backward pass: the longest chains get a head start
 EAGER_INVERSE_SAMPLED = False   # ... also when a loss backward pass follows the sampled one.  That pass hides the
                                 # inverses anyway, and one grouped inverse for all factors after the sampled pass is
@@ -64,9 +72,19 @@ class FisherMaker(GradientMaker):
     def __init__(self, model, config):
         super().__init__(model)
         self.config: FisherConfig = config
+        self.late_inverse_flags = LATE_INVERSE_FLAGS
+        self._late_flags = []
         self.before_inverse_wait = None      # optional callable, run right before the host waits for the inverses
         self.after_factors = None            # optional callable, run when the factors are final and before the loss
                                              # backward pass is enqueued; may return an object with finish()
+
+    def check_late_flags(self):
+        """Reads the flags of the last update whose flags were left unread (late_inverse_flags) and raises
+        torch.linalg.LinAlgError for a factor that was not positive definite.  Called by the next update; call it
+        after the last one."""
+        pending, self._late_flags = self._late_flags, []
+        for late in pending:
+            late.check()
 
     def zero_fisher(self, fvp=False):
         attr = self.config.fvp_attr if fvp else self.config.fisher_attr
@@ -205,7 +223,12 @@ class FisherMaker(GradientMaker):
             if self.before_inverse_wait is not None:
                 self.before_inverse_wait()      # host work of the caller that needs no flags: the device is still busy
             if deferred is not None:
-                deferred.finish(config.fisher_attr)
+                self.check_late_flags()         # of the previous update: read long ago by the device's clock
+                late = deferred.finish_late() if self.late_inverse_flags else None
+                if late is None:
+                    deferred.finish(config.fisher_attr)
+                else:
+                    self._late_flags = late
             if early is not None:
                 early.finish()
         phase_mark('upd_inv')             # what is left of the inverses once the loss backward pass has ended

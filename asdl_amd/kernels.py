@@ -742,6 +742,25 @@ def tril_unpack(tril, n_cols):
 
 
 # ------------------------------------------------------------------------------ damping / inverse
+def identity_where_zero(outs, nonzero, flag_index):
+    """outs[m] <- identity where nonzero.view(-1)[flag_index[m]] == 0 (an all-zero factor, whose inverse was
+    skipped); the other matrices are left alone.  No host synchronisation."""
+    if not outs:
+        return
+    _require_gpu(*outs, nonzero)
+    dev = outs[0].device
+    for o in outs:
+        if o.dtype != torch.float32 or o.ndim != 2 or o.shape[0] != o.shape[1] or not o.is_contiguous():
+            raise ValueError('outs have to be contiguous square float32 matrices')
+    ptrs = device_ptr_array(outs)
+    dims = device_ints(tuple(int(o.shape[0]) for o in outs), dev)
+    index = device_ints(tuple(int(i) for i in flag_index), dev)
+    rc = _lib.load().ak_identity_where_zero(ctypes.c_void_p(ptrs.data_ptr()), ctypes.c_void_p(dims.data_ptr()),
+                                            ctypes.c_void_p(nonzero.data_ptr()), ctypes.c_void_p(index.data_ptr()),
+                                            len(outs), _stream())
+    _lib.check(rc, 'ak_identity_where_zero')
+
+
 def kron_damping(A_list, B_list, damping, eps=1e-7, eig_scale=None):
     """Returns (lam [batch, 2] float32, nonzero [batch, 2] int32), both on the device.  A factor is a square
     [d, d] matrix or, for the low-rank (swift) factors, an [n, d] matrix with n < d rows; ``eig_scale``: optional

@@ -104,6 +104,19 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         return [m for _, m in self.named_modules_for(shape)]
 
     @property
+    def late_inverse_flags(self):
+        """fisher.LATE_INVERSE_FLAGS for this maker: the flags of an inverse update are read by the next one."""
+        return self.fisher_maker.late_inverse_flags
+
+    @late_inverse_flags.setter
+    def late_inverse_flags(self, value):
+        self.fisher_maker.late_inverse_flags = bool(value)
+
+    def check_late_flags(self):
+        """Reads the flags that late_inverse_flags left unread (after the last step, before a checkpoint)."""
+        self.fisher_maker.check_late_flags()
+
+    @property
     def _fisher_attr(self):
         return self.fisher_maker.config.fisher_attr
 

@@ -449,6 +449,16 @@ class DeferredInverses:
         self._chunks = chunks            # [(PendingInverses, [(module, kron), ...]), ...]
         self._context = context
 
+    def finish_late(self):
+        """finish() without its host synchronisation (PendingInverses.finish_late): returns the LateFlags objects
+        whose check() reads the flags later.  None when the context also has unit-wise flags to read, which only
+        finish() does."""
+        if self._context is not None and self._context._unit_flags:
+            return None
+        for pending, _ in self._chunks:
+            pending.join()
+        return [late for late in (pending.finish_late() for pending, _ in self._chunks) if late is not None]
+
     def finish(self, attr):
         if self._context is not None:
             self._context.check_unit_flags()

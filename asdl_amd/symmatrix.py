@@ -100,13 +100,36 @@ def _is_all_none(xs):
     return all(x is None for x in xs)
 
 
+class LateFlags:
+    """Flags of a batch of inverses on their way to pinned host memory (PendingInverses.finish_late).  check() waits
+    for the copy, which has long arrived when it is called a step later, and raises for a factor that was not
+    positive definite."""
+
+    def __init__(self, host, event, records, keep_alive):
+        self._host, self._event, self._records, self._keep_alive = host, event, records, keep_alive
+
+    def check(self):
+        if self._host is None:
+            return
+        self._event.synchronize()
+        host, self._host, self._keep_alive = self._host.tolist(), None, None
+        n = len(self._records)
+        info_host, nz_host = host[:n], host[n:]
+        for (flat, which), inf in zip(self._records, info_host):
+            if nz_host[flat] and inf != 0:
+                raise torch.linalg.LinAlgError(
+                    f'cholesky_inv: the leading minor of order {inf} of kron.{which} + damping was not '
+                    f'positive-definite (reported late: the flags of this update were read after the next one)')
+
+
 class PendingInverses:
     """Inverses that have been enqueued (on side streams) but whose flags have not been read yet.
     finish() joins the streams into the current one, reads all flags with one device-to-host copy,
     raises for a matrix that is not positive definite and stores the inverses on the Kron objects."""
 
-    def __init__(self, records, infos, nz_flat, events, replace, keep_alive=None, futures=()):
+    def __init__(self, records, infos, nz_flat, events, replace, keep_alive=None, futures=(), fresh=None):
         self._records, self._infos, self._nz_flat = records, infos, nz_flat
+        self._fresh = list(fresh) if fresh is not None else [True] * len(records)   # output buffers that held no inverse
         self._keep_alive = keep_alive      # tensors the side-stream kernels still read
         self._events, self._replace = events, replace
         self._futures = list(futures)      # enqueue jobs running on worker threads; each returns an event
@@ -121,6 +144,32 @@ class PendingInverses:
             main = torch.cuda.current_stream()
             for ev in events:
                 main.wait_event(ev)
+
+    def finish_late(self):
+        """finish() without its host synchronisation: the inverses are stored on the Kron objects as if every factor
+        was non-zero and positive definite, the copy of the flags to pinned host memory is enqueued, and the returned
+        LateFlags reads them when asked (a step later, say).  Until then an all-zero factor, whose inverse was
+        skipped, has the identity as its inverse if the buffer is a fresh one (the device fills it in), and its
+        previous inverse otherwise, as in the reference, which skips the update (asdl/symmatrix.py:517, :527)."""
+        if self._done:
+            return None
+        self._done = True
+        self.join()
+        fresh = [(flat, out) for (flat, k, which, out), was_fresh in zip(self._records, self._fresh) if was_fresh]
+        if fresh:
+            kernels.identity_where_zero([out for _, out in fresh], self._nz_flat, [flat for flat, _ in fresh])
+        flags = torch.cat(self._infos + [self._nz_flat])
+        host = torch.empty(flags.shape, dtype=flags.dtype, pin_memory=True)
+        host.copy_(flags, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        for (flat, k, which, out) in self._records:
+            setattr(k, which + '_inv', out)
+            if self._replace:
+                setattr(k, which, None)
+        late = LateFlags(host, event, [(flat, which) for flat, _, which, _ in self._records], (flags, self._keep_alive))
+        self._keep_alive = None
+        return late
 
     def finish(self):
         if self._done:
@@ -198,6 +247,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         groups = {-1: merged}
     order = sorted(groups, key=lambda d: sum(e[1].shape[0] ** 3 for e in groups[d]), reverse=True)
     prepared = []
+    fresh_of = {}                # id(output buffer) -> it held no inverse before
     for d in order:
         entries = groups[d]
         idx = kernels.device_ints(tuple(e[0] for e in entries), dev)
@@ -206,6 +256,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
             old = getattr(k, which + '_inv')
             reuse = old is not None and old.shape == mat.shape and old.is_contiguous() and old.dtype == mat.dtype
             outs.append(old if reuse else torch.empty_like(mat))
+            fresh_of[id(outs[-1])] = not reuse
         info = torch.empty(len(entries), dtype=torch.int32, device=dev)
         prepared.append((entries, outs, lam_flat[idx], nz_flat[idx].contiguous(), info))
     for flat, mat, k, which in low_rank:
@@ -214,6 +265,7 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         old = getattr(k, which + '_inv')
         reuse = old is not None and tuple(old.shape) == (d, d) and old.is_contiguous() and old.dtype == mat.dtype
         out = old if reuse else torch.empty(d, d, dtype=mat.dtype, device=dev)
+        fresh_of[id(out)] = not reuse
         info = torch.empty(1, dtype=torch.int32, device=dev)
         prepared.append(([(flat, mat, k, which)], [out], lam_flat[flat:flat + 1], None, info))
     prepared.sort(key=lambda g: -sum(e[1].shape[0] * e[1].shape[1] ** 2 for e in g[0]))
@@ -270,7 +322,8 @@ def batched_update_inv(krons, damping=_default_damping, calc_A_inv=True, calc_B_
         infos.append(info)
         records.extend((e[0], e[2], e[3], out) for e, out in zip(entries, outs))
     pending = PendingInverses(records, infos, nz_flat, events, replace,
-                              keep_alive=(prepared, lam, nonzero, A_list, B_list), futures=futures)
+                              keep_alive=(prepared, lam, nonzero, A_list, B_list), futures=futures,
+                              fresh=[fresh_of[id(r[3])] for r in records])
     if defer:
         return pending
     pending.finish()

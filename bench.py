@@ -72,6 +72,13 @@ def parse():
     ap.add_argument('--factor-launches', choices=['default', 'single', 'grouped'], default='default',
                     help='single: one launch per Kronecker factor; grouped: the factors of a pass in one grouped launch '
                          '(asdl_amd.fisher.GROUPED_FACTORS); default: the library\'s own setting')
+    ap.add_argument('--inverse-flags', choices=['late', 'now'], default='late',
+                    help='K-FAC workloads: when the host reads the zero / not-positive-definite flags of a step\'s '
+                         'inverses.  now: before it enqueues the preconditioning, as the reference\'s '
+                         'torch.linalg.cholesky does (the library\'s default); late: when the next step gets there '
+                         '(FisherMaker.late_inverse_flags; the last step\'s flags are read inside the timed region), '
+                         'so that the host prepares the next step while the device finishes this one.  Same kernels, '
+                         'same results; an error would be raised one step later')
     ap.add_argument('--traffic-calibration-mib', type=int, default=0,
                     help='before the warm-up, launch one plain copy kernel (ak::copy_bytes_kernel) of this many MiB: '
                          'the known traffic against which a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this '
@@ -270,6 +277,8 @@ def main():
         gm.update_preconditioner = timed_update
     else:
         gm = KfacGradientMaker(model, config, fisher_type=args.fisher, swift=args.swift)
+        gm.late_inverse_flags = args.inverse_flags == 'late'
+    late_flags = getattr(gm, 'late_inverse_flags', False)
     opt = torch.optim.SGD([p for p in model.parameters() if p.requires_grad], lr=1e-4)
 
     def fwd(inp):
@@ -320,6 +329,8 @@ def main():
         # host time and a marker in the queue: 216 pairs per step would slow the measured step by 5 %)
         kernels.enable_timing(i % FACTOR_TIMING_EVERY == 0)
         step()
+    if late_flags:
+        gm.check_late_flags()         # the flags of the last step's inverses
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     kernels.enable_timing(True)
@@ -370,7 +381,8 @@ def main():
                                f'{args.fisher}) on ResNet-50, batch {bs}, 3x224x224 N(0,1) images, 1000 classes, '
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
                                f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights, '
-                               f'cudnn.benchmark {"on" if autotune else "off"}' + (', swift (SKFAC) factors' if args.swift else ''),
+                               f'cudnn.benchmark {"on" if autotune else "off"}' + (', swift (SKFAC) factors' if args.swift else '')
+                               + (', flags of a step\'s inverses read by the host one step late' if late_flags else ''),
                    'batch': bs},
     }
     if sink:

@@ -141,6 +141,15 @@ int ak_conv_patch_sum(const void* x, int dtype, int64_t sn, int64_t sc, int64_t 
                       int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw,
                       float alpha, float beta, float* out, int64_t ldo, ak_stream_t stream);
 
+/* out_list[m] (device array of `count` pointers to contiguous fp32 [dims[m], dims[m]] matrices) <- the identity
+ * where nonzero[flag_index[m]] == 0, i.e. where ak_kron_damping found the factor all zero; the other matrices are not
+ * touched.  dims, flag_index: device int64 [count]; nonzero: the device flags ak_kron_damping wrote.
+ * The reference skips the inverse of an all-zero factor on the host (`if not torch.all(self.A == 0)`,
+ * asdl/symmatrix.py:517, :527); a caller that does not want to read the flags before it preconditions lets such a
+ * factor precondition with the identity instead. */
+int ak_identity_where_zero(float* const* out_list, const int64_t* dims, const int* nonzero,
+                           const int64_t* flag_index, int count, ak_stream_t stream);
+
 /* ak_kron_damping for pairs whose factors may be n x d row matrices: dims = device int64 [batch,4]
  * (rows_A, d_A, rows_B, d_B; rows = 0: square d x d factor, eigenvalue mean trace/d; rows > 0: sum(x^2)/d),
  * eig_scale = device float [batch,2] multiplied into the eigenvalue means (may be null).

@@ -427,8 +427,8 @@ def test_resnet50_batch64_channels_last_properties():
     assert relerr(got, ref) < 1e-3, relerr(got, ref)
 
 
-@pytest.mark.parametrize('early_batch', [False, True])
-def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch, monkeypatch):
+@pytest.mark.parametrize('early_batch,late_flags', [(False, False), (True, False), (False, True)])
+def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch, late_flags, monkeypatch):
     """The very code path bench.py times, at its size: ResNet-50, batch 64, channels-last, bf16 autocast, sampled
     (MC) Fisher without EMA, the grouped inverse on a side stream fed by a worker thread beside the loss backward pass
     (and, with ``early_batch``, a first batch started from inside the hooks of the sampled pass:
@@ -457,6 +457,7 @@ def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch
 
     config = PreconditioningConfig(data_size=bs, damping=damping, ignore_modules=[nn.BatchNorm2d])
     gm = KfacGradientMaker(model, config, fisher_type=FISHER_MC)
+    gm.late_inverse_flags = late_flags      # bench.py's setting: the host reads the flags of a step one step late
     layers = [(n, m) for n, m in model.named_modules() if isinstance(m, (nn.Linear, nn.Conv2d))]
     ins, gouts, raw, handles = {}, {}, {}, []
     benchmark_flag = torch.backends.cudnn.benchmark
@@ -481,6 +482,7 @@ def test_benchmark_path_resnet50_batch64_against_a_sequential_replay(early_batch
         torch.backends.cudnn.benchmark = benchmark_flag
         for h in handles:
             h.remove()
+    gm.check_late_flags()
     torch.cuda.synchronize()
     got = {name: (m.fisher.kron.A_inv.clone(), m.fisher.kron.B_inv.clone(),
                   {pn: p.grad.detach().clone() for pn, p in m.named_parameters(recurse=False)}) for name, m in layers}
@@ -676,6 +678,100 @@ def test_grouped_precondition_and_its_early_preparation_give_the_per_module_resu
     got, _ = run(True, True, False, replace_grad=True)
     for key in ref:
         assert grad_close(got[key], ref[key], 1e-5), key
+
+
+def test_identity_where_zero_touches_only_the_flagged_matrices():
+    from asdl_amd import kernels as K
+    outs = [torch.full((d, d), 7.0, device='cuda') for d in (5, 130, 64)]
+    flags = torch.tensor([1, 1, 9, 0, 0, 3], dtype=torch.int32, device='cuda')
+    K.identity_where_zero(outs, flags, [0, 3, 5])
+    torch.cuda.synchronize()
+    assert torch.all(outs[0] == 7.0) and torch.all(outs[2] == 7.0)
+    assert torch.equal(outs[1], torch.eye(130, device='cuda'))
+
+
+def test_late_flags_of_a_batched_inverse():
+    """PendingInverses.finish_late(): no host synchronisation; a factor that is not positive definite raises when the
+    flags are read (strictly: at once), an all-zero factor's fresh inverse buffer holds the identity, the inverses
+    of the others are those of finish()."""
+    from asdl_amd.symmatrix import Kron, batched_update_inv
+    g = torch.Generator().manual_seed(9)
+
+    def spd(d):
+        X = torch.randn(3 * d, d, generator=g)
+        return (X.T @ X / (3 * d)).cuda()
+
+    mats = [(spd(24), spd(40)), (torch.zeros(16, 16).cuda(), spd(8)), (spd(130), spd(12))]
+    strict = [Kron(A.clone(), B.clone()) for A, B in mats]
+    batched_update_inv(strict, damping=1e-2)
+    late = [Kron(A.clone(), B.clone()) for A, B in mats]
+    flags = batched_update_inv(late, damping=1e-2, defer=True).finish_late()
+    flags.check()                                   # nothing to report
+    flags.check()                                   # a second call is a no-op
+    assert strict[1].A_inv is None and torch.equal(late[1].A_inv, torch.eye(16, device='cuda'))
+    for a, b in zip(strict, late):
+        assert torch.equal(a.B_inv, b.B_inv)
+        assert a.A_inv is None or torch.equal(a.A_inv, b.A_inv)
+    bad = [Kron(spd(24), -torch.eye(8).cuda()), Kron(spd(12), spd(12))]
+    with pytest.raises(torch.linalg.LinAlgError):
+        batched_update_inv([Kron(k.A.clone(), k.B.clone()) for k in bad], damping=1e-2)
+    flags = batched_update_inv(bad, damping=1e-2, defer=True).finish_late()     # enqueued, inverses stored, no error yet
+    assert bad[1].A_inv is not None and bad[0].B_inv is not None
+    with pytest.raises(torch.linalg.LinAlgError, match='reported late'):
+        flags.check()
+
+
+@pytest.mark.parametrize('fisher_type', [FISHER_MC, FISHER_EMP])
+def test_late_inverse_flags_give_the_same_steps(fisher_type, monkeypatch):
+    """FisherMaker.late_inverse_flags (fisher.LATE_INVERSE_FLAGS, off by default, on in bench.py): the flags of an
+    update are read when the next update reaches the same point, so the host never waits for the device inside a
+    step.  Same kernels in the same order: every inverse of three steps is bit for bit the one of the strict order, every
+    preconditioned gradient within 1e-4; each step checks the flags of the one before, check_late_flags() those of
+    the last."""
+    import asdl_amd.symmatrix as sm_mod
+    checks = []
+    plain_check = sm_mod.LateFlags.check
+    monkeypatch.setattr(sm_mod.LateFlags, 'check', lambda self: (checks.append(self), plain_check(self))[1])
+    xs = [torch.randn(8, 16, 12, 12, generator=torch.Generator().manual_seed(50 + i)).cuda()
+          .contiguous(memory_format=torch.channels_last) for i in range(3)]
+    ts = [torch.randint(10, (8,), generator=torch.Generator().manual_seed(60 + i)).cuda() for i in range(3)]
+
+    def run(late):
+        torch.manual_seed(33)
+        model = nn.Sequential(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU(), nn.Conv2d(32, 32, 1), nn.ReLU(),
+                              nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
+        model = model.to(memory_format=torch.channels_last)
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=8, damping=1e-2), fisher_type=fisher_type, seed=5)
+        gm.late_inverse_flags = late
+        assert gm.fisher_maker.late_inverse_flags == late
+
+        fwd = model                 # fp32: the framework's bf16 convolution kernels vary too much from call to call
+        out = {}
+        for step, (x, t) in enumerate(zip(xs, ts)):
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(fwd, x), t)
+            gm.forward_and_backward()
+            for name, m in model.named_modules():
+                if hasattr(m, 'fisher'):
+                    out[(step, name, 'A_inv')] = m.fisher.kron.A_inv.clone()
+                    out[(step, name, 'B_inv')] = m.fisher.kron.B_inv.clone()
+                    out[(step, name, 'grad')] = m.weight.grad.clone()
+        n_pending = len(gm.fisher_maker._late_flags)
+        gm.check_late_flags()
+        assert not gm.fisher_maker._late_flags
+        return out, n_pending
+
+    ref, n = run(False)
+    assert n == 0 and not checks
+    got, n = run(True)
+    # fisher_emp computes its inverses inside the one backward pass it has: no loss backward pass follows, nothing is
+    # deferred and the flags are read at once as before
+    expect_late = fisher_type == FISHER_MC
+    assert (n > 0 and len(checks) == 3 * n) if expect_late else (n == 0 and not checks), (n, len(checks))
+    assert got.keys() == ref.keys() and len(ref) == 27
+    for key in ref:
+        # the raw weight gradients come from the framework's convolution kernels, which do not sum in a fixed order
+        assert relerr(got[key], ref[key]) < 1e-4 if key[2] == 'grad' else torch.equal(got[key], ref[key]), key
 
 
 @pytest.mark.parametrize('pi', [1, 2])
