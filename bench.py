@@ -29,7 +29,7 @@ FACTOR_TIMING_EVERY = 4     # steps between two steps whose factor launches are 
 # known size (--traffic-calibration-mib); counters cannot be read from inside the timed run, so the figure is recorded
 # here, reported only for the configuration it was measured on and marked as such (`traffic_source`).  Algorithmic
 # bytes of the same calls: 31.7e6.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 70.8e6    # FETCH_SIZE + WRITE_SIZE of the factor kernels per step / 108 factors (see profiles/)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 71.1e6    # FETCH_SIZE + WRITE_SIZE of the factor kernels per step / 108 factors (see profiles/)
 
 
 def parse():
