@@ -144,7 +144,9 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         curvature state itself so that a resumed run continues where it stopped: per module name a dict
         ``'<kron|unit>.<attribute>' -> tensor`` holding the Kronecker factors A, B (kept in EMA mode only; without EMA
         they live in scratch memory and only the inverses exist), their inverses A_inv, B_inv, and the unit-wise
-        blocks and their inverses.  Tensors are clones on the device they live on."""
+        blocks and their inverses.  Tensors are clones on the device they live on.  Flags of the last inverse update
+        that late_inverse_flags left unread are read first: a checkpoint never holds unchecked inverses."""
+        self.check_late_flags()
         state = dict(self.state)
         curvature = {}
         for shape in _kernel_shapes:
