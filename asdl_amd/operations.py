@@ -61,6 +61,14 @@ def _autocast_rounds(x):
 
 _FACTOR_CACHE_ATTR = '_asdl_amd_factor_cache'
 
+# A module that is called several times in one forward pass (shared weights), factors not accumulated (no EMA).
+# True, the reference's behaviour (asdl/operations/operation.py:225-233, 265-279): every backward call pairs the A
+# factor of the LAST forward call with the B factor of its own output gradient, takes the pi-damping of that pair,
+# inverts both, and the inverses of the calls are ADDED.  False: the A and the B contributions of the calls are
+# summed and inverted once, (sum A + lam I)^-1, the curvature block that K-FAC defines and that both forms compute
+# when the factors are accumulated.
+PER_CALL_INVERSES = True
+
 
 class Operation:
     supported_operations = {OP_COV_KRON, OP_COV_KRON_INV, OP_COV_SWIFT_KRON, OP_COV_SWIFT_KRON_INV, OP_SAVE_INPUTS,
@@ -152,22 +160,27 @@ class Operation:
             cache[key] = buf
         return buf
 
-    def _factor_inv_mode(self, key, tmp_key, data, swift, square_fn, low_rank_fn, device):
+    def _factor_inv_mode(self, key, tmp_key, data, swift, square_fn, low_rank_fn, device, slot=None):
         """One contribution to the scratch factor of the *_INV operations.  Swift (asdl/operations/operation.py:
         282-299): a factor with fewer samples than columns is the unscaled [n, d] row matrix; a square one is
         scaled by cov_scale only after the damping has been taken from the unscaled factors, which the damping
-        kernel reproduces by un-scaling its eigenvalue mean."""
+        kernel reproduces by un-scaling its eigenvalue mean.  ``slot``: the contribution does not join the
+        factor of the earlier calls but is written to a scratch buffer of its own (per-call factors of a module
+        that is called several times) and returned instead of stored under ``tmp_key``."""
         n, dim = self.swift_rows_cols(data)
-        first = tmp_key not in self._op_results
+        first = slot is not None or tmp_key not in self._op_results
+        cache_key = key if slot is None else f'{key}@{slot}'
         if swift and n < dim:
-            buf = self._scratch_factor(key, dim, device, rows=n)
+            buf = self._scratch_factor(cache_key, dim, device, rows=n)
             low_rank_fn(buf, 1.0, 0.0 if first else 1.0)
             self._op_results['_eig_scale_' + key] = 1.0
         else:
-            buf = self._scratch_factor(key, dim, device)
+            buf = self._scratch_factor(cache_key, dim, device)
             square_fn(buf, self._cov_scale, 0.0 if first else 1.0)
             self._op_results['_eig_scale_' + key] = 1.0 / self._cov_scale if swift else 1.0
-        self._op_results[tmp_key] = buf
+        if slot is None:
+            self._op_results[tmp_key] = buf
+        return buf
 
     def forward_post_process(self, in_data: torch.Tensor, out_data: torch.Tensor):
         with nvtx_range('cov_kron_A'):
@@ -190,6 +203,10 @@ class Operation:
             self._update_factor('A', lambda out, alpha, beta: fn(module, data, out=out, alpha=alpha, beta=beta))
         elif OP_COV_KRON_INV in op_names or OP_COV_SWIFT_KRON_INV in op_names:
             data = self.preprocess_in_data(module, in_data, out_data)
+            if PER_CALL_INVERSES:
+                # the reference's backward hook forms A from the input of the LAST forward call
+                # (asdl/operations/operation.py:232): a later call replaces the factor of an earlier one
+                self._op_results.pop('_A_tmp', None)
             self._factor_inv_mode(
                 'A', '_A_tmp', data, OP_COV_SWIFT_KRON_INV in op_names,
                 lambda out, alpha, beta: self.cov_kron_A(module, data, out=out, alpha=alpha, beta=beta),
@@ -216,11 +233,14 @@ class Operation:
             fn = self.cov_swift_kron_B if n < dim else self.cov_kron_B
             self._update_factor('B', lambda out, alpha, beta: fn(module, grads, out=out, alpha=alpha, beta=beta))
         elif OP_COV_KRON_INV in op_names or OP_COV_SWIFT_KRON_INV in op_names:
-            self._factor_inv_mode(
+            per_call = PER_CALL_INVERSES and self._n_forward > 1
+            buf = self._factor_inv_mode(
                 'B', '_B_tmp', grads, OP_COV_SWIFT_KRON_INV in op_names,
                 lambda out, alpha, beta: self.cov_kron_B(module, grads, out=out, alpha=alpha, beta=beta),
                 lambda out, alpha, beta: self.cov_swift_kron_B(module, grads, out=out, alpha=alpha, beta=beta),
-                grads.device)
+                grads.device, slot=self._n_backward % self._n_forward if per_call else None)
+            if per_call:
+                self._op_results.setdefault('_B_calls', []).append(buf)
             self._n_backward += 1
             # a module called several times in the forward pass is complete after as many backward hooks
             if self._context is not None and self._n_backward % max(self._n_forward, 1) == 0:
@@ -633,6 +653,13 @@ class OperationContext:
         self._pending_inverse = []
         if not ops:
             return
+        shared = [op for op in ops if op._op_results.get('_B_calls')]
+        if shared:
+            ops = [op for op in ops if op not in shared]
+            for op in shared:
+                self._invert_per_call(op)
+            if not ops:
+                return
         krons = []
         for op in ops:
             A = op._op_results.pop('_A_tmp', None)
@@ -653,6 +680,34 @@ class OperationContext:
             store['A_inv'] = outs[(id(kron), 'A')]
             store['B_inv'] = outs[(id(kron), 'B')]
         self._inverse_chunks.append((pending, [(op._module, kron) for op, kron in zip(ops, krons)]))
+
+    def _invert_per_call(self, op):
+        """A module that was called several times (PER_CALL_INVERSES): one (A, B_k) pair per backward call, each with
+        its own pi-damping, and the sum of their inverses.  A rare shape of model: the pairs are inverted at once and
+        their flags read here, with a host synchronisation."""
+        A = op._op_results.pop('_A_tmp', None)
+        B_calls = op._op_results.pop('_B_calls', None)
+        if A is None or not B_calls:
+            raise RuntimeError('cov_kron_inv: the forward and backward hooks did not both run')
+        scales = (op._op_results.pop('_eig_scale_A', 1.0), op._op_results.pop('_eig_scale_B', 1.0))
+        krons = []
+        for B in B_calls:
+            kron = Kron(A, B)
+            if scales != (1.0, 1.0):
+                kron._eig_scale = scales
+            krons.append(kron)
+        batched_update_inv(krons, damping=op._damping, replace=False, defer=False)
+        store = op._op_results.setdefault(OP_COV_KRON, {})
+        for which in ('A_inv', 'B_inv'):
+            total = None
+            for kron in krons:
+                inv = getattr(kron, which)
+                if inv is not None:
+                    total = inv if total is None else total.add_(inv)
+            if total is None:
+                store.pop(which, None)
+            else:
+                store[which] = total
 
     def flush_inverses(self, defer=False):
         """Inverts every queued (A, B) pair in batched passes.  With ``defer=True`` the launches are only

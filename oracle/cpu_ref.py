@@ -507,6 +507,27 @@ class KfacOracle:
         B_inv = None if bool(torch.all(B == 0)) else swift_inv(B, dB)
         return A_inv, B_inv
 
+    def _shared_module_factors(self, name, module, inputs, out_grads, cov_scale, accumulate):
+        """A module that is called several times in one forward pass.  With accumulated factors (OP_COV_KRON)
+        every forward call adds its A and every backward call its B (asdl/operations/operation.py:196-198,
+        262-264 with accumulate_result's ``+=``, :136-137).  Without (OP_COV_KRON_INV, :265-279) every backward
+        call forms A from the input of the LAST forward call (:232), B from its own output gradient, takes the
+        pi-damping of that pair, inverts both and ADDS THE INVERSES to those of the earlier calls."""
+        if accumulate:
+            A = sum(self._factor(module, x, out_grads[0], cov_scale)[0] for x in inputs)
+            B = sum(self._factor(module, inputs[0], g, cov_scale)[1] for g in out_grads)
+            self.A[name] = ema_accumulate(self.A.get(name), A, self.ema_decay)
+            self.B[name] = ema_accumulate(self.B.get(name), B, self.ema_decay)
+            return
+        A_inv = B_inv = None
+        for g in out_grads:
+            A, B = self._factor(module, inputs[-1], g, cov_scale)
+            dA, dB = kron_damping(A, B, self.damping)
+            Ai, Bi = cholesky_inv(A, dA), cholesky_inv(B, dB)
+            A_inv = Ai if A_inv is None else A_inv + Ai
+            B_inv = Bi if B_inv is None else B_inv + Bi
+        self.A_inv[name], self.B_inv[name] = A_inv, B_inv
+
     def forward_and_backward(self, x, t, loss_fn=F.cross_entropy, mc_targets=None):
         model = self.model
         step = self.step
@@ -532,11 +553,19 @@ class KfacOracle:
                     if out.requires_grad:
                         out.register_hook(lambda g, name=name: saved_g.__setitem__(name, g.detach()))
                 handles.append(m.register_forward_hook(norm_hook))
+            # a module may be called several times per forward pass: the inputs are kept in call order, the
+            # output gradients in the order the backward hook fires (asdl/operations/operation.py:188, 225-233)
+            calls_in, calls_g = {}, {}
             for name, m in self.layers:
-                handles.append(m.register_forward_hook(
-                    lambda mod, inp, out, name=name: saved_in.__setitem__(name, inp[0].detach())))
-                handles.append(m.register_full_backward_hook(
-                    lambda mod, gin, gout, name=name: saved_g.__setitem__(name, gout[0].detach())))
+                def fwd_hook(mod, inp, out, name=name):
+                    saved_in[name] = inp[0].detach()
+                    calls_in.setdefault(name, []).append(inp[0].detach())
+
+                def bwd_hook(mod, gin, gout, name=name):
+                    saved_g[name] = gout[0].detach()
+                    calls_g.setdefault(name, []).append(gout[0].detach())
+                handles.append(m.register_forward_hook(fwd_hook))
+                handles.append(m.register_full_backward_hook(bwd_hook))
             if self.seed is not None:
                 torch.random.manual_seed(self.seed)
             y = model(x)
@@ -572,6 +601,11 @@ class KfacOracle:
                         dA, dB = swift_kron_damping(A, B, self.damping)
                         self.A_inv[name] = cholesky_inv(A * cov_scale, dA) if A.shape[0] == A.shape[1] else smw_inv(A, dA)
                         self.B_inv[name] = cholesky_inv(B * cov_scale, dB) if B.shape[0] == B.shape[1] else smw_inv(B, dB)
+                    continue
+                if len(calls_in[name]) > 1:
+                    if self.swift:
+                        raise NotImplementedError('swift factors of a module called more than once are not restated')
+                    self._shared_module_factors(name, m, calls_in[name], calls_g[name], cov_scale, accumulate)
                     continue
                 A, B = self._factor(m, saved_in[name], saved_g[name], cov_scale)
                 if accumulate:

@@ -196,6 +196,44 @@ def main_swift():
     run_kfac('swift_mlpw_fisher_emp_ema-1', get_mlp_wide(), xs, ts, 'fisher_emp', -1, 1e-2, swift=True)
 
 
+class SharedNet(nn.Module):
+    """One Conv2d and one Linear that are each called twice per forward pass (shared weights)."""
+
+    def __init__(self, ch=4, hid=6, out=5):
+        super().__init__()
+        self.stem = nn.Conv2d(3, ch, 3, 1, 1)
+        self.conv = nn.Conv2d(ch, ch, 3, 1, 1)
+        self.fc_in = nn.Linear(ch * 4 * 4, hid)
+        self.fc = nn.Linear(hid, hid)
+        self.head = nn.Linear(hid, out)
+
+    def forward(self, x):
+        x = F.relu(self.stem(x))
+        x = F.relu(self.conv(x))
+        x = F.max_pool2d(F.relu(self.conv(x)), 2)
+        x = F.relu(self.fc_in(x.flatten(1)))
+        x = torch.tanh(self.fc(x))
+        x = F.relu(self.fc(x))
+        return self.head(x)
+
+
+def main_shared():
+    # modules called twice per forward pass: without EMA the reference inverts inside every backward hook call and
+    # adds the inverses up (asdl/operations/operation.py:267-279); with EMA the factors of the calls are summed
+    bs = 8
+    torch.manual_seed(41)
+    xs = [torch.randn(bs, 3, 8, 8) for _ in range(3)]
+    ts = [torch.randint(5, (bs,)) for _ in range(3)]
+    torch.manual_seed(42)
+    run_kfac('shared_fisher_emp_ema-1', SharedNet(), xs, ts, 'fisher_emp', -1, 1e-2)
+    torch.manual_seed(43)
+    run_kfac('shared_fisher_mc_ema-1', SharedNet(), xs, ts, 'fisher_mc', -1, 1e-2, seed=5)
+    torch.manual_seed(44)
+    run_kfac('shared_fisher_emp_ema0.5', SharedNet(), xs, ts, 'fisher_emp', 0.5, 1e-2)
+    torch.manual_seed(45)
+    run_kfac('shared_fisher_mc_ema0.5', SharedNet(), xs, ts, 'fisher_mc', 0.5, 1e-2, seed=6)
+
+
 def run_partitioned(tag, shape, block_size, merge, damping, ema_decay, seed):
     """The reference's Preconditioner driven directly (ShampooGradientMaker never passes it a block size)."""
     from asdl.precondition.shampoo import Preconditioner
@@ -241,9 +279,12 @@ def main():
         return main_bn()
     if len(sys.argv) > 1 and sys.argv[1] == 'swift':
         return main_swift()
+    if len(sys.argv) > 1 and sys.argv[1] == 'shared':
+        return main_shared()
     main_bn()
     main_swift()
     main_blocks()
+    main_shared()
     torch.manual_seed(0)
     bs = 8
     xs = [torch.randn(bs, 5) for _ in range(3)]

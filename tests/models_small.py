@@ -1,6 +1,8 @@
 """Tiny models shared by the oracle tests and the GPU end-to-end tests (the same shapes as
 the fixtures of the reference's test/conftest.py:11-25, plus a padded / strided CNN)."""
+import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 
 def get_mlp(in_dim=5, hid=4, out=4):
@@ -36,6 +38,27 @@ def get_cnn3(in_dim=3, hid=6, out=5):
                          nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(hid, out))
 
 
+class SharedNet(nn.Module):
+    """One Conv2d and one Linear that are each called twice per forward pass (shared weights)."""
+
+    def __init__(self, ch=4, hid=6, out=5):
+        super().__init__()
+        self.stem = nn.Conv2d(3, ch, 3, 1, 1)
+        self.conv = nn.Conv2d(ch, ch, 3, 1, 1)
+        self.fc_in = nn.Linear(ch * 4 * 4, hid)
+        self.fc = nn.Linear(hid, hid)
+        self.head = nn.Linear(hid, out)
+
+    def forward(self, x):
+        x = F.relu(self.stem(x))
+        x = F.relu(self.conv(x))
+        x = F.max_pool2d(F.relu(self.conv(x)), 2)
+        x = F.relu(self.fc_in(x.flatten(1)))
+        x = torch.tanh(self.fc(x))
+        x = F.relu(self.fc(x))
+        return self.head(x)
+
+
 GOLDEN_KFAC = {
     # tag: (model factory, fisher_type, ema_decay, damping, seed, curvature interval, preconditioner interval)
     'mlp_fisher_emp_ema-1': (get_mlp, 'fisher_emp', -1, 1e-2, None, None, 1),
@@ -49,6 +72,11 @@ GOLDEN_KFAC = {
     'cnnbn_fisher_emp_ema-1': (get_cnn_bn, 'fisher_emp', -1, 1e-2, None, None, 1),
     'cnnbn_fisher_emp_ema0.4': (get_cnn_bn, 'fisher_emp', 0.4, 1e-2, None, None, 1),
     'cnnbn_fisher_mc_ema-1': (get_cnn_bn, 'fisher_mc', -1, 1e-2, 3, None, 1),
+    # modules called twice per forward pass
+    'shared_fisher_emp_ema-1': (SharedNet, 'fisher_emp', -1, 1e-2, None, None, 1),
+    'shared_fisher_mc_ema-1': (SharedNet, 'fisher_mc', -1, 1e-2, 5, None, 1),
+    'shared_fisher_emp_ema0.5': (SharedNet, 'fisher_emp', 0.5, 1e-2, None, None, 1),
+    'shared_fisher_mc_ema0.5': (SharedNet, 'fisher_mc', 0.5, 1e-2, 6, None, 1),
     # tags that start with 'swift_': KfacGradientMaker(swift=True)
     'swift_cnn2_fisher_emp_ema-1': (get_cnn2, 'fisher_emp', -1, 1e-2, None, None, 1),
     'swift_cnn2_fisher_mc_ema-1': (get_cnn2, 'fisher_mc', -1, 1e-3, 4, None, 1),

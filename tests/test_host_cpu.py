@@ -375,15 +375,17 @@ def test_load_state_dict_accepts_the_reference_form_and_rejects_unknown_modules(
         gm.load_state_dict({'step': 1, 'curvature': {'nosuch': {'kron.A': torch.eye(2)}}})
 
 
-def test_module_called_twice_in_one_forward_gets_one_inverse_of_the_summed_factors(monkeypatch):
-    """A module that is called twice per forward pass (shared weights), without EMA.  This build sums the two
-    A contributions and the two B contributions and inverts once: (A1 + A2 + lam I)^-1.  The reference inverts inside
-    every backward call and adds the inverses up (asdl/operations/operation.py:267-279: accumulate_result on A_inv /
-    B_inv, and the forward hook keeps only the last input): (A2 + lam I)^-1 + (A2 + lam' I)^-1 with the first call's
-    input lost.  That is a deliberate divergence: the sum of the factors is the curvature block K-FAC defines, and it
-    is what both implementations compute in EMA mode.  No golden run of the reference covers shared modules."""
+@pytest.mark.parametrize('per_call', [True, False])
+def test_module_called_twice_in_one_forward(per_call, monkeypatch):
+    """A module that is called twice per forward pass (shared weights), without EMA.  Default (the reference,
+    asdl/operations/operation.py:225-233, 265-279, pinned by the golden runs 'shared_*'): every backward call inverts
+    the pair (A of the LAST forward call, B of its own output gradient) with the pi-damping of that pair, and the
+    inverses are added.  With operations.PER_CALL_INVERSES = False the contributions are summed and inverted once,
+    (A1 + A2 + lam I)^-1."""
     import oracle.cpu_ref as R
+    from asdl_amd import operations
     cpu_backend.install(monkeypatch)
+    monkeypatch.setattr(operations, 'PER_CALL_INVERSES', per_call)
     torch.manual_seed(5)
 
     class Twice(nn.Module):
@@ -403,15 +405,23 @@ def test_module_called_twice_in_one_forward_gets_one_inverse_of_the_summed_facto
         o.register_hook(lambda g: gouts.append(g.detach()))
     handle = model.lin.register_forward_hook(capture)
     gm = KfacGradientMaker(model, PreconditioningConfig(data_size=10, damping=1e-2), fisher_type=FISHER_EMP)
-    gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
-    gm.forward_and_backward()
+    for _ in range(2):        # the second step reuses the per-call scratch buffers
+        ins.clear(), gouts.clear()
+        model.zero_grad(set_to_none=True)
+        gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+        gm.forward_and_backward()
+        assert len(ins) == 2 and len(gouts) == 2
+        if per_call:
+            A = R.linear_cov_kron_A(ins[-1]) / 10
+            pairs = [R.kron_update_inv(A, R.linear_cov_kron_B(g) / 10, 1e-2) for g in gouts]
+            A_inv, B_inv = sum(p[0] for p in pairs), sum(p[1] for p in pairs)
+        else:
+            A = sum(R.linear_cov_kron_A(a) for a in ins) / 10
+            B = sum(R.linear_cov_kron_B(g) for g in gouts) / 10
+            A_inv, B_inv = R.kron_update_inv(A, B, 1e-2)
+        assert relerr(model.lin.fisher.kron.A_inv, A_inv) < 1e-5
+        assert relerr(model.lin.fisher.kron.B_inv, B_inv) < 1e-5
     handle.remove()
-    assert len(ins) == 2 and len(gouts) == 2
-    A = sum(R.linear_cov_kron_A(a) for a in ins) / 10
-    B = sum(R.linear_cov_kron_B(g) for g in gouts) / 10
-    A_inv, B_inv = R.kron_update_inv(A, B, 1e-2)
-    assert relerr(model.lin.fisher.kron.A_inv, A_inv) < 1e-5
-    assert relerr(model.lin.fisher.kron.B_inv, B_inv) < 1e-5
 
 
 # ------------------------------------------------------------------ FisherMaker invariants (test/grad_maker/test_fisher.py)
