@@ -59,8 +59,9 @@ __device__ __forceinline__ void decode_upper_tile(int id, int T, int& ti, int& t
 
 // The SYRK epilogues read the old result (beta != 0) through a 32-bit buffer descriptor: results of 4 GiB and more
 // cannot be accumulated into.
+// (d + 31: the 32-bit offsets of a partial last block row are formed for rows up to d + 30 before the range check.)
 inline bool syrk_beta_ok(float beta, int64_t d, int64_t ldc) {
-  return beta == 0.f || ((d - 1) * ldc + d) * 4 < 0xFFFFFF00ll;
+  return beta == 0.f || ((d + 31) * ldc + d) * 4 < 0xFFFFFF00ll;
 }
 
 // Symmetric epilogue for one wave's accumulators of a BT x BT output tile at (ti, tj), ti <= tj.
@@ -75,10 +76,14 @@ __device__ __forceinline__ void syrk_epilogue(floatx16 (&acc)[TI][TJ], float* __
   // Phase 1: acc <- alpha * acc (+ beta * C).  All reads of C come before the first store: the compiler cannot
   // prove that a store to C leaves a later read alone, so reads that follow stores are issued one memory latency
   // after another.  The reads go through a buffer descriptor of C: one 32-bit offset register per 32 x 32 block and
-  // lane, the row within the block as a scalar offset, and rows beyond the matrix read as zero without a bounds
-  // test (a load under a per-element condition gets a wait of its own: 16 * TI * TJ memory latencies in a row;
-  // 64-bit addresses and clamped indices for as many loads in flight cost more registers than the widest tile has).
-  // Columns beyond d read whatever lies there inside the buffer; those accumulators are never stored.
+  // lane, the row within the block as a scalar offset (a load under a per-element condition gets a wait of its
+  // own: 16 * TI * TJ memory latencies in a row; 64-bit addresses and clamped indices for as many loads in flight
+  // cost more registers than the widest tile has).  The hardware checks only the vector offset plus the
+  // instruction's immediate against the descriptor's size; the scalar offset is added to the address afterwards,
+  // unchecked.  So the scalar row offset is used only in 32-row blocks that lie wholly inside the matrix (a test
+  // that is uniform over the wave); the one partial block row of a matrix with d % 32 != 0 puts the row into the
+  // vector offset, where rows beyond the matrix are out of range and read as zero.  Lanes of columns beyond d get
+  // an out-of-range vector offset for the same reason (their accumulators are never stored).
 #pragma unroll
   for (int a = 0; a < TI; ++a)
 #pragma unroll
@@ -94,13 +99,26 @@ __device__ __forceinline__ void syrk_epilogue(floatx16 (&acc)[TI][TJ], float* __
     for (int a = 0; a < TI; ++a) {
 #pragma unroll
       for (int b = 0; b < TJ; ++b) {
+        // a lane whose column lies beyond the matrix gets an offset that is out of range whatever the row
+        const bool col_ok = gj0 + 32 * b + l32 < d;
         const uint32_t voff = static_cast<uint32_t>(gi0 + 32 * a + 4 * g) * ldc4 +
                               static_cast<uint32_t>(gj0 + 32 * b + l32) * 4u;
+        if (gi0 + 32 * a + 32 <= d) {
+          const uint32_t vsel = col_ok ? voff : 0xFFFFFF00u;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float c = __builtin_bit_cast(
-              float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, (8 * (r >> 2) + (r & 3)) * ldc4, 0));
-          acc[a][b][r] += beta * c;
+          for (int r = 0; r < 16; ++r) {
+            const float c = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, vsel, (8 * (r >> 2) + (r & 3)) * ldc4, 0));
+            acc[a][b][r] += beta * c;
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const uint32_t vrow = voff + (8 * (r >> 2) + (r & 3)) * ldc4;
+            const float c = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, col_ok ? vrow : 0xFFFFFF00u, 0, 0));
+            acc[a][b][r] += beta * c;
+          }
         }
       }
     }

@@ -440,14 +440,20 @@ def test_shampoo_gpt2_small_full_decoder_bf16_real_gradients():
             print(f'  root {names[k]} axis {j}: oracle {e_ref:.2e} ({it_ref} iterations), here {e_mine:.2e}', flush=True)
             worst_ratio = max(worst_ratio, e_mine / max(e_ref, 1e-30))
             assert e_mine <= max(4 * e_ref, 1e-4), (names[k], j, e_mine, e_ref)
-        # one root of each larger size against the fp64 closed form
+        # one root of each larger size: distance from the fp64 closed form, and (first update; the CPU run of the
+        # 3072-wide iteration takes a minute) the oracle's distance on the same input with the same start vector
         for n in (1024, 2304, 3072):
             k, j = members[n][0]
-            w, V = torch.linalg.eigh(precs[k].statistics[j].double())
-            exact = (V * w.clamp_min(1e-300) ** -0.25) @ V.T
+            exact = _closed_form_root(precs[k].statistics[j], 4)
             e = relerr(precs[k].preconditioners[j], exact)
-            print(f'  root n={n} ({names[k]} axis {j}): distance from the fp64 closed form {e:.2e}', flush=True)
-            assert e < 5e-2, (n, e)
+            if step == 0:
+                root_ref, it_ref, _ = R.compute_power(stats_in[k][j].cpu().clone(), 4, starts[n][0].clone(), ridge_epsilon=1e-6)
+                e_ref = relerr(root_ref, exact)
+                print(f'  root n={n} ({names[k]} axis {j}): oracle {e_ref:.2e} ({it_ref} iterations), here {e:.2e}', flush=True)
+                assert e <= max(4 * e_ref, 1e-4), (n, e, e_ref)
+            else:
+                print(f'  root n={n} ({names[k]} axis {j}): distance from the fp64 closed form {e:.2e}', flush=True)
+                assert e < 1e-2, (n, e)
         gm.precondition()
         worst = 0.0
         for pc, g in zip(precs, raw):
