@@ -247,6 +247,13 @@ int conv_patch_syrk(const void* x, int dtype, int64_t sn, int64_t sc, int64_t sh
                     int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw, float alpha, float beta,
                     float* A, int64_t lda, void* ws, size_t ws_bytes, hipStream_t stream);
 
+// Input factor of a 3 x 3 / stride 1 / padding 1 convolution on a channels-last bf16 input with a multiple of 64
+// channels, from shifted correlations of the input (conv_corr.hip).  The workspace query answers 0, the launcher
+// AK_ERR_UNSUPPORTED, for other layers.
+size_t conv_corr_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw);
+int conv_corr_syrk(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
+                   int pw, float alpha, float beta, float* A, int64_t lda, void* ws, size_t ws_bytes, hipStream_t stream);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_ERR_LAUNCH; }
 
 // Split-K factor shared by the SYRK front ends: enough work groups to fill 256 CUs twice over

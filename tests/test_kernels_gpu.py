@@ -199,6 +199,53 @@ def test_conv_syrk_channels_last_matches_oracle(K, case):
     assert relerr(out, out2.double()) < 1e-5
 
 
+CORR_CASES = [
+    # N, C, H, W: 3 x 3 windows, stride 1, padding 1, a multiple of 64 channels: the shifted-correlation form
+    (2, 64, 5, 7),          # 64-wide tiles, one tile per shift
+    (3, 128, 8, 8),         # 128-wide tiles
+    (2, 256, 4, 6),         # two row tiles of 128
+    (2, 512, 7, 7),         # 256-wide tiles of 8 waves
+    (1, 64, 1, 1),          # a single pixel: only the centre tap sees it
+    (2, 64, 2, 3),          # the first and the last image row are neighbours
+    (2, 64, 1, 9),          # one image row: both row corrections remove the same pixels
+    (3, 192, 6, 5),         # 64-wide tiles, three per shift
+    (16, 64, 28, 28),       # 12544 pixels: row splits
+    (5, 128, 33, 35),       # ragged last split
+]
+
+
+@pytest.mark.parametrize('case', CORR_CASES, ids=[str(c) for c in CORR_CASES])
+def test_conv_syrk_shifted_correlations_match_oracle(K, case):
+    """3 x 3 / stride 1 / padding 1 factors of channels-last bf16 inputs are assembled from 13 shifted correlations of
+    the input and 16 border corrections (csrc/conv_corr.hip) instead of the unfolded matrix: same statistic
+    (asdl/operations/conv.py:80-88), checked against the oracle's unfolded product in fp64, exact symmetry, and
+    accumulation into an existing factor."""
+    N, C, H, W = case
+    from asdl_amd import _lib
+    assert _lib.load().ak_conv_syrk_nhwc_ws_bytes(N, C, H, W, 3, 3, 1, 1, 1, 1) > 0
+    x = _inputs((N, C, H, W), torch.bfloat16, seed=N + 10 * C + H)
+    ref = R.conv_cov_kron_A(x.float().double(), (3, 3), (1, 1), (1, 1))
+    print(f'conv_syrk shifted correlations case={case}', flush=True)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last)
+    out = K.conv_syrk(xg, (3, 3), (1, 1), (1, 1), alpha=1.0 / (H * W))
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5, relerr(out, ref)
+    assert torch.equal(out, out.T)
+    # every 9C x 9C block against its own norm: a wrong correction of one border block must not hide in the total
+    blocks = (out.double().cpu() - ref).reshape(C, 9, C, 9).permute(1, 3, 0, 2)
+    ref_blocks = ref.reshape(C, 9, C, 9).permute(1, 3, 0, 2)
+    for t1 in range(9):
+        for t2 in range(9):
+            if float(ref_blocks[t1, t2].norm()) > 0:
+                assert float(blocks[t1, t2].norm() / ref_blocks[t1, t2].norm()) < 1e-5, (t1, t2)
+            else:
+                assert float(blocks[t1, t2].abs().max()) < 1e-6 * float(ref.abs().max()), (t1, t2)
+    K.conv_syrk(xg, (3, 3), (1, 1), (1, 1), out=out, alpha=0.25 / (H * W), beta=2.0)
+    torch.cuda.synchronize()
+    assert relerr(out, 2.25 * ref) < 1e-5
+    assert torch.equal(out, out.T)
+
+
 @pytest.mark.parametrize('layout', ['nchw', 'channels_last'])
 def test_round_bf16_outside_the_window_kernel_is_a_cast(K, layout):
     """round_bf16 for operands the window kernel does not take (many channels, 1x1 windows, plain rows): the wrappers
