@@ -69,9 +69,9 @@ __device__ __forceinline__ int corr_find(const CorrArgs& a, int w, bool by_tile)
 
 // One work group per (product, row split, tile).
 template <int WR, int WC, int FR, int FC>
-__global__ __launch_bounds__(WR * WC * 64) void corr_products_kernel(CorrArgs a) {
+__device__ __forceinline__ void corr_products_tile(const CorrArgs& a, uint32_t wg, uint32_t nwg) {
   constexpr int BT = DtlCfg<WR, WC, FR, FC, true>::BT;
-  const int w = static_cast<int>(xcd_contiguous_id(blockIdx.x, gridDim.x));
+  const int w = static_cast<int>(xcd_contiguous_id(wg, nwg));
   const CorrProd& cp = a.prod[corr_find(a, w, false)];
   DtlParams p{};
   p.X = cp.X;
@@ -98,14 +98,14 @@ __global__ __launch_bounds__(WR * WC * 64) void corr_products_kernel(CorrArgs a)
 // red[C][29 C]: 13 C columns of the main product, 3 C per image row and image column, C per corner.
 // grid (tiles of all products, 4 * FR * FC): one work group per float4 slot of every thread's accumulators.
 template <int WR, int WC, int FR, int FC>
-__global__ __launch_bounds__(WR * WC * 64) void corr_reduce_kernel(CorrArgs a) {
+__device__ __forceinline__ void corr_reduce_tile(const CorrArgs& a, int tile, int slot) {
   constexpr int NW = WR * WC, BT = 32 * FR * WR;
   constexpr int64_t tile_f4 = BT * BT / 4;
-  const CorrProd& cp = a.prod[corr_find(a, blockIdx.x, true)];
-  const int t = blockIdx.x - cp.first_tile, ntiles = cp.nti * cp.ntj;
+  const CorrProd& cp = a.prod[corr_find(a, tile, true)];
+  const int t = tile - cp.first_tile, ntiles = cp.nti * cp.ntj;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave / WC, wc = wave % WC, g = lane >> 5, l32 = lane & 31;
-  const int slot = blockIdx.y, q = slot & 3, b = (slot >> 2) % FC, aa = (slot >> 2) / FC;
+  const int q = slot & 3, b = (slot >> 2) % FC, aa = (slot >> 2) / FC;
   const floatx4* src = a.part + cp.part_off + t * tile_f4 + slot * (NW * 64) + tid;
   const int64_t stride = ntiles * tile_f4;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -124,6 +124,18 @@ __global__ __launch_bounds__(WR * WC * 64) void corr_reduce_kernel(CorrArgs a) {
   float* dst = a.red + cp.out_off + static_cast<int64_t>(row) * ld + col;
 #pragma unroll
   for (int e = 0; e < 4; ++e) dst[static_cast<int64_t>(e) * ld] = acc[e];
+}
+
+// All products of one layer in one launch: one work group per (product, row split, tile).
+template <int WR, int WC, int FR, int FC>
+__global__ __launch_bounds__(WR * WC * 64) void corr_products_kernel(CorrArgs a) {
+  corr_products_tile<WR, WC, FR, FC>(a, blockIdx.x, gridDim.x);
+}
+
+// grid (tiles of all products, 4 * FR * FC): one work group per float4 slot of every thread's accumulators.
+template <int WR, int WC, int FR, int FC>
+__global__ __launch_bounds__(WR * WC * 64) void corr_reduce_kernel(CorrArgs a) {
+  corr_reduce_tile<WR, WC, FR, FC>(a, blockIdx.x, blockIdx.y);
 }
 
 // The dense factor from the reduced matrix.  One work group per block of CR channels of rows and 64 channels of
@@ -296,12 +308,14 @@ static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W) {
     CorrProd& p = a.prod[i];
     const int64_t ktiles = (p.M + kDtlBK - 1) / kDtlBK, ntiles = static_cast<int64_t>(p.nti) * p.ntj;
     int64_t ns = 1;
-    if (i == 0) {
+    if (i == 0 && ntiles > 0) {
       // the main product fills the device once (the corrections ride in its tail); at least 8 k-tiles per split
       ns = (slots + ntiles / 2) / ntiles;
       const int64_t cap = ktiles / 8 < 1 ? 1 : ktiles / 8;
       if (ns > cap) ns = cap;
       if (ns < 1) ns = 1;
+    } else if (i > 0) {
+      ns = (ktiles + 15) / 16;          // corrections: chains of at most 16 k-tiles
     }
     p.kt_split = static_cast<int32_t>((ktiles + ns - 1) / ns);
     p.nsplit = static_cast<int32_t>((ktiles + p.kt_split - 1) / p.kt_split);
@@ -309,7 +323,7 @@ static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W) {
     p.first_tile = tiles;
     p.part_off = static_cast<int64_t>(part);
     p.out_off = red_col;
-    red_col += static_cast<int64_t>(p.ntj) * bt;
+    red_col += static_cast<int64_t>(p.ntj) * bt;       // C per piece: 13 C, 3 C or C
     items += p.nsplit * static_cast<int>(ntiles);
     tiles += static_cast<int>(ntiles);
     part += static_cast<size_t>(p.nsplit) * ntiles * tile_f4;

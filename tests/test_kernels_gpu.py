@@ -209,8 +209,15 @@ CORR_CASES = [
     (2, 64, 2, 3),          # the first and the last image row are neighbours
     (2, 64, 1, 9),          # one image row: both row corrections remove the same pixels
     (3, 192, 6, 5),         # 64-wide tiles, three per shift
-    (16, 64, 28, 28),       # 12544 pixels: row splits
-    (5, 128, 33, 35),       # ragged last split
+    (16, 64, 28, 28),       # 12544 pixels: row splits; image rows of 14 ... 64 pixels: the main product on windows
+    (5, 128, 33, 35),       # windows of 48 + 16 pixels, ragged last split
+    (4, 64, 14, 14),        # three image rows per pipeline stage
+    (2, 128, 56, 56),       # windows of 64 + 16 pixels
+    (3, 64, 3, 16),         # W a multiple of 16: no padding pixels; three image rows per sample
+    (1, 192, 17, 64),       # the widest image row the windows take
+    (2, 256, 14, 14),       # 32 units of (row channels, column channels)
+    (5, 64, 20, 30),        # 100 image rows: splits of unequal length
+    (7, 64, 5, 65),         # one pixel too wide for the windows: tiles again
 ]
 
 
