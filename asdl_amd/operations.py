@@ -457,6 +457,7 @@ class LayerNorm(_NormOperation):
 
 
 EAGER_COST_FRACTION = 0.6
+_warned_late_fallback = False
 
 
 class DeferredInverses:
@@ -474,7 +475,14 @@ class DeferredInverses:
         whose check() reads the flags later.  None when the context also has unit-wise flags to read, which only
         finish() does."""
         if self._context is not None and self._context._unit_flags:
+            global _warned_late_fallback
+            if not _warned_late_fallback:
+                _warned_late_fallback = True
+                warnings.warn('late_inverse_flags: this model has unit-wise (BatchNorm / LayerNorm) blocks, whose flags '
+                              'are read at once; the flags of the Kronecker factors are read with them.')
             return None
+        if self._context is not None:
+            self._context._unit_flags_deferred = False      # nothing was deferred to this object's finish()
         for pending, _ in self._chunks:
             pending.join()
         return [late for late in (pending.finish_late() for pending, _ in self._chunks) if late is not None]

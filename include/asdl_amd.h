@@ -340,7 +340,8 @@ int ak_kron_precond(const float* Binv, const float* Ainv, float* G, int64_t dB, 
  * AK_ERR_TOO_LARGE and touches nothing.  Calls no hipMalloc / hipFree.  Nothing in the array has to start at zero
  * (both products overwrite their whole output).  All calls on one GPU share the array: calls that may overlap on
  * one GPU (different streams, different threads) race; order them on one stream.  Same results as ak_kron_precond.
- * No counterpart in the reference. */
+ * The first call on a device looks up the array's device address (hipGetSymbolAddress, which may load the library's
+ * code object): make it before a stream capture begins.  No counterpart in the reference. */
 int64_t ak_kron_precond_static_max_floats(void);
 
 /* out <- grad_scale * Binv G Ainv (and bias_out <- grad_scale * Binv bias when bias != NULL) as back-to-back products

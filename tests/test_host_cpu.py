@@ -228,6 +228,24 @@ def test_update_schedule_and_intervals():
     assert [gm4.do_update_preconditioner(s) for s in range(9)] == [True] * 4 + [False] * 3 + [True, False]
 
 
+def test_update_schedules_are_assignable_like_the_reference_attributes():
+    """asdl/precondition/prec_grad_maker.py:85-99, 174-195: the schedules are plain attributes there; an assigned
+    list decides step by step, None hands the decision back to the intervals."""
+    model = get_mlp()
+    gm = KfacGradientMaker(model, PreconditioningConfig(data_size=4, preconditioner_upd_interval=3))
+    assert gm.preconditioner_upd_schedule is None and gm.curvature_upd_schedule is None
+    assert [gm.do_update_preconditioner(s) for s in range(4)] == [True, False, False, True]
+    gm.preconditioner_upd_schedule = [False, True, True, False]
+    assert [gm.do_update_preconditioner(s) for s in range(4)] == [False, True, True, False]
+    assert [gm.do_update_curvature(s) for s in range(4)] == [False, True, True, False]      # follows the preconditioner
+    gm.curvature_upd_schedule = [True, True, False, False]
+    assert [gm.do_update_curvature(s) for s in range(4)] == [True, True, False, False]
+    gm.curvature_upd_schedule = None
+    assert [gm.do_update_curvature(s) for s in range(4)] == [False, True, True, False]
+    gm.preconditioner_upd_schedule = None
+    assert [gm.do_update_preconditioner(s) for s in range(4)] == [True, False, False, True]
+
+
 def test_module_selection_by_ignore_list_and_trainability():
     model = nn.Sequential(nn.Linear(3, 3), nn.ReLU(), nn.Linear(3, 3), nn.Sequential(nn.Linear(3, 2)), nn.Linear(2, 2))
     for p in model[4].parameters():
