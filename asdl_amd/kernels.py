@@ -72,9 +72,22 @@ def _timing_event():
     return _event_pool.pop() if _event_pool else _RawEvent()
 
 
+MFMA_PEAK_FLOPS = {torch.bfloat16: 2.5e15, torch.float32: 157.3e12}      # dense matrix-core peaks of an MI355X
+HBM_PEAK_BYTES = 8.0e12
+
+
+def factor_floor_seconds(flops, dtype, in_bytes, d, beta):
+    """Roofline floor of one factor statistic: its FLOP at the matrix-core peak of the operand type, or its
+    algorithmic bytes (the operand once, the factor written once, and read once when it is accumulated into) at the
+    memory peak, whichever takes longer."""
+    out_bytes = d * d * 4 * (2 if beta != 0.0 else 1)
+    return max(flops / MFMA_PEAK_FLOPS.get(dtype, 157.3e12), (in_bytes + out_bytes) / HBM_PEAK_BYTES)
+
+
 class _Timed:
-    def __init__(self, name, flops, calls=1):
-        self.name, self.flops, self.calls = name, flops, calls      # calls: factors covered by the timed region
+    def __init__(self, name, flops, calls=1, floor=0.0):
+        # calls: factors covered by the timed region; floor: the sum of their roofline floors in seconds
+        self.name, self.flops, self.calls, self.floor = name, flops, calls, floor
 
     def __enter__(self):
         self.timed = _timing_sink is not None and _timing_on
@@ -87,7 +100,7 @@ class _Timed:
         if self.timed:
             end = _timing_event()
             end.record()
-            _timing_sink.append((self.name, self.flops, self.start, end, self.calls))
+            _timing_sink.append((self.name, self.flops, self.start, end, self.calls, self.floor))
         return False
 
 
@@ -341,6 +354,7 @@ class FactorGroup:
     def __init__(self, device):
         self.device = torch.device(device)
         self._rows, self._keep, self._outs, self._flops = [], [], set(), 0
+        self._versions, self._floor = [], 0.0
         self._sizes = {}
         self.plain_only = False      # take X^T X calls only: unfolded inputs are launched at once
         self._slots = [dict(host=None, dev=None, event=None) for _ in range(self.SLOTS)]
@@ -363,17 +377,20 @@ class FactorGroup:
             _group_eligible[key] = ok
         return ok
 
-    def add(self, row, flops, *tensors):
+    def add(self, row, flops, floor, *tensors):
         if row[2] in self._outs:
             self.flush()
         self._rows.append(row)
         self._outs.add(row[2])
         self._keep.append(tensors)
+        self._versions.append(tensors[0]._version)       # the operand must still hold these values at flush()
         self._flops += flops
+        self._floor += floor
 
     def discard(self):
         """Forgets what has been collected without launching it (a pass that ended in an exception)."""
         self._rows, self._keep, self._outs, self._flops = [], [], set(), 0
+        self._versions, self._floor = [], 0.0
 
     def flush(self):
         """Launches what has been collected on the calling thread's launch stream."""
@@ -381,6 +398,14 @@ class FactorGroup:
             return
         rows, self._rows, keep, self._keep = self._rows, [], self._keep, []
         flops, self._flops, self._outs = self._flops, 0, set()
+        versions, self._versions = self._versions, []
+        floor, self._floor = self._floor, 0.0
+        for tensors, version in zip(keep, versions):
+            # the reference forms a factor inside the hook; here the operand is read later, by address
+            if tensors[0]._version != version:
+                raise RuntimeError('an activation or output gradient was modified in place between the hook that '
+                                   'recorded its factor statistic and the grouped launch of the pass; set '
+                                   'asdl_amd.fisher.GROUPED_FACTORS = False for this model')
         if len(rows) == 1:
             # nothing to share a launch with: the single-factor entry points, whose plan search knows more tile
             # sizes and a two-stage reduction
@@ -421,7 +446,7 @@ class FactorGroup:
             slot['dev'] = torch.empty(slot['host'].numel(), dtype=torch.uint8, device=self.device)
             slot['event'] = torch.cuda.Event()
         ws, ws_size, ws_keep = _ws_args(ws_bytes, self.device)
-        with _Timed('syrk_group', flops, calls=len(rows)):
+        with _Timed('syrk_group', flops, calls=len(rows), floor=floor):
             rc = lib.ak_syrk_group_launch(specs_ptr, len(rows), ctypes.c_void_p(slot['host'].data_ptr()),
                                           ctypes.c_void_p(slot['dev'].data_ptr()), slot['host'].numel(),
                                           ws, ws_size, _stream(self.device))
@@ -472,12 +497,12 @@ class DeferredFactors:
         self.group.discard()
 
 
-def _group_take(row, flops, align_key, *tensors):
+def _group_take(row, flops, floor, align_key, *tensors):
     """True when the calling thread has an active group and it has taken the call."""
     grp = getattr(_group, 'active', None)
     if grp is None or (grp.plain_only and row[0] != 0) or not FactorGroup.eligible(row, align_key):
         return False
-    grp.add(row, flops, *tensors)
+    grp.add(row, flops, floor, *tensors)
     return True
 
 
@@ -507,15 +532,17 @@ def syrk_tn(x, out=None, alpha=1.0, beta=0.0, round_bf16=False):
         beta = 0.0
     if out.dtype != torch.float32 or out.shape != (d, d) or out.stride(1) != 1:
         raise ValueError('out has to be a float32 [d, d] tensor with contiguous rows')
+    flops = M * d * (d + 1)
+    floor = factor_floor_seconds(flops, x.dtype, M * d * x.element_size(), d, beta) if _timing_sink is not None else 0.0
     if x.dtype == torch.bfloat16 and getattr(_group, 'active', None) is not None:
         row = [0, x.data_ptr(), out.data_ptr(), out.stride(0), _float_bits(alpha) | (_float_bits(beta) << 32),
                M, d, ldx] + [0] * 8
-        if _group_take(row, M * d * (d + 1), x.data_ptr() & 15, x, out):
+        if _group_take(row, flops, floor, x.data_ptr() & 15, x, out):
             return out
     lib = _lib.load()
     need = _ws_need('ak_syrk_tn_ws_bytes', M, d)
     ws, ws_bytes, keep = _ws_args(need, x.device)
-    with _Timed('syrk_tn', M * d * (d + 1)):
+    with _Timed('syrk_tn', flops, floor=floor):
         rc = lib.ak_syrk_tn(ctypes.c_void_p(x.data_ptr()), _dtype_code(x), M, d, ldx, alpha, beta,
                             ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
     _lib.check(rc, 'ak_syrk_tn')
@@ -561,6 +588,12 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0, ro
             x = _as_bf16(x)
     if code is None:
         code = _dtype_code(x)
+    flops = N * h_out * w_out * d * (d + 1)
+    floor = 0.0
+    if _timing_sink is not None:
+        # a rounded fp32 input is read as fp32 and multiplied as bf16
+        floor = factor_floor_seconds(flops, torch.float32 if code == AK_F32 else torch.bfloat16,
+                                     N * C * H * W * x.element_size(), d, beta)
     if NCHW_VIA_CHANNELS_LAST and x.dtype == torch.bfloat16 and C % 8 == 0 and not few_channels \
             and x.is_contiguous() and C > 1 and N * C * H * W >= (1 << 16):
         # one transposing copy (memory-bound, a few microseconds) buys the direct-to-LDS kernels, which read rows of
@@ -573,11 +606,11 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0, ro
         if x.dtype == torch.bfloat16 and getattr(_group, 'active', None) is not None:
             row = [1, x.data_ptr(), out.data_ptr(), out.stride(0), _float_bits(alpha) | (_float_bits(beta) << 32),
                    N, C, H, W, kh, kw, sh, sw, ph, pw, 0]
-            if _group_take(row, N * h_out * w_out * d * (d + 1), x.data_ptr() & 15, x, out):
+            if _group_take(row, flops, floor, x.data_ptr() & 15, x, out):
                 return out
         need = _ws_need('ak_conv_syrk_nhwc_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
         ws, ws_bytes, keep = _ws_args(need, x.device)
-        with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
+        with _Timed('conv_syrk', flops, floor=floor):
             rc = lib.ak_conv_syrk_nhwc(ctypes.c_void_p(x.data_ptr()), code, N, C, H, W, kh, kw, sh, sw,
                                        ph, pw, alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0),
                                        ws, ws_bytes, _stream())
@@ -587,7 +620,7 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0, ro
     x = _contiguous(x)
     need = _ws_need('ak_conv_syrk_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
     ws, ws_bytes, keep = _ws_args(need, x.device)
-    with _Timed('conv_syrk', N * h_out * w_out * d * (d + 1)):
+    with _Timed('conv_syrk', flops, floor=floor):
         rc = lib.ak_conv_syrk(ctypes.c_void_p(x.data_ptr()), code, N, C, H, W, kh, kw, sh, sw, ph, pw,
                               alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream())
     if rc == AK_ERR_UNSUPPORTED and code == AK_F32_AS_BF16:     # a window too large for the LDS: cast, then the bf16 kernels
