@@ -1,19 +1,20 @@
 // out_m <- (A_m + lam_m I)^-1 for many symmetric positive definite fp32 matrices of DIFFERENT sizes in one call.
 //
-// Per matrix the arithmetic is the recursive blocked Cholesky of chol_inv.hip that carries the triangular inverse
-// along (work matrix W, lower triangle):
-//   F(lo, hi): n <= 128 -> one work group factors the diagonal block in the LDS and inverts the factor (chol_leaf.hpp)
-//              otherwise    F(lo, mid);  T1 = A21 M11^T;  { A22 -= T1 T1^T,  T2 = T1 M11 };  F(mid, hi);  M21 = -M22 T2
-//   out = M^T M.
-// T2 only needs T1 and M11, so it shares a launch with the trailing update: three product launches per node.
+// Per matrix (work matrix W, lower triangle) a right-looking blocked Cholesky that keeps the inverses of its 128 x 128
+// diagonal blocks, then the triangular inverse by levels, then out = M^T M (cg_right_looking below):
+//   for every diagonal block k:  leaf: W_kk -> M_kk = L_kk^-1 (one work group, in the LDS: chol_leaf.hpp);
+//                                panel: L21 = A21 M_kk^T;  update: A22 -= L21 L21^T
+//   for every level of a balanced tree over the blocks:  T2 = L21 M11;  M21 = -M22 T2
+// d^3 FLOP in total, like POTRF + POTRI.  Explicit inverses are taken of 128 x 128 diagonal blocks only, so a panel is
+// as accurate as a triangular solve with a block of that size (measured against fp64 on rank-deficient factors: 1.4-1.7
+// times the error of LAPACK's fp32 potrf + potri; a recursion that multiplied by the inverse of a whole half was at 3-8).
 //
-// What changes is the schedule.  The per-matrix sequences of steps (leaf | products) of ALL matrices are merged into
-// one sequence of "super-steps": super-step s holds, for every matrix whose next step has the type chosen for s,
-// that step.  One launch per super-step: a grouped leaf launch (one work group per diagonal block) or a grouped
-// product launch (one work group per 128 x 128 tile of any product of the step, split-bf16 MFMA tile of gemm_x3.hpp,
-// descriptor found by bisection on the running tile count).  The longest chain (the largest matrix) sets the number
-// of launches; the work of all smaller matrices runs in the shadow of its steps.  ResNet-50 (156 factors, 13 sizes):
-// about 150 launches instead of 620.
+// The per-matrix sequences of steps (leaf | products) of ALL matrices are merged into one sequence of "super-steps":
+// super-step s holds, for every matrix whose next step has the type chosen for s, that step.  One launch per
+// super-step: a grouped leaf launch (one work group per diagonal block) or a grouped product launch (one work group
+// per 128 x 128 tile of any product of the step, split-operand MFMA tile of gemm_x3.hpp, descriptor found through a
+// tile -> product map).  The longest chain (the largest matrix) sets the number of launches; the work of all smaller
+// matrices runs in the shadow of its steps.  ResNet-50 (108 factors, 13 sizes): 121 launches.
 //
 // The plan (descriptor tables, launch sequence) depends on the sizes only; every address in it is an offset into the
 // workspace.  The caller builds it once per size set on the host (ak_chol_group_plan), keeps a device copy, and
@@ -43,6 +44,7 @@ static float CG_HALF_MAX_COND = 65536.f;              // tuning builds: ak_debug
 #else
 constexpr float CG_HALF_MAX_COND = 65536.f;           // a / lam beyond 2^16: the matrix keeps the bf16 three-piece products
 #endif
+constexpr int CG_GROUP = 4;                           // block columns whose updates of the trailing matrix are merged
 constexpr int CG_COPY_ROWS = 8;                       // rows of W one work group of the copy-in kernel writes
 
 struct CgHeader {
@@ -285,6 +287,8 @@ static int64_t cg_pool(int64_t n) {
   return std::max(cg_pool(s1), s1 * s2 + cg_pool(s2));
 }
 
+static inline int64_t cg_align64(int64_t x) { return (x + 63) / 64 * 64; }
+
 static int64_t cg_tiles(const CgProd& p) {
   const int64_t tm = (p.M + 127) / 128, tn = (p.N + 127) / 128;
   return p.tile_mode == TILE_ALL ? tm * tn : tm * (tm + 1) / 2;
@@ -306,45 +310,79 @@ static CgProd cg_prod(int mat, int flags, int kind_a, int kind_b, int M, int N, 
   return p;
 }
 
-static void cg_range(std::vector<CgOp>& ops, int mat, int64_t w, int d, int dp, int64_t t1, int64_t t2, int lo, int hi,
-                     int64_t pool_off) {
+// The right-looking sequence of one matrix: for every diagonal block k of 128 columns
+//   leaf: W_kk -> M_kk = L_kk^-1;   panel: W[below, k] <- W[below, k] M_kk^T = L[below, k] (in place: every work group
+//   reads the 128 x 128 tile it writes, whole, before its epilogue);   update: W22 -= L21 L21^T (lower tiles, K = 128)
+// then the triangular inverse by levels of a balanced tree over the blocks (all nodes of one height are independent
+// and share two launches):   T2 = L21 M11;  W21 <- M21 = -M22 T2.
+// Every product of the factorization phase has as many tiles as the trailing matrix (hundreds for the wide factors).
+struct CgNode { int lo, mid, hi, height; };
+
+static int cg_nodes(std::vector<CgNode>& nodes, int lo, int hi) {
   const int n = hi - lo;
-  if (n <= LEAF) {
-    CgOp op;
-    op.type = CG_LEAF;
-    op.leaf = CgLeafTask{w + static_cast<int64_t>(lo) * dp + lo, mat, lo, n, dp, d, 0};
-    ops.push_back(op);
-    return;
-  }
+  if (n <= LEAF) return 0;
   const int mid = lo + static_cast<int>(cg_half(n));
-  cg_range(ops, mat, w, d, dp, t1, t2, lo, mid, pool_off);
-  const int s1 = mid - lo, s2 = hi - mid;
-  const int64_t W11 = w + static_cast<int64_t>(lo) * dp + lo, W21 = w + static_cast<int64_t>(mid) * dp + lo,
-                W22 = w + static_cast<int64_t>(mid) * dp + mid;
-  const int64_t T1 = t1 + pool_off, T2 = t2 + pool_off;
-  {
-    CgOp op;
-    op.type = CG_PROD;      // T1 = A21 M11^T
-    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_W, CG_KIND_M, s2, s1, s1, 1.f, W21, dp, W11, dp, 0.f, T1, s1,
-                               K_LE_J, TILE_ALL));
-    ops.push_back(op);
+  const int h = 1 + std::max(cg_nodes(nodes, lo, mid), cg_nodes(nodes, mid, hi));
+  nodes.push_back(CgNode{lo, mid, hi, h});
+  return h;
+}
+
+static void cg_right_looking(std::vector<CgOp>& ops, int mat, int64_t w, int d, int dp, int64_t t2) {
+  // Block columns are taken in groups of CG_GROUP: inside a group a block's rank-128 update goes to the remaining
+  // columns of the group only; the trailing matrix behind the group gets ONE update with the whole group as its
+  // contraction (K up to 128 CG_GROUP), i.e. it is read and written once per group instead of once per block.
+  for (int gs = 0; gs < dp; gs += CG_GROUP * LEAF) {
+    const int ge = std::min(gs + CG_GROUP * LEAF, dp);
+    for (int lo = gs; lo < ge; lo += LEAF) {
+      const int n = std::min(LEAF, dp - lo), below = dp - lo - n;
+      CgOp leaf;
+      leaf.type = CG_LEAF;
+      leaf.leaf = CgLeafTask{w + static_cast<int64_t>(lo) * dp + lo, mat, lo, n, dp, d, 0};
+      ops.push_back(leaf);
+      if (below == 0) break;
+      auto at = [&](int r, int c) { return w + static_cast<int64_t>(r) * dp + c; };
+      CgOp panel, update;
+      panel.type = update.type = CG_PROD;
+      panel.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_W, CG_KIND_M, below, n, n, 1.f, at(lo + n, lo), dp,
+                                    at(lo, lo), dp, 0.f, at(lo + n, lo), dp, K_LE_J, TILE_ALL));
+      ops.push_back(panel);
+      const int next = lo + n;
+      if (next < ge) {
+        // the group's remaining columns: the square on the diagonal (lower tiles) and the rows below the group
+        const int sq = ge - next, under = dp - ge;
+        update.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_L, CG_KIND_L, sq, sq, n, -1.f, at(next, lo), dp,
+                                       at(next, lo), dp, 1.f, at(next, next), dp, K_FULL, TILE_LOWER));
+        if (under > 0)
+          update.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_L, CG_KIND_L, under, sq, n, -1.f, at(ge, lo), dp,
+                                         at(next, lo), dp, 1.f, at(ge, next), dp, K_FULL, TILE_ALL));
+      } else {
+        // end of the group: the trailing matrix, with the group's ge - gs columns as the contraction
+        const int under = dp - ge;
+        update.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_L, CG_KIND_L, under, under, ge - gs, -1.f, at(ge, gs), dp,
+                                       at(ge, gs), dp, 1.f, at(ge, ge), dp, K_FULL, TILE_LOWER));
+      }
+      ops.push_back(update);
+    }
   }
-  {
-    CgOp op;
-    op.type = CG_PROD;      // A22 -= T1 T1^T (lower triangle);  T2 = T1 M11
-    op.prods.push_back(cg_prod(mat, CG_FLAG_TRANSB, CG_KIND_L, CG_KIND_L, s2, s2, s1, -1.f, T1, s1, T1, s1, 1.f, W22, dp,
-                               K_FULL, TILE_LOWER));
-    op.prods.push_back(cg_prod(mat, 0, CG_KIND_L, CG_KIND_M, s2, s1, s1, 1.f, T1, s1, W11, dp, 0.f, T2, s1, K_GE_J,
-                               TILE_ALL));
-    ops.push_back(op);
-  }
-  cg_range(ops, mat, w, d, dp, t1, t2, mid, hi, pool_off + static_cast<int64_t>(s1) * s2);
-  {
-    CgOp op;
-    op.type = CG_PROD;      // M21 = -M22 T2
-    op.prods.push_back(cg_prod(mat, 0, CG_KIND_M, CG_KIND_T2, s2, s1, s2, -1.f, W22, dp, T2, s1, 0.f, W21, dp, K_LE_I,
-                               TILE_ALL));
-    ops.push_back(op);
+  std::vector<CgNode> nodes;
+  const int top = cg_nodes(nodes, 0, dp);
+  for (int h = 1; h <= top; ++h) {
+    CgOp first, second;
+    first.type = second.type = CG_PROD;
+    int64_t pool = t2;
+    for (const CgNode& nd : nodes) {
+      if (nd.height != h) continue;
+      const int s1 = nd.mid - nd.lo, s2 = nd.hi - nd.mid;
+      const int64_t W11 = w + static_cast<int64_t>(nd.lo) * dp + nd.lo, W21 = w + static_cast<int64_t>(nd.mid) * dp + nd.lo,
+                    W22 = w + static_cast<int64_t>(nd.mid) * dp + nd.mid;
+      first.prods.push_back(cg_prod(mat, 0, CG_KIND_L, CG_KIND_M, s2, s1, s1, 1.f, W21, dp, W11, dp, 0.f, pool, s1, K_GE_J,
+                                    TILE_ALL));
+      second.prods.push_back(cg_prod(mat, 0, CG_KIND_M, CG_KIND_T2, s2, s1, s2, -1.f, W22, dp, pool, s1, 0.f, W21, dp,
+                                     K_LE_I, TILE_ALL));
+      pool += cg_align64(static_cast<int64_t>(s1) * s2);
+    }
+    ops.push_back(first);
+    ops.push_back(second);
   }
 }
 
@@ -379,7 +417,7 @@ static void cg_build(const int64_t* dims, int count, CgPlan& plan) {
     copy_blocks += (dp + CG_COPY_ROWS - 1) / CG_COPY_ROWS;
     const int64_t t1 = off + cg_align(static_cast<int64_t>(dp) * dp, 64), t2 = t1 + pool;
     off = t2 + pool;
-    cg_range(seq[m], m, cm.w_off, d, dp, t1, t2, 0, dp, 0);
+    cg_right_looking(seq[m], m, cm.w_off, d, dp, t1);     // the T2 panels of one level: at most dp^2 / 4 + 64 per node
     CgOp fin;
     fin.type = CG_PROD;     // out = M^T M, both triangles
     fin.prods.push_back(cg_prod(m, CG_FLAG_TRANSA | CG_FLAG_OUT_USER, CG_KIND_M, CG_KIND_M, d, d, dp, 1.f, cm.w_off, dp,

@@ -618,10 +618,10 @@ def test_chol_inv_grouped_operand_scaling(K, scale, lam_rel):
         assert torch.isfinite(o).all()
         e = relerr(o, ref)
         print(f'  matrix {i}: cond {cond:.1e}, relative error {e:.1e} (fp32 oracle {e_ref:.1e})', flush=True)
-        # The recursion multiplies by explicit inverses of the triangular diagonal blocks where LAPACK solves with
-        # them: on rank-deficient factors its error is 3-8 times that of potrf + potri (measured at cond 70 ... 2e5,
-        # the same for the bf16 three-piece and the fp16 two-piece products), on full-rank ones 1.3-1.6 times.
-        assert e < max(1e-4, 12 * e_ref), (i, cond, e, e_ref)
+        # Explicit inverses are taken of the 128 x 128 diagonal blocks only (LAPACK solves with the factor itself):
+        # measured 1.4-1.7 times the error of potrf + potri on the rank-deficient matrices, 1.3-1.6 on the full-rank
+        # ones.  The contract for inverses is 1e-4; beyond the conditioning that allows it, at most twice the oracle.
+        assert e < max(1e-4, 2 * e_ref), (i, cond, e, e_ref)
 
 
 @pytest.mark.parametrize('d', [2048, 2304, 4096, 4608])
