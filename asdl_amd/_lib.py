@@ -63,8 +63,6 @@ _SIGNATURES = {
     'ak_copy_bytes': (c_int, [c_ptr, c_ptr, c_i64, c_ptr]),
     'ak_absmax_block': (c_i64, []),
     'ak_absmax_grouped': (c_int, [c_ptr, c_int, c_i64, c_ptr]),
-    'ak_kron_precond_fused_max_short': (c_i64, []),
-    'ak_kron_precond_fused': (c_int, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_f32, c_ptr]),
     'ak_tril_pack': (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     'ak_tril_unpack': (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_ptr]),
     'ak_gemm_f32': (c_int, [c_int, c_int, c_i64, c_i64, c_i64, c_f32, c_ptr, c_i64, c_ptr, c_i64, c_f32,

@@ -217,30 +217,6 @@ extern "C" int ak_kron_precond(const float* Binv, const float* Ainv, float* G, i
                               static_cast<hipStream_t>(stream));
 }
 
-namespace ak {
-bool kron_fused_ok(int64_t dB, int64_t dA);
-int kron_precond_fused(const float* Binv, const float* Ainv, const float* G, float* out, int64_t dB, int64_t dA,
-                       float scale, hipStream_t stream);
-}  // namespace ak
-
-extern "C" int ak_kron_precond_fused(const float* Binv, const float* Ainv, const float* G, float* out, int64_t dB,
-                                     int64_t dA, const float* bias, float* bias_out, float grad_scale,
-                                     ak_stream_t stream) {
-  if (Binv == nullptr || Ainv == nullptr || G == nullptr || out == nullptr || out == G || dB <= 0 || dA <= 0 ||
-      dB > (1 << 30) || dA > (1 << 30) || (bias != nullptr && (bias_out == nullptr || bias_out == bias)))
-    return AK_ERR_ARG;
-  if (!ak::kron_fused_ok(dB, dA)) return AK_ERR_TOO_LARGE;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int rc = ak::kron_precond_fused(Binv, Ainv, G, out, dB, dA, grad_scale, s);
-  if (rc != AK_OK) return rc;
-  if (bias != nullptr) {
-    hipLaunchKernelGGL(ak::gemv_kernel, dim3(static_cast<unsigned>((dB + 3) / 4)), dim3(256), 0, s, Binv, bias, bias_out,
-                       dB, grad_scale);
-    return ak::check_launch();
-  }
-  return AK_OK;
-}
-
 extern "C" int64_t ak_kron_precond_static_max_floats(void) { return ak::STATIC_SCRATCH_FLOATS; }
 
 extern "C" int ak_kron_precond_static(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA,

@@ -1037,36 +1037,6 @@ def kron_precond(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
     return grad_w, grad_b
 
 
-def kron_precond_fused_ok(dB, dA):
-    return min(int(dB), int(dA)) <= _lib.load().ak_kron_precond_fused_max_short()
-
-
-def kron_precond_fused(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0, out_w=None, out_b=None):
-    """(out_w, out_b) = (grad_scale * B_inv @ view(grad_w, [dB, dA]) @ A_inv, grad_scale * B_inv @ grad_b), out of
-    place, the two products back to back in one launch with the intermediate in the LDS (true fp32 products).
-    Needs min(dB, dA) <= 1024."""
-    _require_gpu(B_inv, A_inv, grad_w, grad_b, out_w, out_b)
-    dB, dA = B_inv.shape[0], A_inv.shape[0]
-    if grad_w.numel() != dB * dA or not grad_w.is_contiguous() or grad_w.dtype != torch.float32:
-        raise ValueError('grad_w has to be a contiguous float32 tensor with dB * dA elements')
-    if grad_b is not None and (grad_b.numel() != dB or not grad_b.is_contiguous() or grad_b.dtype != torch.float32):
-        raise ValueError('grad_b has to be a contiguous float32 vector with dB elements')
-    if out_w is None:
-        out_w = torch.empty_like(grad_w)
-    if out_b is None and grad_b is not None:
-        out_b = torch.empty_like(grad_b)
-    if out_w.data_ptr() == grad_w.data_ptr() or out_w.shape != grad_w.shape or not out_w.is_contiguous() \
-            or out_w.dtype != torch.float32:
-        raise ValueError('out_w has to be another contiguous float32 tensor of the shape of grad_w')
-    null = ctypes.c_void_p(0)
-    rc = _lib.load().ak_kron_precond_fused(
-        ctypes.c_void_p(B_inv.data_ptr()), ctypes.c_void_p(A_inv.data_ptr()), ctypes.c_void_p(grad_w.data_ptr()),
-        ctypes.c_void_p(out_w.data_ptr()), dB, dA, ctypes.c_void_p(grad_b.data_ptr()) if grad_b is not None else null,
-        ctypes.c_void_p(out_b.data_ptr()) if grad_b is not None else null, grad_scale, _stream())
-    _lib.check(rc, 'ak_kron_precond_fused')
-    return out_w, out_b
-
-
 def kron_precond_static(B_inv, A_inv, grad_w, grad_b=None, grad_scale=1.0):
     """kron_precond through the entry point that brings its own scratch memory (a fixed array inside the library's
     device image, no workspace, no allocation): for callers that must not allocate.  Raises KernelError when

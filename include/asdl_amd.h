@@ -344,16 +344,6 @@ int ak_kron_precond(const float* Binv, const float* Ainv, float* G, int64_t dB, 
  * code object): make it before a stream capture begins.  No counterpart in the reference. */
 int64_t ak_kron_precond_static_max_floats(void);
 
-/* out <- grad_scale * Binv G Ainv (and bias_out <- grad_scale * Binv bias when bias != NULL) as back-to-back products
- * in ONE launch whose [dB, dA] intermediate never leaves the LDS: a work group owns 32 or 64 rows of the result seen
- * with the longer side of G as rows, computes that row panel of the first product into the LDS and multiplies it by
- * the factor of the shorter side from there.  Needs min(dB, dA) <= ak_kron_precond_fused_max_short() (1024: every
- * ResNet-50 layer), else AK_ERR_TOO_LARGE and nothing is touched.  True fp32 products.  out must not alias G
- * (every work group reads all of G), nor bias_out bias.  No workspace.
- * Replaces Kron.mvp (asdl/symmatrix.py:536-548), like ak_kron_precond. */
-int64_t ak_kron_precond_fused_max_short(void);
-int ak_kron_precond_fused(const float* Binv, const float* Ainv, const float* G, float* out, int64_t dB, int64_t dA,
-                          const float* bias, float* bias_out, float grad_scale, ak_stream_t stream);
 int ak_kron_precond_static(const float* Binv, const float* Ainv, float* G, int64_t dB, int64_t dA,
                            float* bias, float grad_scale, ak_stream_t stream);
 

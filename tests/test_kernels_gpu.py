@@ -824,47 +824,6 @@ def test_kron_precond_matches_oracle(K, dB, dA, bias):
         assert relerr(G4.view(dB, dA), 0.5 * rw) < 1e-5
 
 
-@pytest.mark.parametrize('dB,dA,bias', [(5, 7, True), (64, 576, False), (70, 33, True), (512, 4608, False),
-                                        (2048, 512, True), (1000, 2049, True), (256, 256, False), (1024, 1024, True),
-                                        (300, 1024, False), (1030, 520, True), (4608, 4, False)])
-def test_kron_precond_fused_matches_fp64(K, dB, dA, bias):
-    """The back-to-back kernel (intermediate in the LDS) against B_inv G A_inv in fp64, on either orientation (rows or
-    columns of G as the long side), ragged sizes, both row-panel heights (64 rows up to 512 short columns, else 32),
-    and against the two-launch path."""
-    g = torch.Generator().manual_seed(dB * 5 + dA)
-    Bi = torch.randn(dB, dB, generator=g)
-    Bi = (Bi @ Bi.T / dB).cuda()
-    Ai = torch.randn(dA, dA, generator=g)
-    Ai = (Ai @ Ai.T / dA).cuda()
-    G = torch.randn(dB, dA, generator=g).cuda()
-    b = torch.randn(dB, generator=g).cuda() if bias else None
-    assert K.kron_precond_fused_ok(dB, dA)
-    print(f'kron_precond_fused dB={dB} dA={dA}', flush=True)
-    keep = G.clone()
-    out_w, out_b = K.kron_precond_fused(Bi, Ai, G, b, grad_scale=0.25)
-    torch.cuda.synchronize()
-    assert torch.equal(G, keep), 'the input gradient must be left unchanged'
-    ref = 0.25 * Bi.double() @ G.double() @ Ai.double()
-    assert relerr(out_w, ref) < 1e-5, relerr(out_w, ref)
-    if bias:
-        assert relerr(out_b, 0.25 * Bi.double() @ b.double()) < 1e-5
-    two = G.clone()
-    K.kron_precond(Bi, Ai, two, None, grad_scale=0.25)
-    assert relerr(out_w, two) < 1e-5
-
-
-def test_kron_precond_fused_rejects_what_does_not_fit(K):
-    from asdl_amd._lib import KernelError
-    Bi, Ai = torch.eye(1100, device='cuda'), torch.eye(1200, device='cuda')
-    G = torch.ones(1100, 1200, device='cuda')
-    assert not K.kron_precond_fused_ok(1100, 1200)
-    with pytest.raises(KernelError):
-        K.kron_precond_fused(Bi, Ai, G)
-    with pytest.raises(ValueError):
-        K.kron_precond_fused(torch.eye(8, device='cuda'), torch.eye(8, device='cuda'), G[:8, :8].contiguous(),
-                             out_w=None if False else G[:8, :8])       # non-contiguous output
-
-
 # ------------------------------------------------------------------ unit-wise blocks (BatchNorm / LayerNorm)
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('kind,shape', [('bn2d', (6, 16, 7, 5)), ('bn2d_cl', (6, 16, 7, 5)), ('bn2d', (3, 70, 14, 14)),
