@@ -254,6 +254,12 @@ size_t conv_corr_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, in
 int conv_corr_syrk(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
                    int pw, float alpha, float beta, float* A, int64_t lda, void* ws, size_t ws_bytes, hipStream_t stream);
 
+// The same for an fp32 NCHW input: split into three bf16 planes first (products at the accuracy of fp32).
+size_t conv_corr_f32_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw);
+int conv_corr_syrk_f32(const float* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
+                       int pw, float alpha, float beta, float* A, int64_t lda, void* ws, size_t ws_bytes,
+                       hipStream_t stream);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? AK_OK : AK_ERR_LAUNCH; }
 
 // Split-K factor shared by the SYRK front ends: enough work groups to fill 256 CUs twice over

@@ -44,7 +44,10 @@ struct CorrProd {
   int32_t M;                           // positions
   int32_t Ho, Wo, kw, KK, pw;          // virtual convolution (stride 1, no padding above)
   uint32_t mWo, mHo, mKw, mBlk;
-  int32_t ti0, nti, tj0, ntj;          // tiles (ti0 + i, tj0 + j)
+  // Tiles: the row tap's C columns from tile ti0 on, `ntaps` column taps of C columns each from tile tj0 on.  With
+  // an input of three bf16 planes (C = 3 c channels, [hi | mid | lo]) whose planes are whole tiles, only the six plane
+  // pairs that matter are computed: npairs = 6, ppt = c / BT tiles per plane; else npairs = 1, ppt = C / BT.
+  int32_t ti0, tj0, ntaps, ppt, npairs, tpt;    // tpt: tiles per tap in the column direction (C / BT)
   int32_t kt_split, nsplit;            // k-tiles per row split, splits
   int32_t first_item, first_tile;      // running counts over the products
   int64_t part_off;                    // float4 index of partial tile (split 0, tile 0)
@@ -67,6 +70,23 @@ __device__ __forceinline__ int corr_find(const CorrArgs& a, int w, bool by_tile)
   return pi;
 }
 
+// Tile t of a product: (ti, tj) in the virtual Gram matrix, and (row, col) = where the tile starts in the product's
+// [C, ntaps C] block of the reduced matrix, in tiles.
+__device__ __forceinline__ void corr_tile_of(const CorrProd& cp, int t, int& ti, int& tj, int& row, int& col) {
+  const int per_pair = cp.ntaps * cp.ppt * cp.ppt;
+  const int pair = t / per_pair, rem = t - pair * per_pair;
+  const int tap = rem / (cp.ppt * cp.ppt), r2 = rem - tap * cp.ppt * cp.ppt;
+  const int ii = r2 / cp.ppt, jj = r2 - ii * cp.ppt;
+  // plane pairs in the order (0,0) (0,1) (0,2) (1,0) (1,1) (2,0): hi = 0, mid = 1, lo = 2, sum of the two <= 2
+  const int pi = pair < 3 ? 0 : (pair < 5 ? 1 : 2), pj = pair < 3 ? pair : (pair < 5 ? pair - 3 : 0);
+  row = pi * cp.ppt + ii;
+  col = tap * cp.tpt + pj * cp.ppt + jj;
+  ti = cp.ti0 + row;
+  tj = cp.tj0 + col;
+}
+
+__device__ __forceinline__ int corr_ntiles(const CorrProd& cp) { return cp.npairs * cp.ntaps * cp.ppt * cp.ppt; }
+
 // One work group per (product, row split, tile).
 template <int WR, int WC, int FR, int FC>
 __device__ __forceinline__ void corr_products_tile(const CorrArgs& a, uint32_t wg, uint32_t nwg) {
@@ -83,13 +103,21 @@ __device__ __forceinline__ void corr_products_tile(const CorrArgs& a, uint32_t w
   p.Ho = cp.Ho; p.Wo = cp.Wo;
   p.G = a.Cin;
   p.mWo = cp.mWo; p.mHo = cp.mHo; p.mKw = cp.mKw; p.mBlk = cp.mBlk; p.mG = a.mG; p.mKK = 0;
-  const int local = w - cp.first_item, ntiles = cp.nti * cp.ntj;
+  const int local = w - cp.first_item, ntiles = corr_ntiles(cp);
   const int s = local / ntiles, t = local - s * ntiles;
-  const int ti = cp.ti0 + t / cp.ntj, tj = cp.tj0 + t % cp.ntj;
+  int ti, tj, row, col;
+  corr_tile_of(cp, t, ti, tj, row, col);
   const int64_t k_begin = static_cast<int64_t>(s) * cp.kt_split * kDtlBK;
   int64_t k_end = k_begin + static_cast<int64_t>(cp.kt_split) * kDtlBK;
   if (k_end > cp.M) k_end = cp.M;
   const int rows = k_begin < k_end ? static_cast<int>(k_end - k_begin) : 0;
+  if (cp.nsplit == 1) {
+    // the only split: the tile goes straight into the reduced matrix
+    const int64_t ld = static_cast<int64_t>(kCorrPieces) * a.Cin;
+    dtl_tile<WR, WC, FR, FC, true>(p, ti, tj, k_begin, rows, nullptr,
+                                   a.red + cp.out_off + static_cast<int64_t>(row) * BT * ld + static_cast<int64_t>(col) * BT, ld);
+    return;
+  }
   floatx4* partial = a.part + cp.part_off + static_cast<int64_t>(local) * (BT * BT / 4);
   dtl_tile<WR, WC, FR, FC, true>(p, ti, tj, k_begin, rows, partial);
 }
@@ -102,7 +130,10 @@ __device__ __forceinline__ void corr_reduce_tile(const CorrArgs& a, int tile, in
   constexpr int NW = WR * WC, BT = 32 * FR * WR;
   constexpr int64_t tile_f4 = BT * BT / 4;
   const CorrProd& cp = a.prod[corr_find(a, tile, true)];
-  const int t = tile - cp.first_tile, ntiles = cp.nti * cp.ntj;
+  if (cp.nsplit == 1) return;                          // written by the product itself
+  const int t = tile - cp.first_tile, ntiles = corr_ntiles(cp);
+  int ti, tj, trow, tcol;
+  corr_tile_of(cp, t, ti, tj, trow, tcol);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave / WC, wc = wave % WC, g = lane >> 5, l32 = lane & 31;
   const int q = slot & 3, b = (slot >> 2) % FC, aa = (slot >> 2) / FC;
@@ -119,8 +150,8 @@ __device__ __forceinline__ void corr_reduce_tile(const CorrArgs& a, int tile, in
   }
   for (; s < cp.nsplit; ++s) acc += src[s * stride];
   const int ld = kCorrPieces * a.Cin;
-  const int row = (t / cp.ntj) * BT + 32 * FR * wr + 32 * aa + 8 * q + 4 * g;
-  const int col = (t % cp.ntj) * BT + 32 * FC * wc + 32 * b + l32;
+  const int row = trow * BT + 32 * FR * wr + 32 * aa + 8 * q + 4 * g;
+  const int col = tcol * BT + 32 * FC * wc + 32 * b + l32;
   float* dst = a.red + cp.out_off + static_cast<int64_t>(row) * ld + col;
 #pragma unroll
   for (int e = 0; e < 4; ++e) dst[static_cast<int64_t>(e) * ld] = acc[e];
@@ -233,11 +264,61 @@ __global__ __launch_bounds__(kAsmThreads) void corr_assemble_kernel(CorrAsm a) {
   }
 }
 
+// ---- fp32 inputs: three bf16 planes ------------------------------------------------------------------------------
+// An fp32 NCHW input takes the same path on the bf16 matrix cores at the accuracy of fp32 products: every element
+// is split exactly into three bf16 pieces, x = hi + mid + lo (each the remainder rounded to the nearest bf16; the
+// third needs no rounding), written as a channels-last tensor with 3 C channels, [hi | mid | lo] per pixel.  The
+// products above then run on that tensor as they are (3 C channels), and before the assembly the 3 x 3 blocks of
+// every [3 C, 3 C] piece are folded into [C, C]:  x^T y ~= hi^T hi' + (hi^T mid' + mid^T hi') + (hi^T lo' + lo^T hi')
+// + mid^T mid'; the three dropped blocks are below 2^-24 of the product.  The pairs are added in this order so that
+// the fold of a symmetric piece is symmetric to the last bit.
+
+// x: [N, C, HW] fp32 (HW contiguous) -> planes: [N, HW, 3 C] bf16.  One work group per (sample, 32 pixels, 32
+// channels): coalesced 128-byte reads along the pixels, 64-byte runs of channels per pixel and plane on the way out.
+__global__ __launch_bounds__(256) void corr_split_nchw_kernel(const float* __restrict__ x, uint16_t* __restrict__ planes,
+                                                              int C, int HW) {
+  __shared__ float tile[32][33];
+  const int n = blockIdx.z, p0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;          // 32 x 8
+  const float* src = x + (static_cast<int64_t>(n) * C + c0) * HW + p0;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int c = ty + 8 * r;
+    tile[c][tx] = p0 + tx < HW ? src[static_cast<int64_t>(c) * HW + tx] : 0.f;
+  }
+  __syncthreads();
+  uint16_t* dst = planes + (static_cast<int64_t>(n) * HW + p0) * (3 * C) + c0;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int px = ty + 8 * r;
+    if (p0 + px >= HW) continue;
+    const float v = tile[tx][px];
+    const __bf16 hi = static_cast<__bf16>(v);
+    const float r1 = v - static_cast<float>(hi);
+    const __bf16 mid = static_cast<__bf16>(r1);
+    const __bf16 lo = static_cast<__bf16>(r1 - static_cast<float>(mid));
+    uint16_t* q = dst + static_cast<int64_t>(px) * (3 * C) + tx;
+    q[0] = __builtin_bit_cast(uint16_t, hi);
+    q[C] = __builtin_bit_cast(uint16_t, mid);
+    q[2 * C] = __builtin_bit_cast(uint16_t, lo);
+  }
+}
+
+// red3: [3 C][29 * 3 C] (pieces of 3 C columns) -> red: [C][29 * C].  grid (29 C / 256, C).
+__global__ __launch_bounds__(256) void corr_fold_kernel(const float* __restrict__ red3, float* __restrict__ red, int C) {
+  const int col = blockIdx.x * 256 + threadIdx.x, c = blockIdx.y;
+  if (col >= kCorrPieces * C) return;
+  const int pc = col / C, c2 = col - pc * C;
+  const int64_t ld3 = static_cast<int64_t>(kCorrPieces) * 3 * C;
+  auto at = [&](int p, int q) { return red3[static_cast<int64_t>(p * C + c) * ld3 + pc * 3 * C + q * C + c2]; };
+  const float hh = at(0, 0), hm = at(0, 1) + at(1, 0), hl = at(0, 2) + at(2, 0), mm = at(1, 1);
+  red[static_cast<int64_t>(c) * (kCorrPieces * C) + col] = ((hh + hm) + hl) + mm;
+}
+
 // ---- host side ------------------------------------------------------------------------------------------------
 
 struct CorrPlan {
   CorrArgs args;            // X pointers, part and red are filled in per call
-  CorrAsm assemble;
   int bt, items, tiles;
   size_t part_f4, red_floats;
   int64_t x_off[kCorrProds];   // byte offset of each product's first pixel from the tensor
@@ -246,6 +327,7 @@ struct CorrPlan {
 static int corr_tile_width(int64_t C) {
   if (C % 256 == 0 && C >= 512) return 256;
   if (C % 128 == 0) return 128;
+  if (C % 192 == 0) return 192;
   if (C % 64 == 0) return 64;
   return 0;
 }
@@ -269,19 +351,22 @@ static bool corr_eligible(int64_t N, int64_t C, int64_t H, int64_t W, int kh, in
   return true;
 }
 
-static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W) {
+// planes: 1, or 3 when the C channels are the three bf16 planes of C / 3 channels
+static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W, int planes) {
   CorrPlan pl{};
   const int bt = corr_tile_width(C);
   pl.bt = bt;
   const int cb = static_cast<int>(C / bt);
-  const int occ = bt == 64 ? 4 : (bt == 128 ? 2 : 1);
+  // the unneeded plane pairs can be left out when every plane is a whole number of tiles
+  const bool pairs = planes == 3 && (C / 3) % bt == 0;
+  const int occ = bt == 64 ? 4 : (bt == 128 ? 2 : 1);      // work groups per CU
   const int64_t slots = 256 * occ;
   CorrArgs& a = pl.args;
   a.Cin = static_cast<int32_t>(C); a.H = static_cast<int32_t>(H); a.W = static_cast<int32_t>(W);
   a.nprod = kCorrProds;
   a.mG = make_magic(static_cast<uint32_t>(C));
-  auto fill = [&](int i, int64_t x_off, int64_t M, int64_t Ho, int64_t Wo, int kh_v, int kw_v, int pw_v, int ti0, int nti,
-                  int tj0, int ntj) {
+  auto fill = [&](int i, int64_t x_off, int64_t M, int64_t Ho, int64_t Wo, int kh_v, int kw_v, int pw_v, int ti0,
+                  int tj0, int ntaps) {
     CorrProd& p = a.prod[i];
     pl.x_off[i] = x_off;
     p.M = static_cast<int32_t>(M);
@@ -289,24 +374,28 @@ static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W) {
     p.kw = kw_v; p.KK = kh_v * kw_v; p.pw = pw_v;
     p.mWo = make_magic(p.Wo); p.mHo = make_magic(p.Ho); p.mKw = make_magic(kw_v);
     p.mBlk = make_magic(static_cast<uint32_t>(C) * p.KK);
-    p.ti0 = ti0; p.nti = nti; p.tj0 = tj0; p.ntj = ntj;
+    p.ti0 = ti0; p.tj0 = tj0; p.ntaps = ntaps;
+    p.tpt = cb;
+    p.npairs = pairs ? 6 : 1;
+    p.ppt = pairs ? cb / 3 : cb;
   };
   const int64_t px = C * 2;                      // bytes per pixel
-  fill(0, 0, N * H * W, H, W, 3, 5, 2, 2 * cb, cb, 2 * cb, kCorrShifts * cb);
-  fill(1, 0, N * W, 1, W, 1, 3, 0, 0, cb, 0, 3 * cb);                         // image row 0
-  fill(2, (H - 1) * W * px, N * W, 1, W, 1, 3, 0, 0, cb, 0, 3 * cb);          // image row H - 1
-  fill(3, 0, N * H, H, 1, 3, 1, 0, 0, cb, 0, 3 * cb);                         // image column 0
-  fill(4, (W - 1) * px, N * H, H, 1, 3, 1, 0, 0, cb, 0, 3 * cb);              // image column W - 1
+  fill(0, 0, N * H * W, H, W, 3, 5, 2, 2 * cb, 2 * cb, kCorrShifts);
+  fill(1, 0, N * W, 1, W, 1, 3, 0, 0, 0, 3);                         // image row 0
+  fill(2, (H - 1) * W * px, N * W, 1, W, 1, 3, 0, 0, 0, 3);          // image row H - 1
+  fill(3, 0, N * H, H, 1, 3, 1, 0, 0, 0, 3);                         // image column 0
+  fill(4, (W - 1) * px, N * H, H, 1, 3, 1, 0, 0, 0, 3);              // image column W - 1
   for (int r = 0; r < 2; ++r)
     for (int q = 0; q < 2; ++q)
-      fill(5 + 2 * r + q, ((r ? H - 1 : 0) * W + (q ? W - 1 : 0)) * px, N, 1, 1, 1, 1, 0, 0, cb, 0, cb);
+      fill(5 + 2 * r + q, ((r ? H - 1 : 0) * W + (q ? W - 1 : 0)) * px, N, 1, 1, 1, 1, 0, 0, 0, 1);
   int items = 0, tiles = 0;
   size_t part = 0;
   int64_t red_col = 0;
   const size_t tile_f4 = static_cast<size_t>(bt) * bt / 4;
   for (int i = 0; i < kCorrProds; ++i) {
     CorrProd& p = a.prod[i];
-    const int64_t ktiles = (p.M + kDtlBK - 1) / kDtlBK, ntiles = static_cast<int64_t>(p.nti) * p.ntj;
+    const int64_t ktiles = (p.M + kDtlBK - 1) / kDtlBK,
+                  ntiles = static_cast<int64_t>(p.npairs) * p.ntaps * p.ppt * p.ppt;
     int64_t ns = 1;
     if (i == 0 && ntiles > 0) {
       // the main product fills the device once (the corrections ride in its tail); at least 8 k-tiles per split
@@ -323,7 +412,7 @@ static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W) {
     p.first_tile = tiles;
     p.part_off = static_cast<int64_t>(part);
     p.out_off = red_col;
-    red_col += static_cast<int64_t>(p.ntj) * bt;       // C per piece: 13 C, 3 C or C
+    red_col += static_cast<int64_t>(p.ntaps) * C;      // C per piece: 13 C, 3 C or C
     items += p.nsplit * static_cast<int>(ntiles);
     tiles += static_cast<int>(ntiles);
     part += static_cast<size_t>(p.nsplit) * ntiles * tile_f4;
@@ -332,15 +421,15 @@ static CorrPlan corr_plan_build(int64_t N, int64_t C, int64_t H, int64_t W) {
   pl.tiles = tiles;
   pl.part_f4 = part;
   pl.red_floats = static_cast<size_t>(C) * kCorrPieces * C;       // red_col == 29 C
-  pl.assemble.C = static_cast<int32_t>(C);
   return pl;
 }
 
-static CorrPlan corr_plan(int64_t N, int64_t C, int64_t H, int64_t W) {
+static CorrPlan corr_plan(int64_t N, int64_t C, int64_t H, int64_t W, int planes = 1) {
   struct Key {
     int64_t N, C, H, W;
     bool operator==(const Key& o) const { return N == o.N && C == o.C && H == o.H && W == o.W; }
   };
+  H = planes == 3 ? -H : H;      // the two kinds of plan for one shape are two cache entries
   struct Hash {
     size_t operator()(const Key& k) const {
       uint64_t h = 0x9e3779b97f4a7c15ull;
@@ -357,7 +446,7 @@ static CorrPlan corr_plan(int64_t N, int64_t C, int64_t H, int64_t W) {
   auto it = cache.find(key);
   if (it != cache.end()) return it->second;
   if (cache.size() > 1024) cache.clear();
-  const CorrPlan plan = corr_plan_build(N, C, H, W);
+  const CorrPlan plan = corr_plan_build(N, C, H < 0 ? -H : H, W, planes);
   cache.emplace(key, plan);
   return plan;
 }
@@ -393,27 +482,24 @@ size_t conv_corr_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, in
   return corr_ws_layout(corr_plan(N, C, H, W), red_at);
 }
 
-int conv_corr_syrk(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
-                   int pw, float alpha, float beta, float* A, int64_t lda, void* ws, size_t ws_bytes,
-                   hipStream_t stream) {
-  if (!corr_eligible(N, C, H, W, kh, kw, sh, sw, ph, pw) || (reinterpret_cast<uintptr_t>(x) & 15) != 0)
-    return AK_ERR_UNSUPPORTED;
-  CorrPlan pl = corr_plan(N, C, H, W);
-  size_t red_at;
-  const size_t need = corr_ws_layout(pl, red_at);
-  if (ws == nullptr || ws_bytes < need) return AK_ERR_WORKSPACE;
+// All products of the layer on the channels-last bf16 tensor x (C channels), reduced into red [C][29 C].
+static int corr_products(const CorrPlan& plan, const void* x, floatx4* part, float* red, hipStream_t stream) {
+  CorrPlan pl = plan;
   CorrArgs& args = pl.args;
   for (int i = 0; i < kCorrProds; ++i) args.prod[i].X = static_cast<const unsigned char*>(x) + pl.x_off[i];
-  args.part = static_cast<floatx4*>(ws);
-  args.red = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + red_at);
-  int rc;
-  if (pl.bt == 64) rc = corr_launch_cfg<2, 2, 1, 1>(pl, args, stream);
-  else if (pl.bt == 128) rc = corr_launch_cfg<2, 2, 2, 2>(pl, args, stream);
-  else rc = corr_launch_cfg<2, 4, 4, 2>(pl, args, stream);
-  if (rc != AK_OK) return rc;
-  CorrAsm s = pl.assemble;
-  s.red = args.red;
+  args.part = part;
+  args.red = red;
+  if (pl.bt == 64) return corr_launch_cfg<2, 2, 1, 1>(pl, args, stream);
+  if (pl.bt == 128) return corr_launch_cfg<2, 2, 2, 2>(pl, args, stream);
+  if (pl.bt == 192) return corr_launch_cfg<2, 2, 3, 3>(pl, args, stream);
+  return corr_launch_cfg<2, 4, 4, 2>(pl, args, stream);
+}
+
+static int corr_assemble(const float* red, int64_t C, float alpha, float beta, float* A, int64_t lda, hipStream_t stream) {
+  CorrAsm s{};
+  s.red = red;
   s.A = A; s.lda = lda;
+  s.C = static_cast<int32_t>(C);
   s.alpha = alpha; s.beta = beta;
   // channels of rows per work group: 4 (60 KB of LDS) where that still gives a work group per CU
   const dim3 block(kAsmThreads);
@@ -427,6 +513,59 @@ int conv_corr_syrk(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, in
     hipLaunchKernelGGL((corr_assemble_kernel<1>), dim3(static_cast<unsigned>(C / kAsmCC), static_cast<unsigned>(C)),
                        block, 0, stream, s);
   return check_launch();
+}
+
+int conv_corr_syrk(const void* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
+                   int pw, float alpha, float beta, float* A, int64_t lda, void* ws, size_t ws_bytes,
+                   hipStream_t stream) {
+  if (!corr_eligible(N, C, H, W, kh, kw, sh, sw, ph, pw) || (reinterpret_cast<uintptr_t>(x) & 15) != 0)
+    return AK_ERR_UNSUPPORTED;
+  const CorrPlan pl = corr_plan(N, C, H, W);
+  size_t red_at;
+  const size_t need = corr_ws_layout(pl, red_at);
+  if (ws == nullptr || ws_bytes < need) return AK_ERR_WORKSPACE;
+  float* red = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + red_at);
+  const int rc = corr_products(pl, x, static_cast<floatx4*>(ws), red, stream);
+  if (rc != AK_OK) return rc;
+  return corr_assemble(red, C, alpha, beta, A, lda, stream);
+}
+
+// fp32 NCHW input: [planes: N H W 3C bf16][workspace of the 3 C-channel products, its reduced matrix last][red: C x 29 C]
+static size_t corr_f32_layout(int64_t N, int64_t C, int64_t H, int64_t W, const CorrPlan& pl3, size_t& ws3_at,
+                              size_t& red3_in_ws3, size_t& red_at) {
+  const size_t planes = static_cast<size_t>(N) * H * W * 3 * C * 2;
+  ws3_at = (planes + 255) & ~static_cast<size_t>(255);
+  const size_t ws3 = corr_ws_layout(pl3, red3_in_ws3);
+  red_at = (ws3_at + ws3 + 255) & ~static_cast<size_t>(255);
+  return red_at + static_cast<size_t>(C) * kCorrPieces * C * sizeof(float);
+}
+
+size_t conv_corr_f32_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph, int pw) {
+  if (C % 64 != 0 || !corr_eligible(N, 3 * C, H, W, kh, kw, sh, sw, ph, pw)) return 0;
+  size_t a, b, c;
+  return corr_f32_layout(N, C, H, W, corr_plan(N, 3 * C, H, W, 3), a, b, c);
+}
+
+int conv_corr_syrk_f32(const float* x, int64_t N, int64_t C, int64_t H, int64_t W, int kh, int kw, int sh, int sw, int ph,
+                       int pw, float alpha, float beta, float* A, int64_t lda, void* ws, size_t ws_bytes,
+                       hipStream_t stream) {
+  if (C % 64 != 0 || !corr_eligible(N, 3 * C, H, W, kh, kw, sh, sw, ph, pw)) return AK_ERR_UNSUPPORTED;
+  const CorrPlan pl3 = corr_plan(N, 3 * C, H, W, 3);
+  size_t ws3_at, red3_in_ws3, red_at;
+  const size_t need = corr_f32_layout(N, C, H, W, pl3, ws3_at, red3_in_ws3, red_at);
+  if (ws == nullptr || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return AK_ERR_WORKSPACE;
+  unsigned char* base = static_cast<unsigned char*>(ws);
+  uint16_t* planes = reinterpret_cast<uint16_t*>(base);
+  const int HW = static_cast<int>(H * W);
+  hipLaunchKernelGGL(corr_split_nchw_kernel, dim3((HW + 31) / 32, static_cast<unsigned>(C / 32), static_cast<unsigned>(N)),
+                     dim3(256), 0, stream, x, planes, static_cast<int>(C), HW);
+  float* red3 = reinterpret_cast<float*>(base + ws3_at + red3_in_ws3);
+  const int rc = corr_products(pl3, planes, reinterpret_cast<floatx4*>(base + ws3_at), red3, stream);
+  if (rc != AK_OK) return rc;
+  float* red = reinterpret_cast<float*>(base + red_at);
+  hipLaunchKernelGGL(corr_fold_kernel, dim3(static_cast<unsigned>((kCorrPieces * C + 255) / 256), static_cast<unsigned>(C)),
+                     dim3(256), 0, stream, red3, red, static_cast<int>(C));
+  return corr_assemble(red, C, alpha, beta, A, lda, stream);
 }
 
 }  // namespace ak

@@ -585,8 +585,8 @@ extern "C" size_t ak_conv_syrk_ws_bytes(int64_t N, int64_t C, int64_t H, int64_t
   const size_t patch = ak::conv_patch_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw);
   if (patch > 0) return patch;
   ak::ConvPlan a, b;
-  size_t need = 0;
-  if (ak::make_plan(a, 2, N, C, H, W, kh, kw, sh, sw, ph, pw)) need = a.ws_need;
+  size_t need = ak::conv_corr_f32_ws_bytes(N, C, H, W, kh, kw, sh, sw, ph, pw);
+  if (ak::make_plan(a, 2, N, C, H, W, kh, kw, sh, sw, ph, pw) && a.ws_need > need) need = a.ws_need;
   if (ak::make_plan(b, 4, N, C, H, W, kh, kw, sh, sw, ph, pw) && b.ws_need > need) need = b.ws_need;
   return need;
 }
@@ -605,6 +605,12 @@ extern "C" int ak_conv_syrk(const void* x, int dtype, int64_t N, int64_t C, int6
     if (rc != AK_ERR_UNSUPPORTED) return rc;
   }
   if (dtype == AK_F32_AS_BF16) return AK_ERR_UNSUPPORTED;      // rounding on the fly is the window kernel's
+  if (dtype == AK_F32) {
+    // 3 x 3, stride 1, padding 1: shifted correlations of three bf16 planes of the input
+    const int rc = ak::conv_corr_syrk_f32(static_cast<const float*>(x), N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta, A,
+                                          lda, ws, ws_bytes, static_cast<hipStream_t>(stream));
+    if (rc != AK_ERR_UNSUPPORTED) return rc;
+  }
   ak::ConvPlan plan;
   if (!ak::make_plan(plan, dtype == AK_BF16 ? 2 : 4, N, C, H, W, kh, kw, sh, sw, ph, pw)) return AK_ERR_UNSUPPORTED;
   if (lda < plan.p.d) return AK_ERR_ARG;

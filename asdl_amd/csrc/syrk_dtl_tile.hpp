@@ -180,10 +180,11 @@ __device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t wgid, uint32_t nw
 
 // Rows [k_begin, k_begin + rows) of the operand into tile (ti, tj) of one factor.  partial == nullptr: the result is
 // the factor's tile (alpha, beta, mirror image); otherwise the accumulators go to `partial` in accumulator order,
-// [(a, b, q)][thread] float4, for a reduction pass.
+// [(a, b, q)][thread] float4, for a reduction pass.  raw != nullptr: the bare tile goes to a row-major matrix.
 template <int WR, int WC, int FR, int FC, bool GATHER>
 __device__ __forceinline__ void dtl_tile(const DtlParams& p, int ti, int tj, int64_t k_begin, int rows,
-                                         floatx4* __restrict__ partial) {
+                                         floatx4* __restrict__ partial, float* __restrict__ raw = nullptr,
+                                         int64_t raw_ld = 0) {
   using Cfg = DtlCfg<WR, WC, FR, FC, GATHER>;
   constexpr int NW = Cfg::NW, BT = Cfg::BT, NCB = Cfg::NCB, IPW = Cfg::IPW, BK = kDtlBK, S = kDtlStages;
   extern __shared__ __attribute__((aligned(1024))) unsigned char dtl_smem[];
@@ -353,7 +354,17 @@ __device__ __forceinline__ void dtl_tile(const DtlParams& p, int ti, int tj, int
   else mainloop(std::false_type{});
 
   const int64_t gi0 = i0 + 32 * FR * wr, gj0 = j0 + 32 * FC * wc;
-  if (partial == nullptr) {
+  if (raw != nullptr) {
+    // the tile as it is, row-major with leading dimension raw_ld at `raw` (no scaling, no mirror image, no bounds)
+    const int g = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int a = 0; a < FR; ++a)
+#pragma unroll
+      for (int b = 0; b < FC; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          raw[(32 * FR * wr + 32 * a + 8 * (r >> 2) + 4 * g + (r & 3)) * raw_ld + 32 * FC * wc + 32 * b + l32] = acc[a][b][r];
+  } else if (partial == nullptr) {
     dtl_epilogue<FR, FC, GATHER>(acc, p, gi0, gj0, diag, lane);
   } else {
 #pragma unroll

@@ -253,6 +253,34 @@ def test_conv_syrk_shifted_correlations_match_oracle(K, case):
     assert torch.equal(out, out.T)
 
 
+CORR_F32_CASES = [(2, 64, 5, 7), (3, 128, 8, 8), (2, 256, 4, 6), (1, 512, 7, 7), (4, 64, 16, 16), (2, 192, 6, 5),
+                  (8, 64, 32, 32)]
+
+
+@pytest.mark.parametrize('case', CORR_F32_CASES, ids=[str(c) for c in CORR_F32_CASES])
+def test_conv_syrk_fp32_nchw_shifted_correlations_match_oracle(K, case):
+    """fp32 NCHW inputs of 3 x 3 / stride 1 / padding 1 layers: the input is split exactly into three bf16 planes
+    (channels-last, 3 C channels), the shifted correlations run on the bf16 matrix cores, and the plane pairs are
+    folded before the assembly.  The result has to be the fp32 statistic (asdl/operations/conv.py:80-88) to 1e-5,
+    not a bf16-rounded one: inputs with a wide dynamic range inside every patch."""
+    N, C, H, W = case
+    g = torch.Generator().manual_seed(7 * N + C + H)
+    x = torch.randn(N, C, H, W, generator=g) * torch.exp(2 * torch.randn(N, C, H, W, generator=g))
+    ref = R.conv_cov_kron_A(x.double(), (3, 3), (1, 1), (1, 1))
+    print(f'conv_syrk fp32 nchw shifted correlations case={case}', flush=True)
+    xg = x.cuda()
+    out = K.conv_syrk(xg, (3, 3), (1, 1), (1, 1), alpha=1.0 / (H * W))
+    torch.cuda.synchronize()
+    assert relerr(out, ref) < 1e-5, relerr(out, ref)
+    assert torch.equal(out, out.T)
+    # not the statistic of the bf16-rounded input
+    assert relerr(out, R.conv_cov_kron_A(x.bfloat16().double(), (3, 3), (1, 1), (1, 1))) > 1e-4
+    K.conv_syrk(xg, (3, 3), (1, 1), (1, 1), out=out, alpha=0.25 / (H * W), beta=2.0)
+    torch.cuda.synchronize()
+    assert relerr(out, 2.25 * ref) < 1e-5
+    assert torch.equal(out, out.T)
+
+
 @pytest.mark.parametrize('layout', ['nchw', 'channels_last'])
 def test_round_bf16_outside_the_window_kernel_is_a_cast(K, layout):
     """round_bf16 for operands the window kernel does not take (many channels, 1x1 windows, plain rows): the wrappers
