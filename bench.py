@@ -489,9 +489,13 @@ def main():
                                      f'4608 x 4608, damping {args.damping}, BatchNorm ignored, cudnn.benchmark off',
                          'batch': bs}
         if 'roofline' in out:
-            out['roofline']['kernel'] = ('factor statistics of fp32 NCHW operands (conv_syrk_kernel<float>, '
-                                         'conv_patch_syrk_kernel<float>, syrk_tn_kernel<float>: v_mfma_f32_32x32x2_f32), SYRK '
-                                         'FLOP M*d*(d+1) against the fp32 matrix peak')
+            out['roofline']['kernel'] = ('factor statistics of fp32 NCHW operands: the 3x3 stride-1 layers as shifted '
+                                         'correlations of three bf16 planes of the input (corr_split_nchw_kernel, '
+                                         'corr_products_kernel, corr_fold_kernel, corr_assemble_kernel: bf16 matrix '
+                                         'cores, fp32 accuracy), the others on conv_syrk_kernel<float>, '
+                                         'conv_patch_syrk_kernel<float>, syrk_tn_kernel<float> (v_mfma_f32_32x32x2_f32); '
+                                         'SYRK FLOP M*d*(d+1) against the fp32 matrix peak, the rate the reference\'s '
+                                         'fp32 arithmetic is priced at')
     inv = inverse_roofline(w, args.damping) if not args.no_inverse_roofline else None
     if inv is not None:
         out['roofline_inverse'] = inv
