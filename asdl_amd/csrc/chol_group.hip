@@ -254,6 +254,7 @@ static __global__ __launch_bounds__(256) void cg_prod_kernel(CgArgs a, const CgP
   p.kmode = d.kmode; p.tile_mode = d.tile_mode;
   p.active = nullptr; p.active_stride = 0;
   p.split = 3;
+  p.chunked = 0;
   p.scaleA = p.scaleB = 1.f;
   const float* __restrict__ sc = a.scales + static_cast<int64_t>(d.mat) * CG_SCALE_FLOATS;
   if (sc[4] != 0.f) {

@@ -39,6 +39,10 @@ struct GemmParams {
   const int* active;        // optional per-batch flags: batch z runs only if active[z*active_stride] != 0
   int active_stride;
   int split;                // 0: fp32 MFMA; 2 / 3: bf16 MFMA on operands split into that many bf16 pieces (gemm_x3.hpp)
+  int chunked;              // non-zero: the contraction is summed in chunks (a fresh accumulator every 128 / 256 k, added
+                            // to a running total), which keeps the rounding error of a long sum near that of one
+                            // rounding instead of growing with the number of matrix instructions (fp32 kernel, and the
+                            // three-piece kernel for untransposed operands; ignored elsewhere)
   float scaleA, scaleB;     // fp16-piece variant only: powers of two the operands are multiplied by before the split
   float* absmax_out;        // optional (split kernels): max |C| of the result is folded into this word with an integer
                             // atomic maximum on its bit pattern (the caller zeroes it first)
@@ -107,7 +111,10 @@ __device__ __forceinline__ void gemm_frag(float (&f)[8], const float* __restrict
 }
 
 // One BT x BT tile (ti, tj) of batch entry z of the product described by p; lds: [2][2][PANEL] floats.
-template <int TI>
+// CHUNKED: every 8 k-tiles (128 k) the accumulators are added to a running total and start again from zero: the
+// matrix instruction rounds its accumulator once per two k, so a contraction over K rounds K/2 times at the full
+// magnitude of the sum; in chunks, 64 roundings happen at the magnitude of one chunk and K/128 at the full one.
+template <int TI, bool CHUNKED = false>
 __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int tj, int z,
                                               float (*lds)[2][GemmTile<64 * TI>::PANEL]) {
   constexpr int BT = 64 * TI;
@@ -139,6 +146,16 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int t
     for (int b = 0; b < TI; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  constexpr int TT = CHUNKED ? TI : 1;
+  floatx16 tot[TT][TT];
+  if constexpr (CHUNKED) {
+#pragma unroll
+    for (int a = 0; a < TI; ++a)
+#pragma unroll
+      for (int b = 0; b < TI; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tot[a][b][r] = 0.f;
+  }
 
   const int nk = kbeg < kend ? (kend - kbeg + GBK - 1) / GBK : 0;
   floatx4 ra[GemmTile<BT>::CHUNKS], rb[GemmTile<BT>::CHUNKS];
@@ -167,6 +184,16 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int t
       for (int a = 0; a < TI; ++a)
 #pragma unroll
         for (int b = 0; b < TI; ++b) acc[a][b] = mfma_f32(fa[a][m], fb[b][m], acc[a][b]);
+    if constexpr (CHUNKED) {
+      if ((kt & 7) == 7) {
+#pragma unroll
+        for (int a = 0; a < TI; ++a)
+#pragma unroll
+          for (int b = 0; b < TI; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { tot[a][b][r] += acc[a][b][r]; acc[a][b][r] = 0.f; }
+      }
+    }
     if (kt + 1 < nk) {
       gemm_stash<BT>(ra, lds[buf ^ 1][0], a_kc, tid);
       gemm_stash<BT>(rb, lds[buf ^ 1][1], b_kc, tid);
@@ -174,6 +201,14 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int t
     __syncthreads();
   }
 
+  if constexpr (CHUNKED) {
+#pragma unroll
+    for (int a = 0; a < TI; ++a)
+#pragma unroll
+      for (int b = 0; b < TI; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += tot[a][b][r];
+  }
   const bool lower_only = (p.tile_mode == TILE_LOWER);
   const bool mirror = (p.tile_mode == TILE_LOWER_MIRROR) && (ti != tj);
 #pragma unroll
@@ -196,10 +231,10 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int t
     }
 }
 
-template <int TI>
+template <int TI, bool CHUNKED = false>
 static __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(16))) float lds[2][2][GemmTile<64 * TI>::PANEL];
-  gemm_f32_tile<TI>(p, blockIdx.y, blockIdx.x, blockIdx.z, lds);
+  gemm_f32_tile<TI, CHUNKED>(p, blockIdx.y, blockIdx.x, blockIdx.z, lds);
 }
 
 }  // namespace ak
@@ -236,6 +271,7 @@ inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
     // hand), one instantiation per pair of operand layouts; two pieces: the single-buffered loop
     if (p.split == 3 && g_x3_double_buffer) {
       if (p.transA == 0 && p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 1>), grid, dim3(256), 0, stream, q);
+      else if (p.transA == 0 && p.chunked) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 0, true>), grid, dim3(256), 0, stream, q);
       else if (p.transA == 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 1, 0>), grid, dim3(256), 0, stream, q);
       else if (p.transB != 0) hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 1>), grid, dim3(256), 0, stream, q);
       else hipLaunchKernelGGL((gemm_x3_kernel<3, true, 0, 0>), grid, dim3(256), 0, stream, q);
@@ -249,10 +285,12 @@ inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
   // 128 x 128 tiles when they alone fill the 256 CUs twice over, else 64 x 64 tiles (four times the work groups)
   if (work_groups >= 512) {
     dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, batch);
-    hipLaunchKernelGGL(gemm_f32_kernel<2>, grid, dim3(256), 0, stream, p);
+    if (p.chunked) hipLaunchKernelGGL((gemm_f32_kernel<2, true>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(gemm_f32_kernel<2>, grid, dim3(256), 0, stream, p);
   } else {
     dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
-    hipLaunchKernelGGL(gemm_f32_kernel<1>, grid, dim3(256), 0, stream, p);
+    if (p.chunked) hipLaunchKernelGGL((gemm_f32_kernel<1, true>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(gemm_f32_kernel<1>, grid, dim3(256), 0, stream, p);
   }
   return check_launch();
 }
@@ -271,6 +309,7 @@ inline GemmParams make_gemm(int transA, int transB, int M, int N, int K, float a
   p.absmax_out = nullptr;
   p.active = nullptr; p.active_stride = 0;
   p.split = 0;
+  p.chunked = 0;
   return p;
 }
 

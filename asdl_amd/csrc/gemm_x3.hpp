@@ -164,9 +164,14 @@ __device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bo
 }
 
 // One 128 x 128 tile (ti, tj) of batch entry z of the product described by p.
-template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool HALF = false>
+// CHUNKED (three pieces): the products of the leading pieces, which carry the magnitude of the result, have an
+// accumulator of their own that is added to a running total every 8 k-tiles (256 k: 16 roundings at the magnitude of
+// a chunk, K/256 at the full one); the five cross products, 2^-8 and less of that magnitude, share a second one.
+// The sum then carries about one rounding error instead of one that grows with 6 K / 16 accumulator roundings.
+template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool HALF = false, bool CHUNKED = false>
 __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj, int z, AK_LDS3 unsigned char* lds) {
   static_assert(!HALF || (NSPLIT == 2 && !DB), "fp16 pieces: two of them, single-buffered loop");
+  static_assert(!CHUNKED || NSPLIT == 3, "chunked sums: three pieces");
   constexpr int BT = X3_BT, BK = X3_BK;
   constexpr int BUF = 2 * NSPLIT * X3_PLANE;        // both operands' planes of one k-tile
   AK_LDS3 unsigned char* panelA = lds;
@@ -198,6 +203,29 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  constexpr int TT = CHUNKED ? 2 : 1;
+  floatx16 small[TT][TT], tot[TT][TT];
+  if constexpr (CHUNKED) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) small[a][b][r] = tot[a][b][r] = 0.f;
+  }
+  // end of k-tile kt: every eighth one moves the leading products' accumulators into the running total
+  auto end_of_ktile = [&](int kt) {
+    if constexpr (CHUNKED) {
+      if ((kt & 7) == 7) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { tot[a][b][r] += acc[a][b][r]; acc[a][b][r] = 0.f; }
+      }
+    }
+  };
 
   const int nk = kbeg < kend ? (kend - kbeg + BK - 1) / BK : 0;
   const bool interior = i0 + BT <= p.M && j0 + BT <= p.N && (kend - kbeg) % BK == 0;
@@ -221,6 +249,15 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
           // smallest terms first
+          if constexpr (CHUNKED) {
+            small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], small[a][b]);
+            small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], small[a][b]);
+            small[a][b] = x3_mfma<HALF>(fa[a][2], fb[b][0], small[a][b]);
+            small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][1], small[a][b]);
+            small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][0], small[a][b]);
+            acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][0], acc[a][b]);
+            continue;
+          }
           if constexpr (NSPLIT >= 3) {
             acc[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], acc[a][b]);
             acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], acc[a][b]);
@@ -292,7 +329,12 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
             {   // matrix instruction m: (h, a, b) and the term, smallest terms first
               constexpr int PA[6] = {1, 0, 2, 0, 1, 0}, PB[6] = {1, 2, 0, 1, 0, 0};
               const int h = m / 24, ab = (m % 24) / 6, t = m % 6;
-              acc[ab >> 1][ab & 1] = mfma_bf16(fa[h][ab >> 1][PA[t]], fb[h][ab & 1][PB[t]], acc[ab >> 1][ab & 1]);
+              constexpr int SM = CHUNKED ? 1 : 0;       // the cross products' accumulators exist in that variant only
+              if (CHUNKED && t < 5)
+                small[SM * (ab >> 1)][SM * (ab & 1)] =
+                    mfma_bf16(fa[h][ab >> 1][PA[t]], fb[h][ab & 1][PB[t]], small[SM * (ab >> 1)][SM * (ab & 1)]);
+              else
+                acc[ab >> 1][ab & 1] = mfma_bf16(fa[h][ab >> 1][PA[t]], fb[h][ab & 1][PB[t]], acc[ab >> 1][ab & 1]);
             }
             {   // sixth m of the split: float4 u (0..3 of A, 4..7 of B), pair e, piece q
               const int u = m / 6, q = (m % 6) / 2, e = m % 2;
@@ -316,6 +358,7 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
             }
             __builtin_amdgcn_sched_barrier(0);
           }
+          end_of_ktile(kt);
           __syncthreads();
         }
       }
@@ -324,6 +367,7 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
         AK_LDS3 unsigned char* nxt = lds + ((kt + 1) & 1) * BUF;
         if (kt + 1 < nk) stash(nxt);
         multiply(cur);
+        end_of_ktile(kt);
         __syncthreads();
       }
     } else {
@@ -331,6 +375,7 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
       for (int kt = 0; kt < nk; ++kt) {
         if (kt + 1 < nk) fetch(kt + 1);       // next k-tile's global loads fly during this one's MFMAs
         multiply(lds);
+        end_of_ktile(kt);
         __syncthreads();                      // everybody is done reading this k-tile
         if (kt + 1 < nk) stash(lds);
         __syncthreads();
@@ -340,6 +385,14 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
   if (interior) mainloop(std::true_type{});
   else mainloop(std::false_type{});
   (void)g; (void)panelA; (void)panelB;
+  if constexpr (CHUNKED) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] = (tot[a][b][r] + acc[a][b][r]) + small[a][b][r];
+  }
 
   // the partial products of (i, j) and (j, i) are summed in different orders, so a mirrored result takes both
   // triangles of a diagonal tile from the lower one
@@ -395,7 +448,7 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
   }
 }
 
-template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1>
+template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool CHUNKED = false>
 static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char x3_smem[(DB ? 2 : 1) * 2 * NSPLIT * X3_PLANE];
   int ti = blockIdx.y, tj = blockIdx.x;
@@ -403,7 +456,7 @@ static __global__ __launch_bounds__(256) void gemm_x3_kernel(GemmParams p) {
     p.tile_mode &= ~TILE_LINEAR_GRID;
     decode_lower_tile(blockIdx.x, ti, tj);
   }
-  gemm_x3_tile<NSPLIT, DB, AKC, BKC>(p, ti, tj, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
+  gemm_x3_tile<NSPLIT, DB, AKC, BKC, false, CHUNKED>(p, ti, tj, blockIdx.z, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // Grouped products: many independent C_i <- alpha_i * op(A_i) op(B_i) + beta_i * C_i of different sizes in one
@@ -446,6 +499,7 @@ __device__ __forceinline__ bool grouped_lookup(const int64_t* __restrict__ table
   p.tile_mode = (r[9] & 4) ? TILE_LOWER_MIRROR : TILE_ALL;     // symmetric result: lower tiles only, mirrored
   p.active = nullptr; p.active_stride = 0;
   p.split = 0;
+  p.chunked = 0;
   p.scaleA = p.scaleB = 1.f;
   p.absmax_out = reinterpret_cast<float*>(r[14]);
   const int local = w - static_cast<int>(r[11]);

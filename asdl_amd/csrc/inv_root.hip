@@ -337,6 +337,10 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.active = st.active; g.active_stride = 1;
     g.split = g_root_split;
+    // sums in chunks: the error of the root is set by the absolute rounding error of the first iterations' products
+    // against the smallest eigenvalues of M (ridge_eps of the largest); a rank-deficient 1024 x 1024 statistic lost a
+    // factor of six against LAPACK-grade fp32 products with one accumulator rounded at every matrix instruction
+    g.chunked = 1;
     // Every matrix of the iteration is a polynomial of the one symmetric statistic, so every product is symmetric up
     // to rounding: large ones compute the tiles on and below the diagonal only and mirror them (half the work; the
     // results are then exactly symmetric).  Small ones keep the full product.

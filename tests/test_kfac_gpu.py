@@ -921,13 +921,14 @@ def test_grouped_factor_launches_give_the_single_launch_factors(ema, fisher_type
         del taken[:]
         got = run(True, every)
         # per step: B of the four convolutions once per backward pass (the Linear layer's 10 columns are not a
-        # multiple of 8), and with forward grouping A of the four layers that are not the few-channel stem; with
-        # -2 only those of them that are plain X^T X products (kind 0, like every B)
+        # multiple of 8), and with forward grouping A of the three layers that are neither the few-channel stem nor
+        # the 64-channel 3x3 layer (whose factor comes from shifted correlations of its input, launched at once);
+        # with -2 only those of them that are plain X^T X products (kind 0, like every B)
         passes = {FISHER_EMP: 1, FISHER_MC: n_mc, FISHER_EXACT: 10}[fisher_type]
         if plain_forward is None:
             plain_forward = taken.count(0) - 2 * 4 * passes
-            assert 0 < plain_forward < 2 * 4
-        forward = {-1: 0, -2: plain_forward}.get(every[0], 2 * 4)
+            assert 0 < plain_forward < 2 * 3
+        forward = {-1: 0, -2: plain_forward}.get(every[0], 2 * 3)
         assert len(taken) == 2 * 4 * passes + forward and (every[0] < 0 or 1 in taken), (every, taken)
         assert every[0] != -2 or 1 not in taken
         assert got.keys() == ref.keys()
