@@ -49,7 +49,8 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
             if op_class is None:
                 continue
             names = [n for n in names if n in op_class.supported_operations]
-            cxt.register_operation(module, op_class(module, names, model_for_kernel=model))
+            op = op_class(module, names, model_for_kernel=model)
+            cxt.register_operation(module, op)
             has_fwd = any(n in FWD_OPS for n in names)
             has_bwd = any(n in BWD_OPS for n in names)
             if not (has_fwd or has_bwd):
@@ -58,16 +59,16 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
             # only the stored outputs and the unit-wise statistics look at the module's output
             needs_out = OP_SAVE_OUTPUTS in names or any(n in BWD_OPS_WITH_INPUTS for n in names)
 
-            def forward_hook(_module, in_data, out_data, _has_bwd=has_bwd, _needs_out=needs_out):
+            def forward_hook(_module, in_data, out_data, _has_bwd=has_bwd, _needs_out=needs_out, _op=op):
                 x = in_data[0].detach()
                 y = out_data.detach() if _needs_out else None
-                run_hook(lambda: cxt.call_operations_in_forward(_module, x, y), x)
+                run_hook(lambda: _op.forward_post_process(x, y), x)
                 if _has_bwd and out_data.requires_grad:
                     def grad_hook(grad, _m=_module):
                         if not cxt.is_operation_registered(_m):
                             return None          # context already closed
                         g = grad.detach()
-                        run_hook(lambda: cxt.call_operations_in_backward(_m, g), g, backward=True)
+                        run_hook(lambda: _op.backward_pre_process(g, None), g, backward=True)
                         return None
                     handles.append(out_data.register_hook(grad_hook))
                     # the graph edge the hook sits on: a backward pass restricted to these edges still fires

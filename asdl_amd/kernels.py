@@ -416,6 +416,8 @@ class FactorGroup:
                 alpha = struct.unpack('<f', struct.pack('<I', rows[0][4] & 0xffffffff))[0]
                 beta = struct.unpack('<f', struct.pack('<I', rows[0][4] >> 32))[0]
                 if rows[0][0] == 0:
+                    if x.ndim != 2:      # kept as the hook saw it: the [M, d] rows the row describes
+                        x = torch.as_strided(x, (rows[0][5], rows[0][6]), (rows[0][7], 1))
                     syrk_tn(x, out=out, alpha=alpha, beta=beta)
                 else:
                     r = rows[0]
@@ -503,7 +505,58 @@ def _group_take(row, flops, floor, align_key, *tensors):
     if grp is None or (grp.plain_only and row[0] != 0) or not FactorGroup.eligible(row, align_key):
         return False
     grp.add(row, flops, floor, *tensors)
+    _group.last = (row, flops, floor)
     return True
+
+
+class GroupedCall:
+    """A factor call that the active FactorGroup took, remembered by its caller (one per hooked module and factor):
+    operand geometry, the group's row, the result buffer, FLOP count and floor.  On the next pass the caller's hook
+    sees a tensor of the same shape, strides, type and alignment, for which syrk_tn() / conv_syrk() would derive the
+    very same row; again() appends it to the group without going through them."""
+    __slots__ = ('shape', 'stride', 'dtype', 'device', 'align', 'row', 'out', 'flops', 'floor', 'timed', 'extra')
+
+    @staticmethod
+    def begin():
+        """Call before the factor call that is to be remembered."""
+        _group.last = None
+
+    @classmethod
+    def remember(cls, x, out, extra=None):
+        """After the factor call on the hook's tensor ``x`` with result ``out``: the record, or None when the call
+        was launched at once, or read a converted or rearranged copy of ``x`` (whose address the next pass cannot
+        know)."""
+        last = getattr(_group, 'last', None)
+        _group.last = None
+        if last is None:
+            return None
+        row, flops, floor = last
+        if row[1] != x.data_ptr() or row[2] != out.data_ptr():
+            return None
+        rec = cls()
+        rec.shape, rec.stride, rec.dtype, rec.device = x.shape, x.stride(), x.dtype, x.device
+        rec.align = row[1] & 15
+        rec.row, rec.out, rec.flops, rec.floor = list(row), out, flops, floor
+        rec.timed = _timing_sink is not None
+        rec.extra = extra
+        return rec
+
+    def again(self, x, extra=None):
+        """Appends the remembered call, on ``x``, to the active group.  False (nothing done) when ``x`` or the state
+        of the calling thread differs from what the record was made under."""
+        grp = getattr(_group, 'active', None)
+        if grp is None or (grp.plain_only and self.row[0] != 0):
+            return False
+        if x.dtype is not self.dtype or x.shape != self.shape or x.stride() != self.stride or x.device != self.device \
+                or extra != self.extra or (_timing_sink is not None) != self.timed:
+            return False
+        ptr = x.data_ptr()
+        if ptr & 15 != self.align:
+            return False
+        row = list(self.row)
+        row[1] = ptr
+        grp.add(row, self.flops, self.floor, x, self.out)
+        return True
 
 
 # ------------------------------------------------------------------------------ factors

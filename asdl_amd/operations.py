@@ -91,6 +91,7 @@ class Operation:
             if name not in ALL_OPS:
                 raise ValueError(f'Invalid operation name: {name}. {ALL_OPS} are supported.')
         self._op_names = op_names
+        self._inv_only = op_names == {OP_COV_KRON_INV}     # the hooks of this combination may repeat remembered calls
         self._op_results = {}
         self._damping = 1.e-7
         self._cov_scale = 1.
@@ -160,7 +161,25 @@ class Operation:
             cache[key] = buf
         return buf
 
-    def _factor_inv_mode(self, key, tmp_key, data, swift, square_fn, low_rank_fn, device, slot=None):
+    def _remembered_call(self, key, tmp_key, raw, first):
+        """The grouped factor call that this module's hook made on the previous pass, made again on ``raw`` (see
+        kernels.GroupedCall): True when the group has taken it.  Only the square scratch factors of the *_INV
+        operations are remembered; whatever differs from the remembered call goes through _factor_inv_mode()."""
+        cache = getattr(self._module, _FACTOR_CACHE_ATTR, None)
+        rec = cache.get('call' + key) if cache is not None else None
+        if rec is None or cache.get(key) is not rec.out:
+            return False
+        if not rec.again(raw, (self._geometry(), self._cov_scale, first)):
+            return False
+        self._op_results[tmp_key] = rec.out
+        self._op_results['_eig_scale_' + key] = 1.0
+        return True
+
+    def _geometry(self):
+        """What the factor kernels take from the module besides its input (nothing for a Linear layer)."""
+        return None
+
+    def _factor_inv_mode(self, key, tmp_key, data, swift, square_fn, low_rank_fn, device, slot=None, raw=None):
         """One contribution to the scratch factor of the *_INV operations.  Swift (asdl/operations/operation.py:
         282-299): a factor with fewer samples than columns is the unscaled [n, d] row matrix; a square one is
         scaled by cov_scale only after the damping has been taken from the unscaled factors, which the damping
@@ -176,7 +195,13 @@ class Operation:
             self._op_results['_eig_scale_' + key] = 1.0
         else:
             buf = self._scratch_factor(cache_key, dim, device)
+            remember = raw is not None and slot is None and not swift
+            if remember:
+                kernels.GroupedCall.begin()
             square_fn(buf, self._cov_scale, 0.0 if first else 1.0)
+            if remember:
+                getattr(self._module, _FACTOR_CACHE_ATTR)['call' + key] = \
+                    kernels.GroupedCall.remember(raw, buf, (self._geometry(), self._cov_scale, first))
             self._op_results['_eig_scale_' + key] = 1.0 / self._cov_scale if swift else 1.0
         if slot is None:
             self._op_results[tmp_key] = buf
@@ -202,16 +227,19 @@ class Operation:
             fn = self.cov_swift_kron_A if n < dim else self.cov_kron_A
             self._update_factor('A', lambda out, alpha, beta: fn(module, data, out=out, alpha=alpha, beta=beta))
         elif OP_COV_KRON_INV in op_names or OP_COV_SWIFT_KRON_INV in op_names:
-            data = self.preprocess_in_data(module, in_data, out_data)
             if PER_CALL_INVERSES:
                 # the reference's backward hook forms A from the input of the LAST forward call
                 # (asdl/operations/operation.py:232): a later call replaces the factor of an earlier one
                 self._op_results.pop('_A_tmp', None)
+            if OP_COV_KRON_INV in op_names and self._remembered_call('A', '_A_tmp', in_data, '_A_tmp' not in self._op_results):
+                self._n_forward += 1
+                return
+            data = self.preprocess_in_data(module, in_data, out_data)
             self._factor_inv_mode(
                 'A', '_A_tmp', data, OP_COV_SWIFT_KRON_INV in op_names,
                 lambda out, alpha, beta: self.cov_kron_A(module, data, out=out, alpha=alpha, beta=beta),
                 lambda out, alpha, beta: self.cov_swift_kron_A(module, data, out=out, alpha=alpha, beta=beta),
-                in_data.device)
+                in_data.device, raw=in_data)
             self._n_forward += 1
 
     def backward_pre_process(self, out_grads, vector: torch.Tensor = None):
@@ -222,6 +250,12 @@ class Operation:
         module = self._module
         op_names = self._op_names
         if not any(name in BWD_OPS for name in op_names):
+            return
+        if self._inv_only and self._n_forward <= 1 and \
+                self._remembered_call('B', '_B_tmp', out_grads, '_B_tmp' not in self._op_results):
+            self._n_backward += 1
+            if self._context is not None:
+                self._context.queue_inverse(self)
             return
         grads = self.preprocess_out_grads(module, out_grads)
         if OP_SAVE_OUTGRADS in op_names:
@@ -238,7 +272,7 @@ class Operation:
                 'B', '_B_tmp', grads, OP_COV_SWIFT_KRON_INV in op_names,
                 lambda out, alpha, beta: self.cov_kron_B(module, grads, out=out, alpha=alpha, beta=beta),
                 lambda out, alpha, beta: self.cov_swift_kron_B(module, grads, out=out, alpha=alpha, beta=beta),
-                grads.device, slot=self._n_backward % self._n_forward if per_call else None)
+                grads.device, slot=self._n_backward % self._n_forward if per_call else None, raw=out_grads)
             if per_call:
                 self._op_results.setdefault('_B_calls', []).append(buf)
             self._n_backward += 1
@@ -323,6 +357,10 @@ class Linear(Operation):
 class Conv2d(Operation):
     """module.weight: c_out x c_in x k_h x k_w; in_data: lazy n x (c_in k_h k_w) x out_size;
     out_grads: n x c_out x out_size (asdl/operations/conv.py:9-42, 80-103)."""
+
+    def _geometry(self):
+        m = self._module
+        return (m.kernel_size, m.stride, m.padding, m.dilation, m.groups)
 
     @staticmethod
     def preprocess_in_data(module, in_data, out_data):
