@@ -74,6 +74,9 @@ class FisherMaker(GradientMaker):
         self.config: FisherConfig = config
         self.late_inverse_flags = LATE_INVERSE_FLAGS
         self._late_flags = []
+        self.flags_to_caller = False         # set by a caller that enqueues work between the inverses and their flags
+                                             # (the preconditioning) and then reads them itself: take_caller_flags()
+        self._caller_flags = None
         self.before_inverse_wait = None      # optional callable, run right before the host waits for the inverses
         self.after_factors = None            # optional callable, run when the factors are final and before the loss
                                              # backward pass is enqueued; may return an object with finish()
@@ -85,6 +88,12 @@ class FisherMaker(GradientMaker):
         pending, self._late_flags = self._late_flags, []
         for late in pending:
             late.check()
+
+    def take_caller_flags(self):
+        """The unread flags of this call's inverses (flags_to_caller), as a list of objects with check(); None when
+        they have been read already."""
+        pending, self._caller_flags = self._caller_flags, None
+        return pending
 
     def zero_fisher(self, fvp=False):
         attr = self.config.fvp_attr if fvp else self.config.fisher_attr
@@ -199,7 +208,7 @@ class FisherMaker(GradientMaker):
             cxt.finish_registered()
             # The inverses only need the factors: enqueue them now (side streams) and, when a loss backward
             # pass follows, let that pass run on the main stream meanwhile; the flags are read afterwards.
-            deferred = cxt.flush_inverses(defer=loss_grad_after_fisher)
+            deferred = cxt.flush_inverses(defer=loss_grad_after_fisher or self.flags_to_caller)
             self._inverse_cost_prev = cxt.inverse_cost
             self._extract_fisher(cxt)
 
@@ -224,9 +233,12 @@ class FisherMaker(GradientMaker):
                 self.before_inverse_wait()      # host work of the caller that needs no flags: the device is still busy
             if deferred is not None:
                 self.check_late_flags()         # of the previous update: read long ago by the device's clock
-                late = deferred.finish_late() if self.late_inverse_flags else None
+                to_caller = self.flags_to_caller and not self.late_inverse_flags
+                late = deferred.finish_late(config.fisher_attr, warn=self.late_inverse_flags) if (self.late_inverse_flags or to_caller) else None
                 if late is None:
                     deferred.finish(config.fisher_attr)
+                elif to_caller:
+                    self._caller_flags = late
                 else:
                     self._late_flags = late
             if early is not None:

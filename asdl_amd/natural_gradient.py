@@ -6,6 +6,7 @@ Host-side differences from the reference, all result-preserving:
 * inverses of all layers are taken in one batched pass with one host synchronisation,
 * layer ownership across ranks (the reference's partitions) does not exist: one process, one GPU.
 """
+import sys
 from typing import Any, List, Union
 
 import torch
@@ -27,6 +28,16 @@ _norm_classes = (nn.BatchNorm1d, nn.BatchNorm2d, nn.LayerNorm)
 PRECONDITION_STREAMS = 6      # side streams over which precondition() spreads the layers
 OVERLAP_INVERSE_UPDATE = True           # EMA mode: update_preconditioner()'s inverses beside the loss backward pass
 PREPARE_PRECONDITION_EARLY = True      # host side of precondition() while the device still works on the inverses
+FLAGS_AFTER_PRECONDITION = True        # forward_and_backward(): the zero / not-positive-definite flags of the step's
+                                       # inverses are read after the preconditioning has been enqueued instead of
+                                       # before, so that the device has that work in its queue while the host waits and
+                                       # prepares the next step.  What the caller sees is the reference's behaviour: a
+                                       # factor that is not positive definite raises torch.linalg.LinAlgError from
+                                       # this call, with the gradients as the backward pass left them (they are
+                                       # saved before the preconditioning and put back); an all-zero factor without
+                                       # an earlier inverse, for which the reference computes none, has the identity
+                                       # while the gradients are preconditioned (its own gradient is zero, as its
+                                       # inputs or output gradients are) and none afterwards.
 GROUPED_PRECONDITION = True      # all Kronecker-factored modules in three launches instead of one stream-juggled chain per module
 
 __all__ = ['NaturalGradientMaker', 'KfacGradientMaker']
@@ -226,11 +237,18 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             OVERLAP_INVERSE_UPDATE and self.do_accumulate and self.do_update_curvature(step)
             and self.do_update_preconditioner(step))
         self._kron_inverses_current = False
+        # precondition() follows in this very call: it may read the flags of the inverses once it has launched
+        self.fisher_maker.flags_to_caller = bool(FLAGS_AFTER_PRECONDITION)
         try:
             return super().forward_and_backward()
         finally:
             self._inverse_update_follows = False
             self._kron_inverses_current = False
+            self.fisher_maker.flags_to_caller = False
+            unread = self.fisher_maker.take_caller_flags()
+            if unread and sys.exc_info()[0] is None:
+                for late in unread:          # no stage read them (precondition() was replaced, say)
+                    late.check(when=None)
 
     def _curvature_matrices(self, module_name=None):
         matrices, units = [], []
@@ -286,6 +304,46 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
         if grad_scale is None:
             grad_scale = self.grad_scale
         work = self._precondition_work()
+        unread = self.fisher_maker.take_caller_flags()
+        if not unread:
+            self._precondition_launch(work, grad_scale, use_inv)
+            return
+        # FLAGS_AFTER_PRECONDITION: launch on inverses whose flags are still on the device, then read them
+        grads = [g for m, _ in work for g in (getattr(getattr(m, 'weight', None), 'grad', None),
+                                              getattr(getattr(m, 'bias', None), 'grad', None)) if g is not None]
+        saved = self._save_gradients(grads)
+        self._precondition_launch(work, grad_scale, use_inv)
+        try:
+            for late in unread:
+                late.check(when=None)
+        except torch.linalg.LinAlgError:
+            if grads:
+                torch._foreach_copy_(grads, saved)      # as the reference leaves them when its Cholesky raises
+            raise
+
+    def _save_gradients(self, grads):
+        """Copies of ``grads`` in one reusable buffer (one launch per dtype and device)."""
+        if not grads:
+            return []
+        views, buffers = [], getattr(self, '_grad_backup', None)
+        if buffers is None:
+            buffers = self._grad_backup = {}
+        need = {}
+        for g in grads:
+            key = (g.dtype, g.device)
+            need[key] = need.get(key, 0) + g.numel()
+        for key, n in need.items():
+            if key not in buffers or buffers[key].numel() < n:
+                buffers[key] = torch.empty(n, dtype=key[0], device=key[1])
+        used = dict.fromkeys(need, 0)
+        for g in grads:
+            key = (g.dtype, g.device)
+            views.append(buffers[key][used[key]:used[key] + g.numel()].view(g.shape))
+            used[key] += g.numel()
+        torch._foreach_copy_(views, grads)
+        return views
+
+    def _precondition_launch(self, work, grad_scale, use_inv):
         if use_inv and GROUPED_PRECONDITION:
             work = self._precondition_grouped(work, grad_scale)
         grads = [m.weight.grad for m, _ in work if getattr(m, 'weight', None) is not None and m.weight.grad is not None]

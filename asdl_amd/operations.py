@@ -498,6 +498,23 @@ EAGER_COST_FRACTION = 0.6
 _warned_late_fallback = False
 
 
+class LateChunk:
+    """The unread flags of one chunk of DeferredInverses.finish_late() and the modules its Kron objects belong to."""
+
+    def __init__(self, late, targets, attr):
+        self._late, self._targets, self._attr = late, targets, attr
+
+    def check(self, *args, **kwargs):
+        zero = self._late.check(*args, **kwargs)
+        if zero and self._attr is not None:
+            owner = {id(kron): module for module, kron in self._targets}
+            for kron, which in zero:
+                fisher = getattr(owner.get(id(kron)), self._attr, None)
+                if fisher is not None and fisher.has_kron:
+                    setattr(fisher.kron, which + '_inv', None)
+        return zero
+
+
 class DeferredInverses:
     """Inverses enqueued by OperationContext.flush_inverses(defer=True), possibly in several chunks.
     finish(attr) waits for them, raises torch.linalg.LinAlgError for a factor that is not positive definite,
@@ -508,13 +525,14 @@ class DeferredInverses:
         self._chunks = chunks            # [(PendingInverses, [(module, kron), ...]), ...]
         self._context = context
 
-    def finish_late(self):
-        """finish() without its host synchronisation (PendingInverses.finish_late): returns the LateFlags objects
-        whose check() reads the flags later.  None when the context also has unit-wise flags to read, which only
-        finish() does."""
+    def finish_late(self, attr=None, warn=True):
+        """finish() without its host synchronisation (PendingInverses.finish_late): returns objects whose check()
+        reads the flags later (and, like finish(), removes from ``module.<attr>.kron`` the inverse of an all-zero
+        factor that had none before).  None when the context also has unit-wise flags to read, which only finish()
+        does."""
         if self._context is not None and self._context._unit_flags:
             global _warned_late_fallback
-            if not _warned_late_fallback:
+            if warn and not _warned_late_fallback:
                 _warned_late_fallback = True
                 warnings.warn('late_inverse_flags: this model has unit-wise (BatchNorm / LayerNorm) blocks, whose flags '
                               'are read at once; the flags of the Kronecker factors are read with them.')
@@ -523,7 +541,8 @@ class DeferredInverses:
             self._context._unit_flags_deferred = False      # nothing was deferred to this object's finish()
         for pending, _ in self._chunks:
             pending.join()
-        return [late for late in (pending.finish_late() for pending, _ in self._chunks) if late is not None]
+        return [LateChunk(late, targets, attr) for late, targets in
+                ((pending.finish_late(), targets) for pending, targets in self._chunks) if late is not None]
 
     def finish(self, attr):
         if self._context is not None:

@@ -108,18 +108,28 @@ class LateFlags:
     def __init__(self, host, event, records, keep_alive):
         self._host, self._event, self._records, self._keep_alive = host, event, records, keep_alive
 
-    def check(self):
+    def check(self, when='reported late: the flags of this update were read after the next one'):
+        """Raises for a factor that was not positive definite.  Returns the (Kron, 'A' | 'B') whose factor was all
+        zero and had no inverse before: the reference computes none for them (asdl/symmatrix.py:517, :527); the
+        device has put the identity there, and the caller removes it again."""
         if self._host is None:
-            return
-        self._event.synchronize()
+            return []
+        if self._event is not None:
+            self._event.synchronize()
         host, self._host, self._keep_alive = self._host.tolist(), None, None
         n = len(self._records)
         info_host, nz_host = host[:n], host[n:]
-        for (flat, which), inf in zip(self._records, info_host):
-            if nz_host[flat] and inf != 0:
+        zero = []
+        for (flat, k, which, was_fresh), inf in zip(self._records, info_host):
+            if not nz_host[flat]:
+                if was_fresh:
+                    setattr(k, which + '_inv', None)
+                    zero.append((k, which))
+            elif inf != 0:
                 raise torch.linalg.LinAlgError(
                     f'cholesky_inv: the leading minor of order {inf} of kron.{which} + damping was not '
-                    f'positive-definite (reported late: the flags of this update were read after the next one)')
+                    f'positive-definite' + (f' ({when})' if when else ''))
+        return zero
 
 
 class PendingInverses:
@@ -159,15 +169,21 @@ class PendingInverses:
         if fresh:
             kernels.identity_where_zero([out for _, out in fresh], self._nz_flat, [flat for flat, _ in fresh])
         flags = torch.cat(self._infos + [self._nz_flat])
-        host = torch.empty(flags.shape, dtype=flags.dtype, pin_memory=True)
-        host.copy_(flags, non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
+        event = None
+        if flags.is_cuda:
+            host = torch.empty(flags.shape, dtype=flags.dtype, pin_memory=True)
+            host.copy_(flags, non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+        else:
+            host = flags.clone()
         for (flat, k, which, out) in self._records:
             setattr(k, which + '_inv', out)
             if self._replace:
                 setattr(k, which, None)
-        late = LateFlags(host, event, [(flat, which) for flat, _, which, _ in self._records], (flags, self._keep_alive))
+        # (flag index, Kron, side, did the buffer hold no inverse before)
+        late = LateFlags(host, event, [(flat, k, which, was_fresh) for (flat, k, which, _), was_fresh
+                                       in zip(self._records, self._fresh)], (flags, self._keep_alive))
         self._keep_alive = None
         return late
 

@@ -7,8 +7,8 @@ optimizer.step().  bf16 autocast forward/backward, fp32 factors and inverses, fa
 step, BatchNorm excluded (Conv2d + Linear only).  Inputs are synthetic N(0,1) images resident in HBM.
 
 Prints ONE JSON line; see --help for the knobs.  The headline (`value`, `ms_per_step`) is measured with the library's
-defaults; the same steps with the flags of a step's inverses read one step late are reported beside it
-(`late_inverse_flags`).  The `roofline` object is for the dominant kernel family (the factor-statistics kernels):
+defaults (the flags of a step's inverses are read in the step's own call, once its preconditioning is enqueued); the
+same steps with the flags read one step late are reported beside it (`late_inverse_flags`).  The `roofline` object is for the dominant kernel family (the factor-statistics kernels):
 algorithmic FLOP M*d*(d+1) per launch summed over the 108 factors of a step, divided by their summed durations
 measured with events on the launching stream inside the timed region (on every fourth step, to keep the
 instrumentation's own cost small); `floor_ms_per_step` is the sum of the per-launch roofline floors of the same
@@ -76,13 +76,15 @@ def parse():
     ap.add_argument('--factor-launches', choices=['default', 'single', 'grouped'], default='default',
                     help='single: one launch per Kronecker factor; grouped: the factors of a pass in one grouped launch '
                          '(asdl_amd.fisher.GROUPED_FACTORS); default: the library\'s own setting')
-    ap.add_argument('--inverse-flags', choices=['late', 'now'], default='now',
+    ap.add_argument('--inverse-flags', choices=['late', 'now', 'before'], default='now',
                     help='K-FAC workloads: when the host reads the zero / not-positive-definite flags of a step\'s '
-                         'inverses in the headline measurement.  now (default): before it enqueues the preconditioning, as '
-                         'the reference\'s torch.linalg.cholesky does (the library\'s default); late: when the next step gets there '
-                         '(FisherMaker.late_inverse_flags; the last step\'s flags are read inside the timed region), '
-                         'so that the host prepares the next step while the device finishes this one.  Same kernels, '
-                         'same results; an error would be raised one step later')
+                         'inverses in the headline measurement.  now (default, the library\'s default): in the same '
+                         'forward_and_backward() call, once the preconditioning has been enqueued (a bad factor raises '
+                         'from that call with the gradients put back as the backward pass left them, as the '
+                         'reference\'s torch.linalg.cholesky would leave them); before: before the preconditioning is '
+                         'enqueued (asdl_amd.natural_gradient.FLAGS_AFTER_PRECONDITION = False); late: when the next '
+                         'step gets there (FisherMaker.late_inverse_flags; the last step\'s flags are read inside the '
+                         'timed region), an error would be raised one step later.  Same kernels, same results')
     ap.add_argument('--traffic-calibration-mib', type=int, default=0,
                     help='before the warm-up, launch one plain copy kernel (ak::copy_bytes_kernel) of this many MiB: '
                          'the known traffic against which a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this '
@@ -256,7 +258,7 @@ def build_workload(args, name, dev):
     return w
 
 
-def measure_kfac(w, args, steps, warmup, late_flags, factor_timing, phase_steps):
+def measure_kfac(w, args, steps, warmup, flags_mode, factor_timing, phase_steps):
     """Warm-up, then `steps` timed K-FAC steps of workload `w`; returns the wall time per step, the factor launches
     recorded with events inside the timed region, and the per-phase breakdown of extra steps after it."""
     import torch
@@ -268,7 +270,10 @@ def measure_kfac(w, args, steps, warmup, late_flags, factor_timing, phase_steps)
         if hasattr(m, 'fisher'):
             delattr(m, 'fisher')
     gm = KfacGradientMaker(model, w['config'], fisher_type=args.fisher, swift=args.swift)
+    import asdl_amd.natural_gradient as ng_mod
+    late_flags = flags_mode == 'late'
     gm.late_inverse_flags = late_flags
+    ng_mod.FLAGS_AFTER_PRECONDITION = flags_mode != 'before'
     opt = torch.optim.SGD([p for p in model.parameters() if p.requires_grad], lr=1e-4)
 
     def step():
@@ -437,7 +442,7 @@ def main():
     w = build_workload(args, args.workload, dev)
     bs = w['bs']
     late = args.inverse_flags == 'late'
-    res = measure_kfac(w, args, args.steps, args.warmup, late, not args.no_factor_timing, args.phase_steps)
+    res = measure_kfac(w, args, args.steps, args.warmup, args.inverse_flags, not args.no_factor_timing, args.phase_steps)
     out = {
         'metric': 'K-FAC steps/s ResNet-50 bs64',
         'value': res['value'],
@@ -456,9 +461,12 @@ def main():
                                f'bf16 autocast forward/backward, fp32 factors/inverses, damping {args.damping}, '
                                f'BatchNorm {"unit-wise" if args.with_batchnorm else "ignored"}, {args.memory_format} activations and weights, '
                                f'cudnn.benchmark {"on" if w["autotune"] else "off"}' + (', swift (SKFAC) factors' if args.swift else '')
-                               + (', flags of a step\'s inverses read by the host one step late' if late else
-                                  ', the library\'s defaults (flags of a step\'s inverses read before its '
-                                  'preconditioning, as the reference\'s Cholesky raises)'),
+                               + {'late': ', flags of a step\'s inverses read by the host one step late',
+                                  'before': ', flags of a step\'s inverses read before its preconditioning is enqueued',
+                                  'now': ', the library\'s defaults (a factor that is not positive definite raises '
+                                         'from the step\'s own call and leaves the raw gradients, as the reference\'s '
+                                         'Cholesky does; the host reads the flags once the preconditioning is enqueued)'
+                                  }[args.inverse_flags],
                    'batch': bs},
     }
     default_workload = (args.workload == 'resnet50' and bs == 64 and args.fisher == 'fisher_mc'
@@ -505,12 +513,12 @@ def main():
     if default_workload and not args.no_secondary:
         # the same steps with the flags of a step's inverses read one step late (FisherMaker.late_inverse_flags): the
         # host then runs ahead of the device; same kernels, same results, errors raised one update late
-        other = measure_kfac(w, args, args.steps, 2, not late, False, args.phase_steps)
+        other = measure_kfac(w, args, args.steps, 2, 'now' if late else 'late', False, args.phase_steps)
         key = 'late_inverse_flags' if not late else 'default_inverse_flags'
         out[key] = {'ms_per_step': other['ms_per_step'], 'value': other['value'], 'unit': 'steps/s',
                     'note': 'same process, same model; flags of a step\'s inverses read '
                             + ('one step late (not the library\'s default: a factor that is not positive definite '
-                               'raises one update late)' if not late else 'before its preconditioning'),
+                               'raises one update late)' if not late else 'in the same call, after its preconditioning is enqueued'),
                     'phases': other.get('phases')}
     if not args.no_cpu_baseline:
         if args.workload == 'linear4096':

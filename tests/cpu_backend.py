@@ -157,8 +157,15 @@ def unit_wise_mvp(mat, vec_weight, vec_bias, scale=1.0):
     return vec_weight, vec_bias
 
 
+def identity_where_zero(outs, nonzero, flag_index):
+    flags = nonzero.view(-1)
+    for out, i in zip(outs, flag_index):
+        if int(flags[i]) == 0:
+            out.copy_(torch.eye(out.shape[0], dtype=out.dtype))
+
+
 def install(monkeypatch):
     from asdl_amd import kernels
     for name in ['syrk_tn', 'conv_syrk', 'syrk_nt', 'kron_damping', 'chol_inv_batched', 'chol_inv_grouped', 'cholesky_inv',
-                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_inv_grouped', 'unit_wise_mvp', 'conv_patch_sum', 'smw_inv']:
+                 'kron_precond', 'gemm', 'unit_wise_stats', 'unit_wise_inv', 'unit_wise_inv_grouped', 'unit_wise_mvp', 'conv_patch_sum', 'smw_inv', 'identity_where_zero']:
         monkeypatch.setattr(kernels, name, globals()[name])

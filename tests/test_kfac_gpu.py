@@ -738,8 +738,8 @@ def test_identity_where_zero_touches_only_the_flagged_matrices():
 
 def test_late_flags_of_a_batched_inverse():
     """PendingInverses.finish_late(): no host synchronisation; a factor that is not positive definite raises when the
-    flags are read (strictly: at once), an all-zero factor's fresh inverse buffer holds the identity, the inverses
-    of the others are those of finish()."""
+    flags are read (strictly: at once), an all-zero factor's fresh inverse buffer holds the identity until then and
+    the factor has no inverse afterwards (as with finish()), the inverses of the others are those of finish()."""
     from asdl_amd.symmatrix import Kron, batched_update_inv
     g = torch.Generator().manual_seed(9)
 
@@ -752,9 +752,10 @@ def test_late_flags_of_a_batched_inverse():
     batched_update_inv(strict, damping=1e-2)
     late = [Kron(A.clone(), B.clone()) for A, B in mats]
     flags = batched_update_inv(late, damping=1e-2, defer=True).finish_late()
-    flags.check()                                   # nothing to report
-    flags.check()                                   # a second call is a no-op
     assert strict[1].A_inv is None and torch.equal(late[1].A_inv, torch.eye(16, device='cuda'))
+    zero = flags.check()                            # nothing to raise; the all-zero factor is reported ...
+    assert zero == [(late[1], 'A')] and late[1].A_inv is None        # ... and loses the identity it had meanwhile
+    assert flags.check() == []                      # a second call is a no-op
     for a, b in zip(strict, late):
         assert torch.equal(a.B_inv, b.B_inv)
         assert a.A_inv is None or torch.equal(a.A_inv, b.A_inv)
@@ -775,14 +776,16 @@ def test_late_inverse_flags_give_the_same_steps(fisher_type, monkeypatch):
     preconditioned gradient within 1e-4; each step checks the flags of the one before, check_late_flags() those of
     the last."""
     import asdl_amd.symmatrix as sm_mod
+    import asdl_amd.natural_gradient as ng_mod
     checks = []
     plain_check = sm_mod.LateFlags.check
-    monkeypatch.setattr(sm_mod.LateFlags, 'check', lambda self: (checks.append(self), plain_check(self))[1])
+    monkeypatch.setattr(sm_mod.LateFlags, 'check', lambda self, *a, **k: (checks.append(self), plain_check(self, *a, **k))[1])
     xs = [torch.randn(8, 16, 12, 12, generator=torch.Generator().manual_seed(50 + i)).cuda()
           .contiguous(memory_format=torch.channels_last) for i in range(3)]
     ts = [torch.randint(10, (8,), generator=torch.Generator().manual_seed(60 + i)).cuda() for i in range(3)]
 
-    def run(late):
+    def run(late, after=False):
+        monkeypatch.setattr(ng_mod, 'FLAGS_AFTER_PRECONDITION', after)
         torch.manual_seed(33)
         model = nn.Sequential(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU(), nn.Conv2d(32, 32, 1), nn.ReLU(),
                               nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
@@ -819,6 +822,70 @@ def test_late_inverse_flags_give_the_same_steps(fisher_type, monkeypatch):
     for key in ref:
         # the raw weight gradients come from the framework's convolution kernels, which do not sum in a fixed order
         assert relerr(got[key], ref[key]) < 1e-4 if key[2] == 'grad' else torch.equal(got[key], ref[key]), key
+    # the library's default (natural_gradient.FLAGS_AFTER_PRECONDITION): read in the step's own call, once its
+    # preconditioning is enqueued; nothing is left for the next step or the checkpoint
+    del checks[:]
+    got, n = run(False, after=True)
+    assert n == 0 and len(checks) == 3, (n, len(checks))      # also with the single pass of the empirical Fisher
+    for key in ref:
+        assert relerr(got[key], ref[key]) < 1e-4 if key[2] == 'grad' else torch.equal(got[key], ref[key]), key
+
+
+def test_flags_read_after_the_preconditioning_leave_raw_gradients_when_they_raise(monkeypatch):
+    """natural_gradient.FLAGS_AFTER_PRECONDITION: forward_and_backward() enqueues the preconditioning before it reads
+    the flags of the step's inverses.  A factor that is not positive definite (here: every damping value replaced by
+    a large negative one) has to raise torch.linalg.LinAlgError from that very call and leave in .grad what the
+    backward pass wrote there, exactly what the strict order (flags first) leaves; the next step with sound factors
+    works as if nothing had happened."""
+    import asdl_amd.natural_gradient as ng_mod
+    import asdl_amd.symmatrix as sm_mod
+    from asdl_amd import kernels
+    plain_damping = kernels.kron_damping
+    broken = [False]
+
+    def damping(*args, **kwargs):
+        lam, nonzero = plain_damping(*args, **kwargs)
+        return (lam * -1e6 if broken[0] else lam), nonzero
+    monkeypatch.setattr(sm_mod.kernels, 'kron_damping', damping)
+    x = torch.randn(8, 16, 12, 12, generator=torch.Generator().manual_seed(70)).cuda().contiguous(memory_format=torch.channels_last)
+    t = torch.randint(10, (8,), generator=torch.Generator().manual_seed(71)).cuda()
+
+    def run(after):
+        monkeypatch.setattr(ng_mod, 'FLAGS_AFTER_PRECONDITION', after)
+        torch.manual_seed(34)
+        model = nn.Sequential(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU(), nn.Conv2d(32, 32, 1), nn.ReLU(),
+                              nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
+        model = model.to(memory_format=torch.channels_last)
+        gm = KfacGradientMaker(model, PreconditioningConfig(data_size=8, damping=1e-2), fisher_type=FISHER_MC, seed=5)
+        out = {}
+        for step, bad in enumerate((False, True, False)):
+            broken[0] = bad
+            model.zero_grad(set_to_none=True)
+            gm.setup_loss_call(F.cross_entropy, gm.setup_model_call(model, x), t)
+            if bad:
+                with pytest.raises(torch.linalg.LinAlgError, match='positive-definite'):
+                    gm.forward_and_backward()
+            else:
+                gm.forward_and_backward()
+            assert gm.fisher_maker.take_caller_flags() is None
+            for name, p in model.named_parameters():
+                out[(step, name)] = p.grad.clone()
+        return out
+
+    strict, after = run(False), run(True)
+    # the raw gradients of the step that raised: the loss gradient divided by the data size
+    torch.manual_seed(34)
+    model = nn.Sequential(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU(), nn.Conv2d(32, 32, 1), nn.ReLU(),
+                          nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10)).cuda()
+    model = model.to(memory_format=torch.channels_last)
+    F.cross_entropy(model(x), t, reduction='sum').div(8).backward()
+    raw = {name: p.grad for name, p in model.named_parameters()}
+    for (step, name), g in strict.items():
+        assert relerr(after[(step, name)], g) < 1e-4, (step, name)
+        if step == 1:
+            assert relerr(after[(step, name)], raw[name]) < 1e-4 and relerr(g, raw[name]) < 1e-4, name
+        else:
+            assert relerr(g, raw[name]) > 1e-2, name              # preconditioned
 
 
 @pytest.mark.parametrize('pi', [1, 2])
