@@ -26,15 +26,24 @@ constexpr int LEAF_T2_FLOATS = 64 * T1_LD;
 constexpr size_t LEAF_LDS_BYTES = (LEAF * LLD + LEAF_T1_FLOATS + LEAF_T2_FLOATS + 8) * sizeof(float);
 
 // Cholesky factor and its inverse of a PB x PB block held one row per lane (lanes >= PB carry an identity
-// row).  On exit a[] is row `lane` of L (entries right of the diagonal are meaningless) and m[] is column `lane`
-// of L^-1.  Returns 0 or the 1-based index of the first non-positive pivot.
-// Every step is applied to all lanes and all columns without masks: entries above the diagonal and the rows
-// that are already final only ever receive values nobody reads (each broadcast below takes a[k] of a lane j >= k).
-// The broadcasts of one pivot are issued together, ahead of the multiply-adds that use them, so that the wait
-// states between a lane read and its first use are filled with the other lane reads.
+// row).  On exit a[] is row `lane` of L (entries right of the diagonal are meaningless) and m[] is row `lane` of
+// L^-1 (zeros right of the diagonal).  Returns 0 or the 1-based index of the first non-positive pivot.
+//
+// One loop over the pivots does both.  Row i of the inverse is (e_i - sum_{k<i} l_ik m_k) / l_ii; every lane keeps the
+// numerator u_i of its own row, and pivot k, whose row u_k is complete by then, subtracts (l_ik / l_kk) u_k from the
+// rows below it: k + 1 lane reads and as many multiply-adds that do not depend on one another, next to the 15 - k of
+// the factorization's own update, so that every pivot issues the same 16 + 16 and the wait states of the serial
+// pivot chain (lane read, reciprocal square root, scaling, lane read, multiply-add) are filled.  A forward
+// substitution after the factorization costs the same arithmetic as chains of up to 15 dependent multiply-adds,
+// and took as long again as the factorization.
+// Every step is applied to all lanes without masks where that is harmless: entries above the diagonal and the rows
+// that are already final only ever receive values nobody reads (each broadcast below takes a[k] of a lane j >= k);
+// the rows of the inverse are protected by a factor that is zero for the lanes at and above the pivot.
 __device__ __forceinline__ int small_chol_inv(float (&a)[PB], float (&m)[PB], int lane) {
   int bad = 0;
-  float inv_diag[PB];
+  float my_inv = 1.f;
+#pragma unroll
+  for (int j = 0; j < PB; ++j) m[j] = (j == lane) ? 1.f : 0.f;
 #pragma unroll
   for (int k = 0; k < PB; ++k) {
     float akk = lane_bcast(a[k], k);
@@ -44,24 +53,21 @@ __device__ __forceinline__ int small_chol_inv(float (&a)[PB], float (&m)[PB], in
     }
     float inv = __builtin_amdgcn_rsqf(akk);                 // hardware rsqrt, then one Newton step:
     inv = inv * (1.5f - 0.5f * akk * inv * inv);             // keeps the serial pivot chain short
-    inv_diag[k] = inv;
+    my_inv = (lane == k) ? inv : my_inv;
     a[k] *= inv;                    // lane k: a_kk / sqrt(a_kk) = l_kk; lanes below: l_ik
-    float l[PB];
+    const float f = (lane > k) ? a[k] * inv : 0.f;          // l_ik / l_kk for the rows below the pivot
+    float l[PB], u[PB];
 #pragma unroll
     for (int j = k + 1; j < PB; ++j) l[j] = lane_bcast(a[k], j);
 #pragma unroll
+    for (int j = 0; j <= k; ++j) u[j] = lane_bcast(m[j], k);
+#pragma unroll
     for (int j = k + 1; j < PB; ++j) a[j] -= a[k] * l[j];
+#pragma unroll
+    for (int j = 0; j <= k; ++j) m[j] -= f * u[j];
   }
 #pragma unroll
-  for (int i = 0; i < PB; ++i) {   // column `lane` of L^-1 by forward substitution down the rows
-    float l[PB];
-#pragma unroll
-    for (int k = 0; k < i; ++k) l[k] = lane_bcast(a[k], i);
-    float s = (lane == i) ? 1.f : 0.f;
-#pragma unroll
-    for (int k = 0; k < i; ++k) s -= l[k] * m[k];
-    m[i] = (lane <= i) ? s * inv_diag[i] : 0.f;
-  }
+  for (int j = 0; j < PB; ++j) m[j] *= my_inv;
   return bad;
 }
 
@@ -71,7 +77,8 @@ __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
-// Which part of the contraction range a 16x16 output tile (ib, jb) needs when one operand is triangular.
+// Which part of the contraction range a 16x16 output tile (ib, jb) needs when one operand is triangular (the rest
+// multiplies zeros).
 enum LeafK { LK_FULL, LK_LE_J, LK_GE_J, LK_LE_I };
 
 // C[M x N] (=, -=) alpha * A[M x K] * op(B) for small matrices in LDS, all sizes multiples of 16, one 16x16 output
@@ -86,18 +93,22 @@ __device__ __forceinline__ void leaf_gemm(float* __restrict__ C, int ldc, const 
   for (int t = wave; t < TM * TN; t += LEAF_WAVES) {
     const int ib = t / TN, jb = t % TN;
     if (LOWER && jb > ib) continue;
-    int k0 = 0, k1 = K;
-    if (KM == LK_LE_J) k1 = 16 * (jb + 1);
-    if (KM == LK_GE_J) k0 = 16 * jb;
-    if (KM == LK_LE_I) k1 = 16 * (ib + 1);
+    // The whole contraction range, whatever KM says: the triangular operands hold zeros outside their triangle, and
+    // a loop whose bounds depend on the tile waits for the LDS once per step (the recursion is a chain of some thirty
+    // of these products, each as long as its slowest tile).  Here every operand of the tile is requested before
+    // the first matrix instruction is issued.
+    constexpr int KS = K / 4;
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
     const float* pa = A + (16 * ib + li) * lda + lk;
     const float* pb = TB ? B + (16 * jb + li) * ldb + lk : B + lk * ldb + 16 * jb + li;
-    for (int k = k0; k < k1; k += 4) {
-      const float a = pa[k];
-      const float b = TB ? pb[k] : pb[k * ldb];
-      acc = mfma16(a, b, acc);
+    float av[KS], bv[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      av[s] = pa[4 * s];
+      bv[s] = TB ? pb[4 * s] : pb[4 * s * ldb];
     }
+#pragma unroll
+    for (int s = 0; s < KS; ++s) acc = mfma16(av[s], bv[s], acc);
     float* pc = C + (16 * ib + 4 * lk) * ldc + 16 * jb + li;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -116,13 +127,22 @@ __device__ __forceinline__ void leaf_factor(float* __restrict__ Wm, int lo, floa
   if constexpr (N == PB) {
     if (wave == 0) {
       float a[PB], m[PB];
+      // every lane reads a whole row (the lanes beyond the block re-read its last one) with four 16-byte loads that
+      // are all in flight together; a load under a per-element condition would be waited for on its own
+      const floatx4* row = reinterpret_cast<const floatx4*>(Wm + (lo + (lane < PB ? lane : PB - 1)) * LLD + lo);
+      floatx4 q[PB / 4];
 #pragma unroll
-      for (int j = 0; j < PB; ++j)
-        a[j] = (lane < PB && j <= lane) ? Wm[(lo + lane) * LLD + lo + j] : ((j == lane) ? 1.f : 0.f);
+      for (int c = 0; c < PB / 4; ++c) q[c] = row[c];
+#pragma unroll
+      for (int j = 0; j < PB; ++j) a[j] = (lane < PB && j <= lane) ? q[j >> 2][j & 3] : ((j == lane) ? 1.f : 0.f);
       const int bad = small_chol_inv(a, m, lane);
       if (lane < PB) {
+        floatx4* dst = reinterpret_cast<floatx4*>(Wm + (lo + lane) * LLD + lo);
 #pragma unroll
-        for (int j = 0; j < PB; ++j) Wm[(lo + j) * LLD + lo + lane] = m[j];     // m[j] = 0 above the diagonal
+        for (int c = 0; c < PB / 4; ++c) {
+          const floatx4 w = {m[4 * c], m[4 * c + 1], m[4 * c + 2], m[4 * c + 3]};     // zeros above the diagonal
+          dst[c] = w;
+        }
       }
       if (lane == 0 && bad != 0 && *s_bad == 0) *s_bad = lo + bad;
     }
@@ -155,12 +175,22 @@ __device__ __forceinline__ void leaf_block(float* __restrict__ blk, int64_t ld, 
   float* t2 = t1 + LEAF_T1_FLOATS;
   int* s_bad = reinterpret_cast<int*>(t2 + LEAF_T2_FLOATS);
   const int npad = n <= 16 ? 16 : (n <= 32 ? 32 : (n <= 64 ? 64 : 128));
-  for (int i = tid >> 7; i < npad; i += LEAF_THREADS / 128) {
+  {
+    // all of this thread's elements are requested before the first one is stored: a load and its store per turn
+    // would pay the latency of the device memory sixteen times over
+    constexpr int ROWS_PER_TURN = LEAF_THREADS / 128, TURNS = LEAF / ROWS_PER_TURN;
     const int j = tid & 127;
-    if (j < npad) {
-      float v = (i == j) ? 1.f : 0.f;              // identity padding beyond n
-      if (i < n && j < n) v = (j <= i) ? blk[static_cast<int64_t>(i) * ld + j] : 0.f;
-      Wm[i * LLD + j] = v;
+    float v[TURNS];
+#pragma unroll
+    for (int t = 0; t < TURNS; ++t) {
+      const int i = (tid >> 7) + ROWS_PER_TURN * t;
+      v[t] = (i == j) ? 1.f : 0.f;                 // identity padding beyond n
+      if (i < n && j < n) v[t] = (j <= i) ? blk[static_cast<int64_t>(i) * ld + j] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < TURNS; ++t) {
+      const int i = (tid >> 7) + ROWS_PER_TURN * t;
+      if (i < npad && j < npad) Wm[i * LLD + j] = v[t];
     }
   }
   if (tid == 0) *s_bad = 0;
