@@ -26,26 +26,31 @@ enum TileMode {
 };
 
 struct GemmParams {
-  const float* A;
-  const float* B;
-  float* C;
-  float* const* C_list;     // optional: per-batch output pointers (overrides C / sC)
-  int64_t lda, ldb, ldc;
-  int64_t sA, sB, sC;       // batch strides in elements
-  int M, N, K;
-  int transA, transB;
-  float alpha, beta;
-  int kmode, tile_mode;
-  const int* active;        // optional per-batch flags: batch z runs only if active[z*active_stride] != 0
-  int active_stride;
-  int split;                // 0: fp32 MFMA; 2 / 3: bf16 MFMA on operands split into that many bf16 pieces (gemm_x3.hpp)
-  int chunked;              // non-zero: the contraction is summed in chunks (a fresh accumulator every 128 / 256 k, added
-                            // to a running total), which keeps the rounding error of a long sum near that of one
-                            // rounding instead of growing with the number of matrix instructions (fp32 kernel, and the
-                            // three-piece kernel for untransposed operands; ignored elsewhere)
-  float scaleA, scaleB;     // fp16-piece variant only: powers of two the operands are multiplied by before the split
-  float* absmax_out;        // optional (split kernels): max |C| of the result is folded into this word with an integer
-                            // atomic maximum on its bit pattern (the caller zeroes it first)
+  const float* A = nullptr;
+  const float* B = nullptr;
+  float* C = nullptr;
+  float* const* C_list = nullptr;     // optional: per-batch output pointers (overrides C / sC)
+  int64_t lda = 0, ldb = 0, ldc = 0;
+  int64_t sA = 0, sB = 0, sC = 0;     // batch strides in elements
+  int M = 0, N = 0, K = 0;
+  int transA = 0, transB = 0;
+  float alpha = 1.f, beta = 0.f;
+  int kmode = 0, tile_mode = 0;
+  const int* active = nullptr;        // optional per-batch flags: batch z runs only if active[z*active_stride] != 0
+  int active_stride = 0;
+  int split = 0;                      // 0: fp32 MFMA; 2 / 3: bf16 MFMA on operands split into that many bf16 pieces (gemm_x3.hpp)
+  int chunked = 0;                    // non-zero: the contraction is summed in chunks (a fresh accumulator every 128 / 256 k, added
+                                      // to a running total), which keeps the rounding error of a long sum near that of one
+                                      // rounding instead of growing with the number of matrix instructions (fp32 kernel, and the
+                                      // three-piece kernel for untransposed operands; ignored elsewhere)
+  float scaleA = 1.f, scaleB = 1.f;   // fp16-piece variant only: powers of two the operands are multiplied by before the split
+  float* absmax_out = nullptr;        // optional: the largest |C| of the result (of batch entry z: absmax_out[z * absmax_stride]) is
+  int64_t absmax_stride = 0;          // folded into this word with an integer atomic maximum on its bit pattern (the caller
+  int absmax_identity = 0;            // zeroes it first).  absmax_identity: the largest |C - I| instead, and a NaN in C ends up
+                                      // in the word (as torch.max would return it) instead of being skipped
+  float* C2 = nullptr;                // optional second result, same shape and batch layout as C with its own strides:
+  int64_t ldc2 = 0, sC2 = 0;          // C2 = c2_scale * C + c2_diag * I (the next iterate's polynomial of a Newton iteration,
+  float c2_scale = 0.f, c2_diag = 0.f;   // written while C is still in registers)
 };
 
 constexpr int GBT = 128, GBK = 16;     // GBT: granularity of the triangular contraction ranges (both tile sizes)
@@ -108,6 +113,25 @@ __device__ __forceinline__ void gemm_frag(float (&f)[8], const float* __restrict
 #pragma unroll
     for (int m = 0; m < 8; ++m) f[m] = lds[(8 * g + m) * GemmTile<BT>::IC_STRIDE + row];
   }
+}
+
+// Running maximum of |v| (identity: of |v - 1| on the diagonal, |v| off it, and a NaN is kept once it has been seen).
+__device__ __forceinline__ float gemm_fold_absmax(float vmax, float v, bool diagonal, int identity) {
+  if (identity == 0) return fmaxf(vmax, fabsf(v));
+  const float d = fabsf(v - (diagonal ? 1.f : 0.f));
+  return (d > vmax || d != d) ? d : vmax;
+}
+
+// Folds a wave's maxima into the word at `out`.  Non-negative floats order like their bit patterns, and a NaN has a
+// larger pattern than any number.
+__device__ __forceinline__ void gemm_store_absmax(float* out, float vmax, int lane) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float other = __shfl_xor(vmax, o);
+    vmax = (other > vmax || other != other) ? other : vmax;
+  }
+  vmax = fabsf(vmax);       // (a NaN of either sign: the pattern without the sign bit)
+  if (lane == 0) atomicMax(reinterpret_cast<unsigned int*>(out), __builtin_bit_cast(unsigned int, vmax));
 }
 
 // One BT x BT tile (ti, tj) of batch entry z of the product described by p; lds: [2][2][PANEL] floats.
@@ -211,6 +235,8 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int t
   }
   const bool lower_only = (p.tile_mode == TILE_LOWER);
   const bool mirror = (p.tile_mode == TILE_LOWER_MIRROR) && (ti != tj);
+  float* __restrict__ C2 = p.C2 != nullptr ? p.C2 + static_cast<int64_t>(z) * p.sC2 : nullptr;
+  float vmax = 0.f;
 #pragma unroll
   for (int a = 0; a < TI; ++a)
 #pragma unroll
@@ -227,8 +253,15 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmParams& p, int ti, int t
         if (p.beta != 0.f) v += p.beta * *dst;
         *dst = v;
         if (mirror) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
+        vmax = gemm_fold_absmax(vmax, v, gi == gj, p.absmax_identity);
+        if (C2 != nullptr) {
+          const float w = p.c2_scale * v + (gi == gj ? p.c2_diag : 0.f);
+          C2[static_cast<int64_t>(gi) * p.ldc2 + gj] = w;
+          if (mirror) C2[static_cast<int64_t>(gj) * p.ldc2 + gi] = w;
+        }
       }
     }
+  if (p.absmax_out != nullptr) gemm_store_absmax(p.absmax_out + static_cast<int64_t>(z) * p.absmax_stride, vmax, lane);
 }
 
 template <int TI, bool CHUNKED = false>
@@ -298,18 +331,12 @@ inline int launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
 inline GemmParams make_gemm(int transA, int transB, int M, int N, int K, float alpha, const float* A, int64_t lda,
                             const float* B, int64_t ldb, float beta, float* C, int64_t ldc) {
   GemmParams p;
-  p.A = A; p.B = B; p.C = C; p.C_list = nullptr;
+  p.A = A; p.B = B; p.C = C;
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
-  p.sA = p.sB = p.sC = 0;
   p.M = M; p.N = N; p.K = K;
   p.transA = transA; p.transB = transB;
   p.alpha = alpha; p.beta = beta;
   p.kmode = K_FULL; p.tile_mode = TILE_ALL;
-  p.scaleA = p.scaleB = 1.f;
-  p.absmax_out = nullptr;
-  p.active = nullptr; p.active_stride = 0;
-  p.split = 0;
-  p.chunked = 0;
   return p;
 }
 

@@ -422,6 +422,7 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][b][r] *= p.alpha;
   }
+  float* __restrict__ C2 = p.C2 != nullptr ? p.C2 + static_cast<int64_t>(z) * p.sC2 : nullptr;
   float vmax = 0.f;
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -435,17 +436,17 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
         if (gi >= p.M) continue;
         if (lower_only && gi < gj) continue;
         const float v = acc[a][b][r];
-        vmax = fmaxf(vmax, fabsf(v));
+        vmax = gemm_fold_absmax(vmax, v, gi == gj, p.absmax_identity);
         C[static_cast<int64_t>(gi) * p.ldc + gj] = v;
         if (mirror && gi != gj) C[static_cast<int64_t>(gj) * p.ldc + gi] = v;
+        if (C2 != nullptr) {
+          const float w = p.c2_scale * v + (gi == gj ? p.c2_diag : 0.f);
+          C2[static_cast<int64_t>(gi) * p.ldc2 + gj] = w;
+          if (mirror && gi != gj) C2[static_cast<int64_t>(gj) * p.ldc2 + gi] = w;
+        }
       }
     }
-  if (p.absmax_out != nullptr) {
-    // non-negative floats order like their bit patterns; NaN (a larger pattern than any number) propagates
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, o));
-    if (lane == 0) atomicMax(reinterpret_cast<unsigned int*>(p.absmax_out), __builtin_bit_cast(unsigned int, vmax));
-  }
+  if (p.absmax_out != nullptr) gemm_store_absmax(p.absmax_out + static_cast<int64_t>(z) * p.absmax_stride, vmax, lane);
 }
 
 template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool CHUNKED = false>

@@ -4,7 +4,9 @@
 // test evaluated on the device.  The host enqueues the maximum number of iterations; each kernel
 // first reads its matrix's `active` word and returns at once when that matrix has converged (or
 // stopped because its error grew by more than 1.2x, in which case the previous root is kept).
-// All products are fp32 MFMA GEMM tiles (gemm_f32.hpp); reductions are two-stage and deterministic.
+// The products run on the split-operand tile kernel (gemm_x3.hpp; small ones on the fp32 tile of gemm_f32.hpp), summed
+// in chunks; the product that forms the next M also folds max |M - I| into a device word and writes the next step's
+// polynomial, and the iterates alternate between two buffer pairs, so a step is its products and one decision kernel.
 #include "gemm_f32.hpp"
 
 namespace ak {
@@ -31,6 +33,8 @@ struct RootState {
   int* active;      // Newton iteration still running
   int* commit;      // last Newton step accepted
   int* count;
+  int* par;         // which of the two root / M buffers holds the matrix's latest accepted iterate
+  float* errword;   // max |M' - I| of the step under way, folded in by the epilogue of the product that forms M'
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -66,6 +70,8 @@ static __global__ __launch_bounds__(256) void root_init_kernel(RootState st, con
     st.active[z] = 0;
     st.commit[z] = 0;
     st.count[z] = 0;
+    st.par[z] = 0;
+    st.errword[z] = 0.f;
   }
 }
 
@@ -148,21 +154,23 @@ static __global__ void root_zscale_kernel(RootState st, int p) {
   st.zscale[z] = (1.f + p) / (2.f * sqrtf(s));
 }
 
-// grid (RCHUNKS, batch): M = z S, root = z^(1/p) I, partial max |M - I|
+// grid (RCHUNKS, batch): M = z S, T = (1 + 1/p) I - M / p, root = z^(1/p) I, partial max |M - I|
 static __global__ __launch_bounds__(256) void root_start_kernel(RootState st, const float* __restrict__ S,
                                                                 int64_t strideS, float* __restrict__ M,
-                                                                float* __restrict__ root, int64_t strideR, int64_t n,
-                                                                int p) {
+                                                                float* __restrict__ T, float* __restrict__ root,
+                                                                int64_t strideR, int64_t n, int p) {
   __shared__ float red[4];
   const int z = blockIdx.y;
   const float zs = st.zscale[z];
   const float r0 = powf(zs, 1.0f / p);
+  const float alpha = -1.0f / p;
   const int64_t total = n * n;
   float e = 0.f;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
     const bool diag = (i % (n + 1) == 0);
     const float m = zs * S[z * strideS + i];
     M[z * total + i] = m;
+    T[z * total + i] = (diag ? (1.f - alpha) : 0.f) + alpha * m;
     root[z * strideR + i] = diag ? r0 : 0.f;
     e = fmaxf(e, fabsf(m - (diag ? 1.f : 0.f)));
   }
@@ -182,78 +190,51 @@ static __global__ void root_begin_kernel(RootState st, float tol, int max_iter) 
   st.active[z] = (e > tol && max_iter > 0) ? 1 : 0;
 }
 
-// grid (RCHUNKS, batch): T = (1 + 1/p) I - M / p
-static __global__ __launch_bounds__(256) void newton_tmp_kernel(RootState st, const float* __restrict__ M,
-                                                                float* __restrict__ T, int64_t n, int p) {
-  const int z = blockIdx.y;
-  if (st.active[z] == 0) return;
-  const int64_t total = n * n;
-  const float alpha = -1.0f / p;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
-    const bool diag = (i % (n + 1) == 0);
-    T[z * total + i] = (diag ? (1.f - alpha) : 0.f) + alpha * M[z * total + i];
-  }
-}
-
-// grid (RCHUNKS, batch): partial max |Mnew - I|
-static __global__ __launch_bounds__(256) void newton_err_kernel(RootState st, const float* __restrict__ Mnew, int64_t n) {
-  __shared__ float red[4];
-  const int z = blockIdx.y;
-  if (st.active[z] == 0) return;
-  const int64_t total = n * n;
-  float e = 0.f;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
-    const float m = Mnew[z * total + i];
-    const float d = fabsf(m - ((i % (n + 1) == 0) ? 1.f : 0.f));
-    e = (d > e || d != d) ? d : e;        // NaN propagates, as torch.max does
-  }
-  float o;
-#pragma unroll
-  for (int s = 32; s > 0; s >>= 1) { o = __shfl_xor(e, s); e = (o > e || o != o) ? o : e; }
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = e;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float r = red[0];
-    for (int w = 1; w < 4; ++w) r = (red[w] > r || red[w] != red[w]) ? red[w] : r;
-    st.partial[z * RCHUNKS + blockIdx.x] = r;
-  }
-}
-
-// grid (batch): accept / reject the step and decide whether to go on
-static __global__ void newton_decide_kernel(RootState st, float tol, int max_iter) {
+// grid (batch): accept / reject the step and decide whether to go on.  The error of the step is the word the product
+// M' = T^p M folded max |M' - I| into; `wrote`: which buffer pair that step wrote (the matrix's latest iterate if
+// the step is accepted).
+static __global__ void newton_decide_kernel(RootState st, float tol, int max_iter, int wrote) {
   const int z = blockIdx.x;
   if (threadIdx.x != 0) return;
   st.commit[z] = 0;
+  const float e = st.errword[z];
+  st.errword[z] = 0.f;
   if (st.active[z] == 0) return;
-  float e = st.partial[z * RCHUNKS];
-  for (int c = 1; c < RCHUNKS; ++c) {
-    const float x = st.partial[z * RCHUNKS + c];
-    e = (x > e || x != x) ? x : e;
-  }
   const float err = st.err[z];
   if (e > err * 1.2f) {          // diverging: keep the previous root (NaN compares false, like the reference)
     st.active[z] = 0;
     return;
   }
   st.commit[z] = 1;
+  st.par[z] = wrote;
   st.err[z] = e;
   const int c = st.count[z] + 1;
   st.count[z] = c;
   if (!(e > tol && c < max_iter)) st.active[z] = 0;
 }
 
-// grid (RCHUNKS, batch): root <- newroot, M <- Mnew where the step was accepted
-static __global__ __launch_bounds__(256) void newton_commit_kernel(RootState st, float* __restrict__ root,
-                                                                   int64_t strideR, const float* __restrict__ newroot,
-                                                                   float* __restrict__ M, const float* __restrict__ Mnew,
+// grid (RCHUNKS, batch): brings the matrices whose latest iterate sits in the second buffer pair back to the first
+// one (root, M, and T for a matrix that goes on iterating) and resets their marks.  With an even number of iterations
+// per call only the matrices that stopped after an odd number of steps are concerned.
+static __global__ __launch_bounds__(256) void newton_gather_kernel(RootState st, float* __restrict__ root,
+                                                                   int64_t strideR, const float* __restrict__ root1,
+                                                                   float* __restrict__ M, const float* __restrict__ M1,
+                                                                   float* __restrict__ T, const float* __restrict__ T1,
                                                                    int64_t n) {
   const int z = blockIdx.y;
-  if (st.commit[z] == 0) return;
+  if (st.par[z] == 0) return;
+  const bool go_on = st.active[z] != 0;
   const int64_t total = n * n;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += RCHUNKS * 256) {
-    root[z * strideR + i] = newroot[z * total + i];
-    M[z * total + i] = Mnew[z * total + i];
+    root[z * strideR + i] = root1[z * total + i];
+    M[z * total + i] = M1[z * total + i];
+    if (go_on) T[z * total + i] = T1[z * total + i];
   }
+}
+
+// grid (batch): after newton_gather_kernel
+static __global__ void newton_gathered_kernel(RootState st) {
+  if (threadIdx.x == 0) st.par[blockIdx.x] = 0;
 }
 
 // grid (batch)
@@ -266,22 +247,23 @@ static __global__ void root_stats_kernel(RootState st, float* __restrict__ stats
   stats[4 * z + 3] = st.err[z];
 }
 
-static size_t root_state_floats(int batch) { return static_cast<size_t>(batch) * (4 + RCHUNKS + 5) + 16; }
+static size_t root_state_floats(int batch) { return static_cast<size_t>(batch) * (4 + RCHUNKS + 7) + 16; }
 
 }  // namespace ak
 
 extern "C" size_t ak_inv_root_ws_bytes(int64_t n, int batch) {
   if (n <= 0 || batch <= 0) return 0;
-  // M, Mnew, newroot, four product buffers, two vectors, state
-  return (static_cast<size_t>(batch) * (7 * n * n + 2 * n) + ak::root_state_floats(batch)) * sizeof(float);
+  // two M, the second root, two T, four product buffers, two vectors, state
+  return (static_cast<size_t>(batch) * (9 * n * n + 2 * n) + ak::root_state_floats(batch)) * sizeof(float);
 }
 
 namespace ak {
 
-// Workspace layout: M, Mnew, newroot, four product buffers, two vectors, then the per-matrix state; `active`
-// (int32 per matrix, non-zero while its Newton iteration runs) sits at root_active_offset().
+// Workspace layout: M (two buffers), the second root buffer (the first is the caller's result), T (two buffers), four
+// product buffers, two vectors, then the per-matrix state; `active` (int32 per matrix, non-zero while its Newton
+// iteration runs) sits at root_active_offset().
 static size_t root_active_offset(int64_t n, int batch) {
-  return (static_cast<size_t>(batch) * (7 * n * n + 2 * n) + static_cast<size_t>(batch) * (4 + RCHUNKS + 2)) * sizeof(float);
+  return (static_cast<size_t>(batch) * (9 * n * n + 2 * n) + static_cast<size_t>(batch) * (4 + RCHUNKS + 2)) * sizeof(float);
 }
 
 // phases: 1 = power iteration, ridge and start of the Newton iteration; 2 = `iters` Newton iterations; 4 = statistics
@@ -295,9 +277,13 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t nn = n * n;
   float* w = static_cast<float*>(ws);
-  float* M = w;        w += batch * nn;
-  float* Mnew = w;     w += batch * nn;
-  float* newroot = w;  w += batch * nn;
+  float* Mb[2];
+  Mb[0] = w;           w += batch * nn;
+  Mb[1] = w;           w += batch * nn;
+  float* root1 = w;    w += batch * nn;
+  float* Tb[2];
+  Tb[0] = w;           w += batch * nn;
+  Tb[1] = w;           w += batch * nn;
   float* buf[4];
   for (int i = 0; i < 4; ++i) { buf[i] = w; w += batch * nn; }
   float* v = w;        w += batch * n;
@@ -313,6 +299,8 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
   st.active = reinterpret_cast<int*>(w); w += batch;
   st.commit = reinterpret_cast<int*>(w); w += batch;
   st.count = reinterpret_cast<int*>(w); w += batch;
+  st.par = reinterpret_cast<int*>(w); w += batch;
+  st.errword = w; w += batch;
 
   if (reinterpret_cast<unsigned char*>(st.active) != static_cast<unsigned char*>(ws) + root_active_offset(n, batch))
     return AK_ERR_ARG;     // the layout above and root_active_offset() have to agree
@@ -326,13 +314,15 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     }
     hipLaunchKernelGGL(root_ridge_kernel, gc, b256, 0, s, st, S, strideS, n, ridge_eps);
     hipLaunchKernelGGL(root_zscale_kernel, gb, dim3(64), 0, s, st, p);
-    hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, M, out, strideOut, n, p);
+    hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, Mb[0], Tb[0], out, strideOut, n, p);
     hipLaunchKernelGGL(root_begin_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
   }
   if (!(phases & 2)) iters = 0;
 
   const int N = static_cast<int>(n);
-  auto mm = [&](const float* A, int64_t sA, const float* B, int64_t sB, float* C, int64_t sC) {
+  // C = A B for every matrix that still iterates.  next_T (the product that forms M' only): the epilogue also folds
+  // max |C - I| into the matrix's error word and writes the polynomial of the next step, (1 + 1/p) I - C / p.
+  auto mm = [&](const float* A, int64_t sA, const float* B, int64_t sB, float* C, int64_t sC, float* next_T) {
     GemmParams g = make_gemm(0, 0, N, N, N, 1.f, A, n, B, n, 0.f, C, n);
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.active = st.active; g.active_stride = 1;
@@ -341,16 +331,26 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     // against the smallest eigenvalues of M (ridge_eps of the largest); a rank-deficient 1024 x 1024 statistic lost a
     // factor of six against LAPACK-grade fp32 products with one accumulator rounded at every matrix instruction
     g.chunked = 1;
+    if (next_T != nullptr) {
+      g.absmax_out = st.errword; g.absmax_stride = 1; g.absmax_identity = 1;
+      g.C2 = next_T; g.ldc2 = n; g.sC2 = nn;
+      g.c2_scale = -1.0f / p; g.c2_diag = 1.0f + 1.0f / p;
+    }
     // Every matrix of the iteration is a polynomial of the one symmetric statistic, so every product is symmetric up
     // to rounding: large ones compute the tiles on and below the diagonal only and mirror them (half the work; the
     // results are then exactly symmetric).  Small ones keep the full product.
     if (N >= kRootSymmetricMinDim) g.tile_mode = TILE_LOWER_MIRROR;
     return launch_gemm(g, batch, s);
   };
+  // Iteration j of this call reads the buffer pair j % 2 (roots: the caller's `out` and root1; M and T: Mb, Tb) and
+  // writes the other one; an accepted step moves the matrix's mark (st.par) there, so nothing is copied per step.
+  // Every call starts with all marks on pair 0 and ends by bringing the marked matrices back to it.
+  float* const Rb[2] = {out, root1};
+  const int64_t sR[2] = {strideOut, nn};
   for (int it = 0; it < iters; ++it) {
-    float* T = buf[0];
-    hipLaunchKernelGGL(newton_tmp_kernel, gc, b256, 0, s, st, M, T, n, p);
-    int rc = mm(out, strideOut, T, nn, newroot, nn);            // new_root = root T
+    const int a = it & 1, b = a ^ 1;
+    const float* T = Tb[a];
+    int rc = mm(Rb[a], sR[a], T, nn, Rb[b], sR[b], nullptr);      // new_root = root T
     if (rc != AK_OK) return rc;
     // T^p with the multiplication order of MatPower
     const float* tp = nullptr;
@@ -359,7 +359,7 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
       int which = 1;
       for (int done = 1; done < p; done *= 2) {
         float* dst = buf[which];
-        rc = mm(cur, nn, cur, nn, dst, nn);
+        rc = mm(cur, nn, cur, nn, dst, nn, nullptr);
         if (rc != AK_OK) return rc;
         cur = dst;
         which = (which == 1) ? 2 : 1;
@@ -368,14 +368,14 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     } else {
       const float* base = T;        // squares ping-pong in buf[0]/buf[1], the running power in buf[2]/buf[3]
       const float* power = nullptr;
-      int sq = 1, pw = 2;
+      int sq = 0, pw = 2;
       for (int q = p; q > 0; q /= 2) {
         if (q & 1) {
           if (power == nullptr) {
             power = base;
           } else {
             float* dst = buf[pw];
-            rc = mm(base, nn, power, nn, dst, nn);
+            rc = mm(base, nn, power, nn, dst, nn, nullptr);
             if (rc != AK_OK) return rc;
             power = dst;
             pw = (pw == 2) ? 3 : 2;
@@ -383,26 +383,28 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
         }
         if (q / 2 > 0) {
           float* dst = buf[sq];
-          if (power == base) {      // keep the value `power` points at alive
+          if (power == base && base != T) {      // a later square would overwrite the value `power` points at
             float* keep = buf[pw];
             if (hipMemcpyAsync(keep, base, sizeof(float) * batch * nn, hipMemcpyDeviceToDevice, s) != hipSuccess)
               return AK_ERR_LAUNCH;
             power = keep;
             pw = (pw == 2) ? 3 : 2;
           }
-          rc = mm(base, nn, base, nn, dst, nn);
+          rc = mm(base, nn, base, nn, dst, nn, nullptr);
           if (rc != AK_OK) return rc;
           base = dst;
-          sq = (sq == 1) ? 0 : 1;
+          sq = (sq == 0) ? 1 : 0;
         }
       }
       tp = power;
     }
-    rc = mm(tp, nn, M, nn, Mnew, nn);                           // M' = T^p M
+    rc = mm(tp, nn, Mb[a], nn, Mb[b], nn, Tb[b]);                // M' = T^p M, its error, the next T
     if (rc != AK_OK) return rc;
-    hipLaunchKernelGGL(newton_err_kernel, gc, b256, 0, s, st, Mnew, n);
-    hipLaunchKernelGGL(newton_decide_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
-    hipLaunchKernelGGL(newton_commit_kernel, gc, b256, 0, s, st, out, strideOut, newroot, M, Mnew, n);
+    hipLaunchKernelGGL(newton_decide_kernel, gb, dim3(64), 0, s, st, tol, max_iter, b);
+  }
+  if (iters > 0) {
+    hipLaunchKernelGGL(newton_gather_kernel, gc, b256, 0, s, st, out, strideOut, root1, Mb[0], Mb[1], Tb[0], Tb[1], n);
+    hipLaunchKernelGGL(newton_gathered_kernel, gb, dim3(64), 0, s, st);
   }
   if (phases & 4) hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
   return check_launch();
