@@ -8,6 +8,7 @@
 // in chunks; the product that forms the next M also folds max |M - I| into a device word and writes the next step's
 // polynomial, and the iterates alternate between two buffer pairs, so a step is its products and one decision kernel.
 #include "gemm_f32.hpp"
+#include "gemm_planes.hpp"
 
 namespace ak {
 
@@ -20,6 +21,22 @@ constexpr int g_root_split = 3;
 
 constexpr int RCHUNKS = 64;   // partial-reduction chunks per matrix
 constexpr int kRootSymmetricMinDim = 512;   // products of matrices this large compute the lower tiles only
+// Statistics this large iterate on bf16 planes (gemm_planes.hpp): every matrix of the iteration is stored as the three
+// planes of its exact split, written by the product that makes it.  Smaller ones keep fp32 matrices and the tile
+// kernels that split (or multiply in fp32) as they read.
+#ifdef AK_TUNING_HOOKS
+inline int g_root_planes_min = 512;
+#else
+constexpr int g_root_planes_min = 512;
+#endif
+static bool root_uses_planes(int64_t n) { return n >= g_root_planes_min && n <= kPlaneMaxDim; }
+static int64_t root_pad(int64_t n) { return (n + kPlaneTile - 1) / kPlaneTile * kPlaneTile; }
+// floats of the matrix buffers of one statistic: ten plane sets (two roots, two M, two T, four products) of
+// 3 n_pad^2 bf16, or nine fp32 matrices (two M, the second root, two T, four products)
+static size_t root_matrix_floats(int64_t n) {
+  if (root_uses_planes(n)) return static_cast<size_t>(15) * root_pad(n) * root_pad(n);
+  return static_cast<size_t>(9) * n * n;
+}
 
 struct RootState {
   // per matrix, all device memory
@@ -237,6 +254,81 @@ static __global__ void newton_gathered_kernel(RootState st) {
   if (threadIdx.x == 0) st.par[blockIdx.x] = 0;
 }
 
+// ---- the same on bf16 planes --------------------------------------------------------------------------------------
+
+// grid (RCHUNKS, batch): planes of M = z S, T = (1 + 1/p) I - M / p and root = z^(1/p) I over the padded index range
+// (zero outside n x n), partial max |M - I|
+static __global__ __launch_bounds__(256) void root_start_planes_kernel(RootState st, const float* __restrict__ S,
+                                                                       int64_t strideS, __bf16* __restrict__ M,
+                                                                       __bf16* __restrict__ T, __bf16* __restrict__ R,
+                                                                       int64_t set_elems, int64_t n, int64_t n_pad, int p) {
+  __shared__ float red[4];
+  const int z = blockIdx.y;
+  const float zs = st.zscale[z];
+  const float r0 = powf(zs, 1.0f / p);
+  const float alpha = -1.0f / p;
+  const int64_t total = n_pad * n_pad;
+  __bf16* Mz = M + z * set_elems;
+  __bf16* Tz = T + z * set_elems;
+  __bf16* Rz = R + z * set_elems;
+  float e = 0.f;
+  for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < total; at += RCHUNKS * 256) {
+    const int64_t i = at / n_pad, j = at - i * n_pad;
+    const bool inside = i < n && j < n, diag = i == j;
+    float m = 0.f, t = 0.f, r = 0.f;
+    if (inside) {
+      m = zs * S[z * strideS + i * n + j];
+      t = (diag ? (1.f - alpha) : 0.f) + alpha * m;
+      r = diag ? r0 : 0.f;
+      e = fmaxf(e, fabsf(m - (diag ? 1.f : 0.f)));
+    }
+    __bf16 h, mid, l;
+    plane_split(m, h, mid, l);
+    Mz[at] = h; Mz[total + at] = mid; Mz[2 * total + at] = l;
+    plane_split(t, h, mid, l);
+    Tz[at] = h; Tz[total + at] = mid; Tz[2 * total + at] = l;
+    plane_split(r, h, mid, l);
+    Rz[at] = h; Rz[total + at] = mid; Rz[2 * total + at] = l;
+  }
+  e = wave_max(e);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = e;
+  __syncthreads();
+  if (threadIdx.x == 0) st.partial[z * RCHUNKS + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// grid (RCHUNKS, batch): newton_gather_kernel on plane sets (set_words 32-bit words each)
+static __global__ __launch_bounds__(256) void newton_gather_planes_kernel(RootState st, uint32_t* __restrict__ R0,
+                                                                          const uint32_t* __restrict__ R1,
+                                                                          uint32_t* __restrict__ M0,
+                                                                          const uint32_t* __restrict__ M1,
+                                                                          uint32_t* __restrict__ T0,
+                                                                          const uint32_t* __restrict__ T1,
+                                                                          int64_t set_words) {
+  const int z = blockIdx.y;
+  if (st.par[z] == 0) return;
+  const bool go_on = st.active[z] != 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < set_words; i += RCHUNKS * 256) {
+    R0[z * set_words + i] = R1[z * set_words + i];
+    M0[z * set_words + i] = M1[z * set_words + i];
+    if (go_on) T0[z * set_words + i] = T1[z * set_words + i];
+  }
+}
+
+// grid (RCHUNKS, batch): the caller's fp32 result from the planes of the root (their sum is exact)
+static __global__ __launch_bounds__(256) void root_out_planes_kernel(const __bf16* __restrict__ R, int64_t set_elems,
+                                                                     float* __restrict__ out, int64_t strideOut,
+                                                                     int64_t n, int64_t n_pad) {
+  const int z = blockIdx.y;
+  const int64_t total = n_pad * n_pad;
+  const __bf16* Rz = R + z * set_elems;
+  for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < n * n; at += RCHUNKS * 256) {
+    const int64_t i = at / n, j = at - i * n;
+    const int64_t src = i * n_pad + j;
+    out[z * strideOut + at] = (static_cast<float>(Rz[src]) + static_cast<float>(Rz[total + src])) +
+                              static_cast<float>(Rz[2 * total + src]);
+  }
+}
+
 // grid (batch)
 static __global__ void root_stats_kernel(RootState st, float* __restrict__ stats) {
   const int z = blockIdx.x;
@@ -253,8 +345,8 @@ static size_t root_state_floats(int batch) { return static_cast<size_t>(batch) *
 
 extern "C" size_t ak_inv_root_ws_bytes(int64_t n, int batch) {
   if (n <= 0 || batch <= 0) return 0;
-  // two M, the second root, two T, four product buffers, two vectors, state
-  return (static_cast<size_t>(batch) * (9 * n * n + 2 * n) + ak::root_state_floats(batch)) * sizeof(float);
+  // the matrix buffers, two vectors, state
+  return (static_cast<size_t>(batch) * (ak::root_matrix_floats(n) + 2 * n) + ak::root_state_floats(batch)) * sizeof(float);
 }
 
 namespace ak {
@@ -263,7 +355,7 @@ namespace ak {
 // product buffers, two vectors, then the per-matrix state; `active` (int32 per matrix, non-zero while its Newton
 // iteration runs) sits at root_active_offset().
 static size_t root_active_offset(int64_t n, int batch) {
-  return (static_cast<size_t>(batch) * (9 * n * n + 2 * n) + static_cast<size_t>(batch) * (4 + RCHUNKS + 2)) * sizeof(float);
+  return (static_cast<size_t>(batch) * (root_matrix_floats(n) + 2 * n) + static_cast<size_t>(batch) * (4 + RCHUNKS + 2)) * sizeof(float);
 }
 
 // phases: 1 = power iteration, ridge and start of the Newton iteration; 2 = `iters` Newton iterations; 4 = statistics
@@ -277,15 +369,32 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t nn = n * n;
   float* w = static_cast<float*>(ws);
-  float* Mb[2];
-  Mb[0] = w;           w += batch * nn;
-  Mb[1] = w;           w += batch * nn;
-  float* root1 = w;    w += batch * nn;
-  float* Tb[2];
-  Tb[0] = w;           w += batch * nn;
-  Tb[1] = w;           w += batch * nn;
-  float* buf[4];
-  for (int i = 0; i < 4; ++i) { buf[i] = w; w += batch * nn; }
+  const bool planes = root_uses_planes(n);
+  const int64_t n_pad = root_pad(n), set_elems = 3 * n_pad * n_pad;       // bf16 elements of one plane set
+  float* Mb[2] = {nullptr, nullptr};
+  float* root1 = nullptr;
+  float* Tb[2] = {nullptr, nullptr};
+  float* buf[4] = {nullptr, nullptr, nullptr, nullptr};
+  __bf16* pR[2] = {nullptr, nullptr};
+  __bf16* pM[2] = {nullptr, nullptr};
+  __bf16* pT[2] = {nullptr, nullptr};
+  __bf16* pbuf[4] = {nullptr, nullptr, nullptr, nullptr};
+  if (planes) {
+    __bf16* q = reinterpret_cast<__bf16*>(w);
+    for (int i = 0; i < 2; ++i) { pR[i] = q; q += batch * set_elems; }
+    for (int i = 0; i < 2; ++i) { pM[i] = q; q += batch * set_elems; }
+    for (int i = 0; i < 2; ++i) { pT[i] = q; q += batch * set_elems; }
+    for (int i = 0; i < 4; ++i) { pbuf[i] = q; q += batch * set_elems; }
+  } else {
+    float* q = w;
+    Mb[0] = q;           q += batch * nn;
+    Mb[1] = q;           q += batch * nn;
+    root1 = q;           q += batch * nn;
+    Tb[0] = q;           q += batch * nn;
+    Tb[1] = q;           q += batch * nn;
+    for (int i = 0; i < 4; ++i) { buf[i] = q; q += batch * nn; }
+  }
+  w += static_cast<size_t>(batch) * root_matrix_floats(n);
   float* v = w;        w += batch * n;
   float* mv = w;       w += batch * n;
   RootState st;
@@ -314,26 +423,51 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     }
     hipLaunchKernelGGL(root_ridge_kernel, gc, b256, 0, s, st, S, strideS, n, ridge_eps);
     hipLaunchKernelGGL(root_zscale_kernel, gb, dim3(64), 0, s, st, p);
-    hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, Mb[0], Tb[0], out, strideOut, n, p);
+    if (planes)
+      hipLaunchKernelGGL(root_start_planes_kernel, gc, b256, 0, s, st, S, strideS, pM[0], pT[0], pR[0], set_elems, n, n_pad, p);
+    else
+      hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, Mb[0], Tb[0], out, strideOut, n, p);
     hipLaunchKernelGGL(root_begin_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
   }
   if (!(phases & 2)) iters = 0;
 
   const int N = static_cast<int>(n);
-  // C = A B for every matrix that still iterates.  next_T (the product that forms M' only): the epilogue also folds
-  // max |C - I| into the matrix's error word and writes the polynomial of the next step, (1 + 1/p) I - C / p.
-  auto mm = [&](const float* A, int64_t sA, const float* B, int64_t sB, float* C, int64_t sC, float* next_T) {
-    GemmParams g = make_gemm(0, 0, N, N, N, 1.f, A, n, B, n, 0.f, C, n);
-    g.sA = sA; g.sB = sB; g.sC = sC;
+  // The matrices of the iteration by number: two roots, two M, two T, four product buffers.  fp32 form: the first
+  // root is the caller's `out`; plane form: all ten are plane sets of the workspace.
+  enum { R0 = 0, R1, M0, M1, T0, T1, B0, B1, B2, B3, NBUF };
+  float* fptr[NBUF] = {out, root1, Mb[0], Mb[1], Tb[0], Tb[1], buf[0], buf[1], buf[2], buf[3]};
+  int64_t fstride[NBUF];
+  for (int i = 0; i < NBUF; ++i) fstride[i] = nn;
+  fstride[R0] = strideOut;
+  __bf16* pptr[NBUF] = {pR[0], pR[1], pM[0], pM[1], pT[0], pT[1], pbuf[0], pbuf[1], pbuf[2], pbuf[3]};
+  // C = A B for every matrix that still iterates.  next_T >= 0 (the product that forms M' only): the epilogue also
+  // folds max |C - I| into the matrix's error word and writes the polynomial of the next step, (1 + 1/p) I - C / p.
+  auto mm = [&](int ia, int ib, int ic, int next_T) {
+    if (planes) {
+      PlaneGemm g{};
+      g.A = pptr[ia]; g.B = pptr[ib]; g.C = pptr[ic];
+      g.sA = g.sB = g.sC = g.sC2 = set_elems;
+      g.plane_elems = n_pad * n_pad;
+      g.n = N; g.n_pad = static_cast<int>(n_pad); g.T = static_cast<int>(n_pad / kPlaneTile);
+      g.active = st.active;
+      if (next_T >= 0) {
+        g.errword = st.errword;
+        g.C2 = pptr[next_T];
+        g.c2_scale = -1.0f / p; g.c2_diag = 1.0f + 1.0f / p;
+      }
+      return launch_plane_gemm(g, batch, s);
+    }
+    GemmParams g = make_gemm(0, 0, N, N, N, 1.f, fptr[ia], n, fptr[ib], n, 0.f, fptr[ic], n);
+    g.sA = fstride[ia]; g.sB = fstride[ib]; g.sC = fstride[ic];
     g.active = st.active; g.active_stride = 1;
     g.split = g_root_split;
     // sums in chunks: the error of the root is set by the absolute rounding error of the first iterations' products
     // against the smallest eigenvalues of M (ridge_eps of the largest); a rank-deficient 1024 x 1024 statistic lost a
     // factor of six against LAPACK-grade fp32 products with one accumulator rounded at every matrix instruction
     g.chunked = 1;
-    if (next_T != nullptr) {
+    if (next_T >= 0) {
       g.absmax_out = st.errword; g.absmax_stride = 1; g.absmax_identity = 1;
-      g.C2 = next_T; g.ldc2 = n; g.sC2 = nn;
+      g.C2 = fptr[next_T]; g.ldc2 = n; g.sC2 = fstride[next_T];
       g.c2_scale = -1.0f / p; g.c2_diag = 1.0f + 1.0f / p;
     }
     // Every matrix of the iteration is a polynomial of the one symmetric statistic, so every product is symmetric up
@@ -342,70 +476,79 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     if (N >= kRootSymmetricMinDim) g.tile_mode = TILE_LOWER_MIRROR;
     return launch_gemm(g, batch, s);
   };
-  // Iteration j of this call reads the buffer pair j % 2 (roots: the caller's `out` and root1; M and T: Mb, Tb) and
-  // writes the other one; an accepted step moves the matrix's mark (st.par) there, so nothing is copied per step.
-  // Every call starts with all marks on pair 0 and ends by bringing the marked matrices back to it.
-  float* const Rb[2] = {out, root1};
-  const int64_t sR[2] = {strideOut, nn};
+  auto copy = [&](int dst, int src) {
+    const hipError_t e = planes
+        ? hipMemcpyAsync(pptr[dst], pptr[src], sizeof(__bf16) * batch * set_elems, hipMemcpyDeviceToDevice, s)
+        : hipMemcpyAsync(fptr[dst], fptr[src], sizeof(float) * batch * nn, hipMemcpyDeviceToDevice, s);
+    return e == hipSuccess ? AK_OK : AK_ERR_LAUNCH;
+  };
+  // Iteration j of this call reads the buffer pair j % 2 (R, M, T) and writes the other one; an accepted step moves the
+  // matrix's mark (st.par) there, so nothing is copied per step.  Every call starts with all marks on pair 0 and ends
+  // by bringing the marked matrices back to it.
   for (int it = 0; it < iters; ++it) {
     const int a = it & 1, b = a ^ 1;
-    const float* T = Tb[a];
-    int rc = mm(Rb[a], sR[a], T, nn, Rb[b], sR[b], nullptr);      // new_root = root T
+    const int T = T0 + a;
+    int rc = mm(R0 + a, T, R0 + b, -1);                          // new_root = root T
     if (rc != AK_OK) return rc;
     // T^p with the multiplication order of MatPower
-    const float* tp = nullptr;
+    int tp = -1;
     if ((p & (p - 1)) == 0) {
-      const float* cur = T;
-      int which = 1;
+      int cur = T, which = B1;
       for (int done = 1; done < p; done *= 2) {
-        float* dst = buf[which];
-        rc = mm(cur, nn, cur, nn, dst, nn, nullptr);
+        rc = mm(cur, cur, which, -1);
         if (rc != AK_OK) return rc;
-        cur = dst;
-        which = (which == 1) ? 2 : 1;
+        cur = which;
+        which = (which == B1) ? B2 : B1;
       }
       tp = cur;
     } else {
-      const float* base = T;        // squares ping-pong in buf[0]/buf[1], the running power in buf[2]/buf[3]
-      const float* power = nullptr;
-      int sq = 0, pw = 2;
+      int base = T, power = -1;     // squares ping-pong in B0 / B1, the running power in B2 / B3
+      int sq = B0, pw = B2;
       for (int q = p; q > 0; q /= 2) {
         if (q & 1) {
-          if (power == nullptr) {
+          if (power < 0) {
             power = base;
           } else {
-            float* dst = buf[pw];
-            rc = mm(base, nn, power, nn, dst, nn, nullptr);
+            rc = mm(base, power, pw, -1);
             if (rc != AK_OK) return rc;
-            power = dst;
-            pw = (pw == 2) ? 3 : 2;
+            power = pw;
+            pw = (pw == B2) ? B3 : B2;
           }
         }
         if (q / 2 > 0) {
-          float* dst = buf[sq];
           if (power == base && base != T) {      // a later square would overwrite the value `power` points at
-            float* keep = buf[pw];
-            if (hipMemcpyAsync(keep, base, sizeof(float) * batch * nn, hipMemcpyDeviceToDevice, s) != hipSuccess)
-              return AK_ERR_LAUNCH;
-            power = keep;
-            pw = (pw == 2) ? 3 : 2;
+            rc = copy(pw, base);
+            if (rc != AK_OK) return rc;
+            power = pw;
+            pw = (pw == B2) ? B3 : B2;
           }
-          rc = mm(base, nn, base, nn, dst, nn, nullptr);
+          rc = mm(base, base, sq, -1);
           if (rc != AK_OK) return rc;
-          base = dst;
-          sq = (sq == 0) ? 1 : 0;
+          base = sq;
+          sq = (sq == B0) ? B1 : B0;
         }
       }
       tp = power;
     }
-    rc = mm(tp, nn, Mb[a], nn, Mb[b], nn, Tb[b]);                // M' = T^p M, its error, the next T
+    rc = mm(tp, M0 + a, M0 + b, T0 + b);                         // M' = T^p M, its error, the next T
     if (rc != AK_OK) return rc;
     hipLaunchKernelGGL(newton_decide_kernel, gb, dim3(64), 0, s, st, tol, max_iter, b);
   }
   if (iters > 0) {
-    hipLaunchKernelGGL(newton_gather_kernel, gc, b256, 0, s, st, out, strideOut, root1, Mb[0], Mb[1], Tb[0], Tb[1], n);
+    if (planes) {
+      const int64_t words = set_elems / 2;
+      hipLaunchKernelGGL(newton_gather_planes_kernel, gc, b256, 0, s, st, reinterpret_cast<uint32_t*>(pR[0]),
+                         reinterpret_cast<const uint32_t*>(pR[1]), reinterpret_cast<uint32_t*>(pM[0]),
+                         reinterpret_cast<const uint32_t*>(pM[1]), reinterpret_cast<uint32_t*>(pT[0]),
+                         reinterpret_cast<const uint32_t*>(pT[1]), words);
+    } else {
+      hipLaunchKernelGGL(newton_gather_kernel, gc, b256, 0, s, st, out, strideOut, root1, Mb[0], Mb[1], Tb[0], Tb[1], n);
+    }
     hipLaunchKernelGGL(newton_gathered_kernel, gb, dim3(64), 0, s, st);
   }
+  // plane form: the caller's fp32 root is written with the statistics (the last part of a computation in parts)
+  if ((phases & 4) && planes)
+    hipLaunchKernelGGL(root_out_planes_kernel, gc, b256, 0, s, pR[0], set_elems, out, strideOut, n, n_pad);
   if (phases & 4) hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
   return check_launch();
 }
@@ -435,6 +578,46 @@ extern "C" int ak_inv_root_newton_part(int phases, int iters, float* S, int64_t 
 }
 
 #ifdef AK_TUNING_HOOKS
+namespace ak {
+static __global__ void dbg_to_planes_kernel(const float* __restrict__ X, __bf16* __restrict__ P, int64_t n, int64_t n_pad) {
+  const int64_t total = n_pad * n_pad;
+  for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < total; at += static_cast<int64_t>(gridDim.x) * 256) {
+    const int64_t i = at / n_pad, j = at - i * n_pad;
+    const float x = (i < n && j < n) ? X[i * n + j] : 0.f;
+    __bf16 h, m, l;
+    plane_split(x, h, m, l);
+    P[at] = h; P[total + at] = m; P[2 * total + at] = l;
+  }
+}
+}  // namespace ak
+
+// Tuning builds only: C = A B for symmetric fp32 n x n matrices through the plane kernel (ws: 9 n_pad^2 bf16 + 1 float).
+extern "C" int ak_debug_plane_product(const float* A, const float* B, float* C, int64_t n, void* ws, float* err) {
+  using namespace ak;
+  const int64_t n_pad = root_pad(n), set = 3 * n_pad * n_pad;
+  __bf16* pa = static_cast<__bf16*>(ws);
+  __bf16* pb = pa + set;
+  __bf16* pc = pb + set;
+  float* word = reinterpret_cast<float*>(pc + set);
+  hipMemsetAsync(word, 0, 4, nullptr);
+  hipLaunchKernelGGL(dbg_to_planes_kernel, dim3(512), dim3(256), 0, nullptr, A, pa, n, n_pad);
+  hipLaunchKernelGGL(dbg_to_planes_kernel, dim3(512), dim3(256), 0, nullptr, B, pb, n, n_pad);
+  PlaneGemm g{};
+  g.A = pa; g.B = pb; g.C = pc;
+  g.sA = g.sB = g.sC = g.sC2 = set;
+  g.plane_elems = n_pad * n_pad;
+  g.n = static_cast<int>(n); g.n_pad = static_cast<int>(n_pad); g.T = static_cast<int>(n_pad / kPlaneTile);
+  g.errword = word;
+  const int rc = launch_plane_gemm(g, 1, nullptr);
+  if (rc != AK_OK) return rc;
+  hipLaunchKernelGGL(root_out_planes_kernel, dim3(RCHUNKS, 1), dim3(256), 0, nullptr, pc, set, C, n * n, n, n_pad);
+  hipMemcpy(err, word, 4, hipMemcpyDeviceToHost);
+  return check_launch();
+}
+
+// Tuning builds only: the smallest statistic that iterates on bf16 planes.
+extern "C" void ak_debug_set_root_planes_min(int n) { ak::g_root_planes_min = n; }
+
 // Tuning builds only: 0 = the fp32 MFMA kernel, 3 = the three-piece split kernel for the products of the Newton
 // iteration.
 extern "C" void ak_debug_set_root_split(int pieces) { ak::g_root_split = pieces; }

@@ -356,6 +356,9 @@ int ak_kron_precond_static(const float* Binv, const float* Ainv, float* G, int64
  * below tol, or grows by more than 1.2x (then its previous root is kept), the remaining launches return
  * immediately for it.  stats: device float [batch, 4] = {lambda_max, power iterations, newton iterations,
  * final error}.  n >= 2 (the reference returns the identity for n == 1 without any arithmetic).
+ * Statistics of 512 columns and more iterate on three bf16 planes per matrix (the exact split of its fp32 values,
+ * written by the product that makes the matrix; 192-wide tiles, n padded to a multiple of 192 in the workspace):
+ * ak_inv_root_ws_bytes grows to 60 bytes per padded element and statistic (36 per element below that size).
  * Replaces ComputePower / PowerIter / MatPower (asdl/precondition/shampoo.py:465-586). */
 size_t ak_inv_root_ws_bytes(int64_t n, int batch);
 int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
@@ -369,7 +372,8 @@ int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, f
  * 1 = power iteration, ridge and start; 2 = `iters` further Newton iterations; 4 = stats.  All parts of one
  * computation get the same arguments and the same workspace, untouched in between.  Between parts the host may read
  * the `batch` int32 words at ws + ak_inv_root_active_offset(n, batch) (after synchronising with the stream): word b is
- * non-zero while matrix b still iterates.  ak_inv_root_newton == phases 7 with iters = max_iter. */
+ * non-zero while matrix b still iterates.  ak_inv_root_newton == phases 7 with iters = max_iter.  `out` holds the
+ * roots once the part with bit 4 has run (the last one). */
 size_t ak_inv_root_active_offset(int64_t n, int batch);
 int ak_inv_root_newton_part(int phases, int iters, float* S, int64_t n, int batch, int64_t strideS, int p,
                             float ridge_eps, const float* v0, int max_power_iter, float power_tol, int max_iter,
