@@ -61,8 +61,13 @@ def test_inv_root_matches_reference_golden():
     assert checked >= 5
 
 
-@pytest.mark.parametrize('n,p,batch', [(2, 4, 1), (16, 2, 3), (200, 4, 2), (768, 4, 1), (130, 8, 2), (64, 6, 1)])
+@pytest.mark.parametrize('n,p,batch', [(2, 4, 1), (16, 2, 3), (200, 4, 2), (768, 4, 1), (130, 8, 2), (64, 6, 1),
+                                       (520, 4, 2), (1000, 6, 2), (600, 2, 3), (512, 3, 1)])
 def test_inv_root_closed_form(n, p, batch):
+    """(S + ridge I)^(-1/p) against the fp64 closed form, the power iteration and the iteration count against the
+    oracle.  Statistics below 512 columns iterate on fp32 matrices, the others on bf16 planes padded to a multiple
+    of 192 (520 -> 576, 1000 -> 1152); p = 6 and p = 3 take the general power sequence (squares and a running
+    product), p = 2, 4, 8 repeated squaring."""
     g = torch.Generator().manual_seed(n + p)
     S = torch.empty(batch, n, n)
     for b in range(batch):
@@ -99,6 +104,19 @@ def test_inv_root_polled_and_unpolled_enqueue_give_the_same_result():
         X = torch.randn(40 * (b + 1), 96, generator=g)        # one rank-deficient, two full-rank statistics
         S[b] = X.T @ X / X.shape[0]
     v0 = (torch.rand(3, 96, generator=g) * 2 - 1).cuda()
+    r0, st0 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=0)
+    r1, st1 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=3)
+    r2, st2 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0)
+    assert torch.equal(r0, r1) and torch.equal(r0, r2)
+    assert torch.equal(st0, st1) and torch.equal(st0, st2)
+    assert 1 <= float(st0[:, 2].max()) < 100
+    # the same on bf16 planes (576 columns): parts of an odd number of iterations end with the iterates in the second
+    # buffer pair, from which they are brought back before the next part starts
+    S = torch.empty(2, 576, 576)
+    for b in range(2):
+        X = torch.randn(400 * (b + 1), 576, generator=g)
+        S[b] = X.T @ X / X.shape[0]
+    v0 = (torch.rand(2, 576, generator=g) * 2 - 1).cuda()
     r0, st0 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=0)
     r1, st1 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=3)
     r2, st2 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0)
