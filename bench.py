@@ -639,18 +639,23 @@ def main_shampoo(args, dev):
                 f = float(it.sum()) * products * 2.0 * n ** 3
                 flops += f
                 # every fp32 product runs as 6 bf16 piece products; matrices of 512 and up are known to be
-                # symmetric and only their T (T + 1) / 2 tiles of 128 on and below the diagonal are computed
-                tiles = -(-n // 128)
-                executed_flops += 6.0 * f * ((tiles + 1) / (2.0 * tiles) if n >= 512 else 1.0)
+                # symmetric: only the T (T + 1) / 2 tiles of 192 on and above the diagonal of the matrix padded to a
+                # multiple of 192 are computed (the planes kernel)
+                if n >= 512:
+                    tiles = -(-n // 192)
+                    executed_flops += float(it.sum()) * products * 6.0 * 2.0 * (tiles * (tiles + 1) / 2) * 192.0 ** 2 * (192.0 * tiles)
+                else:
+                    executed_flops += 6.0 * f
                 iters.append(int(it.max()))
         algorithmic = flops / secs / 1e12
         # `achieved` is the ALGORITHMIC rate: 2 n^3 per fp32-grade product of the reference's iteration, against the
         # bf16 matrix peak the products are executed on; the executed piece products are the labelled extra
         out['roofline'] = {'bound': 'mfma', 'achieved': algorithmic, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
                            'frac': algorithmic / BF16_MFMA_PEAK_TFLOPS, 'traffic': None,
-                           'kernel': 'products of the coupled Newton iteration (gemm_x3_kernel): 2 n^3 FLOP per product of '
-                                     'the reference; executed_bf16_tflops counts the bf16 MFMA work actually run (6 piece '
-                                     'products per fp32 product, lower tiles only for the symmetric results)',
+                           'kernel': 'products of the coupled Newton iteration (plane_gemm_kernel: matrices kept as three '
+                                     'bf16 planes; gemm_x3_kernel / gemm_f32_kernel below 512 columns): 2 n^3 FLOP per '
+                                     'product of the reference; executed_bf16_tflops counts the bf16 MFMA work actually '
+                                     'run (6 piece products per fp32 product, the tiles on and above the diagonal only)',
                            'executed_bf16_tflops': executed_flops / secs / 1e12,
                            'executed_bf16_frac': executed_flops / secs / 1e12 / BF16_MFMA_PEAK_TFLOPS,
                            'fp32_peak_frac': algorithmic / FP32_MFMA_PEAK_TFLOPS,

@@ -70,20 +70,35 @@ def main(argv=None):
           lambda: _lib.check(lib.ak_copy_bytes(src.data_ptr(), dst.data_ptr(), n, K._stream()), 'ak_copy_bytes'))
     del src, dst
 
-    # unfold of the 3-channel stem fused into its factor kernel (fp32 images, 7x7 window, stride 2, pad 3): the
-    # input is read once; its 17.5 GFLOP run on the fp32 matrix pipe, which is what bounds it
+    # unfold of the 3-channel stem fused into its factor kernel (fp32 images, 7x7 window, stride 2, pad 3), as the
+    # benchmark step runs it: inside a bf16 autocast region the fp32 images are rounded to bf16 while they are read
+    # and the 17.5 GFLOP run on the bf16 matrix cores; the input is read once
     x = nhwc(64, 3, 224, 224, torch.float32)
     out = torch.empty(147, 147, device=dev)
-    timed('stem unfold + A factor, [64,3,224,224] fp32, 7x7/2', ['ak::conv_patch_syrk_kernel', 'ak::conv_patch_reduce_kernel'],
+    timed('stem unfold + A factor, [64,3,224,224] fp32 rounded to bf16, 7x7/2',
+          ['ak::conv_patch_bf16_kernel', 'ak::conv_patch_bf16_reduce_kernel'],
+          x.numel() * 4 + 147 * 147 * 4, lambda: K.conv_syrk(x, (7, 7), (2, 2), (3, 3), out=out, round_bf16=True),
+          note='bound by the window staging and the LDS gathers of its single wave per SIMD, not by memory')
+    timed('stem unfold + A factor, [64,3,224,224] fp32 kept fp32, 7x7/2',
+          ['ak::conv_patch_syrk_kernel', 'ak::conv_patch_reduce_kernel'],
           x.numel() * 4 + 147 * 147 * 4, lambda: K.conv_syrk(x, (7, 7), (2, 2), (3, 3), out=out),
           note='fp32 MFMA bound (17.5 GFLOP: 0.11 ms at 157.3 TFLOP/s), listed for its unfold traffic')
 
-    # unfold of a 3x3 convolution fused into the bf16 factor kernel, d = 576 (layer1): below the ridge of
-    # 2500 TFLOP/s / 8 TB/s = 312 FLOP/B, (d + 1) / 2 = 288 FLOP per input byte
+    # a 3x3 stride-1 convolution's A factor from shifted correlations of its input, d = 576 (layer1): 13 shifts of a
+    # [C, C] correlation instead of the [9C, 9C] product of the unfolded input, the input read from the L2 / MALL
     x = nhwc(64, 64, 56, 56)
     out = torch.empty(576, 576, device=dev)
-    timed('3x3 unfold + A factor, [64,64,56,56] bf16, d=576', ['ak::syrk_dtl_kernel<..., true>', 'ak::syrk_dtl_finalize_kernel'],
+    timed('3x3 A factor by shifted correlations, [64,64,56,56] bf16, d=576',
+          ['ak::corr_products_kernel', 'ak::corr_reduce_kernel', 'ak::corr_assemble_kernel'],
           x.numel() * 2 + 576 * 576 * 4, lambda: K.conv_syrk(x, (3, 3), (1, 1), (1, 1), out=out))
+
+    # the unfold of a strided 3x3 convolution fused into the gathered bf16 factor kernel, d = 1152 (layer2.0)
+    x = nhwc(64, 128, 56, 56)
+    out = torch.empty(1152, 1152, device=dev)
+    timed('3x3/2 unfold + A factor, [64,128,56,56] bf16, d=1152',
+          ['ak::syrk_dtl_kernel<..., true>', 'ak::syrk_dtl_finalize_blk_kernel'],
+          x.numel() * 2 + 1152 * 1152 * 4, lambda: K.conv_syrk(x, (3, 3), (2, 2), (1, 1), out=out),
+          note='MFMA bound (33 GFLOP by the SYRK count: 13 us at the bf16 peak), listed for its gather traffic')
 
     # plain factors of 1x1 convolutions with few channels: (d + 1) / 2 FLOP per byte, memory bound for d <= 512
     for c, hw in ((64, 56), (256, 56), (512, 28)):
@@ -95,12 +110,12 @@ def main(argv=None):
               ['ak::syrk_dtl_kernel<..., false>', 'ak::syrk_dtl_finalize_kernel'],
               g.numel() * 2 + 2 * c * c * 4, lambda g=g, out=out: K.syrk_tn(g, out=out, alpha=0.95, beta=0.05))
 
-    # the split-K sum / EMA / mirror pass on its own is visible in the kernel trace only; the largest one of the
-    # step belongs to this factor (d = 4608, 3136 rows)
+    # the widest factor of the step with EMA (d = 4608, 3136 rows): the assembly of the shifted correlations reads the
+    # old factor and writes the new one
     x = nhwc(64, 512, 7, 7)
     out = torch.zeros(4608, 4608, device=dev)
-    timed('3x3 unfold + A factor with EMA, [64,512,7,7] bf16, d=4608',
-          ['ak::syrk_dtl_kernel<..., true>', 'ak::syrk_dtl_finalize_kernel'],
+    timed('3x3 A factor by shifted correlations with EMA, [64,512,7,7] bf16, d=4608',
+          ['ak::corr_products_kernel', 'ak::corr_reduce_kernel', 'ak::corr_assemble_kernel'],
           x.numel() * 2 + 2 * 4608 * 4608 * 4, lambda: K.conv_syrk(x, (3, 3), (1, 1), (1, 1), out=out, alpha=0.95, beta=0.05),
           note='result-bound: 85 MB read and 85 MB written for 1.6 MB of input')
 
