@@ -81,6 +81,7 @@ _SIGNATURES = {
     'ak_inv_root_newton': (c_int, [c_ptr, c_i64, c_int, c_i64, c_int, c_f32, c_ptr, c_int, c_f32, c_int, c_f32,
                                    c_ptr, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
     'ak_inv_root_active_offset': (c_size, [c_i64, c_int]),
+    'ak_inv_root_plane_format': (c_int, [c_i64, c_int, c_f32]),
     'ak_inv_root_newton_part': (c_int, [c_int, c_int, c_ptr, c_i64, c_int, c_i64, c_int, c_f32, c_ptr, c_int, c_f32,
                                         c_int, c_f32, c_ptr, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
 }

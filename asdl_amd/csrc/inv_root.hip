@@ -7,6 +7,8 @@
 // The products run on the split-operand tile kernel (gemm_x3.hpp; small ones on the fp32 tile of gemm_f32.hpp), summed
 // in chunks; the product that forms the next M also folds max |M - I| into a device word and writes the next step's
 // polynomial, and the iterates alternate between two buffer pairs, so a step is its products and one decision kernel.
+#include <cmath>
+#include <cstdlib>
 #include "gemm_f32.hpp"
 #include "gemm_planes.hpp"
 
@@ -30,6 +32,34 @@ inline int g_root_planes_min = 512;
 constexpr int g_root_planes_min = 512;
 #endif
 static bool root_uses_planes(int64_t n) { return n >= g_root_planes_min && n <= kPlaneMaxDim; }
+
+// Scales of the two-plane fp16 form (gemm_planes.hpp).  M, the polynomials T and their powers are bounded by the
+// normalisation of the iteration: ||M_0||_F = (1 + p) / 2, T <= (1 + 1/p) I and T^k <= e for a positive definite
+// statistic, so 2^12 keeps them (and a fair excess of an indefinite input) below the fp16 maximum.  The root is kept
+// without its factor z^(1/p): it grows from I to (z A)^(-1/p) <= lambda_min(M_0)^(-1/p), and the ridge bounds
+// lambda_min(M_0) >= ridge_eps (1 + p) / (2 sqrt(n)) from below (lambda_max from the power iteration; a value that is
+// low by a factor f moves the bound by f^(1/p), which the four spare bits cover).  The root's scale must not be below
+// one (the identity it starts from needs its 22 bits too), so the bound has to stay below 2^12: p = 4 with a ridge
+// of 1e-6 gives 70, p = 2 at the same ridge 8000 and more.  Beyond that, without a ridge, or with a power above 8 the
+// iteration stays on the bf16 planes, which have the range of fp32.
+constexpr float kRootScaleM = 4096.f;
+static bool root_fp16_allowed() {
+  static const bool on = [] {
+    const char* e = std::getenv("ASDL_AMD_ROOT_FP16_PLANES");
+    return e == nullptr || e[0] != '0';
+  }();
+  return on;
+}
+// 0: not on fp16 planes; else the scale of the root's planes
+static float root_fp16_scale(int64_t n, int p, float ridge_eps) {
+  if (!root_fp16_allowed() || !root_uses_planes(n) || p > 8 || !(ridge_eps > 0.f)) return 0.f;
+  const double lam = static_cast<double>(ridge_eps) * (1 + p) / (2.0 * std::sqrt(static_cast<double>(n)));
+  const double bound = std::pow(lam, -1.0 / p);                 // of the root's largest eigenvalue
+  if (!(bound < 1e30)) return 0.f;
+  const int e = 12 - static_cast<int>(std::ceil(std::log2(bound)));
+  if (e < 0) return 0.f;
+  return static_cast<float>(std::ldexp(1.0, e < 12 ? e : 12));
+}
 static int64_t root_pad(int64_t n) { return (n + kPlaneTile - 1) / kPlaneTile * kPlaneTile; }
 // floats of the matrix buffers of one statistic: ten plane sets (two roots, two M, two T, four products) of
 // 3 n_pad^2 bf16, or nine fp32 matrices (two M, the second root, two T, four products)
@@ -257,20 +287,24 @@ static __global__ void newton_gathered_kernel(RootState st) {
 // ---- the same on bf16 planes --------------------------------------------------------------------------------------
 
 // grid (RCHUNKS, batch): planes of M = z S, T = (1 + 1/p) I - M / p and root = z^(1/p) I over the padded index range
-// (zero outside n x n), partial max |M - I|
+// (zero outside n x n), partial max |M - I|.  NP = 2 (fp16 planes): M and T scaled by scale_m, the root without its
+// factor z^(1/p): scale_r I.
+template <int NP>
 static __global__ __launch_bounds__(256) void root_start_planes_kernel(RootState st, const float* __restrict__ S,
                                                                        int64_t strideS, __bf16* __restrict__ M,
                                                                        __bf16* __restrict__ T, __bf16* __restrict__ R,
-                                                                       int64_t set_elems, int64_t n, int64_t n_pad, int p) {
+                                                                       int64_t set_elems, int64_t n, int64_t n_pad, int p,
+                                                                       float scale_m, float scale_r) {
   __shared__ float red[4];
   const int z = blockIdx.y;
   const float zs = st.zscale[z];
-  const float r0 = powf(zs, 1.0f / p);
+  const float r0 = NP == 2 ? scale_r : powf(zs, 1.0f / p);
+  const float sm = NP == 2 ? scale_m : 1.f;
   const float alpha = -1.0f / p;
   const int64_t total = n_pad * n_pad;
-  __bf16* Mz = M + z * set_elems;
-  __bf16* Tz = T + z * set_elems;
-  __bf16* Rz = R + z * set_elems;
+  unsigned short* Mz = reinterpret_cast<unsigned short*>(M) + z * set_elems;
+  unsigned short* Tz = reinterpret_cast<unsigned short*>(T) + z * set_elems;
+  unsigned short* Rz = reinterpret_cast<unsigned short*>(R) + z * set_elems;
   float e = 0.f;
   for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < total; at += RCHUNKS * 256) {
     const int64_t i = at / n_pad, j = at - i * n_pad;
@@ -282,13 +316,17 @@ static __global__ __launch_bounds__(256) void root_start_planes_kernel(RootState
       r = diag ? r0 : 0.f;
       e = fmaxf(e, fabsf(m - (diag ? 1.f : 0.f)));
     }
-    __bf16 h, mid, l;
-    plane_split(m, h, mid, l);
-    Mz[at] = h; Mz[total + at] = mid; Mz[2 * total + at] = l;
-    plane_split(t, h, mid, l);
-    Tz[at] = h; Tz[total + at] = mid; Tz[2 * total + at] = l;
-    plane_split(r, h, mid, l);
-    Rz[at] = h; Rz[total + at] = mid; Rz[2 * total + at] = l;
+    unsigned short o[3];
+    const int64_t dst = plane_index(i, j, n_pad);
+    plane_bits<NP>(m * sm, o);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) Mz[q * total + dst] = o[q];
+    plane_bits<NP>(t * sm, o);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) Tz[q * total + dst] = o[q];
+    plane_bits<NP>(r, o);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) Rz[q * total + dst] = o[q];
   }
   e = wave_max(e);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = e;
@@ -314,18 +352,31 @@ static __global__ __launch_bounds__(256) void newton_gather_planes_kernel(RootSt
   }
 }
 
-// grid (RCHUNKS, batch): the caller's fp32 result from the planes of the root (their sum is exact)
+// grid (RCHUNKS, batch): the caller's fp32 result from the planes of the root (their sum is exact).  NP = 2: the planes
+// hold scale_r times the root without its factor z^(1/p); zscale == nullptr: no such factor (plain product).
+template <int NP>
 static __global__ __launch_bounds__(256) void root_out_planes_kernel(const __bf16* __restrict__ R, int64_t set_elems,
                                                                      float* __restrict__ out, int64_t strideOut,
-                                                                     int64_t n, int64_t n_pad) {
+                                                                     int64_t n, int64_t n_pad, const float* zscale, int p,
+                                                                     float scale_r) {
   const int z = blockIdx.y;
   const int64_t total = n_pad * n_pad;
-  const __bf16* Rz = R + z * set_elems;
-  for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < n * n; at += RCHUNKS * 256) {
-    const int64_t i = at / n, j = at - i * n;
-    const int64_t src = i * n_pad + j;
-    out[z * strideOut + at] = (static_cast<float>(Rz[src]) + static_cast<float>(Rz[total + src])) +
-                              static_cast<float>(Rz[2 * total + src]);
+  if constexpr (NP == 3) {
+    const __bf16* Rz = R + z * set_elems;
+    for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < n * n; at += RCHUNKS * 256) {
+      const int64_t i = at / n, j = at - i * n;
+      const int64_t src = plane_index(i, j, n_pad);
+      out[z * strideOut + at] = (static_cast<float>(Rz[src]) + static_cast<float>(Rz[total + src])) +
+                                static_cast<float>(Rz[2 * total + src]);
+    }
+  } else {
+    const _Float16* Rz = reinterpret_cast<const _Float16*>(R) + z * set_elems;
+    const float mul = (zscale != nullptr ? powf(zscale[z], 1.0f / p) : 1.f) / scale_r;
+    for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < n * n; at += RCHUNKS * 256) {
+      const int64_t i = at / n, j = at - i * n;
+      const int64_t src = plane_index(i, j, n_pad);
+      out[z * strideOut + at] = mul * (static_cast<float>(Rz[src]) + static_cast<float>(Rz[total + src]));
+    }
   }
 }
 
@@ -370,7 +421,11 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
   const int64_t nn = n * n;
   float* w = static_cast<float*>(ws);
   const bool planes = root_uses_planes(n);
-  const int64_t n_pad = root_pad(n), set_elems = 3 * n_pad * n_pad;       // bf16 elements of one plane set
+  // two fp16 planes where the ridge bounds the root, else three bf16 planes; every part of a computation in parts
+  // gets the same ridge_eps and p, hence the same answer
+  const float scale_r = root_fp16_scale(n, p, ridge_eps);
+  const int np = scale_r > 0.f ? 2 : 3;
+  const int64_t n_pad = root_pad(n), set_elems = np * n_pad * n_pad;      // 16-bit elements of one plane set
   float* Mb[2] = {nullptr, nullptr};
   float* root1 = nullptr;
   float* Tb[2] = {nullptr, nullptr};
@@ -423,8 +478,12 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     }
     hipLaunchKernelGGL(root_ridge_kernel, gc, b256, 0, s, st, S, strideS, n, ridge_eps);
     hipLaunchKernelGGL(root_zscale_kernel, gb, dim3(64), 0, s, st, p);
-    if (planes)
-      hipLaunchKernelGGL(root_start_planes_kernel, gc, b256, 0, s, st, S, strideS, pM[0], pT[0], pR[0], set_elems, n, n_pad, p);
+    if (planes && np == 2)
+      hipLaunchKernelGGL(root_start_planes_kernel<2>, gc, b256, 0, s, st, S, strideS, pM[0], pT[0], pR[0], set_elems, n, n_pad,
+                         p, kRootScaleM, scale_r);
+    else if (planes)
+      hipLaunchKernelGGL(root_start_planes_kernel<3>, gc, b256, 0, s, st, S, strideS, pM[0], pT[0], pR[0], set_elems, n, n_pad,
+                         p, 1.f, 1.f);
     else
       hipLaunchKernelGGL(root_start_kernel, gc, b256, 0, s, st, S, strideS, Mb[0], Tb[0], out, strideOut, n, p);
     hipLaunchKernelGGL(root_begin_kernel, gb, dim3(64), 0, s, st, tol, max_iter);
@@ -455,7 +514,12 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
         g.C2 = pptr[next_T];
         g.c2_scale = -1.0f / p; g.c2_diag = 1.0f + 1.0f / p;
       }
-      return launch_plane_gemm(g, batch, s);
+      // fp16 planes: the two roots carry scale_r, every other matrix kRootScaleM
+      const float sa = ia <= R1 ? scale_r : kRootScaleM, sb = ib <= R1 ? scale_r : kRootScaleM;
+      g.in_unscale = 1.0f / (sa * sb);
+      g.c_scale = ic <= R1 ? scale_r : kRootScaleM;
+      g.c2_plane_scale = kRootScaleM;
+      return launch_plane_gemm(g, np, batch, s);
     }
     GemmParams g = make_gemm(0, 0, N, N, N, 1.f, fptr[ia], n, fptr[ib], n, 0.f, fptr[ic], n);
     g.sA = fstride[ia]; g.sB = fstride[ib]; g.sC = fstride[ic];
@@ -547,8 +611,13 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
     hipLaunchKernelGGL(newton_gathered_kernel, gb, dim3(64), 0, s, st);
   }
   // plane form: the caller's fp32 root is written with the statistics (the last part of a computation in parts)
-  if ((phases & 4) && planes)
-    hipLaunchKernelGGL(root_out_planes_kernel, gc, b256, 0, s, pR[0], set_elems, out, strideOut, n, n_pad);
+  if ((phases & 4) && planes) {
+    if (np == 2)
+      hipLaunchKernelGGL(root_out_planes_kernel<2>, gc, b256, 0, s, pR[0], set_elems, out, strideOut, n, n_pad, st.zscale, p,
+                         scale_r);
+    else
+      hipLaunchKernelGGL(root_out_planes_kernel<3>, gc, b256, 0, s, pR[0], set_elems, out, strideOut, n, n_pad, nullptr, p, 1.f);
+  }
   if (phases & 4) hipLaunchKernelGGL(root_stats_kernel, gb, dim3(64), 0, s, st, stats);
   return check_launch();
 }
@@ -561,6 +630,11 @@ extern "C" int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t stride
                                   ak_stream_t stream) {
   return ak::inv_root_run(7, max_iter, S, n, batch, strideS, p, ridge_eps, v0, max_power_iter, power_tol, max_iter, tol,
                           out, strideOut, stats, ws, ws_bytes, stream);
+}
+
+extern "C" int ak_inv_root_plane_format(int64_t n, int p, float ridge_eps) {
+  if (n <= 0 || !ak::root_uses_planes(n)) return 0;
+  return ak::root_fp16_scale(n, p, ridge_eps) > 0.f ? 2 : 3;
 }
 
 extern "C" size_t ak_inv_root_active_offset(int64_t n, int batch) {
@@ -584,9 +658,11 @@ static __global__ void dbg_to_planes_kernel(const float* __restrict__ X, __bf16*
   for (int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; at < total; at += static_cast<int64_t>(gridDim.x) * 256) {
     const int64_t i = at / n_pad, j = at - i * n_pad;
     const float x = (i < n && j < n) ? X[i * n + j] : 0.f;
-    __bf16 h, m, l;
-    plane_split(x, h, m, l);
-    P[at] = h; P[total + at] = m; P[2 * total + at] = l;
+    unsigned short o[3];
+    plane_bits<3>(x, o);
+    unsigned short* Q = reinterpret_cast<unsigned short*>(P);
+    const int64_t dst = plane_index(i, j, n_pad);
+    Q[dst] = o[0]; Q[total + dst] = o[1]; Q[2 * total + dst] = o[2];
   }
 }
 }  // namespace ak
@@ -608,9 +684,9 @@ extern "C" int ak_debug_plane_product(const float* A, const float* B, float* C, 
   g.plane_elems = n_pad * n_pad;
   g.n = static_cast<int>(n); g.n_pad = static_cast<int>(n_pad); g.T = static_cast<int>(n_pad / kPlaneTile);
   g.errword = word;
-  const int rc = launch_plane_gemm(g, 1, nullptr);
+  const int rc = launch_plane_gemm(g, 3, 1, nullptr);
   if (rc != AK_OK) return rc;
-  hipLaunchKernelGGL(root_out_planes_kernel, dim3(RCHUNKS, 1), dim3(256), 0, nullptr, pc, set, C, n * n, n, n_pad);
+  hipLaunchKernelGGL(root_out_planes_kernel<3>, dim3(RCHUNKS, 1), dim3(256), 0, nullptr, pc, set, C, n * n, n, n_pad, nullptr, 1, 1.f);
   hipMemcpy(err, word, 4, hipMemcpyDeviceToHost);
   return check_launch();
 }

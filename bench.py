@@ -630,6 +630,11 @@ def main_shampoo(args, dev):
                                'head frozen), 8 x 1024 uniform random tokens, bf16 autocast forward/backward, '
                                'fp32 statistics and roots', 'batch': bs}}
     if root_records:
+        from asdl_amd import _lib
+
+        def plane_format(n, exp):
+            return int(_lib.load().ak_inv_root_plane_format(n, exp, config.damping))
+
         secs = sum(a.elapsed_time(b) for a, b, _ in root_records) * 1e-3
         flops, executed_flops, iters = 0.0, 0.0, []
         for _, _, stats in root_records:
@@ -638,12 +643,13 @@ def main_shampoo(args, dev):
                 products = 2 + (exp - 1).bit_length()      # root T, T^p by squaring (p a power of two), T^p M
                 f = float(it.sum()) * products * 2.0 * n ** 3
                 flops += f
-                # every fp32 product runs as 6 bf16 piece products; matrices of 512 and up are known to be
-                # symmetric: only the T (T + 1) / 2 tiles of 192 on and above the diagonal of the matrix padded to a
-                # multiple of 192 are computed (the planes kernel)
+                # matrices of 512 and up are known to be symmetric: only the T (T + 1) / 2 tiles of 192 on and above
+                # the diagonal of the matrix padded to a multiple of 192 are computed (the planes kernel), as 3 fp16
+                # piece products per fp32-grade product where the ridge bounds the root (2 planes), else 6 bf16 ones
                 if n >= 512:
                     tiles = -(-n // 192)
-                    executed_flops += float(it.sum()) * products * 6.0 * 2.0 * (tiles * (tiles + 1) / 2) * 192.0 ** 2 * (192.0 * tiles)
+                    pieces = 3.0 if plane_format(n, exp) == 2 else 6.0
+                    executed_flops += float(it.sum()) * products * pieces * 2.0 * (tiles * (tiles + 1) / 2) * 192.0 ** 2 * (192.0 * tiles)
                 else:
                     executed_flops += 6.0 * f
                 iters.append(int(it.max()))
@@ -652,10 +658,11 @@ def main_shampoo(args, dev):
         # bf16 matrix peak the products are executed on; the executed piece products are the labelled extra
         out['roofline'] = {'bound': 'mfma', 'achieved': algorithmic, 'peak': BF16_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
                            'frac': algorithmic / BF16_MFMA_PEAK_TFLOPS, 'traffic': None,
-                           'kernel': 'products of the coupled Newton iteration (plane_gemm_kernel: matrices kept as three '
-                                     'bf16 planes; gemm_x3_kernel / gemm_f32_kernel below 512 columns): 2 n^3 FLOP per '
-                                     'product of the reference; executed_bf16_tflops counts the bf16 MFMA work actually '
-                                     'run (6 piece products per fp32 product, the tiles on and above the diagonal only)',
+                           'kernel': 'products of the coupled Newton iteration (plane_gemm_kernel: matrices kept as two '
+                                     'fp16 planes where the ridge bounds the root, else three bf16 planes; gemm_x3_kernel / '
+                                     'gemm_f32_kernel below 512 columns): 2 n^3 FLOP per product of the reference; '
+                                     'executed_bf16_tflops counts the 16-bit MFMA work actually run (3 fp16 or 6 bf16 piece '
+                                     'products per fp32 product, the tiles on and above the diagonal only)',
                            'executed_bf16_tflops': executed_flops / secs / 1e12,
                            'executed_bf16_frac': executed_flops / secs / 1e12 / BF16_MFMA_PEAK_TFLOPS,
                            'fp32_peak_frac': algorithmic / FP32_MFMA_PEAK_TFLOPS,

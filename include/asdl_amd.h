@@ -356,11 +356,16 @@ int ak_kron_precond_static(const float* Binv, const float* Ainv, float* G, int64
  * below tol, or grows by more than 1.2x (then its previous root is kept), the remaining launches return
  * immediately for it.  stats: device float [batch, 4] = {lambda_max, power iterations, newton iterations,
  * final error}.  n >= 2 (the reference returns the identity for n == 1 without any arithmetic).
- * Statistics of 512 columns and more iterate on three bf16 planes per matrix (the exact split of its fp32 values,
- * written by the product that makes the matrix; 192-wide tiles, n padded to a multiple of 192 in the workspace):
- * ak_inv_root_ws_bytes grows to 60 bytes per padded element and statistic (36 per element below that size).
+ * Statistics of 512 columns and more iterate on 16-bit planes written by the product that makes each matrix
+ * (192-wide tiles, n padded to a multiple of 192 in the workspace): two fp16 planes (22 bits of the power-of-two
+ * scaled value, three matrix instructions per fp32-grade product) where ridge_eps, p and n bound the root's largest
+ * eigenvalue, (ridge_eps (1 + p) / (2 sqrt(n)))^(-1/p), below 4096 and p <= 8; else three bf16 planes (the exact split
+ * of the fp32 value, six matrix instructions).  ak_inv_root_plane_format tells which: 0 = fp32 matrices (n < 512),
+ * 2, 3.  The environment variable ASDL_AMD_ROOT_FP16_PLANES=0 (read once) keeps every statistic on bf16 planes.
+ * ak_inv_root_ws_bytes is 60 bytes per padded element and statistic on planes, 36 per element below that size.
  * Replaces ComputePower / PowerIter / MatPower (asdl/precondition/shampoo.py:465-586). */
 size_t ak_inv_root_ws_bytes(int64_t n, int batch);
+int ak_inv_root_plane_format(int64_t n, int p, float ridge_eps);
 int ak_inv_root_newton(float* S, int64_t n, int batch, int64_t strideS, int p, float ridge_eps,
                        const float* v0, int max_power_iter, float power_tol, int max_iter, float tol,
                        float* out, int64_t strideOut, float* stats, void* ws, size_t ws_bytes,

@@ -11,7 +11,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from asdl_amd import PreconditioningConfig, ShampooGradientMaker, kernels as K, compute_power
+from asdl_amd import PreconditioningConfig, ShampooGradientMaker, kernels as K, compute_power, _lib
 from conftest import GOLDEN
 from models_small import GOLDEN_SHAMPOO, get_mlp
 from oracle import cpu_ref as R
@@ -65,9 +65,10 @@ def test_inv_root_matches_reference_golden():
                                        (520, 4, 2), (1000, 6, 2), (600, 2, 3), (512, 3, 1)])
 def test_inv_root_closed_form(n, p, batch):
     """(S + ridge I)^(-1/p) against the fp64 closed form, the power iteration and the iteration count against the
-    oracle.  Statistics below 512 columns iterate on fp32 matrices, the others on bf16 planes padded to a multiple
-    of 192 (520 -> 576, 1000 -> 1152); p = 6 and p = 3 take the general power sequence (squares and a running
-    product), p = 2, 4, 8 repeated squaring."""
+    oracle.  Statistics below 512 columns iterate on fp32 matrices, the others on 16-bit planes padded to a multiple
+    of 192 (520 -> 576, 1000 -> 1152), here two fp16 planes each (the ridge of 1e-6 bounds the root below 4096; the
+    bf16 planes have their own test below); p = 6 and p = 3 take the general power sequence (squares and a running product),
+    p = 2, 4, 8 repeated squaring."""
     g = torch.Generator().manual_seed(n + p)
     S = torch.empty(batch, n, n)
     for b in range(batch):
@@ -110,19 +111,46 @@ def test_inv_root_polled_and_unpolled_enqueue_give_the_same_result():
     assert torch.equal(r0, r1) and torch.equal(r0, r2)
     assert torch.equal(st0, st1) and torch.equal(st0, st2)
     assert 1 <= float(st0[:, 2].max()) < 100
-    # the same on bf16 planes (576 columns): parts of an odd number of iterations end with the iterates in the second
-    # buffer pair, from which they are brought back before the next part starts
+    # the same on 16-bit planes (576 columns; p = 4: two fp16 planes; p = 2 with a ridge of 1e-7: the ridge does not
+    # bound the root below 4096, three bf16 planes): parts of an odd number of iterations end with the iterates in the second buffer pair,
+    # from which they are brought back before the next part starts
     S = torch.empty(2, 576, 576)
     for b in range(2):
         X = torch.randn(400 * (b + 1), 576, generator=g)
         S[b] = X.T @ X / X.shape[0]
     v0 = (torch.rand(2, 576, generator=g) * 2 - 1).cuda()
-    r0, st0 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=0)
-    r1, st1 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0, poll_every=3)
-    r2, st2 = K.inv_root_newton(S.cuda().clone(), 4, 1e-6, v0)
-    assert torch.equal(r0, r1) and torch.equal(r0, r2)
-    assert torch.equal(st0, st1) and torch.equal(st0, st2)
-    assert 1 <= float(st0[:, 2].max()) < 100
+    for p, eps, planes in ((4, 1e-6, 2), (2, 1e-7, 3)):
+        assert _lib.load().ak_inv_root_plane_format(576, p, eps) == planes
+        r0, st0 = K.inv_root_newton(S.cuda().clone(), p, eps, v0, poll_every=0)
+        r1, st1 = K.inv_root_newton(S.cuda().clone(), p, eps, v0, poll_every=3)
+        r2, st2 = K.inv_root_newton(S.cuda().clone(), p, eps, v0)
+        assert torch.equal(r0, r1) and torch.equal(r0, r2)
+        assert torch.equal(st0, st1) and torch.equal(st0, st2)
+        assert 1 <= float(st0[:, 2].max()) < 100
+
+
+def test_inv_root_plane_formats_and_their_fallbacks():
+    """Which statistics iterate on which storage: fp32 matrices below 512 columns; two fp16 planes where ridge, power
+    and size bound the root's largest eigenvalue below 4096; three bf16 planes else (no ridge, a small ridge with a
+    low power, powers above 8).  A well-conditioned statistic without a ridge (bf16 planes) against the closed form."""
+    fmt = _lib.load().ak_inv_root_plane_format
+    assert fmt(130, 8, 1e-6) == 0 and fmt(511, 4, 1e-6) == 0
+    assert fmt(768, 4, 1e-6) == 2 and fmt(3072, 4, 1e-6) == 2 and fmt(1000, 6, 1e-6) == 2 and fmt(512, 3, 1e-6) == 2
+    assert fmt(600, 2, 1e-6) == 2 and fmt(768, 2, 1e-3) == 2 and fmt(3072, 4, 1e-13) == 2
+    assert fmt(768, 2, 1e-6) == 3 and fmt(3072, 4, 1e-14) == 3
+    assert fmt(768, 4, 0.0) == 3 and fmt(768, 4, 1e-30) == 3 and fmt(768, 10, 1e-6) == 3
+    g = torch.Generator().manual_seed(5)
+    n = 600
+    X = torch.randn(4 * n, n, generator=g)
+    S = (X.T @ X / (4 * n)).unsqueeze(0)
+    v0 = torch.rand(1, n, generator=g) * 2 - 1
+    for p, eps in ((4, 0.0), (4, 1e-6), (2, 1e-7)):
+        assert fmt(n, p, eps) == (2 if eps == 1e-6 else 3)
+        root, stats = K.inv_root_newton(S.cuda().clone(), p, eps, v0.cuda())
+        lam = float(stats[0, 0])
+        w, V = torch.linalg.eigh(S[0].double() + eps * lam * torch.eye(n, dtype=torch.float64))
+        ref = V @ torch.diag(w ** (-1.0 / p)) @ V.T
+        assert relerr(root[0], ref) < 1e-5, (p, eps, relerr(root[0], ref))
 
 
 def test_compute_power_api_and_1x1():
