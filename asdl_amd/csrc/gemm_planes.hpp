@@ -43,6 +43,7 @@ struct PlaneGemm {
   __bf16* C2;               // optional
   float* errword;           // optional, one word per batch entry
   const int* active;        // optional: entry z runs only if active[z] != 0
+  int* overflow;            // optional, fp16 form: word z is set when a value of C or C2 does not fit the fp16 range
   int64_t sA, sB, sC, sC2;  // elements between the plane sets of consecutive batch entries
   int64_t plane_elems;      // n_pad * n_pad
   int n, n_pad, T;          // T = n_pad / kPlaneTile
@@ -96,6 +97,7 @@ __device__ __forceinline__ void plane_epilogue(const PlaneGemm& p, int ti, int t
   const bool off_diag = ti != tj;
   const float unscale = NP == 2 ? p.in_unscale : 1.f, cs = NP == 2 ? p.c_scale : 1.f, c2s = NP == 2 ? p.c2_plane_scale : 1.f;
   float vmax = 0.f;
+  bool fits = true;
   // one 32 x 32 block of the wave; the block numbers are compile-time constants (a loop the compiler does not unroll
   // would index the accumulators with a variable, i.e. keep them in memory)
   auto block = [&](auto a_tag, auto b_tag) {
@@ -112,6 +114,7 @@ __device__ __forceinline__ void plane_epilogue(const PlaneGemm& p, int ti, int t
           const bool inside = gi + e < p.n && gj < p.n, diagonal = gi + e == gj;
           if (inside && (off_diag || gi + e <= gj)) vmax = gemm_fold_absmax(vmax, v, diagonal, 1);
           unsigned short o[3];
+          if constexpr (NP == 2) fits = fits && fabsf(v * cs) <= 65504.f;      // (false for a NaN too)
           plane_bits<NP>(v * cs, o);
           // a diagonal tile keeps its upper triangle and mirrors it element by element: the next product reads
           // this matrix as its own transpose, which it has to be exactly
@@ -126,6 +129,7 @@ __device__ __forceinline__ void plane_epilogue(const PlaneGemm& p, int ti, int t
           }
           if (C2 != nullptr) {
             const float w = p.c2_scale * v + ((diagonal && inside) ? p.c2_diag : 0.f);
+            if constexpr (NP == 2) fits = fits && fabsf(w * c2s) <= 65504.f;
             plane_bits<NP>(w * c2s, o);
 #pragma unroll
             for (int s = 0; s < NP; ++s) {
@@ -153,6 +157,7 @@ __device__ __forceinline__ void plane_epilogue(const PlaneGemm& p, int ti, int t
   block(J1{}, J0{}); block(J1{}, J1{}); block(J1{}, J2{});
   block(J2{}, J0{}); block(J2{}, J1{}); block(J2{}, J2{});
   if (p.errword != nullptr) gemm_store_absmax(p.errword + z, vmax, lane);
+  if (NP == 2 && p.overflow != nullptr && !fits) atomicOr(p.overflow + z, 1);
 }
 
 // One 192 x 192 tile (ti <= tj) of batch entry z.  4 waves (2 x 2), 3 x 3 blocks of 32 x 32 per wave.

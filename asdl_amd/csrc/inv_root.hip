@@ -82,6 +82,7 @@ struct RootState {
   int* count;
   int* par;         // which of the two root / M buffers holds the matrix's latest accepted iterate
   float* errword;   // max |M' - I| of the step under way, folded in by the epilogue of the product that forms M'
+  int* ovf;         // fp16 planes: a product of the step under way left the fp16 range
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -119,6 +120,7 @@ static __global__ __launch_bounds__(256) void root_init_kernel(RootState st, con
     st.count[z] = 0;
     st.par[z] = 0;
     st.errword[z] = 0.f;
+    st.ovf[z] = 0;
   }
 }
 
@@ -246,9 +248,13 @@ static __global__ void newton_decide_kernel(RootState st, float tol, int max_ite
   st.commit[z] = 0;
   const float e = st.errword[z];
   st.errword[z] = 0.f;
+  const int overflow = st.ovf[z];
+  st.ovf[z] = 0;
   if (st.active[z] == 0) return;
   const float err = st.err[z];
-  if (e > err * 1.2f) {          // diverging: keep the previous root (NaN compares false, like the reference)
+  // diverging: keep the previous root (NaN compares false, like the reference).  A step whose products left the range
+  // of the fp16 planes (a statistic far from positive definite) is dropped the same way.
+  if (overflow != 0 || e > err * 1.2f) {
     st.active[z] = 0;
     return;
   }
@@ -390,7 +396,7 @@ static __global__ void root_stats_kernel(RootState st, float* __restrict__ stats
   stats[4 * z + 3] = st.err[z];
 }
 
-static size_t root_state_floats(int batch) { return static_cast<size_t>(batch) * (4 + RCHUNKS + 7) + 16; }
+static size_t root_state_floats(int batch) { return static_cast<size_t>(batch) * (4 + RCHUNKS + 8) + 16; }
 
 }  // namespace ak
 
@@ -465,6 +471,7 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
   st.count = reinterpret_cast<int*>(w); w += batch;
   st.par = reinterpret_cast<int*>(w); w += batch;
   st.errword = w; w += batch;
+  st.ovf = reinterpret_cast<int*>(w); w += batch;
 
   if (reinterpret_cast<unsigned char*>(st.active) != static_cast<unsigned char*>(ws) + root_active_offset(n, batch))
     return AK_ERR_ARG;     // the layout above and root_active_offset() have to agree
@@ -509,6 +516,7 @@ static int inv_root_run(int phases, int iters, float* S, int64_t n, int batch, i
       g.plane_elems = n_pad * n_pad;
       g.n = N; g.n_pad = static_cast<int>(n_pad); g.T = static_cast<int>(n_pad / kPlaneTile);
       g.active = st.active;
+      g.overflow = st.ovf;
       if (next_T >= 0) {
         g.errword = st.errword;
         g.C2 = pptr[next_T];
