@@ -202,17 +202,18 @@ __device__ __forceinline__ void plane_tile(const PlaneGemm& p, int ti, int tj, i
   // one block of one k-tile is 1 KB of consecutive bytes of the plane: block column (6 ti + cb), rows 16 kt ..
   const uint32_t lane_off = static_cast<uint32_t>(lane) * 16u;
   const uint32_t colblock_bytes = static_cast<uint32_t>(p.n_pad) * 64u;
-  auto issue_loads = [&](int kt, int stage) {
+  auto issue_load = [&](int kt, int stage, int l) {
     const uint32_t r = static_cast<uint32_t>(kt * BK) * 64u + lane_off;
+    const int blk = wave + 4 * l;                  // 0 .. 35 = (P * 3 + q) * 6 + cb
+    const int P = blk / 18, q = (blk / 6) % 3, cb = blk % 6;
+    const uint32_t col = static_cast<uint32_t>((P == 0 ? ti : tj) * NCB + cb) * colblock_bytes;
+    // (P differs between the waves of one instruction slot: both descriptors, one select)
+    const u32x4 d = P == 0 ? rsrc[0] : rsrc[1];
+    load_to_lds(d, lds0 + stage * STAGE + blk * BLOCK, kt < nk ? r + q * plane_bytes + col : 0u);
+  };
+  auto issue_loads = [&](int kt, int stage) {
 #pragma unroll
-    for (int l = 0; l < LOADS; ++l) {
-      const int blk = wave + 4 * l;                // 0 .. 35 = (P * 3 + q) * 6 + cb
-      const int P = blk / 18, q = (blk / 6) % 3, cb = blk % 6;
-      const uint32_t col = static_cast<uint32_t>((P == 0 ? ti : tj) * NCB + cb) * colblock_bytes;
-      // (P differs between the waves of one instruction slot: both descriptors, one select)
-      const u32x4 d = P == 0 ? rsrc[0] : rsrc[1];
-      load_to_lds(d, lds0 + stage * STAGE + blk * BLOCK, kt < nk ? r + q * plane_bytes + col : 0u);
-    }
+    for (int l = 0; l < LOADS; ++l) issue_load(kt, stage, l);
   };
 
   floatx16 acc[FR][FC], tot[FR][FC];
@@ -244,12 +245,19 @@ __device__ __forceinline__ void plane_tile(const PlaneGemm& p, int ti, int tj, i
   // The nine matrix instructions of one pair of planes, with the three fragment reads of a group that a later pair
   // needs spread between them (what: 0 none, 1 plane `plane` of A into fa[plane], 2 plane `plane` of B into fb[plane],
   // 3 plane 0 of B into fb0_next).
-  auto pair_step = [&](const bf16x8 (&ca)[FR], const bf16x8 (&cb)[FC], auto what_tag, auto plane_tag, int soff) {
+  // first_load >= 0: loads first_load .. first_load + 2 of k-tile load_kt go out one by one between the matrix
+  // instructions (a wave alone on its SIMD cannot afford the issue time of nine in a row)
+  auto pair_step = [&](const bf16x8 (&ca)[FR], const bf16x8 (&cb)[FC], auto what_tag, auto plane_tag, int soff,
+                       int first_load = -1, int load_kt = 0) {
     constexpr int WHAT = decltype(what_tag)::value, PLANE = decltype(plane_tag)::value;
 #pragma unroll
     for (int m = 0; m < FR * FC; ++m) {
       const int a = m / FC, b = m % FC;
       acc[a][b] = mfma_bf16(ca[a], cb[b], acc[a][b]);
+      if (first_load >= 0 && m % 3 == 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_load(load_kt, load_kt & (S - 1), first_load + m / 3);
+      }
       if (WHAT != 0 && m % 3 == 1) {
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (WHAT == 1) read_a(fa[PLANE], soff, PLANE, m / 3);
@@ -277,11 +285,10 @@ __device__ __forceinline__ void plane_tile(const PlaneGemm& p, int ti, int tj, i
     // done with k-tile kt - 1, whose stage the loads of k-tile kt + 3 fill
     wait_vmcnt<LOADS>();
     __syncthreads();
-    issue_loads(kt + 3, (kt + 3) & (S - 1));
-    pair_step(fa[0], fb[1], I2{}, I2{}, soff);
-    pair_step(fa[0], fb[2], I1{}, I2{}, soff_next);
-    if constexpr (NEXT_B0 == 3) pair_step(fa[0], b0, I3{}, I0{}, soff_next);
-    else pair_step(fa[0], b0, I2{}, I0{}, soff_next);
+    pair_step(fa[0], fb[1], I2{}, I2{}, soff, 0, kt + 3);
+    pair_step(fa[0], fb[2], I1{}, I2{}, soff_next, 3, kt + 3);
+    if constexpr (NEXT_B0 == 3) pair_step(fa[0], b0, I3{}, I0{}, soff_next, 6, kt + 3);
+    else pair_step(fa[0], b0, I2{}, I0{}, soff_next, 6, kt + 3);
   };
 
   issue_loads(0, 0);
@@ -354,16 +361,17 @@ __device__ __forceinline__ void plane_tile_h2(const PlaneGemm& p, int ti, int tj
   // The 24 blocks of a k-tile (operand P, plane q, column block cb) are dealt to the waves round-robin.
   const uint32_t lane_off = static_cast<uint32_t>(lane) * 16u;
   const uint32_t colblock_bytes = static_cast<uint32_t>(p.n_pad) * 64u;
-  auto issue_loads = [&](int kt, int stage) {
+  auto issue_load = [&](int kt, int stage, int l) {
     const uint32_t r = static_cast<uint32_t>(kt * BK) * 64u + lane_off;
+    const int blk = wave + 4 * l;                  // 0 .. 23 = (P * 2 + q) * 6 + cb
+    const int P = blk / 12, q = (blk / 6) % 2, cb = blk % 6;
+    const uint32_t col = static_cast<uint32_t>((P == 0 ? ti : tj) * NCB + cb) * colblock_bytes;
+    const u32x4 d = P == 0 ? rsrc[0] : rsrc[1];
+    load_to_lds(d, lds0 + stage * STAGE + blk * BLOCK, kt < nk ? r + q * plane_bytes + col : 0u);
+  };
+  auto issue_loads = [&](int kt, int stage) {
 #pragma unroll
-    for (int l = 0; l < LOADS; ++l) {
-      const int blk = wave + 4 * l;                // 0 .. 23 = (P * 2 + q) * 6 + cb
-      const int P = blk / 12, q = (blk / 6) % 2, cb = blk % 6;
-      const uint32_t col = static_cast<uint32_t>((P == 0 ? ti : tj) * NCB + cb) * colblock_bytes;
-      const u32x4 d = P == 0 ? rsrc[0] : rsrc[1];
-      load_to_lds(d, lds0 + stage * STAGE + blk * BLOCK, kt < nk ? r + q * plane_bytes + col : 0u);
-    }
+    for (int l = 0; l < LOADS; ++l) issue_load(kt, stage, l);
   };
 
   floatx16 acc[FR][FC], tot[FR][FC];
@@ -392,13 +400,20 @@ __device__ __forceinline__ void plane_tile_h2(const PlaneGemm& p, int ti, int tj
   };
   using f16x8 = _Float16 __attribute__((ext_vector_type(8)));
   // what: 1 plane 0 of A, 2 plane 1 of B (both of this k-tile), 3 plane 1 of A and plane 0 of B of the next k-tile
-  auto pair_step = [&](const bf16x8 (&ca)[FR], const bf16x8 (&cb)[FC], auto what_tag, int soff) {
+  // first_load >= 0: loads first_load .. first_load + 2 of k-tile load_kt go out one by one between the matrix
+  // instructions (a wave alone on its SIMD cannot afford the issue time of six in a row)
+  auto pair_step = [&](const bf16x8 (&ca)[FR], const bf16x8 (&cb)[FC], auto what_tag, int soff, int first_load, int load_kt,
+                       int load_stage) {
     constexpr int WHAT = decltype(what_tag)::value;
 #pragma unroll
     for (int m = 0; m < FR * FC; ++m) {
       const int a = m / FC, b = m % FC;
       acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ca[a]), __builtin_bit_cast(f16x8, cb[b]),
                                                          acc[a][b], 0, 0, 0);
+      if (first_load >= 0 && m % 3 == 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_load(load_kt, load_stage, first_load + m / 3);
+      }
       if (m % 3 == 1) {
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (WHAT == 1) read_a(soff, 0, m / 3);
@@ -434,14 +449,13 @@ __device__ __forceinline__ void plane_tile_h2(const PlaneGemm& p, int ti, int tj
     for (int kt = kt0; kt < kt1; ++kt) {
       const int next = stage + 1 == S ? 0 : stage + 1, fill = stage == 0 ? S - 1 : stage - 1;
       const int soff = stage * STAGE, soff_next = next * STAGE;
-      pair_step(fa[1], fb[0], I1{}, soff);
+      pair_step(fa[1], fb[0], I1{}, soff, -1, 0, 0);
       // k-tile kt + 1 has landed for this wave, then for all; and all waves are done with k-tile kt - 1, whose stage
       // the loads of k-tile kt + S - 1 fill
       wait_vmcnt<(S - 3) * LOADS>();
       __syncthreads();
-      issue_loads(kt + S - 1, fill);
-      pair_step(fa[0], fb[0], I2{}, soff);
-      pair_step(fa[0], fb[1], I3{}, soff_next);
+      pair_step(fa[0], fb[0], I2{}, soff, 0, kt + S - 1, fill);
+      pair_step(fa[0], fb[1], I3{}, soff_next, 3, kt + S - 1, fill);
       stage = next;
     }
 #pragma unroll
