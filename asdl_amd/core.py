@@ -18,13 +18,64 @@ _supported_module_classes = (nn.Linear, nn.Conv2d, nn.BatchNorm1d, nn.BatchNorm2
 __all__ = ['extend', 'no_centered_cov', 'module_wise_assignments', 'modules_to_assign']
 
 
+def _model_fingerprint(model):
+    """What the module-wise assignments depend on: the module tree (identities, in order) and, for every supported
+    leaf, the identities and requires_grad flags of its weight and bias.  ~50 us for a ResNet-50."""
+    ids, flags = [], []
+    stack = [model]
+    while stack:
+        m = stack.pop()
+        ids.append(id(m))
+        if isinstance(m, _supported_module_classes):
+            params = m._parameters
+            w, b = params.get('weight'), params.get('bias')
+            flags.append((id(w), w is not None and w.requires_grad, id(b), b is not None and b.requires_grad))
+        children = m._modules
+        if children:
+            stack.extend(c for c in reversed(children.values()) if c is not None)
+    return tuple(ids), tuple(flags)
+
+
+def _assignment_plan(model, op_names, ignore_modules, map_rule, plan_key):
+    """[(module, op names, operation class)] of extend().  With a ``plan_key`` (a hashable that stands for map_rule)
+    the list of the previous call with the same arguments is reused as long as the model's fingerprint is the same:
+    walking the modules by name and applying the rules costs ten times the fingerprint, once per step."""
+    def build():
+        plan = []
+        for module, names in module_wise_assignments(model, *op_names, ignore_modules=ignore_modules, map_rule=map_rule):
+            if len(names) == 0:
+                continue
+            op_class = get_op_class(module)
+            if op_class is None:
+                continue
+            plan.append((module, [n for n in names if n in op_class.supported_operations], op_class))
+        return plan
+
+    if plan_key is None:
+        return build()
+    try:
+        key = (plan_key, tuple(op_names), tuple(m if isinstance(m, (str, type)) else id(m) for m in ignore_modules or ()))
+        hash(key)
+    except TypeError:
+        return build()
+    cache = model.__dict__.setdefault('_asdl_amd_assignment_plans', {})
+    fingerprint = _model_fingerprint(model)
+    hit = cache.get(key)
+    if hit is not None and hit[0] == fingerprint:
+        return hit[1]
+    plan = build()
+    cache[key] = (fingerprint, plan)
+    return plan
+
+
 @contextmanager
 def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, stream=None,
-           factor_stream=None) -> OperationContext:
+           factor_stream=None, plan_key=None) -> OperationContext:
     """``stream``: as in the reference, the hook operations run under ``torch.cuda.stream(stream)``.
     ``factor_stream``: a kernels.FactorStream; the hook operations launch on its side stream, ordered after the
     kernels that produced their inputs, so that the statistics kernels overlap the forward / backward kernels that
-    follow; OperationContext.join_factor_stream() orders the consumers after them."""
+    follow; OperationContext.join_factor_stream() orders the consumers after them.
+    ``plan_key``: see _assignment_plan (callers whose map_rule is a fixed function of the key)."""
     handles = []
     cxt = OperationContext(vectors=vectors)
     use_stream = torch.cuda.is_available() and stream is not None
@@ -42,14 +93,8 @@ def extend(model, *op_names, ignore_modules=None, map_rule=None, vectors=None, s
         fs.run(fn, *tensors, backward=backward)
 
     try:
-        for module, names in module_wise_assignments(model, *op_names, ignore_modules=ignore_modules, map_rule=map_rule):
-            if len(names) == 0:
-                continue
-            op_class = get_op_class(module)
-            if op_class is None:
-                continue
-            names = [n for n in names if n in op_class.supported_operations]
-            op = op_class(module, names, model_for_kernel=model)
+        for module, names, op_class in _assignment_plan(model, op_names, ignore_modules, map_rule, plan_key):
+            op = op_class(module, list(names), model_for_kernel=model)
             cxt.register_operation(module, op)
             has_fwd = any(n in FWD_OPS for n in names)
             has_bwd = any(n in BWD_OPS for n in names)
@@ -111,7 +156,7 @@ def no_centered_cov(model: nn.Module, shapes, ignore_modules=None, cvp=False, ve
             f'"{SHAPE_UNIT_WISE}" are supported. '
             'Exclude such modules with PreconditioningConfig(ignore_modules=[...]).')
     return extend(model, *shapes, ignore_modules=ignore_modules, map_rule=map_rule, vectors=vectors, stream=stream,
-                  factor_stream=factor_stream)
+                  factor_stream=factor_stream, plan_key=('no_centered_cov', bool(calc_inv)))
 
 
 def named_supported_modules(model):

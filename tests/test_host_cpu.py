@@ -259,6 +259,34 @@ def test_module_selection_by_ignore_list_and_trainability():
         assert list(KfacGradientMaker(model_c, PreconditioningConfig(data_size=1)).module_dict.keys()) == ['0']
 
 
+def test_hooked_modules_follow_the_model_between_steps():
+    """The list of hooked modules is kept between calls of no_centered_cov() and rebuilt when the module tree, a
+    parameter object or a requires_grad flag has changed (the reference walks the modules at every call)."""
+    from asdl_amd.core import no_centered_cov
+    model = nn.Sequential(nn.Linear(3, 3), nn.ReLU(), nn.Linear(3, 3), nn.BatchNorm1d(3))
+
+    def hooked(**kw):
+        with no_centered_cov(model, ['kron'], **kw) as cxt:
+            return [m for m in model.modules() if cxt.is_operation_registered(m) and m is not model]
+
+    assert hooked(ignore_modules=[nn.BatchNorm1d]) == [model[0], model[2]]
+    assert hooked(ignore_modules=[nn.BatchNorm1d]) == [model[0], model[2]]            # from the kept list
+    assert len(model.__dict__['_asdl_amd_assignment_plans']) == 1
+    for p in model[0].parameters():
+        p.requires_grad_(False)
+    assert hooked(ignore_modules=[nn.BatchNorm1d]) == [model[2]]                      # a frozen layer drops out
+    model[0].weight.requires_grad_(True)
+    assert hooked(ignore_modules=[nn.BatchNorm1d]) == [model[0], model[2]]
+    new = nn.Linear(3, 3)
+    model[2] = new                                                                    # a replaced module is picked up
+    assert hooked(ignore_modules=[nn.BatchNorm1d]) == [model[0], new]
+    model[0].weight = nn.Parameter(torch.zeros(3, 3), requires_grad=False)            # a replaced parameter too
+    model[0].bias.requires_grad_(False)
+    assert hooked(ignore_modules=[nn.BatchNorm1d]) == [new]
+    assert hooked(ignore_modules=[new, nn.BatchNorm1d]) == []                         # other arguments, other list
+    assert len(model.__dict__['_asdl_amd_assignment_plans']) == 2
+
+
 def test_config_defaults_match_reference():
     c = PreconditioningConfig()
     assert (c.num_total_steps, c.preconditioner_upd_interval, c.preconditioner_warmup_steps) == (None, 1, 0)
