@@ -13,7 +13,8 @@ algorithmic FLOP M*d*(d+1) per launch summed over the 108 factors of a step, div
 measured with events on the launching stream inside the timed region (on every fourth step, to keep the
 instrumentation's own cost small); `floor_ms_per_step` is the sum of the per-launch roofline floors of the same
 launches.  `roofline_inverse` times the damped Cholesky inverses of the step's factors stand-alone.  `secondary`
-holds brief runs of the single-layer (linear4096) and the fp32 ResNet-18 (resnet18_cifar) configurations.
+holds brief runs of the single-layer (linear4096), the fp32 ResNet-18 (resnet18_cifar) and the Shampoo (shampoo_gpt2)
+configurations.
 `cpu_baseline` times the CPU oracle's K-FAC step (same formulas in PyTorch CPU ops) on the host cores of the same box.
 """
 import argparse
@@ -70,7 +71,7 @@ def parse():
     ap.add_argument('--no-factor-timing', action='store_true')
     ap.add_argument('--no-secondary', action='store_true',
                     help='default workload only: skip the second measurement with the other setting of --inverse-flags '
-                         'and the brief runs of the linear4096 and resnet18_cifar workloads (the `secondary` object)')
+                         'and the brief runs of the linear4096, resnet18_cifar and shampoo_gpt2 workloads (the `secondary` object)')
     ap.add_argument('--no-inverse-roofline', action='store_true',
                     help='skip the stand-alone timing of the damped inverses (the `roofline_inverse` object)')
     ap.add_argument('--factor-launches', choices=['default', 'single', 'grouped'], default='default',
@@ -547,6 +548,12 @@ def main():
             w2.clear()
             del r2
             torch.cuda.empty_cache()
+        # the Shampoo configuration: ten steps, one of them with a root update (every tenth step has one)
+        sh = main_shampoo(args, dev, steps=10, warmup=2, emit=False)
+        secondary['shampoo_gpt2'] = {k: sh[k] for k in ('metric', 'value', 'unit', 'ms_per_step', 'steps', 'warmup', 'dtype',
+                                                        'roofline') if k in sh}
+        del sh
+        torch.cuda.empty_cache()
         out['secondary'] = secondary
     print(json.dumps(out))
 
@@ -570,7 +577,9 @@ def cpu_baseline_resnet18(args):
             'sample': f'one K-FAC step of the CPU oracle (PyTorch CPU ops, {cores} threads) on the full workload took {dt:.1f} s'}
 
 
-def main_shampoo(args, dev):
+def main_shampoo(args, dev, steps=None, warmup=None, emit=True):
+    """The Shampoo workload; emit=False: a brief run for the `secondary` object of the default line (no CPU leg),
+    returned instead of printed."""
     import torch
     import torch.nn.functional as F
     import bench_models
@@ -610,19 +619,21 @@ def main_shampoo(args, dev):
         gm.forward_and_backward()
         opt.step()
 
-    for i in range(args.warmup):
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    for i in range(warmup):
         step()
     del root_records[:]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     out = {
         'metric': 'Shampoo steps/s GPT-2-small decoder, 8x1024 tokens',
-        'value': args.steps / elapsed, 'unit': 'steps/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
-        'ms_per_step': elapsed / args.steps * 1e3, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'value': steps / elapsed, 'unit': 'steps/s', 'n_gpus': 1, 'steps': steps, 'warmup': warmup,
+        'ms_per_step': elapsed / steps * 1e3, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16', 'data': 'synthetic',
         'config': {'workload': 'Shampoo step (L/R statistics and preconditioning of the 49 trainable weight matrices '
                                'every step, inverse 4th roots every 10 steps, epsilon 1e-6) on a 12-layer '
@@ -669,6 +680,8 @@ def main_shampoo(args, dev):
                            'root_updates_timed': len(root_records),
                            'ms_per_root_update': secs / len(root_records) * 1e3,
                            'newton_iterations_max': max(iters)}
+    if not emit:
+        return out
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline_shampoo(args)
     print(json.dumps(out))
