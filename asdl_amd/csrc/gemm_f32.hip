@@ -233,7 +233,7 @@ extern "C" int ak_kron_precond_static(const float* Binv, const float* Ainv, floa
 
 extern "C" int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, int64_t total_tiles,
                                    ak_stream_t stream) {
-  if (pieces != 0 && pieces != 2 && pieces != 3 && pieces != 22) return AK_ERR_ARG;
+  if (pieces != 0 && pieces != 2 && pieces != 3 && pieces != 22 && pieces != 23) return AK_ERR_ARG;
   if (count < 0 || total_tiles < 0 || total_tiles > (1ll << 30)) return AK_ERR_ARG;
   if (count == 0 || total_tiles == 0) return AK_OK;
   if (table == nullptr) return AK_ERR_ARG;
@@ -242,6 +242,7 @@ extern "C" int ak_gemm_f32_grouped(int pieces, const int64_t* table, int count, 
   if (pieces == 0) hipLaunchKernelGGL(ak::gemm_f32_grouped_kernel, grid, dim3(256), 0, s, table, count);
   else if (pieces == 2) hipLaunchKernelGGL(ak::gemm_x3_grouped_kernel<2>, grid, dim3(256), 0, s, table, count);
   else if (pieces == 22) hipLaunchKernelGGL((ak::gemm_x3_grouped_kernel<2, true>), grid, dim3(256), 0, s, table, count);
+  else if (pieces == 23) hipLaunchKernelGGL((ak::gemm_x3_grouped_kernel<2, true, true>), grid, dim3(256), 0, s, table, count);
   else hipLaunchKernelGGL(ak::gemm_x3_grouped_kernel<3>, grid, dim3(256), 0, s, table, count);
   return ak::check_launch();
 }

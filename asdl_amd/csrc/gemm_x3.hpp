@@ -164,14 +164,15 @@ __device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bo
 }
 
 // One 128 x 128 tile (ti, tj) of batch entry z of the product described by p.
-// CHUNKED (three pieces): the products of the leading pieces, which carry the magnitude of the result, have an
+// CHUNKED: the products of the leading pieces, which carry the magnitude of the result, have an
 // accumulator of their own that is added to a running total every 8 k-tiles (256 k: 16 roundings at the magnitude of
-// a chunk, K/256 at the full one); the five cross products, 2^-8 and less of that magnitude, share a second one.
+// a chunk, K/256 at the full one); the cross products (five of three pieces, two of two), 2^-8 and less of that
+// magnitude, share a second one.
 // The sum then carries about one rounding error instead of one that grows with 6 K / 16 accumulator roundings.
 template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool HALF = false, bool CHUNKED = false>
 __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj, int z, AK_LDS3 unsigned char* lds) {
   static_assert(!HALF || (NSPLIT == 2 && !DB), "fp16 pieces: two of them, single-buffered loop");
-  static_assert(!CHUNKED || NSPLIT == 3, "chunked sums: three pieces");
+  static_assert(!CHUNKED || NSPLIT >= 2, "chunked sums: split operands");
   constexpr int BT = X3_BT, BK = X3_BK;
   constexpr int BUF = 2 * NSPLIT * X3_PLANE;        // both operands' planes of one k-tile
   AK_LDS3 unsigned char* panelA = lds;
@@ -250,9 +251,11 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
         for (int b = 0; b < 2; ++b) {
           // smallest terms first
           if constexpr (CHUNKED) {
-            small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], small[a][b]);
-            small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], small[a][b]);
-            small[a][b] = x3_mfma<HALF>(fa[a][2], fb[b][0], small[a][b]);
+            if constexpr (NSPLIT >= 3) {
+              small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], small[a][b]);
+              small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], small[a][b]);
+              small[a][b] = x3_mfma<HALF>(fa[a][2], fb[b][0], small[a][b]);
+            }
             small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][1], small[a][b]);
             small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][0], small[a][b]);
             acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][0], acc[a][b]);
@@ -518,7 +521,7 @@ __device__ __forceinline__ float x3_half_scale(float absmax) {
   return ldexpf(1.f, 14 - e);
 }
 
-template <int NSPLIT, bool HALF = false>
+template <int NSPLIT, bool HALF = false, bool CHUNKED = false>
 static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
   __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
   GemmParams p;
@@ -533,7 +536,7 @@ static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64
   }
   // two work groups per CU with the single-buffered loop serve the mix of long and short contractions of a
   // grouped launch better than one work group with the double-buffered loop (measured: 0.99 against 1.25 ms)
-  gemm_x3_tile<NSPLIT, false, -1, -1, HALF>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
+  gemm_x3_tile<NSPLIT, false, -1, -1, HALF, CHUNKED>(p, ti, tj, 0, (AK_LDS3 unsigned char*)x3_smem);
 }
 
 // The same with true fp32 products (v_mfma_f32_32x32x2_f32, one accumulation per k): 128 x 128 tiles as above.

@@ -100,14 +100,15 @@ def _axis_statistic(grad, axis, out, alpha, beta):
         kernels.syrk_nt(grad.movedim(axis, 0).reshape(grad.shape[axis], -1).contiguous(), out=out, alpha=alpha, beta=beta)
 
 
-HALF_PIECE_STATISTICS = True      # the grouped (large) statistics on two fp16 pieces per element instead of true fp32
-                                  # products: 5.9 -> 4.1 ms per step on the GPT-2-small stack, relative error 2.7e-7
-                                  # (fp32 products: 4.1e-7); the matrix instructions' accumulation leaves the diagonal
-                                  # 2-3 % of a ridge of 1e-6 lambda_max low (fp32 products: 0.3-1 %), and 10 % for
-                                  # the 768-wide statistics, which therefore stay below GROUPED_STATISTIC_MIN_DIM
+HALF_PIECE_STATISTICS = True      # the grouped statistics on two fp16 pieces per element instead of true fp32 products,
+                                  # summed in chunks of 256 k (the leading products in an accumulator of their own that
+                                  # joins a running total): 5.9 -> 2.7 ms per step on the GPT-2-small stack, relative
+                                  # error 2.7e-7 (fp32 products: 4.1e-7).  What the matrix instructions' accumulation
+                                  # leaves the diagonal low: 1-5 % of a ridge of 1e-6 lambda_max (fp32 products:
+                                  # 0.3-1 %; one accumulator for the whole sum: 2-3 % at 2304 columns and up, 10 % at 768)
 HALF_PIECE_PRECONDITION = True     # grouped preconditioning on two fp16 pieces per element (kernels.KronPrecondPlan does the same)
 GROUPED_PRECONDITION = True      # matrix-shaped parameters: all their preconditioning products in two launches
-GROUPED_STATISTIC_MIN_DIM = 1024  # statistics of this size and up go into one grouped launch (with GROUPED_PRECONDITION)
+GROUPED_STATISTIC_MIN_DIM = 768   # statistics of this size and up go into one grouped launch (with GROUPED_PRECONDITION)
 
 
 def _precondition_block(grad, preconditioners):
@@ -295,7 +296,7 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
         """Statistics of every axis (asdl/precondition/shampoo.py:331-339).  The large ones of matrix-shaped
         parameters (GROUPED_STATISTIC_MIN_DIM and up), G G^T or G^T G, run in one grouped launch (lower tiles, mirrored:
         exactly symmetric; the EMA folded into alpha / beta): on two fp16 pieces per element with the gradient's range
-        measured by one pass (HALF_PIECE_STATISTICS), else with true fp32 products.  Small statistics stay on the fp32
+        measured by one pass and sums in chunks (HALF_PIECE_STATISTICS), else with true fp32 products.  Small statistics stay on the fp32
         SYRK kernels, one at a time: the inverse roots of small, ill-conditioned statistics magnify what a different
         summation order changes in the last bits, and the golden runs of the reference pin those."""
         grouped, _ = self._split_groupable()
@@ -326,7 +327,7 @@ class ShampooGradientMaker(PreconditionedGradientMaker):
             if specs:
                 if half:
                     kernels.absmax_grouped(vectors, dev)
-                kernels.gemm_grouped_raw(specs, dev, pieces=22 if half else 0)
+                kernels.gemm_grouped_raw(specs, dev, pieces=23 if half else 0)
         for preconditioner in self.preconditioners:
             preconditioner.update_statistics(skip_axes=done.get(id(preconditioner), ()))
 

@@ -283,10 +283,12 @@ int ak_gemm_f32_split(int pieces, int transA, int transB, int64_t M, int64_t N, 
  * matrix cores (pieces = 2 or 3 as in ak_gemm_f32_split) or with true fp32 products (pieces = 0, the fp32 MFMA, one
  * accumulation per k; needs no alignment), or on two fp16 pieces per element (pieces = 22: 22 significant bits, three
  * partial products; each operand is multiplied by the power of two that brings its largest magnitude, read from the
- * float word absmax_A / absmax_B names, into (2^13, 2^14]).  `table` is DEVICE memory, `count` rows of 16 int64:
+ * float word absmax_A / absmax_B names, into (2^13, 2^14]; pieces = 23: the same, summed in chunks of 256 k: the
+ * products of the leading pieces in an accumulator of their own that joins a running total, which keeps the rounding
+ * of a long sum near that of a single one).  `table` is DEVICE memory, `count` rows of 16 int64:
  *   A, B, C (addresses), lda, ldb, ldc, M, N, K, transA | transB << 1 | symmetric << 2, alpha and beta (float
  *   bit patterns in the low and the high 32 bits), first_tile, absmax_A, absmax_B, absmax_C, 0
- * (absmax_A, absmax_B: addresses of float words, required for pieces = 22, ignored otherwise; absmax_C: 0 or the
+ * (absmax_A, absmax_B: addresses of float words, required for pieces = 22 and 23, ignored otherwise; absmax_C: 0 or the
  * address of a float word into which the split kernels fold max |C_i| by an integer atomic maximum on the bit pattern:
  * zero it first)
  * (symmetric: M == N and op(A) op(B) is symmetric, e.g. G G^T: only the tiles on and below the diagonal are
