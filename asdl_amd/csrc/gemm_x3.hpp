@@ -166,8 +166,9 @@ __device__ __forceinline__ bf16x8 x3_frag(AK_LDS3 const unsigned char* plane, bo
 // One 128 x 128 tile (ti, tj) of batch entry z of the product described by p.
 // CHUNKED: the products of the leading pieces, which carry the magnitude of the result, have an
 // accumulator of their own that is added to a running total every 8 k-tiles (256 k: 16 roundings at the magnitude of
-// a chunk, K/256 at the full one); the cross products (five of three pieces, two of two), 2^-8 and less of that
-// magnitude, share a second one.
+// a chunk, K/256 at the full one); the five cross products of three pieces, 2^-8 and less of that magnitude, share a
+// second one (with two pieces the two cross products stay with the leading one: a third set of accumulators would
+// halve the work groups per CU).
 // The sum then carries about one rounding error instead of one that grows with 6 K / 16 accumulator roundings.
 template <int NSPLIT, bool DB, int AKC = -1, int BKC = -1, bool HALF = false, bool CHUNKED = false>
 __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj, int z, AK_LDS3 unsigned char* lds) {
@@ -204,15 +205,18 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  constexpr int TT = CHUNKED ? 2 : 1;
-  floatx16 small[TT][TT], tot[TT][TT];
+  constexpr int TT = CHUNKED ? 2 : 1, TS = (CHUNKED && NSPLIT >= 3) ? 2 : 1;
+  floatx16 small[TS][TS], tot[TT][TT];
   if constexpr (CHUNKED) {
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) small[a][b][r] = tot[a][b][r] = 0.f;
+        for (int r = 0; r < 16; ++r) {
+          tot[a][b][r] = 0.f;
+          if constexpr (NSPLIT >= 3) small[a][b][r] = 0.f;
+        }
   }
   // end of k-tile kt: every eighth one moves the leading products' accumulators into the running total
   auto end_of_ktile = [&](int kt) {
@@ -250,12 +254,10 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
           // smallest terms first
-          if constexpr (CHUNKED) {
-            if constexpr (NSPLIT >= 3) {
-              small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], small[a][b]);
-              small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], small[a][b]);
-              small[a][b] = x3_mfma<HALF>(fa[a][2], fb[b][0], small[a][b]);
-            }
+          if constexpr (CHUNKED && NSPLIT >= 3) {
+            small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][1], small[a][b]);
+            small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][2], small[a][b]);
+            small[a][b] = x3_mfma<HALF>(fa[a][2], fb[b][0], small[a][b]);
             small[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][1], small[a][b]);
             small[a][b] = x3_mfma<HALF>(fa[a][1], fb[b][0], small[a][b]);
             acc[a][b] = x3_mfma<HALF>(fa[a][0], fb[b][0], acc[a][b]);
@@ -394,7 +396,10 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
 #pragma unroll
       for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] = (tot[a][b][r] + acc[a][b][r]) + small[a][b][r];
+        for (int r = 0; r < 16; ++r) {
+          acc[a][b][r] = tot[a][b][r] + acc[a][b][r];
+          if constexpr (NSPLIT >= 3) acc[a][b][r] += small[a][b][r];
+        }
   }
 
   // the partial products of (i, j) and (j, i) are summed in different orders, so a mirrored result takes both
@@ -522,7 +527,7 @@ __device__ __forceinline__ float x3_half_scale(float absmax) {
 }
 
 template <int NSPLIT, bool HALF = false, bool CHUNKED = false>
-static __global__ __launch_bounds__(256) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
+static __global__ __launch_bounds__(256, 2) void gemm_x3_grouped_kernel(const int64_t* __restrict__ table, int count) {
   __shared__ __attribute__((aligned(16))) unsigned char x3_smem[2 * NSPLIT * X3_PLANE];
   GemmParams p;
   int ti, tj;

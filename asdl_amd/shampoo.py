@@ -102,7 +102,7 @@ def _axis_statistic(grad, axis, out, alpha, beta):
 
 HALF_PIECE_STATISTICS = True      # the grouped statistics on two fp16 pieces per element instead of true fp32 products,
                                   # summed in chunks of 256 k (the leading products in an accumulator of their own that
-                                  # joins a running total): 5.9 -> 2.7 ms per step on the GPT-2-small stack, relative
+                                  # joins a running total): 5.9 -> 1.9 ms per step on the GPT-2-small stack, relative
                                   # error 2.7e-7 (fp32 products: 4.1e-7).  What the matrix instructions' accumulation
                                   # leaves the diagonal low: 1-5 % of a ridge of 1e-6 lambda_max (fp32 products:
                                   # 0.3-1 %; one accumulator for the whole sum: 2-3 % at 2304 columns and up, 10 % at 768)
