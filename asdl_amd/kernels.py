@@ -520,6 +520,7 @@ class GroupedCall:
     def begin():
         """Call before the factor call that is to be remembered."""
         _group.last = None
+        _group.last_direct = None
 
     @classmethod
     def remember(cls, x, out, extra=None):
@@ -556,6 +557,56 @@ class GroupedCall:
         row = list(self.row)
         row[1] = ptr
         grp.add(row, self.flops, self.floor, x, self.out)
+        return True
+
+
+class DirectCall:
+    """A factor call that was launched at once (no group took it), remembered by its caller like a GroupedCall: the
+    library function and its argument list, the workspace it needs, FLOP count and floor.  again() launches it on a
+    tensor of the same shape, strides, type and alignment without going through conv_syrk() again."""
+    __slots__ = ('shape', 'stride', 'dtype', 'device', 'align', 'name', 'fn', 'args', 'need', 'out', 'flops', 'floor',
+                 'timed', 'extra')
+
+    @staticmethod
+    def note(name, fn, args, need, x, out, flops, floor):
+        """Called by the factor function right before its launch: args[0] is x's address, args[-3:] are the
+        workspace, its size and the stream."""
+        _group.last_direct = (name, fn, args, need, x.data_ptr(), out, flops, floor)
+
+    @classmethod
+    def remember(cls, x, out, extra=None):
+        last = getattr(_group, 'last_direct', None)
+        _group.last_direct = None
+        if last is None:
+            return None
+        name, fn, args, need, ptr, out_used, flops, floor = last
+        if ptr != x.data_ptr() or out_used is not out:
+            return None          # the call read a converted or rearranged copy of x
+        rec = cls()
+        rec.shape, rec.stride, rec.dtype, rec.device = x.shape, x.stride(), x.dtype, x.device
+        rec.align = ptr & 15
+        rec.name, rec.fn, rec.args, rec.need, rec.out, rec.flops, rec.floor = name, fn, list(args), need, out, flops, floor
+        rec.timed = _timing_sink is not None
+        rec.extra = extra
+        return rec
+
+    def again(self, x, extra=None):
+        grp = getattr(_group, 'active', None)
+        if grp is not None and not grp.plain_only:
+            return False         # a group that takes every kind of row is open: the factor function decides
+        if x.dtype is not self.dtype or x.shape != self.shape or x.stride() != self.stride or x.device != self.device \
+                or extra != self.extra or (_timing_sink is not None) != self.timed:
+            return False
+        ptr = x.data_ptr()
+        if ptr & 15 != self.align:
+            return False
+        args = self.args
+        args[0] = ctypes.c_void_p(ptr)
+        args[-3], args[-2], keep = _ws_args(self.need, x.device)
+        args[-1] = _stream()
+        with _Timed(self.name, self.flops, floor=self.floor):
+            rc = self.fn(*args)
+        _lib.check(rc, self.name)
         return True
 
 
@@ -663,12 +714,13 @@ def conv_syrk(x, kernel_size, stride, padding, out=None, alpha=1.0, beta=0.0, ro
                 return out
         need = _ws_need('ak_conv_syrk_nhwc_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)
         ws, ws_bytes, keep = _ws_args(need, x.device)
+        args = [ctypes.c_void_p(x.data_ptr()), code, N, C, H, W, kh, kw, sh, sw, ph, pw, alpha, beta,
+                ctypes.c_void_p(out.data_ptr()), out.stride(0), ws, ws_bytes, _stream()]
         with _Timed('conv_syrk', flops, floor=floor):
-            rc = lib.ak_conv_syrk_nhwc(ctypes.c_void_p(x.data_ptr()), code, N, C, H, W, kh, kw, sh, sw,
-                                       ph, pw, alpha, beta, ctypes.c_void_p(out.data_ptr()), out.stride(0),
-                                       ws, ws_bytes, _stream())
+            rc = lib.ak_conv_syrk_nhwc(*args)
         if rc != AK_ERR_UNSUPPORTED:
             _lib.check(rc, 'ak_conv_syrk_nhwc')
+            DirectCall.note('conv_syrk', lib.ak_conv_syrk_nhwc, args, need, x, out, flops, floor)
             return out
     x = _contiguous(x)
     need = _ws_need('ak_conv_syrk_ws_bytes', N, C, H, W, kh, kw, sh, sw, ph, pw)

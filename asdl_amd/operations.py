@@ -162,14 +162,14 @@ class Operation:
         return buf
 
     def _remembered_call(self, key, tmp_key, raw, first):
-        """The grouped factor call that this module's hook made on the previous pass, made again on ``raw`` (see
-        kernels.GroupedCall): True when the group has taken it.  Only the square scratch factors of the *_INV
+        """The factor call that this module's hook made on the previous pass, made again on ``raw`` (see
+        kernels.GroupedCall, kernels.DirectCall): True when the group has taken it or it has been launched.  Only the square scratch factors of the *_INV
         operations are remembered; whatever differs from the remembered call goes through _factor_inv_mode()."""
         cache = getattr(self._module, _FACTOR_CACHE_ATTR, None)
         rec = cache.get('call' + key) if cache is not None else None
         if rec is None or cache.get(key) is not rec.out:
             return False
-        if not rec.again(raw, (self._geometry(), self._cov_scale, first)):
+        if not rec.again(raw, (self._geometry(), self._cov_scale, first, _autocast_rounds(raw))):
             return False
         self._op_results[tmp_key] = rec.out
         self._op_results['_eig_scale_' + key] = 1.0
@@ -200,8 +200,11 @@ class Operation:
                 kernels.GroupedCall.begin()
             square_fn(buf, self._cov_scale, 0.0 if first else 1.0)
             if remember:
-                getattr(self._module, _FACTOR_CACHE_ATTR)['call' + key] = \
-                    kernels.GroupedCall.remember(raw, buf, (self._geometry(), self._cov_scale, first))
+                extra = (self._geometry(), self._cov_scale, first, _autocast_rounds(raw))
+                rec = kernels.GroupedCall.remember(raw, buf, extra)
+                if rec is None:
+                    rec = kernels.DirectCall.remember(raw, buf, extra)      # launched at once: that launch, then
+                getattr(self._module, _FACTOR_CACHE_ATTR)['call' + key] = rec
             self._op_results['_eig_scale_' + key] = 1.0 / self._cov_scale if swift else 1.0
         if slot is None:
             self._op_results[tmp_key] = buf

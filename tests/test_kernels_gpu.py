@@ -320,6 +320,36 @@ def test_conv_syrk_channels_last_ema_accumulate(K):
     assert relerr(out, ref) < TOL_FACTOR_F32
 
 
+@pytest.mark.parametrize('C,H', [(64, 14), (16, 12)])     # shifted correlations; the gathered kernel
+def test_remembered_direct_launch_repeats_the_factor_call(K, C, H):
+    """kernels.DirectCall: a hook remembers the library call its factor function made and repeats it on the tensor
+    of the next pass (another address, other values) without going through conv_syrk(): the same factor as a fresh
+    call bit for bit, and no launch at all for a tensor that would not give the same call."""
+    xs = [_inputs((4, C, H, H), torch.bfloat16, seed).cuda().contiguous(memory_format=torch.channels_last) for seed in (3, 4)]
+    out = torch.empty(9 * C, 9 * C, device='cuda')
+    K.GroupedCall.begin()
+    K.conv_syrk(xs[0], (3, 3), (1, 1), (1, 1), out=out, alpha=0.25, beta=0.0)
+    assert K.DirectCall.remember(xs[0].clone(), out, 'same') is None         # not the tensor the call read
+    K.GroupedCall.begin()
+    K.conv_syrk(xs[0], (3, 3), (1, 1), (1, 1), out=out, alpha=0.25, beta=0.0)
+    assert K.DirectCall.remember(xs[0], torch.empty_like(out), 'same') is None      # not the buffer it wrote
+    K.GroupedCall.begin()
+    K.conv_syrk(xs[0], (3, 3), (1, 1), (1, 1), out=out, alpha=0.25, beta=0.0)
+    rec = K.DirectCall.remember(xs[0], out, 'same')
+    assert rec is not None and K.DirectCall.remember(xs[0], out, 'same') is None    # a note is taken once
+    first = out.clone()
+    assert rec.again(xs[1], 'same')
+    fresh = K.conv_syrk(xs[1], (3, 3), (1, 1), (1, 1), alpha=0.25)
+    assert torch.equal(out, fresh) and not torch.equal(out, first)
+    out.fill_(-1.0)
+    assert not rec.again(xs[1], 'other')                                       # the caller's own state differs
+    assert not rec.again(xs[1][:2], 'same')                                    # another shape
+    assert not rec.again(xs[1].float(), 'same')                                # another type
+    assert not rec.again(xs[1].contiguous(), 'same')                           # other strides (NCHW)
+    assert float(out.min()) == -1.0 and float(out.max()) == -1.0               # none of them launched anything
+    assert rec.again(xs[0], 'same') and torch.equal(out, first)
+
+
 @pytest.mark.parametrize('M,d,ld', [(4096, 64, 64), (20000, 64, 64), (3000, 1000, 1000), (777, 256, 320),
                                     (100000, 128, 128), (33, 2048, 2048), (3000, 1600, 1600), (1500, 2560, 2568)])
 def test_syrk_tn_bf16_split_k_and_strided(K, M, d, ld):
