@@ -255,8 +255,8 @@ class FisherMaker(GradientMaker):
 
     def _extract_fisher(self, cxt: OperationContext):
         attr = self.config.fisher_attr
-        for module in self.model.modules():
-            if getattr(module, attr, None) is None and cxt.is_operation_registered(module):
+        for module in cxt.registered_modules():       # (in the order of model.modules(), which registered them)
+            if getattr(module, attr, None) is None:
                 fisher = cxt.cov_symmatrix(module, pop=True)
                 if fisher is not None:
                     setattr(module, attr, fisher)

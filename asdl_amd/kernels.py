@@ -189,7 +189,11 @@ def device_ptr_array(tensors):
     if arr is None:
         if len(_ptr_cache) > 4096:
             _ptr_cache.clear()
-        arr = torch.tensor(ptrs, dtype=torch.int64).to(dev)
+        # staged through pinned memory and copied asynchronously on the launch stream, like device_table(): a
+        # pageable copy would block the caller behind everything that stream has queued
+        host = torch.tensor(ptrs, dtype=torch.int64).pin_memory()
+        with _on_launch_stream():
+            arr = host.to(dev, non_blocking=True)
         _ptr_cache[key] = arr
     return arr
 

@@ -322,24 +322,31 @@ class NaturalGradientMaker(PreconditionedGradientMaker):
             raise
 
     def _save_gradients(self, grads):
-        """Copies of ``grads`` in one reusable buffer (one launch per dtype and device)."""
+        """Copies of ``grads`` in one reusable buffer (one launch per dtype and device).  The views into the buffer
+        depend on the gradients' shapes, types and devices only and are kept from step to step."""
         if not grads:
             return []
-        views, buffers = [], getattr(self, '_grad_backup', None)
-        if buffers is None:
-            buffers = self._grad_backup = {}
-        need = {}
-        for g in grads:
-            key = (g.dtype, g.device)
-            need[key] = need.get(key, 0) + g.numel()
-        for key, n in need.items():
-            if key not in buffers or buffers[key].numel() < n:
-                buffers[key] = torch.empty(n, dtype=key[0], device=key[1])
-        used = dict.fromkeys(need, 0)
-        for g in grads:
-            key = (g.dtype, g.device)
-            views.append(buffers[key][used[key]:used[key] + g.numel()].view(g.shape))
-            used[key] += g.numel()
+        key = tuple((g.shape, g.dtype, g.device) for g in grads)
+        memo = getattr(self, '_grad_backup_views', None)
+        if memo is None or memo[0] != key:
+            buffers = getattr(self, '_grad_backup', None)
+            if buffers is None:
+                buffers = self._grad_backup = {}
+            need = {}
+            for g in grads:
+                k = (g.dtype, g.device)
+                need[k] = need.get(k, 0) + g.numel()
+            for k, n in need.items():
+                if k not in buffers or buffers[k].numel() < n:
+                    buffers[k] = torch.empty(n, dtype=k[0], device=k[1])
+            used = dict.fromkeys(need, 0)
+            views = []
+            for g in grads:
+                k = (g.dtype, g.device)
+                views.append(buffers[k][used[k]:used[k] + g.numel()].view(g.shape))
+                used[k] += g.numel()
+            memo = self._grad_backup_views = (key, views)
+        views = memo[1]
         torch._foreach_copy_(views, grads)
         return views
 

@@ -596,6 +596,9 @@ class OperationContext:
     def is_operation_registered(self, module):
         return module in self._operations
 
+    def registered_modules(self):
+        return list(self._operations)
+
     def register_operation(self, module, operation):
         operation._context = self
         self._operations[module] = operation
