@@ -4,9 +4,11 @@
 // test evaluated on the device.  The host enqueues the maximum number of iterations; each kernel
 // first reads its matrix's `active` word and returns at once when that matrix has converged (or
 // stopped because its error grew by more than 1.2x, in which case the previous root is kept).
-// The products run on the split-operand tile kernel (gemm_x3.hpp; small ones on the fp32 tile of gemm_f32.hpp), summed
-// in chunks; the product that forms the next M also folds max |M - I| into a device word and writes the next step's
-// polynomial, and the iterates alternate between two buffer pairs, so a step is its products and one decision kernel.
+// Statistics of 512 columns and more keep every matrix of the iteration as 16-bit planes and multiply them with the
+// plane kernel (gemm_planes.hpp); smaller ones keep fp32 matrices and run on the split-operand tile kernel (gemm_x3.hpp)
+// or the fp32 tile of gemm_f32.hpp.  All sum in chunks; the product that forms the next M also folds max |M - I| into a
+// device word and writes the next step's polynomial, and the iterates alternate between two buffer pairs, so a step is
+// its products and one decision kernel.
 #include <cmath>
 #include <cstdlib>
 #include "gemm_f32.hpp"
