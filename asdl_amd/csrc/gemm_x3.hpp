@@ -377,13 +377,23 @@ __device__ __forceinline__ void gemm_x3_tile(const GemmParams& p, int ti, int tj
       }
     } else {
       __syncthreads();
-      for (int kt = 0; kt < nk; ++kt) {
+      auto one_ktile = [&](int kt) {
         if (kt + 1 < nk) fetch(kt + 1);       // next k-tile's global loads fly during this one's MFMAs
         multiply(lds);
-        end_of_ktile(kt);
         __syncthreads();                      // everybody is done reading this k-tile
         if (kt + 1 < nk) stash(lds);
         __syncthreads();
+      };
+      if constexpr (CHUNKED) {
+        // two nested loops: with one loop and a conditional flush the compiler evaluates the flush (a move and an
+        // addition per accumulator register) at every k-tile and selects
+        for (int kt0 = 0; kt0 < nk; kt0 += 8) {
+          const int kt1 = kt0 + 8 < nk ? kt0 + 8 : nk;
+          for (int kt = kt0; kt < kt1; ++kt) one_ktile(kt);
+          end_of_ktile(7);
+        }
+      } else {
+        for (int kt = 0; kt < nk; ++kt) one_ktile(kt);
       }
     }
   };
